@@ -1,0 +1,72 @@
+"""Page ids of one pool: who is free, who is taken.
+
+As in the reference (src/engine/block_manager.cpp:17-127) the free ids form a LIFO stack that
+first hands out 0, 1, 2, ... and hands a freed id out again next, a map of taken ids catches a
+second free or a foreign id, and taking several pages is all or nothing.
+"""
+from __future__ import annotations
+
+from typing import Iterable, List
+
+
+class OutOfPages(RuntimeError):
+    pass
+
+
+class PageError(RuntimeError):
+    """A page id that is out of range, freed twice, or freed without having been taken."""
+
+
+class BlockManager:
+    def __init__(self, num_pages: int):
+        if num_pages < 0:
+            raise ValueError(f"num_pages must not be negative, got {num_pages}")
+        self.num_pages = int(num_pages)
+        self._free: List[int] = list(range(self.num_pages - 1, -1, -1))  # pop() gives 0 first
+        self._taken = [False] * self.num_pages
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    @property
+    def num_taken(self) -> int:
+        return self.num_pages - len(self._free)
+
+    def utilization(self) -> float:
+        return self.num_taken / self.num_pages if self.num_pages else 0.0
+
+    def can_allocate(self, n: int) -> bool:
+        return n <= len(self._free)
+
+    def allocate(self, n: int) -> List[int]:
+        if n < 0:
+            raise ValueError(f"cannot take {n} pages")
+        if n > len(self._free):
+            raise OutOfPages(f"{n} pages wanted, {len(self._free)} of {self.num_pages} free")
+        out = []
+        for _ in range(n):
+            p = self._free.pop()
+            self._taken[p] = True
+            out.append(p)
+        return out
+
+    def free(self, pages: Iterable[int]) -> None:
+        pages = list(pages)
+        seen = set()
+        for p in pages:  # check all before changing anything
+            if not isinstance(p, int) or not 0 <= p < self.num_pages:
+                raise PageError(f"page id {p!r} is outside 0..{self.num_pages - 1}")
+            if not self._taken[p] or p in seen:
+                raise PageError(f"page {p} is freed twice or was never taken")
+            seen.add(p)
+        for p in pages:
+            self._taken[p] = False
+            self._free.append(p)
+
+    def is_taken(self, page: int) -> bool:
+        return self._taken[page]
+
+    def reset(self) -> None:
+        self._free = list(range(self.num_pages - 1, -1, -1))
+        self._taken = [False] * self.num_pages

@@ -1,0 +1,70 @@
+"""The description of a model as data: parts, their parameters, and the order they run in.
+
+An architecture's builder turns its typed configuration into a :class:`ModelSpec`.  Nothing in
+a spec names the architecture it came from: a part is ``kind`` (a key of a part registry) plus
+``params`` (its sizes and constants) plus ``weights`` (logical weight name -> tensor name in the
+checkpoint).  The reference wires these by hand for one model (src/model/llama.cpp:398-412,
+568-706); here the wiring is a value that another builder can fill differently, layer by layer.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional
+
+
+@dataclass
+class PartSpec:
+    """One part: which implementation (``kind``), with which constants, fed by which tensors."""
+
+    kind: str
+    params: Dict[str, Any] = field(default_factory=dict)
+    weights: Dict[str, str] = field(default_factory=dict)
+
+
+@dataclass
+class BlockSpec:
+    """A residual block: how a mixer and a feed-forward are arranged around the residual stream.
+
+    ``kind`` chooses the arrangement (``"prenorm"``: x + mixer(norm(x)), then x + ffn(norm(x)),
+    src/model/llama.cpp:324-379).
+    """
+
+    kind: str
+    mixer_norm: PartSpec
+    mixer: PartSpec
+    ffn_norm: PartSpec
+    ffn: PartSpec
+
+
+@dataclass
+class LayerRun:
+    """One entry of the execution order: run block ``block`` on cache ``cache``.
+
+    A block may appear in several entries (its weights are used again); ``cache`` is the index
+    of the per-layer cache it reads, and writes when ``writes_cache`` holds.  An entry with
+    ``writes_cache=False`` reads what an earlier entry with the same ``cache`` wrote.
+    """
+
+    block: int
+    cache: int
+    writes_cache: bool = True
+
+
+@dataclass
+class ModelSpec:
+    vocab_size: int
+    hidden_size: int
+    max_positions: int
+    embedding: PartSpec
+    blocks: List[BlockSpec]
+    order: List[LayerRun]
+    final_norm: PartSpec
+    head: PartSpec
+    bos_token_id: Optional[int] = None
+    eos_token_ids: tuple = ()
+    # tensor name -> name of the tensor it may merely repeat (a tied head stored a second time);
+    # such a tensor is accepted in a checkpoint when it equals the original and is not loaded
+    duplicates: Dict[str, str] = field(default_factory=dict)
+
+    def num_caches(self) -> int:
+        return 1 + max((r.cache for r in self.order), default=-1)

@@ -1,0 +1,239 @@
+// Attention over the paged key/value cache, one query token at a time, for gfx950.
+// Compiled once per head size (-DHEAD_DIM=n, a multiple of 16 up to 256).
+//
+// A work item is (query token, kv head, chunk of the query heads that share it, split of the
+// key range).  The 256 threads of a workgroup are arranged as key slots x dimension lanes:
+// LPK consecutive lanes hold one key row between them (EPL dims each), so a wavefront reads
+// 64/LPK whole rows per access, which are adjacent in a pool laid out
+// [page, kv_head, slot_in_page, head_dim].  Every lane group keeps a running (max, sum, output)
+// of its own for each query head; they are merged across the wave by shuffles, across waves
+// through LDS and across splits by a second kernel.  Softmax and both products are float32.
+//
+// Formula (reference: src/op/kernels/cuda/paged_attention_kernel.cu:111-199 for one token,
+// src/op/kernels/cuda/prefill_attention_kernel.cu:66-141 for a chunk): the query at position P
+// reads keys max(0, P+1-window)..P of its sequence through the block table, head h uses kv head
+// h / (H/KVH), scores are scaled by `scale`, softmax subtracts the maximum and divides by the
+// plain sum.  A prompt portion is handled as its tokens one by one: each reads the cache, which
+// the step has already filled up to and including that token.
+#include "common.h"
+
+#ifndef HEAD_DIM
+#error "HEAD_DIM must be defined"
+#endif
+static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256, "head size: multiple of 16, at most 256");
+
+#define ATT_THREADS 256
+#define GT 4  // query heads handled together by one workgroup
+
+template <typename T> struct Lanes {
+    static constexpr int per16 = 16 / sizeof(T);                 // elements in a 16-byte access
+    static constexpr int want = (HEAD_DIM + per16 - 1) / per16;  // lanes if each took 16 bytes
+    static constexpr int LPK = want <= 1 ? 1 : want <= 2 ? 2 : want <= 4 ? 4 : want <= 8 ? 8 : 16;
+    static constexpr int EPL = HEAD_DIM / LPK;
+    static_assert(LPK * EPL == HEAD_DIM, "lanes x elements must cover a head");
+    static constexpr int KPI = ATT_THREADS / LPK;  // keys per workgroup iteration
+};
+
+__device__ __forceinline__ float scale_of(float m, float m_new) { return m == -INFINITY ? 0.f : expf(m - m_new); }
+
+template <typename T>
+__global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
+    const T* __restrict__ q, int q_stride, const T* __restrict__ kpool, const T* __restrict__ vpool,
+    const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ seq_of_token,
+    const int32_t* __restrict__ positions, T* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int H, int KVH, int page_size, int window, float scale, int nsplit) {
+    using L = Lanes<T>;
+    constexpr int LPK = L::LPK, EPL = L::EPL, KPI = L::KPI, HD = HEAD_DIM;
+    constexpr int WAVES = ATT_THREADS / WAVE;
+
+    const int t = blockIdx.x;
+    const int G = H / KVH;
+    const int chunks = (G + GT - 1) / GT;
+    const int g = blockIdx.y / chunks;
+    const int chunk = blockIdx.y % chunks;
+    const int h0 = g * G + chunk * GT;
+    const int gc = min(GT, G - chunk * GT);
+    const int split = blockIdx.z;
+
+    const int pos = positions[t];
+    const int seq = seq_of_token[t];
+    const int hi = pos + 1;
+    const int lo = window > 0 ? max(0, hi - window) : 0;
+    const int per_split = (hi - lo + nsplit - 1) / nsplit;
+    const int k0 = lo + split * per_split;
+    const int k1 = min(hi, k0 + per_split);
+
+    const int tid = threadIdx.x;
+    const int sub = tid % LPK;
+    const int kslot = tid / LPK;
+    const int32_t* table = block_table + static_cast<size_t>(seq) * table_stride;
+
+    float qreg[GT][EPL];
+#pragma unroll
+    for (int i = 0; i < GT; ++i) {
+        if (i < gc) {
+            VecIO<T, EPL>::load(q + static_cast<size_t>(t) * q_stride + static_cast<size_t>(h0 + i) * HD + sub * EPL, qreg[i]);
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) qreg[i][e] *= scale;
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) qreg[i][e] = 0.f;
+        }
+    }
+
+    float m[GT], l[GT], acc[GT][EPL];
+#pragma unroll
+    for (int i = 0; i < GT; ++i) {
+        m[i] = -INFINITY;
+        l[i] = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) acc[i][e] = 0.f;
+    }
+
+    const int iters = (k1 > k0) ? (k1 - k0 + KPI - 1) / KPI : 0;
+    for (int it = 0; it < iters; ++it) {
+        const int j = k0 + it * KPI + kslot;
+        const bool valid = j < k1;
+        float kk[EPL], vv[EPL];
+        if (valid) {
+            const int page = table[j / page_size];
+            const int off = j % page_size;
+            const size_t base = ((static_cast<size_t>(page) * KVH + g) * page_size + off) * HD + sub * EPL;
+            VecIO<T, EPL>::load(kpool + base, kk);
+            VecIO<T, EPL>::load(vpool + base, vv);
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) { kk[e] = 0.f; vv[e] = 0.f; }
+        }
+#pragma unroll
+        for (int i = 0; i < GT; ++i) {
+            float s = 0.f;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) s += qreg[i][e] * kk[e];
+#pragma unroll
+            for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, WAVE);
+            if (valid) {
+                const float m_new = fmaxf(m[i], s);
+                const float corr = scale_of(m[i], m_new);
+                const float p = expf(s - m_new);
+                l[i] = l[i] * corr + p;
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) acc[i][e] = acc[i][e] * corr + p * vv[e];
+                m[i] = m_new;
+            }
+        }
+    }
+
+    // merge the lane groups of a wave (lanes with equal `sub`)
+#pragma unroll
+    for (int o = LPK; o < WAVE; o <<= 1) {
+#pragma unroll
+        for (int i = 0; i < GT; ++i) {
+            const float m_o = __shfl_xor(m[i], o, WAVE);
+            const float l_o = __shfl_xor(l[i], o, WAVE);
+            const float m_new = fmaxf(m[i], m_o);
+            const float a = scale_of(m[i], m_new);
+            const float b = scale_of(m_o, m_new);
+            l[i] = l[i] * a + l_o * b;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                const float acc_o = __shfl_xor(acc[i][e], o, WAVE);
+                acc[i][e] = acc[i][e] * a + acc_o * b;
+            }
+            m[i] = m_new;
+        }
+    }
+
+    __shared__ float sm_m[WAVES][GT];
+    __shared__ float sm_l[WAVES][GT];
+    __shared__ float sm_acc[WAVES][GT][HD];
+    const int wave = tid / WAVE;
+    const int lane = tid % WAVE;
+    if (lane < LPK) {
+#pragma unroll
+        for (int i = 0; i < GT; ++i) {
+            if (lane == 0) { sm_m[wave][i] = m[i]; sm_l[wave][i] = l[i]; }
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) sm_acc[wave][i][lane * EPL + e] = acc[i][e];
+        }
+    }
+    __syncthreads();
+
+    for (int idx = tid; idx < gc * HD; idx += ATT_THREADS) {
+        const int i = idx / HD;
+        const int dim = idx % HD;
+        float M = sm_m[0][i];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) M = fmaxf(M, sm_m[w][i]);
+        float Lsum = 0.f, O = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const float sc = scale_of(sm_m[w][i], M);
+            Lsum += sm_l[w][i] * sc;
+            O += sm_acc[w][i][dim] * sc;
+        }
+        const int h = h0 + i;
+        if (nsplit == 1) {
+            st(out + static_cast<size_t>(t) * H * HD + static_cast<size_t>(h) * HD + dim, O / Lsum);
+        } else {
+            const size_t p = (static_cast<size_t>(t) * H + h) * nsplit + split;
+            part_o[p * HD + dim] = O;
+            if (dim == 0) { part_ml[p * 2] = M; part_ml[p * 2 + 1] = Lsum; }
+        }
+    }
+}
+
+// Merge the partial (max, sum, output) of the splits of one (token, head).
+template <typename T>
+__global__ void merge_splits_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                    T* __restrict__ out, int H, int nsplit) {
+    const int t = blockIdx.x, h = blockIdx.y;
+    const size_t p0 = (static_cast<size_t>(t) * H + h) * nsplit;
+    float M = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[(p0 + s) * 2]);
+    for (int dim = threadIdx.x; dim < HEAD_DIM; dim += blockDim.x) {
+        float Lsum = 0.f, O = 0.f;
+        for (int s = 0; s < nsplit; ++s) {
+            const float sc = scale_of(part_ml[(p0 + s) * 2], M);
+            Lsum += part_ml[(p0 + s) * 2 + 1] * sc;
+            O += part_o[(p0 + s) * HEAD_DIM + dim] * sc;
+        }
+        st(out + static_cast<size_t>(t) * H * HEAD_DIM + static_cast<size_t>(h) * HEAD_DIM + dim, O / Lsum);
+    }
+}
+
+template <typename T>
+static int launch(const void* q, int q_stride, const void* kpool, const void* vpool, const void* block_table,
+                  int table_stride, const void* seq_of_token, const void* positions, void* out, void* part_o,
+                  void* part_ml, int T_tokens, int H, int KVH, int page_size, int window, float scale, int nsplit,
+                  hipStream_t stream) {
+    const int G = H / KVH;
+    const int chunks = (G + GT - 1) / GT;
+    dim3 grid(T_tokens, KVH * chunks, nsplit);
+    token_attention_kernel<T><<<grid, ATT_THREADS, 0, stream>>>(
+        (const T*)q, q_stride, (const T*)kpool, (const T*)vpool, (const int32_t*)block_table, table_stride,
+        (const int32_t*)seq_of_token, (const int32_t*)positions, (T*)out, (float*)part_o, (float*)part_ml, H, KVH,
+        page_size, window, scale, nsplit);
+    int err = NI_LAUNCH_RESULT();
+    if (err || nsplit == 1) return err;
+    merge_splits_kernel<T><<<dim3(T_tokens, H), 64, 0, stream>>>((const float*)part_o, (const float*)part_ml, (T*)out,
+                                                                H, nsplit);
+    return NI_LAUNCH_RESULT();
+}
+
+NI_EXPORT int ni_attention_head_dim() { return HEAD_DIM; }
+
+// part_o: float [T, H, nsplit, HEAD_DIM], part_ml: float [T, H, nsplit, 2]; unused when nsplit == 1.
+NI_EXPORT int ni_token_attention(const void* q, int q_stride, const void* kpool, const void* vpool,
+                                 const void* block_table, int table_stride, const void* seq_of_token,
+                                 const void* positions, void* out, void* part_o, void* part_ml, int T_tokens, int H,
+                                 int KVH, int page_size, int window, float scale, int nsplit, int dtype,
+                                 hipStream_t stream) {
+    if (T_tokens <= 0) return 0;
+    if (H % KVH != 0 || nsplit < 1 || nsplit > 65535 || page_size < 1) return -1;
+    if (dtype == 0)
+        return launch<float>(q, q_stride, kpool, vpool, block_table, table_stride, seq_of_token, positions, out,
+                             part_o, part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, stream);
+    return launch<bf16_t>(q, q_stride, kpool, vpool, block_table, table_stride, seq_of_token, positions, out, part_o,
+                          part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, stream);
+}

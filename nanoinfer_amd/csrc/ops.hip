@@ -1,0 +1,236 @@
+// Row-wise and element-wise kernels of a decoder step for gfx950: embedding gather,
+// residual-add + RMSNorm, rotation table, rotation + paged key/value write, SwiGLU.
+//
+// Conventions shared by all of them:
+//   * the residual stream is float32; activations that feed a matrix product are the
+//     compute type (float or bfloat16); all arithmetic is float32;
+//   * a key/value pool is laid out [page, kv_head, slot_in_page, head_dim];
+//   * every entry point is extern "C", takes raw device pointers and a hipStream_t, and
+//     returns 0 or the hipError_t of its launch.  Shapes are checked by the host wrapper.
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+// out[t, :] = table[ids[t], :]   (src/op/kernels/cuda/embedding_kernel.cu:30-48 of the reference;
+// ids are range-checked on the host before upload, an id outside the table never reaches here.)
+template <typename T>
+__global__ void embedding_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table,
+                                 float* __restrict__ out, int d, int vocab) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    if (id < 0 || id >= vocab) return;  // unreachable after the host check; never read out of bounds
+    const T* row = table + static_cast<size_t>(id) * d;
+    float* o = out + static_cast<size_t>(t) * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = ld(row + i);
+}
+
+// ---------------------------------------------------------------- add + RMSNorm
+// v = h[row] + pending[row];  out = v * rsqrt(mean(v^2) + eps) * w
+// Without `rows` the sum is written back to h (the residual stream moves on) and out has T rows.
+// With `rows` (a gather before the output head) h is left alone and out row r comes from h[rows[r]].
+// Formula: src/op/kernels/cuda/rmsnorm_kernel.cu:50-103 of the reference.
+template <typename TP, typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TP* __restrict__ pending,
+                                   const float* __restrict__ w, TO* __restrict__ out,
+                                   const int32_t* __restrict__ rows, int d, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
+    float* hrow = h + src * d;
+    const TP* prow = pending ? pending + src * d : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = hrow[i];
+        if (prow) v += ld(prow + i);
+        if (!rows && prow) hrow[i] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(d) + eps);
+    TO* orow = out + static_cast<size_t>(r) * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = hrow[i];
+        if (rows && prow) v += ld(prow + i);
+        st(orow + i, (v * inv) * w[i]);
+    }
+}
+
+// h[row] += pending[row] without a norm (the last residual sum when no norm follows).
+template <typename TP>
+__global__ void residual_add_kernel(float* __restrict__ h, const TP* __restrict__ pending, size_t n) {
+    size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) h[i] += ld(pending + i);
+}
+
+// ---------------------------------------------------------------- rotation table
+// cos/sin[pos, p] of the float32 product pos * inv_freq[p]
+// (src/op/kernels/cuda/rope_kernel.cu:129-131 of the reference; the frequencies come from the host).
+__global__ void rope_table_kernel(const float* __restrict__ inv_freq, float* __restrict__ cos_t,
+                                  float* __restrict__ sin_t, int max_pos, int half) {
+    size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= static_cast<size_t>(max_pos) * half) return;
+    int pos = static_cast<int>(idx / half);
+    int p = static_cast<int>(idx % half);
+    float angle = static_cast<float>(pos) * inv_freq[p];
+    cos_t[idx] = cosf(angle);
+    sin_t[idx] = sinf(angle);
+}
+
+// ---------------------------------------------------------------- rotation + key/value write
+// qkv is [T, (H + 2*KVH) * hd]: q heads, then k heads, then v heads.  Queries are rotated in
+// place; rotated keys and plain values go to the pools at slot_mapping[t] (= page*page_size + slot;
+// negative: this layer does not write).  Pairs are (j, j + rot/2) inside the first `rot` dims of a
+// head, which is the pairing of the checkpoint's row order (the reference permutes rows at export,
+// tools/export_llama3.py:571-583, and rotates neighbours, src/op/kernels/cuda/rope_kernel.cu:32-84).
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
+                                     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                     const int32_t* __restrict__ slot_mapping, T* __restrict__ kpool,
+                                     T* __restrict__ vpool, int H, int KVH, int hd, int rot, int page_size) {
+    const int t = blockIdx.x;
+    const int half = rot / 2;
+    const int row_width = (H + 2 * KVH) * hd;
+    T* row = qkv + static_cast<size_t>(t) * row_width;
+    const int pos = positions[t];
+    const float* c = cos_t ? cos_t + static_cast<size_t>(pos) * half : nullptr;
+    const float* s = sin_t ? sin_t + static_cast<size_t>(pos) * half : nullptr;
+    const int slot = slot_mapping ? slot_mapping[t] : -1;
+    const int page = slot >= 0 ? slot / page_size : 0;
+    const int off = slot >= 0 ? slot % page_size : 0;
+
+    // q and k heads: rotate pairs; dims beyond `rot` pass through.
+    const int per_head = hd - half;  // `half` pairs + (hd - rot) pass-through dims
+    for (int item = threadIdx.x; item < (H + KVH) * per_head; item += blockDim.x) {
+        const int head = item / per_head;
+        const int j = item % per_head;
+        T* hp = row + static_cast<size_t>(head) * hd;
+        const bool is_k = head >= H;
+        T* dst = nullptr;
+        if (is_k && slot >= 0)
+            dst = kpool + ((static_cast<size_t>(page) * KVH + (head - H)) * page_size + off) * hd;
+        if (j < half) {
+            float x0 = ld(hp + j), x1 = ld(hp + j + half);
+            float cs = c[j], sn = s[j];
+            float y0 = x0 * cs - x1 * sn;
+            float y1 = x0 * sn + x1 * cs;
+            if (!is_k) {
+                st(hp + j, y0);
+                st(hp + j + half, y1);
+            } else if (dst) {
+                st(dst + j, y0);
+                st(dst + j + half, y1);
+            }
+        } else {
+            const int dim = rot + (j - half);
+            if (is_k && dst) dst[dim] = hp[dim];
+        }
+    }
+    if (slot >= 0) {
+        for (int item = threadIdx.x; item < KVH * hd; item += blockDim.x) {
+            const int g = item / hd, dim = item % hd;
+            vpool[((static_cast<size_t>(page) * KVH + g) * page_size + off) * hd + dim] =
+                row[static_cast<size_t>(H + KVH + g) * hd + dim];
+        }
+    }
+}
+
+// ---------------------------------------------------------------- SwiGLU
+// out[t, i] = silu(gu[t, i]) * gu[t, I + i]   (src/op/kernels/cuda/swiglu_kernel.cu:31-39 of the
+// reference, with expf instead of the fast intrinsic).
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t n) {
+    size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= n) return;
+    size_t t = idx / I;
+    int i = static_cast<int>(idx % I);
+    float g = ld(gu + t * 2 * I + i);
+    float u = ld(gu + t * 2 * I + I + i);
+    st(out + idx, g / (1.0f + expf(-g)) * u);
+}
+
+// ---------------------------------------------------------------- float32 <- any
+template <typename T>
+__global__ void to_float_kernel(const T* __restrict__ in, float* __restrict__ out, size_t n) {
+    size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = ld(in + i);
+}
+
+// ================================================================ entry points
+// dtype codes: 0 = float32, 1 = bfloat16
+
+static inline unsigned blocks_for(size_t n, unsigned per) { return static_cast<unsigned>((n + per - 1) / per); }
+
+NI_EXPORT int ni_embedding(const void* ids, const void* table, void* out, int T, int d, int vocab,
+                           int table_dtype, hipStream_t stream) {
+    if (T <= 0) return 0;
+    if (table_dtype == 0)
+        embedding_kernel<float><<<T, 256, 0, stream>>>((const int32_t*)ids, (const float*)table, (float*)out, d, vocab);
+    else
+        embedding_kernel<bf16_t><<<T, 256, 0, stream>>>((const int32_t*)ids, (const bf16_t*)table, (float*)out, d, vocab);
+    return NI_LAUNCH_RESULT();
+}
+
+NI_EXPORT int ni_add_rmsnorm(void* h, const void* pending, const void* w, void* out, const void* rows,
+                             int n_rows, int d, float eps, int dtype, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    const int threads = d >= 1024 ? 256 : (d >= 256 ? 128 : 64);
+    if (dtype == 0)
+        add_rmsnorm_kernel<float, float><<<n_rows, threads, 0, stream>>>(
+            (float*)h, (const float*)pending, (const float*)w, (float*)out, (const int32_t*)rows, d, eps);
+    else
+        add_rmsnorm_kernel<bf16_t, bf16_t><<<n_rows, threads, 0, stream>>>(
+            (float*)h, (const bf16_t*)pending, (const float*)w, (bf16_t*)out, (const int32_t*)rows, d, eps);
+    return NI_LAUNCH_RESULT();
+}
+
+NI_EXPORT int ni_residual_add(void* h, const void* pending, size_t n, int dtype, hipStream_t stream) {
+    if (n == 0) return 0;
+    if (dtype == 0)
+        residual_add_kernel<float><<<blocks_for(n, 256), 256, 0, stream>>>((float*)h, (const float*)pending, n);
+    else
+        residual_add_kernel<bf16_t><<<blocks_for(n, 256), 256, 0, stream>>>((float*)h, (const bf16_t*)pending, n);
+    return NI_LAUNCH_RESULT();
+}
+
+NI_EXPORT int ni_rope_table(const void* inv_freq, void* cos_t, void* sin_t, int max_pos, int half,
+                            hipStream_t stream) {
+    size_t n = static_cast<size_t>(max_pos) * half;
+    if (n == 0) return 0;
+    rope_table_kernel<<<blocks_for(n, 256), 256, 0, stream>>>((const float*)inv_freq, (float*)cos_t, (float*)sin_t,
+                                                              max_pos, half);
+    return NI_LAUNCH_RESULT();
+}
+
+NI_EXPORT int ni_rope_kv_write(void* qkv, const void* positions, const void* cos_t, const void* sin_t,
+                               const void* slot_mapping, void* kpool, void* vpool, int T, int H, int KVH, int hd,
+                               int rot, int page_size, int dtype, hipStream_t stream) {
+    if (T <= 0) return 0;
+    if (dtype == 0)
+        rope_kv_write_kernel<float><<<T, 256, 0, stream>>>((float*)qkv, (const int32_t*)positions, (const float*)cos_t,
+                                                           (const float*)sin_t, (const int32_t*)slot_mapping,
+                                                           (float*)kpool, (float*)vpool, H, KVH, hd, rot, page_size);
+    else
+        rope_kv_write_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)qkv, (const int32_t*)positions,
+                                                            (const float*)cos_t, (const float*)sin_t,
+                                                            (const int32_t*)slot_mapping, (bf16_t*)kpool,
+                                                            (bf16_t*)vpool, H, KVH, hd, rot, page_size);
+    return NI_LAUNCH_RESULT();
+}
+
+NI_EXPORT int ni_swiglu(const void* gu, void* out, int T, int I, int dtype, hipStream_t stream) {
+    size_t n = static_cast<size_t>(T) * I;
+    if (n == 0) return 0;
+    if (dtype == 0)
+        swiglu_kernel<float><<<blocks_for(n, 256), 256, 0, stream>>>((const float*)gu, (float*)out, I, n);
+    else
+        swiglu_kernel<bf16_t><<<blocks_for(n, 256), 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, n);
+    return NI_LAUNCH_RESULT();
+}
+
+NI_EXPORT int ni_to_float(const void* in, void* out, size_t n, int dtype, hipStream_t stream) {
+    if (n == 0) return 0;
+    if (dtype == 0)
+        to_float_kernel<float><<<blocks_for(n, 256), 256, 0, stream>>>((const float*)in, (float*)out, n);
+    else
+        to_float_kernel<bf16_t><<<blocks_for(n, 256), 256, 0, stream>>>((const bf16_t*)in, (float*)out, n);
+    return NI_LAUNCH_RESULT();
+}

@@ -1,0 +1,282 @@
+"""Python face of the HIP kernels: loads the compiled libraries through ``ctypes`` and checks,
+on the host, that operand shapes, types and devices are what each kernel and its grid assume.
+
+There is no fallback: when a library cannot be built or loaded, or a tensor is not on the GPU,
+the call raises.  Matrix products are the one thing taken from a library (``torch.matmul`` ->
+rocBLAS/hipBLASLt), as the reference takes them from cuBLAS (src/op/kernels/cuda/matmul_kernel.cu:76-86).
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Dict, Optional
+
+import torch
+
+from ..csrc import build as _build
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+_libs: Dict[str, ctypes.CDLL] = {}
+
+
+def _load(target) -> ctypes.CDLL:
+    name, sources, defines = target
+    lib = _libs.get(name)
+    if lib is None:
+        path = _build.library_path(name, sources, defines)
+        try:
+            lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelError(f"cannot load the compiled kernels {path}: {e}") from e
+        _libs[name] = lib
+    return lib
+
+
+def core() -> ctypes.CDLL:
+    return _load(_build.CORE)
+
+
+def sampling_lib() -> ctypes.CDLL:
+    return _load(_build.SAMPLING)
+
+
+def attention_lib(head_dim: int) -> ctypes.CDLL:
+    return _load(_build.attention_target(head_dim))
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise KernelError(f"compute type {dtype} is not supported (float32 or bfloat16)") from None
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _gpu(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
+    _need(t.is_cuda, f"{name} must live on the GPU (no CPU fallback exists)")
+    _need(t.is_contiguous(), f"{name} must be contiguous")
+    if dtype is not None:
+        _need(t.dtype == dtype, f"{name} must be {dtype}, is {t.dtype}")
+    if shape is not None:
+        _need(tuple(t.shape) == tuple(shape), f"{name} must have shape {tuple(shape)}, has {tuple(t.shape)}")
+
+
+def _check(err: int, what: str) -> None:
+    if err != 0:
+        raise KernelError(f"{what}: launch failed with HIP error {err}")
+
+
+# ------------------------------------------------------------------ row-wise / element-wise
+
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out[t] = table[ids[t]]`` as float32; ``ids`` were range-checked by the caller."""
+    T = ids.shape[0]
+    vocab, d = table.shape
+    _gpu(ids, "ids", torch.int32, (T,))
+    _gpu(table, "table")
+    _gpu(out, "out", torch.float32, (T, d))
+    _check(core().ni_embedding(_ptr(ids), _ptr(table), _ptr(out), T, d, vocab, dtype_code(table.dtype), _stream()),
+           "embedding")
+    return out
+
+
+def add_rmsnorm(h: torch.Tensor, pending: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``h += pending`` (when no ``rows``) and ``out = rmsnorm(h) * weight``; with ``rows`` only those
+    rows are read and ``h`` stays as it is."""
+    T, d = h.shape
+    _gpu(h, "h", torch.float32)
+    _gpu(weight, "weight", torch.float32, (d,))
+    n = T if rows is None else rows.shape[0]
+    _gpu(out, "out", None, (n, d))
+    if pending is not None:
+        _gpu(pending, "pending", out.dtype, (T, d))
+    if rows is not None:
+        _gpu(rows, "rows", torch.int32, (n,))
+    _check(core().ni_add_rmsnorm(_ptr(h), _ptr(pending), _ptr(weight), _ptr(out), _ptr(rows), n, d,
+                                 ctypes.c_float(eps), dtype_code(out.dtype), _stream()), "add_rmsnorm")
+    return out
+
+
+def residual_add(h: torch.Tensor, pending: torch.Tensor) -> torch.Tensor:
+    _gpu(h, "h", torch.float32)
+    _gpu(pending, "pending", None, h.shape)
+    _check(core().ni_residual_add(_ptr(h), _ptr(pending), ctypes.c_size_t(h.numel()), dtype_code(pending.dtype),
+                                  _stream()), "residual_add")
+    return h
+
+
+def rope_table(inv_freq: torch.Tensor, max_pos: int):
+    """cos and sin of ``pos * inv_freq[p]`` in float32, each ``[max_pos, len(inv_freq)]``."""
+    _gpu(inv_freq, "inv_freq", torch.float32)
+    half = inv_freq.shape[0]
+    cos = torch.empty(max_pos, half, dtype=torch.float32, device=inv_freq.device)
+    sin = torch.empty_like(cos)
+    _check(core().ni_rope_table(_ptr(inv_freq), _ptr(cos), _ptr(sin), max_pos, half, _stream()), "rope_table")
+    return cos, sin
+
+
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[torch.Tensor],
+                  sin: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor], kpool: Optional[torch.Tensor],
+                  vpool: Optional[torch.Tensor], H: int, KVH: int, hd: int) -> None:
+    """Rotate the query and key heads of ``qkv`` ([T, (H+2KVH)*hd]) and store keys and values in
+    the pools ([pages, KVH, page_size, hd]) at ``slot_mapping`` (absent: nothing is stored)."""
+    T = qkv.shape[0]
+    _gpu(qkv, "qkv", None, (T, (H + 2 * KVH) * hd))
+    _gpu(positions, "positions", torch.int32, (T,))
+    rot = 0
+    if cos is not None:
+        rot = 2 * cos.shape[1]
+        _need(rot <= hd, f"rotary size {rot} exceeds the head size {hd}")
+        _gpu(cos, "cos", torch.float32)
+        _gpu(sin, "sin", torch.float32, cos.shape)
+    page_size = 1
+    if slot_mapping is not None:
+        _gpu(slot_mapping, "slot_mapping", torch.int32, (T,))
+        _need(kpool is not None and vpool is not None, "a slot mapping needs both pools")
+        _gpu(kpool, "kpool", qkv.dtype)
+        _gpu(vpool, "vpool", qkv.dtype, kpool.shape)
+        _need(kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd,
+              f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
+        page_size = kpool.shape[2]
+    _check(core().ni_rope_kv_write(_ptr(qkv), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
+                                   _ptr(kpool), _ptr(vpool), T, H, KVH, hd, rot, page_size,
+                                   dtype_code(qkv.dtype), _stream()), "rope_kv_write")
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out = silu(gate_up[:, :I]) * gate_up[:, I:]``."""
+    T, two_i = gate_up.shape
+    _need(two_i % 2 == 0, "gate_up needs an even width")
+    _gpu(gate_up, "gate_up")
+    _gpu(out, "out", gate_up.dtype, (T, two_i // 2))
+    _check(core().ni_swiglu(_ptr(gate_up), _ptr(out), T, two_i // 2, dtype_code(gate_up.dtype), _stream()), "swiglu")
+    return out
+
+
+def to_float(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _gpu(x, "x")
+    _gpu(out, "out", torch.float32, x.shape)
+    _check(core().ni_to_float(_ptr(x), _ptr(out), ctypes.c_size_t(x.numel()), dtype_code(x.dtype), _stream()),
+           "to_float")
+    return out
+
+
+# ------------------------------------------------------------------ attention
+
+def choose_splits(n_tokens: int, kv_heads: int, group: int, max_keys: int) -> int:
+    """How many pieces the key range of every token is cut into, so that a small batch still
+    fills the 256 compute units.  One piece never holds fewer than 256 keys."""
+    chunks = (group + 3) // 4
+    items = max(1, n_tokens * kv_heads * chunks)
+    want = max(1, 1024 // items)
+    return int(max(1, min(want, (max_keys + 255) // 256, 64)))
+
+
+def token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
+                    seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, H: int, KVH: int,
+                    hd: int, scale: float, window: Optional[int], nsplit: int,
+                    workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention of every token of ``qkv`` over the paged cache of its sequence.
+
+    ``qkv`` is [T, >= H*hd] with the (rotated) query heads first; the pools already hold the keys
+    and values of all positions up to each token's own.  ``workspace`` (float32, at least
+    ``T*H*nsplit*(hd+2)`` elements) is needed when ``nsplit > 1``.
+    """
+    T = qkv.shape[0]
+    _gpu(qkv, "qkv")
+    _need(qkv.shape[1] >= H * hd, "qkv is narrower than the query heads")
+    _need(H % KVH == 0, f"{H} query heads do not divide into {KVH} kv heads")
+    _gpu(kpool, "kpool", qkv.dtype)
+    _gpu(vpool, "vpool", qkv.dtype, kpool.shape)
+    _need(kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd,
+          f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
+    _gpu(block_table, "block_table", torch.int32)
+    _need(block_table.dim() == 2, "block_table must be [sequences, pages]")
+    _gpu(seq_of_token, "seq_of_token", torch.int32, (T,))
+    _gpu(positions, "positions", torch.int32, (T,))
+    _gpu(out, "out", qkv.dtype, (T, H * hd))
+    part_o = part_ml = None
+    if nsplit > 1:
+        need = T * H * nsplit * (hd + 2)
+        _need(workspace is not None and workspace.dtype == torch.float32 and workspace.numel() >= need,
+              f"attention workspace of {need} floats needed for {nsplit} splits")
+        _gpu(workspace, "workspace")
+        flat = workspace.view(-1)
+        part_o = flat[: T * H * nsplit * hd]
+        part_ml = flat[T * H * nsplit * hd: need]
+    lib = attention_lib(hd)
+    _check(lib.ni_token_attention(_ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table),
+                                  block_table.shape[1], _ptr(seq_of_token), _ptr(positions), _ptr(out),
+                                  _ptr(part_o), _ptr(part_ml), T, H, KVH, kpool.shape[2],
+                                  int(window) if window else 0, ctypes.c_float(scale), nsplit,
+                                  dtype_code(qkv.dtype), _stream()), "token_attention")
+    return out
+
+
+# ------------------------------------------------------------------ sampling
+
+def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    R, V = logits.shape
+    _gpu(logits, "logits", torch.float32)
+    if out is None:
+        out = torch.empty(R, dtype=torch.int32, device=logits.device)
+    _gpu(out, "out", torch.int32, (R,))
+    _check(sampling_lib().ni_argmax(_ptr(logits), _ptr(out), R, V, _stream()), "argmax")
+    return out
+
+
+def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
+           top_p: torch.Tensor, penalty: torch.Tensor, pen_ids: torch.Tensor, pen_off: torch.Tensor,
+           uniform: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    R, V = logits.shape
+    _gpu(logits, "logits", torch.float32)
+    _gpu(work, "work", torch.float32, (R, V))
+    for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+                        ("top_p", top_p, torch.float32), ("penalty", penalty, torch.float32),
+                        ("uniform", uniform, torch.float32), ("out", out, torch.int32)):
+        _gpu(t, name, dt, (R,))
+    _gpu(pen_off, "pen_off", torch.int32, (R + 1,))
+    _gpu(pen_ids, "pen_ids", torch.int32)
+    _check(sampling_lib().ni_sample(_ptr(logits), _ptr(work), _ptr(temperature), _ptr(top_k), _ptr(top_p),
+                                    _ptr(penalty), _ptr(pen_ids), _ptr(pen_off), _ptr(uniform), _ptr(out), R, V,
+                                    _stream()), "sample")
+    return out
+
+
+# ------------------------------------------------------------------ matrix product (library)
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x . weight^T`` with ``weight`` stored [out, in]; float32 inputs are multiplied in true
+    float32 (the reduced-precision matrix modes of the library are switched off at import)."""
+    _need(x.is_cuda and weight.is_cuda, "linear needs GPU tensors")
+    _need(x.dtype == weight.dtype, f"linear: activation {x.dtype} and weight {weight.dtype} differ")
+    _need(x.shape[-1] == weight.shape[1], f"linear: {tuple(x.shape)} x {tuple(weight.shape)}^T")
+    return torch.matmul(x, weight.t(), out=out)
+
+
+def require_gpu() -> torch.device:
+    if not torch.cuda.is_available():
+        raise KernelError("no GPU is visible: nanoinfer_amd runs on an MI355X only and has no CPU path")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+torch.backends.cuda.matmul.allow_tf32 = False
+torch.backends.cudnn.allow_tf32 = False

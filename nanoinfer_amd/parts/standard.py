@@ -1,0 +1,284 @@
+"""The parts that the Llama family is assembled from.  Each takes its sizes and constants from
+``spec.params`` and its tensors by the names in ``spec.weights``; none knows the model it is in.
+
+Kinds registered here: embedding ``table``; norm ``rmsnorm``; position ``rope`` and ``none``;
+mixer ``attention``; feed_forward ``swiglu``; block ``prenorm``; head ``linear``.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional
+
+import numpy as np
+import torch
+
+from .. import kernels as K
+from ..config.spec import BlockSpec, PartSpec
+from ..registry import get_part, register_part
+from .base import CacheNeed, KVNeed, LayerCache, Part, Runtime, WeightRequest
+
+
+def build_part(family: str, spec: PartSpec, tensors: Dict[str, torch.Tensor], rt: Runtime) -> Part:
+    """Instantiate the registered class for ``spec.kind`` with the tensors it asked for."""
+    cls = get_part(family, spec.kind)
+    return cls(spec, {logical: tensors[name] for logical, name in spec.weights.items()}, rt)
+
+
+def requests_of(family: str, spec: PartSpec) -> List[WeightRequest]:
+    return get_part(family, spec.kind).weight_requests(spec)
+
+
+# ------------------------------------------------------------------ embedding
+
+@register_part("embedding", "table")
+class TableEmbedding(Part):
+    """``h[t] = E[id[t]]``, no scaling (src/op/embedding.cpp:14-70, kernel embedding_kernel.cu:30-48).
+    params: vocab_size, hidden_size.  weights: weight [vocab, hidden]."""
+
+    @classmethod
+    def weight_requests(cls, spec):
+        return [WeightRequest(spec.weights["weight"], (spec.params["vocab_size"], spec.params["hidden_size"]))]
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        self.vocab_size = int(spec.params["vocab_size"])
+        self.hidden_size = int(spec.params["hidden_size"])
+        self.weight = rt.matrix(spec.weights["weight"], weights["weight"])
+
+    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+        out = torch.empty(token_ids.shape[0], self.hidden_size, dtype=torch.float32, device=self.rt.device)
+        return K.embedding(token_ids, self.weight, out)
+
+
+# ------------------------------------------------------------------ norm
+
+@register_part("norm", "rmsnorm")
+class RMSNorm(Part):
+    """``x * rsqrt(mean(x^2) + eps) * w`` in float32 (src/op/rmsnorm.cpp:14-69, rmsnorm_kernel.cu:50-103).
+    params: size, eps.  weights: weight [size]."""
+
+    @classmethod
+    def weight_requests(cls, spec):
+        return [WeightRequest(spec.weights["weight"], (spec.params["size"],))]
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        self.size = int(spec.params["size"])
+        self.eps = float(spec.params["eps"])
+        self.weight = rt.vector32(spec.weights["weight"], weights["weight"])
+
+    def forward(self, h: torch.Tensor, pending: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None):
+        n = h.shape[0] if rows is None else rows.shape[0]
+        out = torch.empty(n, self.size, dtype=self.rt.dtype, device=self.rt.device)
+        return K.add_rmsnorm(h, pending, self.weight, self.eps, out, rows)
+
+
+# ------------------------------------------------------------------ position
+
+def rope_inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[dict]) -> np.ndarray:
+    """Frequency of each rotated pair in float32 arithmetic, with llama3 scaling when given:
+    long waves divided by ``factor``, short ones kept, a linear blend between
+    (src/op/kernels/cuda/rope_kernel.cu:108-127, src/op/kernels/cpu/rope_kernel.cpp:121-139)."""
+    f32 = np.float32
+    half = rotary_dim // 2
+    out = np.empty(half, dtype=f32)
+    for p in range(half):
+        freq = f32(1.0) / f32(np.power(f32(theta), f32(f32(2 * p) / f32(rotary_dim)), dtype=f32))
+        if scaling is not None:
+            factor, low, high = f32(scaling["factor"]), f32(scaling["low_freq_factor"]), f32(scaling["high_freq_factor"])
+            orig = f32(scaling["original_max_position_embeddings"])
+            wavelen = f32(f32(2.0) * f32(math.pi) / freq)
+            if wavelen >= f32(orig / low):
+                freq = f32(freq / factor)
+            elif wavelen > f32(orig / high):
+                smooth = f32(f32(orig / wavelen - low) / f32(high - low))
+                freq = f32(f32(f32(1.0) - smooth) * freq / factor + smooth * freq)
+        out[p] = freq
+    return out
+
+
+@register_part("position", "rope")
+class RotaryPosition(Part):
+    """Rotation of pairs by ``pos * f_p``.  params: rotary_dim, theta, scaling (dict or None),
+    max_positions.  One table per distinct set of constants is shared by all layers."""
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        self.rotary_dim = int(p["rotary_dim"])
+        self.max_positions = int(p["max_positions"])
+        if self.rotary_dim % 2 or self.rotary_dim <= 0:
+            raise ValueError(f"rotary_dim {self.rotary_dim} must be positive and even")
+        scaling = p.get("scaling")
+        key = ("rope", self.rotary_dim, float(p["theta"]), self.max_positions,
+               None if scaling is None else tuple(sorted(scaling.items())))
+        if key not in rt.shared:
+            inv = torch.from_numpy(rope_inverse_frequencies(self.rotary_dim, float(p["theta"]), scaling)).to(rt.device)
+            rt.shared[key] = K.rope_table(inv, self.max_positions)
+        self.cos, self.sin = rt.shared[key]
+
+    def tables(self):
+        return self.cos, self.sin
+
+
+@register_part("position", "none")
+class NoPosition(Part):
+    """No position encoding: keys and queries are used as projected."""
+
+    max_positions = None
+
+    def tables(self):
+        return None
+
+
+# ------------------------------------------------------------------ mixer
+
+@register_part("mixer", "attention")
+class Attention(Part):
+    """Grouped-query causal attention over the paged cache (src/op/attention.cpp:101-198).
+
+    params: hidden_size, num_heads, num_kv_heads, head_dim, scale (None: 1/sqrt(head_dim)),
+    window (None: all keys), position (a PartSpec of family ``position``).
+    weights: q [H*hd, d], k [KVH*hd, d], v [KVH*hd, d], o [d, H*hd]; no bias.
+    The three input projections are stacked into one matrix at load, so one product feeds the
+    rotation-and-cache-write kernel directly.
+    """
+
+    @classmethod
+    def weight_requests(cls, spec):
+        p, w = spec.params, spec.weights
+        d, H, KVH, hd = p["hidden_size"], p["num_heads"], p["num_kv_heads"], p["head_dim"]
+        return [WeightRequest(w["q"], (H * hd, d)), WeightRequest(w["k"], (KVH * hd, d)),
+                WeightRequest(w["v"], (KVH * hd, d)), WeightRequest(w["o"], (d, H * hd))]
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        self.hidden_size = int(p["hidden_size"])
+        self.H = int(p["num_heads"])
+        self.KVH = int(p["num_kv_heads"])
+        self.hd = int(p["head_dim"])
+        if self.H % self.KVH:
+            raise ValueError(f"{self.H} query heads do not divide into {self.KVH} kv heads")
+        self.scale = float(p["scale"]) if p.get("scale") is not None else 1.0 / math.sqrt(self.hd)
+        self.window = None if p.get("window") is None else int(p["window"])
+        K.attention_lib(self.hd)  # refuses an unsupported head size now, not at the first step
+        pos_spec: PartSpec = p["position"]
+        self.position = get_part("position", pos_spec.kind)(pos_spec, {}, rt)
+        names = spec.weights
+        fused_name = "|".join((names["q"], names["k"], names["v"]))
+        key = ("matrix", fused_name, rt.dtype)
+        if key not in rt.shared:
+            rt.shared[key] = torch.cat([weights["q"], weights["k"], weights["v"]], dim=0).to(
+                device=rt.device, dtype=rt.dtype).contiguous()
+        self.w_qkv = rt.shared[key]
+        self.w_o = rt.matrix(names["o"], weights["o"])
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(kv=KVNeed(self.KVH, self.hd, self.window))
+
+    def forward(self, x: torch.Tensor, ctx, cache: LayerCache) -> torch.Tensor:
+        T = x.shape[0]
+        qkv = K.linear(x, self.w_qkv)
+        tables = self.position.tables()
+        cos, sin = tables if tables is not None else (None, None)
+        K.rope_kv_write(qkv, ctx.positions, cos, sin, cache.slot_mapping if cache.writes else None,
+                        cache.kpool, cache.vpool, self.H, self.KVH, self.hd)
+        out = torch.empty(T, self.H * self.hd, dtype=x.dtype, device=x.device)
+        max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window)
+        nsplit = K.choose_splits(T, self.KVH, self.H // self.KVH, max_keys)
+        ws = ctx.workspace(T * self.H * nsplit * (self.hd + 2)) if nsplit > 1 else None
+        K.token_attention(qkv, cache.kpool, cache.vpool, cache.block_table, ctx.seq_of_token, ctx.positions, out,
+                          self.H, self.KVH, self.hd, self.scale, self.window, nsplit, ws)
+        return K.linear(out, self.w_o)
+
+
+# ------------------------------------------------------------------ feed-forward
+
+@register_part("feed_forward", "swiglu")
+class SwiGLU(Part):
+    """``down(silu(gate(x)) * up(x))`` (src/model/llama.cpp:364-379, swiglu_kernel.cu:31-39).
+    params: hidden_size, intermediate_size.  weights: gate [I, d], up [I, d], down [d, I].
+    gate and up are stacked so one product yields both halves."""
+
+    @classmethod
+    def weight_requests(cls, spec):
+        p, w = spec.params, spec.weights
+        d, i = p["hidden_size"], p["intermediate_size"]
+        return [WeightRequest(w["gate"], (i, d)), WeightRequest(w["up"], (i, d)), WeightRequest(w["down"], (d, i))]
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        self.intermediate_size = int(spec.params["intermediate_size"])
+        names = spec.weights
+        key = ("matrix", names["gate"] + "|" + names["up"], rt.dtype)
+        if key not in rt.shared:
+            rt.shared[key] = torch.cat([weights["gate"], weights["up"]], dim=0).to(
+                device=rt.device, dtype=rt.dtype).contiguous()
+        self.w_gate_up = rt.shared[key]
+        self.w_down = rt.matrix(names["down"], weights["down"])
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        gu = K.linear(x, self.w_gate_up)
+        act = torch.empty(x.shape[0], self.intermediate_size, dtype=x.dtype, device=x.device)
+        K.swiglu(gu, act)
+        return K.linear(act, self.w_down)
+
+
+# ------------------------------------------------------------------ block
+
+@register_part("block", "prenorm")
+class PreNormBlock:
+    """``h += mixer(norm1(h)); h += ffn(norm2(h))`` (src/model/llama.cpp:324-379).
+
+    The residual stream ``h`` is float32.  The last addend is handed on as ``pending`` and is
+    summed into ``h`` by the next norm, in float32, in the same pass that normalises.
+    """
+
+    family = "block"
+    kind = "prenorm"
+
+    @classmethod
+    def weight_requests(cls, spec: BlockSpec) -> List[WeightRequest]:
+        return (requests_of("norm", spec.mixer_norm) + requests_of("mixer", spec.mixer)
+                + requests_of("norm", spec.ffn_norm) + requests_of("feed_forward", spec.ffn))
+
+    def __init__(self, spec: BlockSpec, tensors: Dict[str, torch.Tensor], rt: Runtime):
+        self.spec = spec
+        self.mixer_norm = build_part("norm", spec.mixer_norm, tensors, rt)
+        self.mixer = build_part("mixer", spec.mixer, tensors, rt)
+        self.ffn_norm = build_part("norm", spec.ffn_norm, tensors, rt)
+        self.ffn = build_part("feed_forward", spec.ffn, tensors, rt)
+
+    def cache_need(self) -> CacheNeed:
+        return self.mixer.cache_need()
+
+    def forward(self, h, pending, ctx, cache: LayerCache):
+        x = self.mixer_norm.forward(h, pending)
+        a = self.mixer.forward(x, ctx, cache)
+        x = self.ffn_norm.forward(h, a)
+        f = self.ffn.forward(x, ctx)
+        return h, f
+
+
+# ------------------------------------------------------------------ head
+
+@register_part("head", "linear")
+class LinearHead(Part):
+    """``logits = x . W^T`` in float32 output (src/model/llama.cpp:383-386).  params: vocab_size,
+    hidden_size.  weights: weight [vocab, hidden]; a tied head names the embedding's tensor and
+    shares its device buffer."""
+
+    @classmethod
+    def weight_requests(cls, spec):
+        return [WeightRequest(spec.weights["weight"], (spec.params["vocab_size"], spec.params["hidden_size"]))]
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        self.vocab_size = int(spec.params["vocab_size"])
+        self.weight = rt.matrix(spec.weights["weight"], weights["weight"])
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if x.dtype == torch.float32:
+            return K.linear(x, self.weight)
+        return torch.mm(x, self.weight.t(), out_dtype=torch.float32)

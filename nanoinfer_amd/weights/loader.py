@@ -1,0 +1,122 @@
+"""Tensors of a model folder, by name, checked against what the model's parts ask for.
+
+The reference trusts running offsets into its own file format and validates neither size nor
+shape (src/model/llama.cpp:568-706).  Here the parts state the names and shapes they need, the
+file states what it holds, and every difference is reported in ONE error: tensors that are
+missing, tensors nobody asked for, tensors of the wrong shape.
+
+Types: a tensor is handed on as stored (bfloat16 stays bfloat16, float32 stays float32, float16
+is widened to float32, integer tables become int32); the parts place matrices in the compute type
+and one-dimensional parameters in float32.
+"""
+from __future__ import annotations
+
+import json
+import os
+from typing import Any, Dict, List, Tuple
+
+import torch
+
+from ..config.model_config import read_config_json
+from ..config.spec import ModelSpec
+from ..registry import architecture_of, get_part
+from .safetensors_io import SafetensorsFile, WeightFileError, write_safetensors
+
+
+class WeightMismatchError(WeightFileError):
+    """The checkpoint does not hold exactly the tensors the model needs."""
+
+    def __init__(self, path: str, missing: List[str], unexpected: List[str],
+                 wrong_shape: List[Tuple[str, Tuple[int, ...], Tuple[int, ...]]]):
+        self.path = path
+        self.missing = missing
+        self.unexpected = unexpected
+        self.wrong_shape = wrong_shape
+        lines = [f"{path} does not match the model:"]
+        if missing:
+            lines.append(f"  missing ({len(missing)}): " + ", ".join(missing))
+        if unexpected:
+            lines.append(f"  unexpected ({len(unexpected)}): " + ", ".join(unexpected))
+        if wrong_shape:
+            lines.append(f"  wrong shape ({len(wrong_shape)}): " + ", ".join(
+                f"{n} is {list(got)}, expected {list(want)}" for n, want, got in wrong_shape))
+        super().__init__("\n".join(lines))
+
+
+def expected_tensors(spec: ModelSpec) -> Dict[str, Tuple[int, ...]]:
+    """Name -> shape of every tensor the parts of ``spec`` ask for (a name asked for twice, as
+    by a tied head, must be asked for with one shape)."""
+    requests = list(get_part("embedding", spec.embedding.kind).weight_requests(spec.embedding))
+    for b in spec.blocks:
+        requests += get_part("block", b.kind).weight_requests(b)
+    requests += get_part("norm", spec.final_norm.kind).weight_requests(spec.final_norm)
+    requests += get_part("head", spec.head.kind).weight_requests(spec.head)
+    out: Dict[str, Tuple[int, ...]] = {}
+    for r in requests:
+        shape = tuple(int(s) for s in r.shape)
+        if r.name in out and out[r.name] != shape:
+            raise WeightFileError(f"tensor {r.name!r} is asked for with shapes {out[r.name]} and {shape}")
+        out[r.name] = shape
+    return out
+
+
+def _as_stored(t: torch.Tensor) -> torch.Tensor:
+    if t.dtype in (torch.bfloat16, torch.float32):
+        return t
+    if t.dtype in (torch.float16, torch.float64):
+        return t.to(torch.float32)
+    if t.dtype in (torch.int64, torch.int16, torch.int8, torch.uint8, torch.int32):
+        return t.to(torch.int32)
+    raise WeightFileError(f"tensor type {t.dtype} cannot be used")
+
+
+def load_tensors(folder: str, spec: ModelSpec) -> Dict[str, torch.Tensor]:
+    """The tensors ``spec`` needs from ``folder/model.safetensors`` (CPU views of the mapped file)."""
+    path = os.path.join(folder, "model.safetensors")
+    f = SafetensorsFile(path)
+    want = expected_tensors(spec)
+    have = set(f.names())
+    missing = sorted(n for n in want if n not in have)
+    unexpected = []
+    for n in sorted(have - set(want)):
+        orig = spec.duplicates.get(n)
+        if orig in have and tuple(f.shape(n)) == tuple(f.shape(orig)) and torch.equal(f.tensor(n), f.tensor(orig)):
+            continue  # a second copy of a tensor the model shares
+        unexpected.append(n)
+    wrong = sorted((n, want[n], f.shape(n)) for n in want if n in have and tuple(f.shape(n)) != want[n])
+    if missing or unexpected or wrong:
+        raise WeightMismatchError(path, missing, unexpected, wrong)
+    return {n: _as_stored(f.tensor(n)) for n in want}
+
+
+def write_model_folder(folder: str, config_json: Dict[str, Any], tensors: Dict[str, torch.Tensor]) -> str:
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as fh:
+        json.dump(config_json, fh, indent=2)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors, {"format": "pt"})
+    return folder
+
+
+_TORCH_DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
+
+
+def make_random_model(folder: str, config_json: Dict[str, Any], seed: int, dtype: str = "bfloat16",
+                      **init) -> str:
+    """Random-weights mode: write ``config.json`` and ``model.safetensors`` for the architecture
+    that ``config_json`` names, from a seed.  ``dtype`` is the type the matrices are stored in."""
+    if dtype not in _TORCH_DTYPES:
+        raise WeightFileError(f"dtype {dtype!r} is not one of {sorted(_TORCH_DTYPES)}")
+    arch = architecture_of(config_json)
+    cfg = arch.config_from_dict(config_json)
+    tensors = arch.random_weights(cfg, seed, dtype=_TORCH_DTYPES[dtype], **init)
+    out = dict(cfg.to_dict())
+    out["torch_dtype"] = "bfloat16" if _TORCH_DTYPES[dtype] == torch.bfloat16 else "float32"
+    return write_model_folder(folder, out, tensors)
+
+
+def read_model_folder(folder: str):
+    """``(architecture, typed configuration, spec)`` of a model folder, chosen by ``config.json``."""
+    raw = read_config_json(folder)
+    arch = architecture_of(raw)
+    cfg = arch.config_from_dict(raw)
+    return arch, cfg, arch.build_spec(cfg)

@@ -1,0 +1,34 @@
+"""Small configurations for the tests.  A and B differ in every size and option; C has sizes that
+are neither powers of two nor multiples of a wavefront."""
+
+TINY_A = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 64, "num_hidden_layers": 2, "num_attention_heads": 4, "num_key_value_heads": 2,
+    "head_dim": 16, "intermediate_size": 160, "vocab_size": 256, "rms_norm_eps": 1e-5,
+    "rope_theta": 10000.0, "rope_scaling": None, "max_position_embeddings": 256,
+    "tie_word_embeddings": True, "hidden_act": "silu", "bos_token_id": 1, "eos_token_id": 2,
+}
+
+TINY_B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 192, "num_hidden_layers": 3, "num_attention_heads": 6, "num_key_value_heads": 1,
+    "head_dim": 32, "intermediate_size": 512, "vocab_size": 1000, "rms_norm_eps": 1e-6,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 4.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 64},
+    "max_position_embeddings": 512, "tie_word_embeddings": False, "hidden_act": "silu",
+    "bos_token_id": 0, "eos_token_id": [998, 999],
+}
+
+# hidden size that is not heads x head_dim, odd vocabulary, five query heads on five kv heads
+TINY_C = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 100, "num_hidden_layers": 2, "num_attention_heads": 5, "num_key_value_heads": 5,
+    "head_dim": 48, "intermediate_size": 136, "vocab_size": 777, "rms_norm_eps": 3e-6,
+    "rope_theta": 25000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 2.0,
+                     "original_max_position_embeddings": 32},
+    "max_position_embeddings": 640, "tie_word_embeddings": True, "hidden_act": "silu",
+}
+
+ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
