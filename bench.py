@@ -1,0 +1,205 @@
+"""Decode and prefill throughput of the engine on one MI355X, Llama 3.2 1B shape, random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--layers L]
+
+A step is one decode step of a batch of 8 requests whose prompts of 2,048 random tokens are in
+the cache (context limit 4,096): the step function runs the 8 new tokens as one batch, the
+argmax kernel picks the next ones, and they come back to the host, as in generation.  ``value``
+is decoded tokens per second.  The same line carries the prefill of one 2,048-token prompt (in
+portions of 512, as the configuration says), the decode step's fraction of the HBM roofline, and
+decode at batch 1 and 64.  Peaks are MI355X's published ones: HBM 8 TB/s, dense bf16 MFMA
+2.5 PFLOP/s, fp32 157.3 TFLOP/s.  The reference publishes no numbers for this model, so
+``vs_baseline`` is null.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import random
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+LLAMA_1B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 2048, "num_hidden_layers": 16, "num_attention_heads": 32, "num_key_value_heads": 8,
+    "head_dim": 64, "intermediate_size": 8192, "vocab_size": 128256, "rms_norm_eps": 1e-5,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "max_position_embeddings": 131072, "tie_word_embeddings": True, "hidden_act": "silu",
+    "bos_token_id": 128000, "eos_token_id": 128001,
+}
+FULL_LAYERS = 16
+PROMPT_LEN = 2048
+CONTEXT_LEN = 4096
+PREFILL_CHUNK = 512
+BLOCK_SIZE = 16
+HBM_PEAK = 8.0e12
+FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def log(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def decode_bytes(cfg: dict, batch: int, mean_context: float, elem: int) -> float:
+    """Bytes a decode step has to read: every matrix once (the tied head is the embedding
+    matrix), the norm weights, and the keys and values of the live requests."""
+    d, L, H, KVH, hd = cfg["hidden_size"], cfg["num_hidden_layers"], cfg["num_attention_heads"], \
+        cfg["num_key_value_heads"], cfg["head_dim"]
+    I, V = cfg["intermediate_size"], cfg["vocab_size"]
+    per_layer = (H * hd * d + 2 * KVH * hd * d + d * H * hd + 3 * I * d) * elem + 2 * d * 4
+    weights = L * per_layer + V * d * elem + d * 4
+    kv = batch * mean_context * L * 2 * KVH * hd * elem
+    return weights + kv
+
+
+def prefill_flops(cfg: dict, tokens: int) -> float:
+    """Matrix products of every layer on every token, causal attention, and the head on one row."""
+    d, L, H, KVH, hd = cfg["hidden_size"], cfg["num_hidden_layers"], cfg["num_attention_heads"], \
+        cfg["num_key_value_heads"], cfg["head_dim"]
+    I, V = cfg["intermediate_size"], cfg["vocab_size"]
+    linear = 2.0 * tokens * L * (H * hd * d + 2 * KVH * hd * d + d * H * hd + 3 * I * d)
+    attention = L * H * 4.0 * hd * (tokens * (tokens + 1) / 2.0)
+    return linear + attention + 2.0 * V * d
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+
+    import nanoinfer_amd  # noqa: F401
+    from nanoinfer_amd import kernels as K
+    from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
+    from nanoinfer_amd.weights.loader import make_random_model
+
+    torch.cuda.set_device(0)
+    cfg = dict(LLAMA_1B)
+    cfg["num_hidden_layers"] = args.layers
+    dtype = {"bf16": "bfloat16", "fp32": "float32"}[args.dtype]
+    elem = 2 if args.dtype == "bf16" else 4
+    rng = random.Random(0)
+    V = cfg["vocab_size"]
+
+    with tempfile.TemporaryDirectory(prefix="nanoinfer-bench-") as folder:
+        t0 = time.perf_counter()
+        make_random_model(folder, cfg, seed=0, dtype=dtype)
+        log(f"random model written in {time.perf_counter() - t0:.1f} s")
+        max_batch = args.batch if args.no_points else max(args.batch, 64)
+        t0 = time.perf_counter()
+        runner = ModelRunner(folder, dtype=dtype, page_size=BLOCK_SIZE, max_tokens=max_batch * CONTEXT_LEN,
+                             max_requests=max_batch)
+        log(f"model loaded in {time.perf_counter() - t0:.1f} s")
+
+    def prompt():
+        return [rng.randrange(V) for _ in range(PROMPT_LEN)]
+
+    def measure_prefill():
+        """One prompt of 2,048 tokens in portions of 512; the last portion yields the first token."""
+        times = []
+        for rep in range(3):
+            toks = prompt()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for s in range(0, PROMPT_LEN, PREFILL_CHUNK):
+                last = s + PREFILL_CHUNK >= PROMPT_LEN
+                logits = runner.step([StepEntry("p", toks[s:s + PREFILL_CHUNK], [PREFILL_CHUNK - 1] if last else [])])
+            K.argmax(logits).tolist()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            runner.release("p")
+        return min(times[1:])
+
+    def measure_decode(batch: int, steps: int, warmup: int):
+        ids = [f"d{i}" for i in range(batch)]
+        tokens = []
+        for i in ids:   # fill the cache: whole prompts, one request a step
+            logits = runner.step([StepEntry(i, prompt(), [PROMPT_LEN - 1])])
+            tokens.append(K.argmax(logits).tolist()[0])
+        log(f"batch {batch}: prompts are in the cache")
+
+        def one_step(toks):
+            logits = runner.step([StepEntry(i, [t], [0]) for i, t in zip(ids, toks)])
+            return K.argmax(logits).tolist()
+
+        for _ in range(warmup):
+            tokens = one_step(tokens)
+        torch.cuda.synchronize()
+        first_ctx = runner.computed_tokens(ids[0])
+        t = time.perf_counter()
+        for _ in range(steps):
+            tokens = one_step(tokens)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        mean_ctx = first_ctx + (steps + 1) / 2.0
+        for i in ids:
+            runner.release(i)
+        return dt / steps, mean_ctx
+
+    log("prefill ...")
+    prefill_s = measure_prefill()
+    log(f"prefill of {PROMPT_LEN}: {prefill_s * 1e3:.2f} ms")
+    step_s, mean_ctx = measure_decode(args.batch, args.steps, args.warmup)
+    log(f"decode batch {args.batch}: {step_s * 1e3:.3f} ms a step")
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            n = max(20, min(args.steps, 100))
+            s, _ = measure_decode(b, n, max(5, args.warmup // 2))
+            points[f"decode_b{b}"] = round(b / s, 1)
+            log(f"decode batch {b}: {s * 1e3:.3f} ms a step")
+
+    achieved = decode_bytes(cfg, args.batch, mean_ctx, elem) / step_s
+    flops = prefill_flops(cfg, PROMPT_LEN)
+    result = {
+        "metric": "decode tok/s at batch 8 (Llama 3.2 1B shape, context 4096)",
+        "value": round(args.batch / step_s, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": args.dtype,
+        "data": "synthetic: random weights (seed 0), uniform random token ids",
+        "config": {
+            "model": "llama-3.2-1b-shape", "layers": args.layers, "layers_full_model": FULL_LAYERS,
+            "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
+            "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+            "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
+            "tied_embeddings": True, "global_batch": args.batch, "prompt_len": PROMPT_LEN,
+            "seq_len": CONTEXT_LEN, "decode_context_mean": round(mean_ctx, 1), "kv_block_size": BLOCK_SIZE,
+            "prefill_chunk": PREFILL_CHUNK, "parallelism": "single-gpu",
+        },
+        "prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN, "ms": round(prefill_s * 1e3, 3),
+                    "frac": round(flops / prefill_s / FLOP_PEAK[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},
+        "points": points,
+    }
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -110,6 +110,8 @@ class ModelRunner:
         self.cache = KVCacheManager(self.model.cache_needs(), self.page_size, num_pages, max_requests,
                                     dtype=torch_dtype, device=self.device)
         self.vocab_size = self.spec.vocab_size
+        self.max_positions = self.model.max_positions
+        self.eos_token_ids = tuple(self.spec.eos_token_ids)
         self._done: Dict[Hashable, int] = {}   # tokens of each live request already in the cache
         self._scratch: Optional[torch.Tensor] = None
 
