@@ -279,26 +279,32 @@ def temperature_scale(logits: torch.Tensor, temperature: float) -> torch.Tensor:
 def filtered_distribution(logits: torch.Tensor, top_k: int, top_p: float) -> torch.Tensor:
     """Probabilities after top-k and top-p, renormalised, in vocabulary order.
 
-    Keep the ``k`` largest logits, softmax, then keep the shortest prefix of the
-    descending order whose mass reaches ``top_p`` and renormalise.
-    src/op/kernels/cpu/sampling_kernel.cpp:134-180 (order: top-k, softmax, top-p, renormalise;
-    src/sampler/configurable_sampler.cpp:93-120).
+    Keep the logits that are at least the k-th largest, softmax, then walk the descending order
+    until the mass reaches ``top_p`` and keep every token at least as probable as the one where
+    it did; renormalise.  Equal values at a cut are kept together (the reference's GPU kernel
+    cuts by a threshold on the value as well, src/op/kernels/cuda/sampling_kernel.cu:202-296).
+    Order of the stages: src/op/kernels/cpu/sampling_kernel.cpp:134-180,
+    src/sampler/configurable_sampler.cpp:93-120.
     """
     V = logits.shape[0]
     order = sorted(range(V), key=lambda i: (-float(logits[i]), i))
-    keep = order[:top_k] if 0 < top_k < V else order
+    keep = order
+    if 0 < top_k < V:
+        kth = float(logits[order[top_k - 1]])
+        keep = [i for i in order if float(logits[i]) >= kth]
     m = max(float(logits[i]) for i in keep)
     e = {i: math.exp(float(logits[i]) - m) for i in keep}
     z = sum(e.values())
     probs = {i: e[i] / z for i in keep}
     if 0.0 < top_p < 1.0:
         cum = 0.0
-        kept = []
+        cut = keep[-1]
         for i in keep:
-            kept.append(i)
             cum += probs[i]
             if cum >= top_p:
+                cut = i
                 break
+        kept = [i for i in keep if float(logits[i]) >= float(logits[cut])]
         z = sum(probs[i] for i in kept)
         probs = {i: probs[i] / z for i in kept}
     out = torch.zeros(V, dtype=F64)

@@ -1,0 +1,170 @@
+"""The cache manager's books: no page lost, held twice or freed twice, under random orders of
+requests; windows give pages back; state slots follow the requests.  Host-only."""
+import random
+
+import pytest
+import torch
+
+from nanoinfer_amd.cache.block_manager import BlockManager, OutOfPages, PageError
+from nanoinfer_amd.cache.manager import CacheError, KVCacheManager, StateSlots
+from nanoinfer_amd.parts.base import CacheNeed, KVNeed, StateNeed
+
+
+def full(n_caches=2, kvh=2, hd=16):
+    return {c: CacheNeed(kv=KVNeed(kvh, hd)) for c in range(n_caches)}
+
+
+# ------------------------------------------------------------------ page ids
+
+def test_block_manager_order_and_reuse():
+    bm = BlockManager(4)
+    assert bm.allocate(2) == [0, 1]               # test/test_engine/test_block_manager.cpp:159-175
+    bm.free([1])
+    assert bm.allocate(1) == [1]                  # LIFO: the page freed last is handed out next
+    bm.free([0])
+    assert bm.allocate(3) == [0, 2, 3]
+    assert bm.num_free == 0 and bm.utilization() == 1.0
+
+
+def test_block_manager_all_or_nothing_and_double_free():
+    bm = BlockManager(3)
+    a = bm.allocate(2)
+    with pytest.raises(OutOfPages):
+        bm.allocate(2)
+    assert bm.num_free == 1                        # the failed call changed nothing
+    bm.free(a)
+    with pytest.raises(PageError):
+        bm.free([a[0]])                            # freed twice
+    with pytest.raises(PageError):
+        bm.free([7])                               # foreign id
+    b = bm.allocate(1)
+    with pytest.raises(PageError):
+        bm.free([b[0], b[0]])                      # twice in one call: nothing is freed
+    assert bm.is_taken(b[0]) and bm.num_free == 2
+    bm.reset()
+    assert bm.num_free == 3 and bm.allocate(1) == [0]
+
+
+# ------------------------------------------------------------------ reserve / release
+
+def test_pages_follow_tokens():
+    m = KVCacheManager(full(), page_size=16, num_pages=8, max_requests=4)
+    assert len(m.groups) == 1 and m.groups[0].cache_ids == [0, 1]        # same need, one group, one table
+    assert m.reserve("a", 17) and m.block_table(0, "a") == [0, 1]        # ceil(17 / 16)
+    assert m.reserve("a", 32) and m.block_table(0, "a") == [0, 1]        # still inside the second page
+    assert m.reserve("a", 33) and m.block_table(0, "a") == [0, 1, 2]
+    assert m.num_tokens("a") == 33 and m.free_pages() == 5
+    assert m.reserve("b", 1) and m.block_table(0, "b") == [3]
+    assert not m.reserve("b", 16 * 5 + 1)                                # five more pages, four free
+    assert m.block_table(0, "b") == [3] and m.num_tokens("b") == 1       # unchanged by the refusal
+    m.check()
+    m.release("a")
+    assert m.free_pages() == 7
+    assert m.reserve("c", 40) and m.block_table(0, "c") == [2, 1, 0]     # handed out again, last freed first
+    with pytest.raises(CacheError):
+        m.release("a")
+    with pytest.raises(CacheError):
+        m.reserve("c", 10)                                               # a request does not shrink
+    m.check()
+    m.reset()
+    assert m.free_pages() == 8 and not m.live_requests()
+
+
+def test_can_reserve_all_counts_the_whole_step():
+    m = KVCacheManager(full(), page_size=4, num_pages=5, max_requests=2)
+    assert m.can_reserve_all([("a", 8), ("b", 12)])
+    assert not m.can_reserve_all([("a", 9), ("b", 12)])
+    assert m.reserve("a", 8)
+    assert m.can_reserve_all([("a", 12), ("b", 8)]) and not m.can_reserve_all([("a", 12), ("b", 9)])
+    assert m.reserve("b", 1)
+    assert not m.can_reserve_all([("c", 1)])                             # no third state slot
+    assert not m.reserve("c", 1)
+    m.check()
+
+
+def test_groups_by_need_have_pages_of_their_own():
+    needs = {0: CacheNeed(kv=KVNeed(2, 16)), 1: CacheNeed(kv=KVNeed(2, 16, window=8)),
+             2: CacheNeed(kv=KVNeed(2, 16)), 3: CacheNeed(kv=KVNeed(1, 32)),
+             4: CacheNeed(state=StateNeed((3, 5)))}
+    m = KVCacheManager(needs, page_size=4, num_pages=6, max_requests=3)
+    assert [g.cache_ids for g in m.groups] == [[0, 2], [1], [3]]
+    assert m.reserve("a", 10)
+    assert [m.block_table(g, "a") for g in range(3)] == [[0, 1, 2]] * 3   # each group counts from its own 0
+    # the window group gives back what a query at position 10 cannot reach: keys before 3 -> no whole page yet
+    assert m.release_passed("a", 10) == 0
+    assert m.reserve("a", 14) and m.release_passed("a", 14) == 1          # first key needed 7 -> page 0 goes
+    assert m.block_table(1, "a") == [-1, 1, 2, 3] and m.block_table(0, "a") == [0, 1, 2, 3]
+    assert m.groups[1].pages.num_free == 3 and m.groups[0].pages.num_free == 2
+    assert m.reserve("a", 24) and m.release_passed("a", 24) == 3          # first key needed 17 -> pages 1..3 go
+    assert m.block_table(1, "a") == [-1, -1, -1, -1, 0, 4]                # page 0 came back and was used again first
+    m.check()
+    m.release("a")
+    assert all(g.pages.num_free == 6 for g in m.groups)
+    m.check()
+
+
+def test_state_slots_follow_requests():
+    slots = StateSlots(2)
+    assert slots.take("a") == 0 and slots.take("b") == 1
+    with pytest.raises(OutOfPages):
+        slots.take("c")
+    with pytest.raises(CacheError):
+        slots.take("a")
+    assert slots.give_back("a") == 0 and slots.take("c") == 0
+    with pytest.raises(CacheError):
+        slots.give_back("a")
+    # the manager hands a slot to every request even when no cache holds state
+    m = KVCacheManager(full(), page_size=4, num_pages=8, max_requests=2)
+    assert m.reserve("x", 1) and m.reserve("y", 1) and {m.state_slot("x"), m.state_slot("y")} == {0, 1}
+    m.release("x")
+    assert m.reserve("z", 1) and m.state_slot("z") == 0
+    assert not m.state                                                   # nothing to allocate for this model
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_keep_the_books(seed):
+    rng = random.Random(seed)
+    window = rng.choice([None, 6, 20])
+    needs = {0: CacheNeed(kv=KVNeed(2, 16)), 1: CacheNeed(kv=KVNeed(2, 16, window=window))}
+    ps = rng.choice([1, 4, 16])
+    m = KVCacheManager(needs, page_size=ps, num_pages=rng.randint(6, 20), max_requests=4)
+    live = {}
+    next_id = 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.25 and len(live) < 6:
+            rid, want = next_id, rng.randint(1, 3 * ps)
+            next_id += 1
+            before = [g.pages.num_free for g in m.groups]
+            if m.reserve(rid, want):
+                live[rid] = want
+                m.release_passed(rid, want)
+            else:
+                assert [g.pages.num_free for g in m.groups] == before and not m.has(rid)
+        elif op < 0.75 and live:
+            rid = rng.choice(list(live))
+            want = live[rid] + rng.randint(1, 2 * ps)
+            before = [list(m.block_table(g, rid)) for g in range(len(m.groups))]
+            if m.reserve(rid, want):
+                live[rid] = want
+                m.release_passed(rid, want)
+            else:
+                assert [m.block_table(g, rid) for g in range(len(m.groups))] == before
+        elif live:
+            rid = rng.choice(list(live))
+            m.release(rid)
+            del live[rid]
+        m.check()
+        for rid, n in live.items():
+            assert m.num_tokens(rid) == n
+            for g in m.groups:
+                table = g.tables[rid]
+                assert len(table) == m.pages_for(n)
+                first = g.first_needed_page(n)
+                assert all(p >= 0 for p in table[first:])               # everything still readable is there
+                if g.need.window is not None:
+                    assert all(p == -1 for p in table[:first])           # everything passed has been given back
+    for rid in list(live):
+        m.release(rid)
+    m.check()
+    assert all(g.pages.num_free == g.pages.num_pages for g in m.groups) and m.slots.num_free == 4

@@ -1,0 +1,266 @@
+"""Replay of the same requests cut in different ways, in float32 and bfloat16, against the plain
+implementation: whole; most in one step and the last 32 tokens one by one; portions of changing
+size down to two tokens; mixed with other requests on so few pages that they are used again.
+Driven through ModelRunner.step in-process, and through bin/trace_run as a user would."""
+import json
+import os
+import random
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_common import TOL, assert_close, model_folder, plain_logits, random_tokens
+from tiny_configs import ALL
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PAGE = {"A": 16, "B": 8, "C": 4}
+LENGTHS = {"A": (7, 19, 33, 70), "B": (1, 40, 77, 130, 200), "C": (2, 50, 65, 97)}
+
+
+# ------------------------------------------------------------------ traces
+
+def whole(requests):
+    return [([(rid, list(toks), list(range(len(toks))))], [rid]) for rid, toks in requests.items()]
+
+
+def tail_one_by_one(requests, tail=32):
+    steps = []
+    for rid, toks in requests.items():
+        n = len(toks)
+        head = max(1, n - tail)
+        steps.append(([(rid, list(toks[:head]), list(range(head)))], []))
+        for i in range(head, n):
+            steps.append(([(rid, [toks[i]], [0])], [rid] if i == n - 1 else []))
+        if head == n:
+            steps[-1] = (steps[-1][0], [rid])
+    return steps
+
+
+def changing_portions(requests, sizes=(7, 2, 13, 3, 2, 29, 5, 2, 64, 11)):
+    steps = []
+    for rid, toks in requests.items():
+        at, k = 0, 0
+        while at < len(toks):
+            n = min(sizes[k % len(sizes)], len(toks) - at)
+            if len(toks) - at - n == 1:      # never leave a single token: the smallest portion is two
+                n += 1
+            k += 1
+            steps.append(([(rid, list(toks[at:at + n]), list(range(n)))], [rid] if at + n == len(toks) else []))
+            at += n
+    return steps
+
+
+def mixed(requests, seed, max_live=4):
+    """Up to ``max_live`` requests at a time: some bring a portion of their prompt (a random first
+    part of the request counts as prompt), others single tokens; a request may sit a step out."""
+    rng = random.Random(seed)
+    waiting = list(requests.items())
+    live = {}     # rid -> [tokens, done, prompt_len]
+    steps = []
+    while waiting or live:
+        while waiting and len(live) < max_live and (not live or rng.random() < 0.6):
+            rid, toks = waiting.pop(0)
+            live[rid] = [list(toks), 0, rng.randint(1, len(toks))]
+        entries, ended = [], []
+        for rid in list(live):
+            toks, done, plen = live[rid]
+            if len(live) > 1 and rng.random() < 0.2:
+                continue                      # left out of this step, goes on later
+            if done < plen:
+                n = min(plen - done, rng.choice([2, 3, 5, 8, 17, 40]))
+                if plen - done - n == 1 and done + n + 1 <= len(toks):
+                    n += 1
+            else:
+                n = 1
+            want = sorted(rng.sample(range(n), rng.randint(0, n))) if n > 1 else [0]
+            entries.append((rid, toks[done:done + n], want))
+            live[rid][1] = done + n
+            if done + n == len(toks):
+                ended.append(rid)
+                del live[rid]
+        if entries:
+            steps.append((entries, ended))
+    return steps
+
+
+def max_live_tokens(steps, requests, page):
+    """The most tokens live requests hold at once, each rounded up to a multiple of 64."""
+    held, worst = {}, 0
+    for entries, ended in steps:
+        for rid, toks, _ in entries:
+            held[rid] = held.get(rid, 0) + len(toks)
+        worst = max(worst, sum(-(-n // 64) * 64 for n in held.values()))
+        for rid in ended:
+            del held[rid]
+    return worst
+
+
+def run_in_process(folder, dtype, page, steps, max_tokens):
+    from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
+
+    runner = ModelRunner(folder, dtype=dtype, page_size=page, max_tokens=max_tokens, max_requests=4)
+    got = {}
+    given_back = set()      # pages that some finished request held
+    reused = False
+    for entries, ended in steps:
+        out = runner.step([StepEntry(r, t, w) for r, t, w in entries], end=())
+        row = 0
+        for r, t, w in entries:
+            reused = reused or any(p in given_back for p in runner.cache.block_table(0, r))
+            base = runner.computed_tokens(r) - len(t)
+            for i in w:
+                got[(r, base + i)] = out[row].clone()
+                row += 1
+        assert (out is None and row == 0) or out.shape[0] == row
+        for r in ended:
+            given_back.update(runner.cache.block_table(0, r))
+            runner.release(r)
+    runner.cache.check()
+    assert runner.cache.free_pages() == runner.cache.num_pages and not runner.cache.live_requests()
+    return got, reused
+
+
+def compare(got, requests, folder, dtype, what):
+    assert got, "nothing was compared"
+    by_request = {}
+    for (rid, pos), row in got.items():
+        by_request.setdefault(rid, []).append((pos, row))
+    for rid, rows in by_request.items():
+        want = plain_logits(folder, tuple(requests[rid]), dtype)
+        rows.sort(key=lambda x: x[0])
+        idx = [p for p, _ in rows]
+        assert_close(torch.stack([r for _, r in rows]), want[idx], dtype, f"{what}, request {rid}, positions {idx[0]}..{idx[-1]}")
+
+
+def make_requests(name, seed=0):
+    vocab = ALL[name]["vocab_size"]
+    return {f"r{i}": random_tokens(vocab, n, seed * 100 + i) for i, n in enumerate(LENGTHS[name])}
+
+
+# ------------------------------------------------------------------ tests
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_each_request_alone_and_whole(name, dtype):
+    folder, requests = model_folder(name), make_requests(name)
+    steps = whole(requests)
+    got, _ = run_in_process(folder, dtype, PAGE[name], steps, max_live_tokens(steps, requests, PAGE[name]))
+    assert len(got) == sum(len(t) for t in requests.values())
+    compare(got, requests, folder, dtype, f"{name} whole")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_last_32_tokens_one_by_one(name, dtype):
+    folder, requests = model_folder(name), make_requests(name)
+    steps = tail_one_by_one(requests)
+    got, _ = run_in_process(folder, dtype, PAGE[name], steps, max_live_tokens(steps, requests, PAGE[name]))
+    assert len(got) == sum(len(t) for t in requests.values())
+    compare(got, requests, folder, dtype, f"{name} tail")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_portions_of_changing_size(name, dtype):
+    folder, requests = model_folder(name), make_requests(name)
+    steps = changing_portions(requests)
+    assert min(len(t) for e, _ in steps for _, t, _ in e if len(t) > 1) == 2
+    got, _ = run_in_process(folder, dtype, PAGE[name], steps, max_live_tokens(steps, requests, PAGE[name]))
+    compare(got, requests, folder, dtype, f"{name} portions")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_requests_on_few_pages(name, dtype):
+    folder = model_folder(name)
+    vocab = ALL[name]["vocab_size"]
+    lengths = list(LENGTHS[name]) + [23, 64, 5, 48, 100]
+    requests = {f"m{i}": random_tokens(vocab, n, 500 + i) for i, n in enumerate(lengths)}
+    steps = mixed(requests, seed=11)
+    assert max(len(e) for e, _ in steps) == 4                          # four live at once did happen
+    assert any(len(e) > 1 and any(len(t) > 1 for _, t, _ in e) and any(len(t) == 1 for _, t, _ in e) for e, _ in steps)
+    got, reused = run_in_process(folder, dtype, PAGE[name], steps, max_live_tokens(steps, requests, PAGE[name]))
+    assert reused, "the pool was large enough that no page was used twice"
+    compare(got, requests, folder, dtype, f"{name} mixed")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(dtype):
+    """A short prompt, then some four hundred tokens one at a time: positions far beyond the prompt,
+    many page boundaries, the split key range of the decode path."""
+    name = "B"
+    folder = model_folder(name)
+    toks = random_tokens(ALL[name]["vocab_size"], 420, 77)
+    steps = [([("long", list(toks[:3]), [0, 1, 2])], [])]
+    steps += [([("long", [t], [0])], []) for t in toks[3:]]
+    steps[-1] = (steps[-1][0], ["long"])
+    got, _ = run_in_process(folder, dtype, PAGE[name], steps, 448)
+    compare(got, {"long": toks}, folder, dtype, "long decoding")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens_of_a_sequence(name, dtype):
+    """Position 0 alone, then 1, then 2: a context of one key, the first page's first slots."""
+    folder = model_folder(name)
+    toks = random_tokens(ALL[name]["vocab_size"], 4, 5)
+    steps = [([("f", [t], [0])], []) for t in toks]
+    got, _ = run_in_process(folder, dtype, PAGE[name], steps + [([], ["f"])], 64)
+    compare(got, {"f": toks}, folder, dtype, "first tokens")
+    steps = [([("g", list(toks[:1]), [0]), ("h", list(toks[:2]), [0, 1])], ["g", "h"])]
+    got, _ = run_in_process(folder, dtype, PAGE[name], steps, 128)
+    compare(got, {"g": toks[:1], "h": toks[:2]}, folder, dtype, "two short requests")
+
+
+def test_stored_bfloat16_weights_give_the_same_logits_in_both_stores():
+    """A folder stored in bfloat16 and run in float32 uses exactly the stored values."""
+    folder = model_folder("A", stored="bfloat16")
+    requests = {"x": random_tokens(256, 40, 3)}
+    for dtype in ("float32", "bfloat16"):
+        got, _ = run_in_process(folder, dtype, 16, whole(requests), 64)
+        compare(got, requests, folder, dtype, f"stored bf16 run {dtype}")
+
+
+# ------------------------------------------------------------------ the program, as a user runs it
+
+def run_trace_program(folder, dtype, steps, max_tokens, out_dir, extra=()):
+    lines = [json.dumps({"step": i, "entries": [{"id": r, "tokens": list(t), "want": list(w)} for r, t, w in entries],
+                         "end": ended}) for i, (entries, ended) in enumerate(steps)]
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", out_dir,
+           "--max-tokens", str(max_tokens), *extra]
+    proc = subprocess.run(cmd, input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done ")] == [f"done {i}" for i in range(len(steps))]
+    return proc
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(dtype, tmp_path):
+    name = "B"
+    folder = model_folder(name)
+    vocab = ALL[name]["vocab_size"]
+    requests = {f"t{i}": random_tokens(vocab, n, 900 + i) for i, n in enumerate((30, 64, 90, 12, 57, 101))}
+    steps = mixed(requests, seed=5)
+    out_dir = str(tmp_path / "out")
+    run_trace_program(folder, dtype, steps, max_live_tokens(steps, requests, 16), out_dir)
+    held, got = {}, {}
+    for i, (entries, ended) in enumerate(steps):
+        n_want = sum(len(w) for _, _, w in entries)
+        path = os.path.join(out_dir, f"{i}.f32")
+        if n_want == 0:
+            assert not os.path.exists(path)
+        else:
+            data = np.fromfile(path, dtype="<f4").reshape(n_want, vocab)
+        row = 0
+        for r, t, w in entries:
+            base = held.get(r, 0)
+            for j in w:
+                got[(r, base + j)] = torch.from_numpy(data[row].copy())
+                row += 1
+            held[r] = base + len(t)
+    compare(got, requests, folder, dtype, "trace_run mixed")

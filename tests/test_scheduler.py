@@ -1,0 +1,221 @@
+"""The scheduler's decisions, and the engine loop over a runner and a sampler that need no GPU.
+
+The fake runner keeps real cache books (a KVCacheManager without pools) and returns logits whose
+argmax is a known function of the request, as the reference's mock model does with a fixed
+argmax of 3 (test/test_engine/test_engine.cpp:11-80)."""
+import pytest
+import torch
+
+from nanoinfer_amd.cache.block_manager import OutOfPages
+from nanoinfer_amd.cache.manager import KVCacheManager
+from nanoinfer_amd.engine.llm import Engine
+from nanoinfer_amd.engine.scheduler import EngineConfig, RequestRefused, RequestState, Scheduler
+from nanoinfer_amd.parts.base import CacheNeed, KVNeed
+from nanoinfer_amd.sampling.params import SamplingParams
+
+VOCAB = 50
+
+
+class FakeRunner:
+    """Books like the real runner; logits put the mass on (last token + 1) % VOCAB."""
+
+    def __init__(self, page_size=4, num_pages=16, max_requests=8, max_positions=1000, eos=()):
+        self.cache = KVCacheManager({0: CacheNeed(kv=KVNeed(1, 16))}, page_size, num_pages, max_requests)
+        self.device = torch.device("cpu")
+        self.vocab_size = VOCAB
+        self.max_positions = max_positions
+        self.eos_token_ids = tuple(eos)
+        self._done = {}
+        self.steps = []          # [(request, n_tokens, wants)] of every step, for the assertions
+
+    def release(self, request):
+        if request in self._done:
+            del self._done[request]
+            self.cache.release(request)
+
+    def step(self, entries, end=()):
+        totals = [(e.request, self._done.get(e.request, 0) + len(e.tokens)) for e in entries]
+        if not self.cache.can_reserve_all(totals):
+            raise OutOfPages("fake runner: the scheduler planned more than the cache holds")
+        rows = []
+        for e, (_, total) in zip(entries, totals):
+            assert self.cache.reserve(e.request, total)
+            self._done[e.request] = total
+            for w in e.want:
+                row = torch.zeros(VOCAB)
+                row[(int(e.tokens[w]) + 1) % VOCAB] = 5.0
+                rows.append(row)
+        self.steps.append([(e.request, len(e.tokens), list(e.want)) for e in entries])
+        self.cache.check()
+        return torch.stack(rows) if rows else None
+
+
+class ArgmaxSampler:
+    def sample(self, logits, params, generated, counters):
+        assert len(params) == len(generated) == len(counters) == logits.shape[0]
+        return logits.argmax(dim=-1).tolist()
+
+
+def make_engine(**kw):
+    runner_kw = {k: kw.pop(k) for k in list(kw) if k in ("page_size", "num_pages", "max_requests", "max_positions", "eos")}
+    runner = FakeRunner(**runner_kw)
+    cfg = EngineConfig(block_size=runner.cache.page_size, num_cache_blocks=runner.cache.num_pages, **kw)
+    return Engine(config=cfg, runner=runner, sampler=ArgmaxSampler()), runner
+
+
+def test_first_token_comes_with_the_last_prompt_portion():
+    # test/test_engine/test_engine.cpp:121-143: prefill yields the first token in the same step
+    eng, runner = make_engine()
+    rid = eng.add_request([7, 8, 9], max_new_tokens=3, params=SamplingParams.greedy())
+    assert eng.get_request(rid).state == RequestState.WAITING
+    assert eng.step() == []
+    r = eng.get_request(rid)
+    assert r.generated == [10] and r.num_computed == 3 and r.state == RequestState.RUNNING
+    assert runner.steps[0] == [(rid, 3, [2])]
+    eng.step()                                     # one token per decode step (test_engine.cpp:145-163)
+    assert r.generated == [10, 11] and runner.steps[1] == [(rid, 1, [0])]
+    done = eng.step()
+    assert [d.request_id for d in done] == [rid] and r.generated == [10, 11, 12] and r.finish_reason == "length"
+    assert not eng.has_work() and not runner.cache.live_requests()        # pages and slot are back
+    # the last sampled token is never fed: 1 prompt step + 2 decode steps for 3 tokens
+    assert len(runner.steps) == 3
+
+
+def test_running_first_then_fcfs_fill():
+    # test/test_engine/test_scheduler.cpp:78-117
+    eng, runner = make_engine(max_batch_size=2, num_pages=64)
+    a = eng.add_request([1, 2], 4)
+    b = eng.add_request([3], 4)
+    c = eng.add_request([4], 4)
+    for r in (a, b, c):
+        eng.get_request(r).params = SamplingParams.greedy()
+    eng.step()
+    assert [x[0] for x in runner.steps[0]] == [a, b]          # the batch cap keeps c waiting
+    eng.step()
+    assert [x[0] for x in runner.steps[1]] == [a, b]          # running requests come first, every step
+    assert eng.scheduler.stats()["num_waiting"] == 1
+    eng.run()
+    assert [eng.get_request(r).finish_reason for r in (a, b, c)] == ["length"] * 3
+    first_c = next(i for i, s in enumerate(runner.steps) if any(x[0] == c for x in s))
+    assert first_c == 4                                       # c enters when a and b have finished (4 steps each)
+
+
+def test_max_sequences_caps_running_requests():
+    eng, runner = make_engine(max_sequences=1, num_pages=64)
+    a, b = eng.add_request([1], 2), eng.add_request([2], 2)
+    eng.step()
+    assert eng.scheduler.stats()["num_running"] == 1 and eng.scheduler.stats()["num_waiting"] == 1
+    eng.run()
+    assert all(len(s) == 1 for s in runner.steps)
+
+
+def test_token_budget_cuts_prompts_into_portions():
+    eng, runner = make_engine(max_num_batched_tokens=8, prefill_chunk_size=6, num_pages=64)
+    a = eng.add_request(list(range(1, 11)), 2)                # 10 prompt tokens
+    b = eng.add_request(list(range(20, 25)), 2)               # 5 prompt tokens
+    for r in (a, b):
+        eng.get_request(r).params = SamplingParams.greedy()
+    eng.step()
+    assert runner.steps[0] == [(a, 6, []), (b, 2, [])]        # chunk cap 6, then what is left of the budget
+    eng.step()
+    # a's rest (4, sampling) and b's rest (3, sampling): both portions end at the prompt's last token
+    assert runner.steps[1] == [(a, 4, [3]), (b, 3, [2])]
+    eng.step()
+    assert runner.steps[2] == [(a, 1, [0]), (b, 1, [0])]
+    assert all(sum(n for _, n, _ in s) <= 8 for s in runner.steps)
+
+
+def test_decode_tokens_go_before_prompt_portions():
+    eng, runner = make_engine(max_num_batched_tokens=5, prefill_chunk_size=4, num_pages=64)
+    a = eng.add_request(list(range(12)), 3)
+    eng.step()                                                # a: 4 of 12
+    b = eng.add_request([1], 3)
+    eng.step()                                                # a: 4 more; b admitted with 1 token
+    assert runner.steps[1] == [(a, 4, []), (b, 1, [0])]
+    eng.step()                                                # b decodes first, a gets the rest of the budget
+    assert runner.steps[2] == [(b, 1, [0]), (a, 4, [3])]
+
+
+def test_stop_token_ends_a_request_and_is_kept():
+    # src/engine/inference_request.cpp:61-73: the stop token is appended, then the request ends
+    eng, runner = make_engine(eos=(12,), num_pages=64)
+    rid = eng.add_request([9], 10, SamplingParams.greedy())
+    eng.run()
+    r = eng.get_request(rid)
+    assert r.generated == [10, 11, 12] and r.finish_reason == "stop"
+
+
+def test_requests_that_can_never_fit_are_refused():
+    eng, runner = make_engine(page_size=4, num_pages=4, max_positions=1000)      # 16 tokens in all
+    with pytest.raises(RequestRefused):
+        eng.add_request(list(range(10)), 8)                   # 10 + 8 - 1 = 17 > 16
+    eng.add_request(list(range(10)), 7)                       # 16 fits
+    with pytest.raises(RequestRefused):
+        eng.add_request([], 3)
+    with pytest.raises(RequestRefused):
+        eng.add_request([1], 0)
+    with pytest.raises(ValueError):
+        eng.add_request([VOCAB], 3)
+    eng2, _ = make_engine(num_pages=64, max_positions=12)
+    with pytest.raises(RequestRefused):
+        eng2.add_request(list(range(10)), 4)                  # the model's positions end at 12
+    eng3, _ = make_engine(num_pages=64, max_model_len=8)
+    with pytest.raises(RequestRefused):
+        eng3.add_request(list(range(8)), 2)
+
+
+def test_waiting_request_waits_for_pages():
+    eng, runner = make_engine(page_size=4, num_pages=4)       # 16 tokens
+    a = eng.add_request(list(range(9)), 4, SamplingParams.greedy())    # 3 pages
+    b = eng.add_request(list(range(7)), 2, SamplingParams.greedy())    # 2 pages: does not fit beside a
+    eng.step()
+    assert [x[0] for x in runner.steps[0]] == [a] and eng.get_request(b).state == RequestState.WAITING
+    eng.run()
+    assert eng.scheduler.num_preemptions == 0
+    assert eng.get_request(b).generated == [7, 8] and eng.get_request(a).generated == [9, 10, 11, 12]
+
+
+def test_running_out_of_pages_preempts_the_youngest():
+    eng, runner = make_engine(page_size=4, num_pages=4, max_num_batched_tokens=64)
+    a = eng.add_request([1, 2, 3, 4, 5, 6, 7], 9, SamplingParams.greedy())   # 7 -> 15 tokens: ends in 4 pages
+    b = eng.add_request([11, 12, 13, 14, 15, 16, 17], 9, SamplingParams.greedy())
+    eng.step()                                                # both admitted: 2 pages each, pool full
+    assert [x[0] for x in runner.steps[0]] == [a, b]
+    eng.step()                                                # position 7 still lies in each one's second page
+    assert eng.scheduler.num_preemptions == 0
+    eng.step()                                                # position 8 needs a third page: b, the youngest, gives way
+    rb = eng.get_request(b)
+    assert eng.scheduler.num_preemptions == 1 and rb.preemptions == 1
+    assert rb.state == RequestState.WAITING and rb.num_computed == 0 and eng.scheduler.waiting[0] is rb
+    assert rb.generated == [18, 19] and [x[0] for x in runner.steps[2]] == [a]      # what b generated is kept
+    assert not runner.cache.has(b)
+    eng.run()
+    ra = eng.get_request(a)
+    assert ra.generated == list(range(8, 17)) and rb.generated == list(range(18, 27))
+    assert ra.finish_reason == rb.finish_reason == "length"
+    # b was recomputed from position 0 with its generated tokens as part of the prompt
+    again = [s for s in runner.steps if any(x[0] == b and x[1] > 1 for x in s)]
+    assert len(again) == 2 and again[1][0][1] == 9            # 7 prompt + 2 generated
+    assert not runner.cache.live_requests() and runner.cache.free_pages() == 4
+
+
+def test_engine_never_plans_more_than_fits():
+    """Random traffic on a small pool: every step the runner can reserve what was planned (the
+    fake runner raises otherwise), every request finishes with the right tokens."""
+    import random
+    rng = random.Random(0)
+    eng, runner = make_engine(page_size=4, num_pages=12, max_requests=6, max_sequences=6, max_batch_size=4,
+                              max_num_batched_tokens=16, prefill_chunk_size=8)
+    want = {}
+    for _ in range(40):
+        for _ in range(rng.randint(0, 2)):
+            prompt = [rng.randrange(VOCAB) for _ in range(rng.randint(1, 20))]
+            n = rng.randint(1, 12)
+            rid = eng.add_request(prompt, n, SamplingParams.greedy())
+            want[rid] = [(prompt[-1] + 1 + i) % VOCAB for i in range(n)]
+        eng.step()
+    eng.run()
+    for rid, tokens in want.items():
+        assert eng.get_request(rid).generated == tokens
+    assert runner.cache.free_pages() == 12 and eng.scheduler.stats()["num_finished"] == len(want)
+    assert all(len(s) <= 4 and sum(n for _, n, _ in s) <= 16 for s in runner.steps)
