@@ -122,7 +122,7 @@ def library_path(name: str, sources: List[str], defines: Optional[Dict[str, obje
 # What the framework is made of.  Attention is compiled per head size.
 CORE = ("ni_ops", ["ops.hip"], {})
 SAMPLING = ("ni_sampling", ["sampling.hip"], {})
-COMMON_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128)
+COMMON_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)
 
 
 def attention_target(head_dim: int):

@@ -1,0 +1,344 @@
+"""Each HIP kernel alone against its plain reference, at sizes other than the engine's tests use:
+widths and vocabularies that are no power of two, head sizes in steps of 16, odd page sizes."""
+import math
+import random
+
+import pytest
+import torch
+
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+# kernels do float32 arithmetic on exactly the given inputs; what is left is summation order
+# (float32) plus the rounding of the stored result (bfloat16: 2^-9 relative)
+KTOL = {"float32": 3e-6, "bfloat16": 6e-3}
+
+
+def dev(t, dtype=None):
+    return t.to("cuda", dtype) if dtype is not None else t.to("cuda")
+
+
+def rel(got, want):
+    return float((got.double().cpu() - want.double()).abs().max() / max(1e-30, float(want.double().abs().max())))
+
+
+@pytest.fixture(scope="module")
+def K():
+    from nanoinfer_amd import kernels
+    return kernels
+
+
+def test_missing_gpu_tensor_is_refused(K):
+    with pytest.raises(K.KernelError):
+        K.embedding(torch.zeros(2, dtype=torch.int32), torch.zeros(4, 4), torch.zeros(2, 4))
+    with pytest.raises(Exception) as e:
+        K.attention_lib(40)                       # not a multiple of 16: refused with a reason, never run
+    assert "multiple of 16" in str(e.value)
+    with pytest.raises(Exception):
+        K.attention_lib(272)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embedding(K, dtype):
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn(1003, 70, generator=g).to(DT[dtype])
+    ids = torch.randint(0, 1003, (37,), generator=g).to(torch.int32)
+    out = K.embedding(dev(ids), dev(table), torch.empty(37, 70, device="cuda"))
+    assert torch.equal(out.cpu(), P.embedding(table.float(), ids.tolist()).float())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("d", [1, 50, 257, 2048, 4100])
+def test_add_rmsnorm(K, dtype, d):
+    g = torch.Generator().manual_seed(d)
+    T = 9
+    h = torch.randn(T, d, generator=g) * 3
+    pending = torch.randn(T, d, generator=g).to(DT[dtype])
+    w = 1 + 0.1 * torch.randn(d, generator=g)
+    eps = 3e-6
+    hd, out = dev(h.clone()), torch.empty(T, d, device="cuda", dtype=DT[dtype])
+    K.add_rmsnorm(hd, dev(pending), dev(w), eps, out)
+    total = h.double() + pending.double()
+    assert rel(hd, total) < 1e-6                                     # the residual stream moved on, in float32
+    assert rel(out, P.rmsnorm(total, w, eps)) < KTOL[dtype]
+    # reference vector: [1..d], weight 1 (test/test_op/test_layer_rmsnorm.cpp:112-136)
+    x = torch.arange(1, d + 1, dtype=torch.float32)[None]
+    out1 = K.add_rmsnorm(dev(x.clone()), None, dev(torch.ones(d)), 1e-5, torch.empty(1, d, device="cuda", dtype=DT[dtype]))
+    assert rel(out1, x.double() / math.sqrt(float((x.double() ** 2).mean()) + 1e-5)) < KTOL[dtype]
+    # gathered rows leave h alone and may repeat a row
+    rows = torch.tensor([4, 0, 4, 8], dtype=torch.int32)
+    hd2 = dev(h.clone())
+    out2 = K.add_rmsnorm(hd2, dev(pending), dev(w), eps, torch.empty(4, d, device="cuda", dtype=DT[dtype]), dev(rows))
+    assert torch.equal(hd2.cpu(), h)
+    assert rel(out2, P.rmsnorm(total[rows.long()], w, eps)) < KTOL[dtype]
+
+
+def test_rope_table_matches_plain(K):
+    from nanoinfer_amd.parts.standard import rope_inverse_frequencies
+    scaling = {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": 128}
+    for hd, theta, sc in [(48, 10000.0, None), (64, 500000.0, scaling), (16, 1234.5, scaling)]:
+        inv = rope_inverse_frequencies(hd, theta, sc)
+        assert (inv == P.rope_frequencies(hd, theta, sc)).all()          # bit for bit: same float32 steps
+        cos, sin = K.rope_table(dev(torch.from_numpy(inv)), 3000)
+        s, c = P.rope_tables(range(3000), inv)
+        assert float((sin.double().cpu() - s).abs().max()) < 2e-6 and float((cos.double().cpu() - c).abs().max()) < 2e-6
+
+
+def plain_rotate_half(x, sin, cos, rot):
+    """[T, heads, hd] with pairs (j, j + rot/2) inside the first rot dims."""
+    half = rot // 2
+    x = x.double()
+    out = x.clone()
+    s, c = sin[:, None, :], cos[:, None, :]
+    out[..., :half] = x[..., :half] * c - x[..., half:rot] * s
+    out[..., half:rot] = x[..., :half] * s + x[..., half:rot] * c
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,KVH,hd,rot,ps", [(4, 2, 16, 16, 4), (6, 1, 32, 32, 8), (5, 5, 48, 24, 5), (8, 2, 128, 128, 16)])
+def test_rope_and_cache_write(K, dtype, H, KVH, hd, rot, ps):
+    g = torch.Generator().manual_seed(hd)
+    T, pages = 11, 9
+    qkv = torch.randn(T, (H + 2 * KVH) * hd, generator=g).to(DT[dtype])
+    positions = torch.tensor([0, 1, 2, 3, 40, 41, 7, 300, 301, 302, 5], dtype=torch.int32)
+    inv = P.rope_frequencies(rot, 10000.0, None)
+    cos, sin = K.rope_table(dev(torch.from_numpy(inv)), 512)
+    slots = torch.tensor(random.Random(0).sample(range(pages * ps), T), dtype=torch.int32)
+    kpool = torch.full((pages, KVH, ps, hd), 9.0, dtype=DT[dtype], device="cuda")
+    vpool = torch.full((pages, KVH, ps, hd), 9.0, dtype=DT[dtype], device="cuda")
+    buf = dev(qkv.clone())
+    K.rope_kv_write(buf, dev(positions), cos, sin, dev(slots), kpool, vpool, H, KVH, hd)
+    s, c = P.rope_tables(positions.tolist(), inv)
+    q_ref = plain_rotate_half(qkv[:, :H * hd].reshape(T, H, hd), s, c, rot)
+    k_ref = plain_rotate_half(qkv[:, H * hd:(H + KVH) * hd].reshape(T, KVH, hd), s, c, rot)
+    v_ref = qkv[:, (H + KVH) * hd:].reshape(T, KVH, hd).double()
+    assert rel(buf[:, :H * hd].reshape(T, H, hd), q_ref) < KTOL[dtype]
+    assert torch.equal(buf[:, H * hd:].cpu(), qkv[:, H * hd:])                       # k and v columns are left as they were
+    kp, vp = kpool.cpu(), vpool.cpu()
+    touched = torch.zeros(pages, ps, dtype=torch.bool)
+    for t in range(T):
+        page, off = int(slots[t]) // ps, int(slots[t]) % ps
+        touched[page, off] = True
+        assert rel(kp[page, :, off, :], k_ref[t]) < KTOL[dtype]
+        assert torch.equal(vp[page, :, off, :].double(), v_ref[t])
+    assert bool((kp.float()[~touched[:, None, :].expand(pages, KVH, ps)] == 9.0).all())   # nothing else was written
+    # the flat address is ((page * KVH + head) * page_size + slot) * hd, the pool's declared order
+    t0 = 3
+    page, off = int(slots[t0]) // ps, int(slots[t0]) % ps
+    flat = vpool.view(-1)
+    addr = ((page * KVH + (KVH - 1)) * ps + off) * hd
+    assert torch.equal(flat[addr:addr + hd].cpu().double(), v_ref[t0, KVH - 1])
+
+
+def test_rope_quarter_turn_vector(K):
+    # test/test_cuda_kernel/test_rope_kernel.cpp:20-118 in this engine's pairing: sin 1, cos 0 turns (2, 2) into (-2, 2)
+    qkv = torch.full((1, 3 * 16), 2.0, device="cuda")
+    cos = torch.zeros(2, 8, device="cuda")
+    sin = torch.ones(2, 8, device="cuda")
+    K.rope_kv_write(qkv, dev(torch.tensor([1], dtype=torch.int32)), cos, sin, None, None, None, 1, 1, 16)
+    assert torch.equal(qkv[0, :8].cpu(), torch.full((8,), -2.0)) and torch.equal(qkv[0, 8:16].cpu(), torch.full((8,), 2.0))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_swiglu(K, dtype):
+    g = torch.Generator().manual_seed(1)
+    gu = (torch.randn(7, 2 * 137, generator=g) * 3).to(DT[dtype])
+    out = K.swiglu(dev(gu), torch.empty(7, 137, device="cuda", dtype=DT[dtype]))
+    assert rel(out, P.swiglu(gu[:, :137].double(), gu[:, 137:].double())) < KTOL[dtype]
+    one = K.swiglu(torch.ones(1, 2, device="cuda"), torch.empty(1, 1, device="cuda"))
+    assert abs(float(one) - 0.7310586) < 1e-6                          # test/test_op/test_layer_swiglu.cpp:65-108
+
+
+# ------------------------------------------------------------------ attention over pages
+
+def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boost=None):
+    """Sequences of ``lens`` keys each; the last ``q_lens`` of each are this step's queries.  The
+    cache is filled through a shuffled block table; everything else in the pools is NaN so that a
+    read outside a sequence's own keys poisons the result."""
+    rng = random.Random(seed)
+    g = torch.Generator().manual_seed(seed)
+    B = len(lens)
+    pages_per = [-(-n // ps) for n in lens]
+    total_pages = sum(pages_per) + 3
+    ids = list(range(total_pages))
+    rng.shuffle(ids)
+    width = max(pages_per)
+    table = torch.full((B, width), -1, dtype=torch.int32)
+    kpool = torch.full((total_pages, KVH, ps, hd), float("nan"))
+    vpool = torch.full((total_pages, KVH, ps, hd), float("nan"))
+    ks, vs, qs, seq_of, positions = [], [], [], [], []
+    at = 0
+    for b, n in enumerate(lens):
+        k = torch.randn(n, KVH, hd, generator=g).to(DT[dtype]).float()
+        v = torch.randn(n, KVH, hd, generator=g).to(DT[dtype]).float()
+        q = torch.randn(n, H, hd, generator=g).to(DT[dtype]).float()
+        if boost is not None:
+            bb, key_at, query_at, factor = boost
+            if bb == b:
+                k[key_at] *= factor
+                q[query_at] = k[key_at].repeat_interleave(H // KVH, 0) / factor * 4
+        for p in range(pages_per[b]):
+            table[b, p] = ids[at]
+            lo, hi = p * ps, min(n, (p + 1) * ps)
+            kpool[ids[at], :, :hi - lo] = k[lo:hi].transpose(0, 1)
+            vpool[ids[at], :, :hi - lo] = v[lo:hi].transpose(0, 1)
+            at += 1
+        ks.append(k), vs.append(v), qs.append(q)
+        for i in range(n - q_lens[b], n):
+            seq_of.append(b), positions.append(i)
+    T = len(seq_of)
+    qkv = torch.zeros(T, (H + 2 * KVH) * hd)
+    row = 0
+    for b, n in enumerate(lens):
+        for i in range(n - q_lens[b], n):
+            qkv[row, :H * hd] = qs[b][i].reshape(-1)
+            row += 1
+    out = torch.empty(T, H * hd, device="cuda", dtype=DT[dtype])
+    ws = torch.empty(max(1, T * H * nsplit * (hd + 2)), device="cuda") if nsplit > 1 else None
+    K.token_attention(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table),
+                      dev(torch.tensor(seq_of, dtype=torch.int32)), dev(torch.tensor(positions, dtype=torch.int32)),
+                      out, H, KVH, hd, 1.0 / math.sqrt(hd), window, nsplit, ws)
+    want = torch.cat([P.causal_attention(qs[b], ks[b], vs[b], range(n), window=window)[n - q_lens[b]:].reshape(q_lens[b], H * hd)
+                      for b, n in enumerate(lens)])
+    return out, want, (qs, ks, vs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,KVH,hd,ps", [(4, 2, 16, 16), (6, 1, 32, 8), (5, 5, 48, 5), (32, 8, 64, 16), (3, 3, 80, 16),
+                                         (8, 2, 96, 4), (2, 1, 112, 16), (16, 2, 128, 16), (2, 2, 256, 16)])
+def test_attention_head_sizes_and_groups(K, dtype, H, KVH, hd, ps):
+    lens, q_lens = [1, 37, 130, 64], [1, 37, 2, 1]
+    for nsplit in (1, 3):
+        out, want, _ = paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, None, hd + nsplit, nsplit)
+        assert not torch.isnan(out).any(), "a key outside the sequence's own pages was read"
+        assert rel(out, want) < KTOL[dtype], (H, KVH, hd, ps, nsplit)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_window_edges(K, dtype):
+    for window in (1, 7, 16, 33):
+        out, want, _ = paged_case(K, dtype, 4, 2, 32, 8, [50, 9, 33], [50, 9, 2], window, window, 1)
+        assert not torch.isnan(out).any()
+        assert rel(out, want) < KTOL[dtype], window
+    out, want, _ = paged_case(K, dtype, 4, 2, 32, 8, [300], [1], 200, 3, 4)
+    assert rel(out, want) < KTOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_finds_a_far_key_among_hundreds(K, dtype):
+    """One early key is made to match the last query: the output must be that key's value, which
+    random keys would never show.  Key 37 sits in the middle of a page, key 16 on a page's first
+    slot, key 15 on a page's last; splits cut the range in other places."""
+    for key_at in (37, 16, 15, 0, 699):
+        for nsplit in (1, 5):
+            out, want, (qs, ks, vs) = paged_case(K, dtype, 8, 2, 64, 16, [700], [1], None, 9, nsplit,
+                                                 boost=(0, key_at, 699, 6.0))
+            assert rel(out, want) < KTOL[dtype]
+            got = out.double().cpu().reshape(8, 64)
+            expect = vs[0][key_at].double().repeat_interleave(4, 0)
+            assert float((got - expect).abs().max()) < 0.05, key_at     # the one key took all the weight
+
+
+def test_attention_uniform_keys_reference_vector(K):
+    # test/test_cuda_kernel/test_paged_attention_kernel.cpp:18-84: K = 0.1, V = 0.2, ctx 10, hd 128, 4 heads on 2 -> 0.2
+    H, KVH, hd, ps = 4, 2, 128, 16
+    kpool = torch.full((2, KVH, ps, hd), 0.1, device="cuda")
+    vpool = torch.full((2, KVH, ps, hd), 0.2, device="cuda")
+    qkv = torch.full((1, (H + 2 * KVH) * hd), 0.3, device="cuda")
+    out = torch.empty(1, H * hd, device="cuda")
+    K.token_attention(qkv, kpool, vpool, dev(torch.tensor([[1, 0]], dtype=torch.int32)),
+                      dev(torch.tensor([0], dtype=torch.int32)), dev(torch.tensor([9], dtype=torch.int32)), out,
+                      H, KVH, hd, 1 / math.sqrt(hd), None, 1)
+    assert float((out - 0.2).abs().max()) < 1e-6
+
+
+# ------------------------------------------------------------------ sampling
+
+def test_argmax_planted_maxima_and_ties(K):
+    # test/test_cuda_kernel/test_argmax_kernel.cpp:18-65
+    V = 10000
+    rows = torch.zeros(6, V)
+    for r, at in enumerate((100, 5000, 9999, 0)):
+        rows[r, at] = 10.0
+    rows[4, 7] = rows[4, 3] = rows[4, 9000] = 2.0          # equal maxima: the lowest index
+    rows[5] = -1.0
+    rows[5, 4321] = -0.5
+    assert K.argmax(dev(rows)).tolist() == [100, 5000, 9999, 0, 3, 4321]
+    g = torch.Generator().manual_seed(0)
+    big = torch.randn(3, 128256, generator=g)
+    assert K.argmax(dev(big)).tolist() == big.argmax(-1).tolist()
+
+
+def sample_rows(K, logits, temperature, top_k, top_p, penalty, generated, uniform):
+    R, V = logits.shape
+    pen_ids, pen_off = [], [0]
+    for g in generated:
+        pen_ids += sorted(set(g))
+        pen_off.append(len(pen_ids))
+    f32, i32 = torch.float32, torch.int32
+    out = torch.empty(R, dtype=i32, device="cuda")
+    K.sample(dev(logits), torch.empty(R, V, device="cuda"), dev(torch.tensor(temperature, dtype=f32)),
+             dev(torch.tensor(top_k, dtype=i32)), dev(torch.tensor(top_p, dtype=f32)), dev(torch.tensor(penalty, dtype=f32)),
+             dev(torch.tensor(pen_ids or [0], dtype=i32)), dev(torch.tensor(pen_off, dtype=i32)),
+             dev(torch.tensor(uniform, dtype=f32)), out)
+    return out.tolist()
+
+
+def plain_pick(logits, temperature, top_k, top_p, penalty, generated, u):
+    l = logits.double()
+    if penalty != 1.0:
+        l = P.repetition_penalty(l, generated, penalty)
+    if temperature <= 0:
+        return P.argmax(l)
+    l = P.temperature_scale(l, temperature)
+    return P.inverse_cdf(P.filtered_distribution(l, top_k, top_p), u)
+
+
+@pytest.mark.parametrize("V", [50, 1000, 5003])
+def test_sampling_matches_plain(K, V):
+    g = torch.Generator().manual_seed(V)
+    rng = random.Random(V)
+    cases = []
+    for _ in range(48):
+        cases.append(dict(temperature=rng.choice([0.0, 0.5, 0.8, 1.0, 1.7]), top_k=rng.choice([0, 0, 1, 5, 40]),
+                          top_p=rng.choice([1.0, 1.0, 0.9, 0.5, 0.1]), penalty=rng.choice([1.0, 1.0, 1.3]),
+                          generated=[rng.randrange(V) for _ in range(rng.randint(0, 6))],
+                          u=(rng.randrange(1, 1 << 20)) / float(1 << 20)))
+    logits = torch.randn(len(cases), V, generator=g) * 2.5
+    got = sample_rows(K, logits, [c["temperature"] for c in cases], [c["top_k"] for c in cases],
+                      [c["top_p"] for c in cases], [c["penalty"] for c in cases], [c["generated"] for c in cases],
+                      [c["u"] for c in cases])
+    for r, c in enumerate(cases):
+        want = plain_pick(logits[r], c["temperature"], c["top_k"], c["top_p"], c["penalty"], c["generated"], c["u"])
+        if got[r] != want:
+            # a draw that falls within rounding of a boundary of the cumulative distribution may take
+            # either neighbour: accept only if u is that close to the boundary between the two
+            l = logits[r].double()
+            if c["penalty"] != 1.0:
+                l = P.repetition_penalty(l, c["generated"], c["penalty"])
+            probs = P.filtered_distribution(P.temperature_scale(l, c["temperature"]), c["top_k"], c["top_p"])
+            cum = torch.cumsum(probs, 0)
+            lo, hi = sorted((got[r], want))
+            assert probs[got[r]] > 0 and abs(float(cum[lo]) - c["u"]) < 1e-5, (r, c, got[r], want)
+
+
+def test_sampling_closed_forms(K):
+    V = 10
+    logits = torch.tensor([[2.0, -1.0, 3.0, 0.0, -2.0, 1.0, 0.5, -0.5, 1.5, -1.5]]).repeat(5, 1)
+    # top-k 1 is argmax whatever u; a tiny temperature too; greedy with a penalty moves the maximum
+    got = sample_rows(K, logits, [1.0, 1e-4, 0.0, 0.0, 1.0], [1, 0, 0, 0, 0], [1.0, 1.0, 1.0, 1.0, 0.3],
+                      [1.0, 1.0, 1.0, 10.0, 1.0], [[], [], [], [2], []], [0.99, 0.5, 0.5, 0.5, 0.7])
+    assert got[:3] == [2, 2, 2]
+    assert got[3] == 0                      # 3.0 / 10 = 0.3 < 2.0: the penalised token loses
+    assert got[4] == 2                      # top-p 0.3: the most probable token alone carries it
+    # same seed, same token; other u, possibly other token, but always inside the top-k set
+    logits = torch.randn(1, 777, generator=torch.Generator().manual_seed(4)).repeat(64, 1)
+    us = [(i + 1) / 64 for i in range(64)]
+    got = sample_rows(K, logits, [1.0] * 64, [5] * 64, [1.0] * 64, [1.0] * 64, [[]] * 64, us)
+    top5 = set(logits[0].topk(5).indices.tolist())
+    assert set(got) <= top5 and len(set(got)) > 1
+    again = sample_rows(K, logits, [1.0] * 64, [5] * 64, [1.0] * 64, [1.0] * 64, [[]] * 64, us)
+    assert again == got

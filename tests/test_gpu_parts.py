@@ -1,0 +1,311 @@
+"""Each part alone, built from a spec as the model builds it, against the plain functions; the
+order of layers as data; and a toy mixer with state of its own that is registered, built and
+stepped from here, without a change to the framework's files."""
+import math
+
+import pytest
+import torch
+
+import plain_llama as P
+from gpu_common import TOL, model_folder, random_tokens
+from tiny_configs import ALL, TINY_B
+
+pytestmark = pytest.mark.gpu
+
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def rel(got, want):
+    return float((got.double().cpu() - want.double()).abs().max() / float(want.double().abs().max()))
+
+
+def runtime(dtype):
+    from nanoinfer_amd.parts.base import Runtime
+    return Runtime(DT[dtype], torch.device("cuda", 0))
+
+
+def test_parts_fail_loudly_without_their_sizes():
+    from nanoinfer_amd.config.spec import PartSpec
+    from nanoinfer_amd.parts.standard import Attention
+    spec = PartSpec("attention", {"hidden_size": 64, "num_heads": 4, "num_kv_heads": 2, "head_dim": 24,
+                                  "position": PartSpec("none")}, {"q": "q", "k": "k", "v": "v", "o": "o"})
+    w = {"q": torch.zeros(96, 64), "k": torch.zeros(48, 64), "v": torch.zeros(48, 64), "o": torch.zeros(64, 96)}
+    with pytest.raises(Exception) as e:
+        Attention(spec, w, runtime("float32"))
+    assert "multiple of 16" in str(e.value)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_norm_embedding_head_feed_forward(dtype):
+    from nanoinfer_amd.config.spec import PartSpec
+    from nanoinfer_amd.parts.standard import build_part
+    rt = runtime(dtype)
+    g = torch.Generator().manual_seed(0)
+    d, I, V, T = 100, 136, 777, 13
+    tensors = {"n": 1 + 0.1 * torch.randn(d, generator=g), "e": 0.1 * torch.randn(V, d, generator=g),
+               "g": 0.1 * torch.randn(I, d, generator=g), "u": 0.1 * torch.randn(I, d, generator=g),
+               "d": 0.1 * torch.randn(d, I, generator=g)}
+    rounded = {k: (v.to(DT[dtype]).double() if v.dim() == 2 else v.double()) for k, v in tensors.items()}
+    norm = build_part("norm", PartSpec("rmsnorm", {"size": d, "eps": 1e-3}, {"weight": "n"}), tensors, rt)
+    h = torch.randn(T, d, generator=g)
+    x = norm.forward(h.cuda(), None)
+    assert x.dtype == DT[dtype] and rel(x, P.rmsnorm(h, tensors["n"], 1e-3)) < TOL[dtype]
+    emb = build_part("embedding", PartSpec("table", {"vocab_size": V, "hidden_size": d}, {"weight": "e"}), tensors, rt)
+    ids = torch.randint(0, V, (T,), generator=g).to(torch.int32)
+    assert torch.equal(emb.forward(ids.cuda()).double().cpu(), rounded["e"][ids.long()])
+    head = build_part("head", PartSpec("linear", {"vocab_size": V, "hidden_size": d}, {"weight": "e"}), tensors, rt)
+    assert head.weight.data_ptr() == emb.weight.data_ptr()                    # tied: one buffer on the device
+    xin = x
+    logits = head.forward(xin)
+    assert logits.dtype == torch.float32 and rel(logits, P.linear(xin.double().cpu(), rounded["e"])) < TOL[dtype]
+    ffn = build_part("feed_forward", PartSpec("swiglu", {"hidden_size": d, "intermediate_size": I},
+                                              {"gate": "g", "up": "u", "down": "d"}), tensors, rt)
+    y = ffn.forward(xin, None)
+    xd = xin.double().cpu()
+    want = P.linear(P.swiglu(P.linear(xd, rounded["g"]), P.linear(xd, rounded["u"])), rounded["d"])
+    assert rel(y, want) < TOL[dtype]
+
+
+def test_position_part_shares_one_table():
+    from nanoinfer_amd.config.spec import PartSpec
+    from nanoinfer_amd.parts.standard import build_part
+    rt = runtime("float32")
+    sc = dict(TINY_B["rope_scaling"])
+    sc.pop("rope_type")
+    spec = PartSpec("rope", {"rotary_dim": 32, "theta": 500000.0, "scaling": sc, "max_positions": 300})
+    a = build_part("position", spec, {}, rt)
+    b = build_part("position", spec, {}, rt)
+    assert a.tables()[0].data_ptr() == b.tables()[0].data_ptr()
+    s, c = P.rope_tables(range(300), P.rope_frequencies(32, 500000.0, sc))
+    assert float((a.tables()[1].double().cpu() - s).abs().max()) < 2e-6
+    assert float((a.tables()[0].double().cpu() - c).abs().max()) < 2e-6
+    assert build_part("position", PartSpec("none"), {}, rt).tables() is None
+
+
+# ------------------------------------------------------------------ a model from a spec written here
+
+def tiny_spec(mixer_kinds, order, d=64, H=4, KVH=2, hd=16, I=96, V=128, window=None, position="rope", state_size=None):
+    from nanoinfer_amd.config.spec import BlockSpec, LayerRun, ModelSpec, PartSpec
+    pos = PartSpec("rope", {"rotary_dim": hd, "theta": 10000.0, "scaling": None, "max_positions": 256}) \
+        if position == "rope" else PartSpec("none")
+    blocks = []
+    for i, kind in enumerate(mixer_kinds):
+        pre = f"L{i}."
+        if kind == "attention":
+            mixer = PartSpec("attention", {"hidden_size": d, "num_heads": H, "num_kv_heads": KVH, "head_dim": hd,
+                                           "scale": None, "window": window[i] if window else None, "position": pos},
+                             {"q": pre + "q", "k": pre + "k", "v": pre + "v", "o": pre + "o"})
+        else:
+            mixer = PartSpec(kind, {"hidden_size": d, "state_size": state_size}, {"inp": pre + "inp", "out": pre + "out"})
+        blocks.append(BlockSpec("prenorm", PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": pre + "n1"}), mixer,
+                                PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": pre + "n2"}),
+                                PartSpec("swiglu", {"hidden_size": d, "intermediate_size": I},
+                                         {"gate": pre + "g", "up": pre + "u", "down": pre + "d"})))
+    return ModelSpec(V, d, 256, PartSpec("table", {"vocab_size": V, "hidden_size": d}, {"weight": "emb"}), blocks,
+                     [LayerRun(*o) for o in order], PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": "nf"}),
+                     PartSpec("linear", {"vocab_size": V, "hidden_size": d}, {"weight": "emb"}))
+
+
+def random_tensors(spec, seed):
+    from nanoinfer_amd.weights.loader import expected_tensors
+    g = torch.Generator().manual_seed(seed)
+    return {n: (1 + 0.05 * torch.randn(s, generator=g)) if len(s) == 1 else 0.08 * torch.randn(s, generator=g)
+            for n, s in expected_tensors(spec).items()}
+
+
+class SpecRunner:
+    """A ModelRunner over a spec and tensors given directly (no folder): the same Model, cache manager
+    and step function, reached through the constructor's pieces."""
+
+    def __new__(cls, spec, tensors, dtype, page_size=8, max_tokens=512):
+        from nanoinfer_amd.cache.manager import KVCacheManager
+        from nanoinfer_amd.engine.model import Model
+        from nanoinfer_amd.engine.runner import ModelRunner
+        r = ModelRunner.__new__(ModelRunner)
+        r.device = torch.device("cuda", 0)
+        r.dtype = DT[dtype]
+        r.spec = spec
+        r.rt = runtime(dtype)
+        r.model = Model(spec, tensors, r.rt)
+        r.page_size = page_size
+        r.cache = KVCacheManager(r.model.cache_needs(), page_size, max_tokens // page_size, 4, dtype=DT[dtype], device=r.device)
+        r.vocab_size, r.max_positions, r.eos_token_ids = spec.vocab_size, r.model.max_positions, ()
+        r._done, r._scratch = {}, None
+        return r
+
+
+def plain_spec_forward(spec, tensors, tokens, extra_mixers=None):
+    """The plain implementation applied to a spec: same functions, parts chosen by the spec."""
+    T = len(tokens)
+    t64 = {k: v.double() for k, v in tensors.items()}
+    h = P.embedding(t64[spec.embedding.weights["weight"]], tokens)
+    kv = {}
+    for run in spec.order:
+        b = spec.blocks[run.block]
+        x = P.rmsnorm(h, t64[b.mixer_norm.weights["weight"]], b.mixer_norm.params["eps"])
+        m = b.mixer
+        if m.kind == "attention":
+            p = m.params
+            H, KVH, hd = p["num_heads"], p["num_kv_heads"], p["head_dim"]
+            q = P.linear(x, P.permute_reverse(t64[m.weights["q"]], H)).reshape(T, H, hd)
+            if run.writes_cache:
+                k = P.linear(x, P.permute_reverse(t64[m.weights["k"]], KVH)).reshape(T, KVH, hd)
+                v = P.linear(x, t64[m.weights["v"]]).reshape(T, KVH, hd)
+            if p["position"].kind == "rope":
+                pp = p["position"].params
+                s, c = P.rope_tables(range(T), P.rope_frequencies(pp["rotary_dim"], pp["theta"], pp["scaling"]))
+                q = P.rope_interleaved(q, s, c)
+                if run.writes_cache:
+                    k = P.rope_interleaved(k, s, c)
+            if run.writes_cache:
+                kv[run.cache] = (k, v)
+            k, v = kv[run.cache]
+            a = P.linear(P.causal_attention(q, k, v, range(T), window=p["window"]).reshape(T, H * hd), t64[m.weights["o"]])
+        else:
+            a = extra_mixers[m.kind](x, t64, m)
+        h = h + a
+        x = P.rmsnorm(h, t64[b.ffn_norm.weights["weight"]], b.ffn_norm.params["eps"])
+        f = b.ffn
+        h = h + P.linear(P.swiglu(P.linear(x, t64[f.weights["gate"]]), P.linear(x, t64[f.weights["up"]])), t64[f.weights["down"]])
+    return P.linear(P.rmsnorm(h, t64[spec.final_norm.weights["weight"]], spec.final_norm.params["eps"]),
+                    t64[spec.head.weights["weight"]])
+
+
+def step_in_portions(runner, tokens, sizes, rid="s"):
+    from nanoinfer_amd.engine.runner import StepEntry
+    outs, at, k = [], 0, 0
+    while at < len(tokens):
+        n = min(sizes[k % len(sizes)], len(tokens) - at)
+        outs.append(runner.step([StepEntry(rid, tokens[at:at + n], list(range(n)))]))
+        at, k = at + n, k + 1
+    runner.release(rid)
+    return torch.cat(outs)
+
+
+def test_order_of_layers_is_data():
+    """A block run twice on caches of its own, a layer that reads another layer's cache, a layer
+    with a window and one without position encoding: all from one list, no new code."""
+    tokens = list(random_tokens(128, 60, 1))
+    cases = {
+        "plain order": (["attention", "attention"], [(0, 0), (1, 1)], None, "rope"),
+        "block 0 twice": (["attention", "attention"], [(0, 0), (1, 1), (0, 2)], None, "rope"),
+        "layer 1 reads layer 0's cache": (["attention", "attention"], [(0, 0, True), (1, 0, False)], None, "rope"),
+        "window on layer 1": (["attention", "attention"], [(0, 0), (1, 1)], [None, 9], "rope"),
+        "no position encoding": (["attention"], [(0, 0)], None, "none"),
+    }
+    for what, (kinds, order, window, position) in cases.items():
+        spec = tiny_spec(kinds, order, window=window, position=position)
+        tensors = random_tensors(spec, 3)
+        want = plain_spec_forward(spec, tensors, tokens)
+        runner = SpecRunner(spec, tensors, "float32")
+        if what == "window on layer 1":
+            assert len(runner.cache.groups) == 2            # a window is another need: pages of its own
+        for sizes in ([60], [7, 2, 13, 1, 1, 1]):
+            got = step_in_portions(runner, tokens, sizes)
+            assert rel(got, want) < TOL["float32"], (what, sizes)
+        runner.cache.check()
+        assert all(g.pages.num_free == g.pages.num_pages for g in runner.cache.groups)
+    with pytest.raises(ValueError):
+        from nanoinfer_amd.engine.model import Model
+        bad = tiny_spec(["attention", "attention"], [(0, 0, False), (1, 0, True)])
+        Model(bad, random_tensors(bad, 0), runtime("float32"))     # reads a cache nobody has written yet
+
+
+def test_windowed_layer_gives_pages_back_while_running():
+    from nanoinfer_amd.engine.runner import StepEntry
+    spec = tiny_spec(["attention", "attention"], [(0, 0), (1, 1)], window=[None, 9])
+    tensors = random_tensors(spec, 4)
+    runner = SpecRunner(spec, tensors, "float32", page_size=4, max_tokens=256)
+    tokens = list(random_tokens(128, 100, 2))
+    want = plain_spec_forward(spec, tensors, tokens)
+    outs = [runner.step([StepEntry("w", tokens[:20], list(range(20)))])]
+    windowed = next(g for g in runner.cache.groups if g.need.window == 9)
+    full = next(g for g in runner.cache.groups if g.need.window is None)
+    for t in tokens[20:]:
+        outs.append(runner.step([StepEntry("w", [t], [0])]))
+        assert windowed.pages.num_taken <= 4                       # 9 keys span at most 3 pages, plus the new one
+    assert full.pages.num_taken == 25 and windowed.tables["w"][:20] == [-1] * 20
+    assert rel(torch.cat(outs), want) < TOL["float32"]
+    runner.release("w")
+
+
+# ------------------------------------------------------------------ a toy mixer with state
+
+def register_toy_mixer():
+    from nanoinfer_amd.parts.base import CacheNeed, Part, StateNeed, WeightRequest
+    from nanoinfer_amd.registry import register_part
+
+    @register_part("mixer", "toy_decay")
+    class ToyDecayMixer(Part):
+        """y_t = out(s_t), s_t = 0.5 * s_{t-1} + inp(x_t): a running state of fixed size per request,
+        kept in a state slot between steps.  Written with library tensor operations: it shows the
+        interface, it is no product kernel."""
+
+        @classmethod
+        def weight_requests(cls, spec):
+            d, n = spec.params["hidden_size"], spec.params["state_size"]
+            return [WeightRequest(spec.weights["inp"], (n, d)), WeightRequest(spec.weights["out"], (d, n))]
+
+        def __init__(self, spec, weights, rt):
+            super().__init__(spec, weights, rt)
+            self.n = spec.params["state_size"]
+            self.inp = rt.matrix(spec.weights["inp"], weights["inp"])
+            self.out = rt.matrix(spec.weights["out"], weights["out"])
+
+        def cache_need(self):
+            return CacheNeed(state=StateNeed((self.n,), torch.float32))
+
+        def forward(self, x, ctx, cache):
+            u = (x @ self.inp.t()).float()
+            states = torch.empty_like(u)
+            for start, length, total, slot in zip(ctx.q_start, ctx.q_len, ctx.context_len, ctx.state_slot):
+                s = cache.state[slot]
+                if total == length:           # the request's first tokens: start from nothing
+                    s = torch.zeros_like(s)
+                for i in range(start, start + length):
+                    s = 0.5 * s + u[i]
+                    states[i] = s
+                cache.state[slot] = s
+            return states.to(x.dtype) @ self.out.t()
+
+    return ToyDecayMixer
+
+
+def plain_toy(x, t64, m):
+    u = P.linear(x, t64[m.weights["inp"]])
+    s = torch.zeros(u.shape[1], dtype=torch.float64)
+    rows = []
+    for i in range(u.shape[0]):
+        s = 0.5 * s + u[i]
+        rows.append(s.clone())
+    return P.linear(torch.stack(rows), t64[m.weights["out"]])
+
+
+def test_toy_mixer_with_state_is_registered_built_and_stepped():
+    from nanoinfer_amd.engine.runner import StepEntry
+    register_toy_mixer()
+    spec = tiny_spec(["attention", "toy_decay", "attention"], [(0, 0), (1, 1), (2, 2)], state_size=24)
+    tensors = random_tensors(spec, 5)
+    runner = SpecRunner(spec, tensors, "float32", page_size=8, max_tokens=512)
+    assert len(runner.cache.groups) == 1 and runner.cache.groups[0].cache_ids == [0, 2]
+    assert list(runner.cache.state) == [1] and tuple(runner.cache.state[1].shape) == (4, 24)
+    reqs = {"p": list(random_tokens(128, 41, 6)), "q": list(random_tokens(128, 29, 7)), "r": list(random_tokens(128, 17, 8))}
+    want = {k: plain_spec_forward(spec, tensors, v, {"toy_decay": plain_toy}) for k, v in reqs.items()}
+    got = {k: [] for k in reqs}
+    done = {k: 0 for k in reqs}
+    plan = [{"p": 5}, {"p": 3, "q": 9}, {"q": 1, "p": 1}, {"p": 20, "q": 1, "r": 17}, {"q": 18, "p": 12}]
+    for stepplan in plan:
+        entries = [StepEntry(k, reqs[k][done[k]:done[k] + n], list(range(n))) for k, n in stepplan.items()]
+        out = runner.step(entries, end=[k for k, n in stepplan.items() if done[k] + n == len(reqs[k])])
+        row = 0
+        for k, n in stepplan.items():
+            got[k].append(out[row:row + n])
+            row += n
+            done[k] += n
+    for k in reqs:
+        assert done[k] == len(reqs[k]) and rel(torch.cat(got[k]), want[k]) < TOL["float32"], k
+    # the slot of a finished request is handed out again and starts from nothing
+    out = runner.step([StepEntry("again", reqs["r"], list(range(17)))], end=["again"])
+    assert rel(out, want["r"]) < TOL["float32"]
+    runner.cache.check()
+    assert runner.cache.slots.num_free == 4
