@@ -122,6 +122,7 @@ def library_path(name: str, sources: List[str], defines: Optional[Dict[str, obje
 # What the framework is made of.  Attention is compiled per head size.
 CORE = ("ni_ops", ["ops.hip"], {})
 SAMPLING = ("ni_sampling", ["sampling.hip"], {})
+SKINNY = ("ni_skinny_gemm", ["gemv.hip"], {})
 COMMON_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)
 
 
@@ -134,5 +135,5 @@ def attention_target(head_dim: int):
 
 def build_all(head_dims: Iterable[int] = COMMON_HEAD_DIMS, force: bool = True, verbose: bool = True) -> List[str]:
     """Compile every library (attention for the given head sizes)."""
-    targets = [CORE, SAMPLING] + [attention_target(h) for h in head_dims]
+    targets = [CORE, SAMPLING, SKINNY] + [attention_target(h) for h in head_dims]
     return [library_path(n, s, d, force=force, verbose=verbose) for n, s, d in targets]

@@ -1,0 +1,209 @@
+// Skinny matrix products for decoding on gfx950: y[M, N] = x[M, K] . W[N, K]^T with M <= 64,
+// where the time is the time to stream W from HBM once.
+//
+// One workgroup of 8 wavefronts owns NT tiles of 16 output columns.  Its wavefronts split K:
+// wavefront w takes the 128-byte pieces w, w+8, ... of every row.  A piece is loaded straight
+// from global memory in MFMA operand layout (lane l: row l%16 of the tile, 32 bytes at offset
+// (l/16)*32 of the piece) and multiplied against the matching piece of x with
+// v_mfma_f32_16x16x32_bf16 (two per piece) or v_mfma_f32_16x16x4_f32 (eight per piece): W is the
+// A operand (rows = output columns n), x^T the B operand (columns = batch rows m), so each
+// loaded byte of W is used for up to 16 rows of x per instruction, and M up to 64 costs four
+// instructions per piece.  The MFMA's k index is only a label, so the same lane-to-k mapping on
+// both operands is all that is required.  Partial sums meet in LDS.
+//
+// Epilogues: store (compute type or float32), or SwiGLU over paired tiles (tile 2j from the gate
+// rows, tile 2j+1 from the up rows of a stacked [2I, K] matrix): out[m, n] = silu(g) * u.
+// float32 inputs are multiplied in true float32 (no reduced-precision MFMA).
+#include <type_traits>
+
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+#define GV_WAVES 8
+#define GV_THREADS (GV_WAVES * WAVE)
+
+template <typename T> struct Piece;   // 32 bytes of one row, and the MFMAs that consume it
+template <> struct Piece<bf16_t> {
+    static constexpr int ELEMS = 16;          // per lane
+    uint4 lo, hi;
+    __device__ __forceinline__ void load(const bf16_t* p) {
+        lo = reinterpret_cast<const uint4*>(p)[0];
+        hi = reinterpret_cast<const uint4*>(p)[1];
+    }
+    __device__ __forceinline__ void zero() { lo = make_uint4(0, 0, 0, 0); hi = lo; }
+    static __device__ __forceinline__ floatx4_t mma(const Piece& a, const Piece& b, floatx4_t c) {
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a.lo), __builtin_bit_cast(bf16x8_t, b.lo), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a.hi), __builtin_bit_cast(bf16x8_t, b.hi), c, 0, 0, 0);
+        return c;
+    }
+};
+template <> struct Piece<float> {
+    static constexpr int ELEMS = 8;
+    float v[8];
+    __device__ __forceinline__ void load(const float* p) {
+        float4 a = reinterpret_cast<const float4*>(p)[0], b = reinterpret_cast<const float4*>(p)[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+    __device__ __forceinline__ void zero() {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = 0.f;
+    }
+    static __device__ __forceinline__ floatx4_t mma(const Piece& a, const Piece& b, floatx4_t c) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[i], b.v[i], c, 0, 0, 0);
+        return c;
+    }
+};
+
+enum { EPI_STORE = 0, EPI_SWIGLU = 1 };
+
+template <typename T, typename TOUT, int MB, int NT, int EPI>
+__global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __restrict__ x, const T* __restrict__ W,
+                                                                 TOUT* __restrict__ y, int M, int N, int K, int I) {
+    constexpr int EL = Piece<T>::ELEMS;
+    constexpr int CH = 4 * EL;                       // k elements in a 128-byte piece of a row
+    const int tid = threadIdx.x;
+    const int wave = tid / WAVE, lane = tid % WAVE;
+    const int r = lane % 16, kg = lane / 16;
+    const int wg = blockIdx.x;
+
+    // weight row that this lane reads in each tile; tiles may hang over the edge of the matrix, then
+    // the row index is clamped (never read past W) and the result is not stored
+    const int n_limit = (EPI == EPI_SWIGLU) ? I : N;
+    const T* wrow[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int col0 = (EPI == EPI_SWIGLU) ? (wg * (NT / 2) + nt / 2) * 16 : (wg * NT + nt) * 16;
+        const int shift = (EPI == EPI_SWIGLU && (nt % 2)) ? I : 0;      // odd tiles of a pair come from the up rows
+        wrow[nt] = W + static_cast<size_t>(min(col0 + r, n_limit - 1) + shift) * K;
+    }
+    const T* xrow[MB];
+    bool xok[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = mb * 16 + r;
+        xok[mb] = m < M;
+        xrow[mb] = x + static_cast<size_t>(min(m, M - 1)) * K;
+    }
+
+    floatx4_t acc[NT][MB];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    // two pieces per trip, all their loads issued before the first multiply, to keep enough bytes in flight
+    const int pieces = (K + CH - 1) / CH;
+    for (int c = wave; c < pieces; c += 2 * GV_WAVES) {
+        Piece<T> xb[2][MB], wa[2][NT];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int k = (c + u * GV_WAVES) * CH + kg * EL;
+            const bool kok = k < K;                  // K is a multiple of EL: a lane's 32 bytes are all in or all out
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                if (kok) wa[u][nt].load(wrow[nt] + k); else wa[u][nt].zero();
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                if (kok && xok[mb]) xb[u][mb].load(xrow[mb] + k); else xb[u][mb].zero();
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = Piece<T>::mma(wa[u][nt], xb[u][mb], acc[nt][mb]);
+    }
+
+    // partial sums of the wavefronts meet in LDS: red[wave][tile][lane * 4 + i]
+    __shared__ float red[GV_WAVES][NT * MB][WAVE * 4];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave][nt * MB + mb][lane * 4 + i] = acc[nt][mb][i];
+    __syncthreads();
+
+    // D[n_local][m_local] of a tile sits at lane = (n_local / 4) * 16 + m_local, register n_local % 4
+    constexpr int NOUT = (EPI == EPI_SWIGLU) ? NT / 2 : NT;      // output tiles of the workgroup
+    const int out_n0 = wg * NOUT * 16;
+    const int out_width = (EPI == EPI_SWIGLU) ? I : N;
+    for (int item = tid; item < MB * 16 * NOUT * 16; item += GV_THREADS) {
+        const int n_in = item % (NOUT * 16);
+        const int m = item / (NOUT * 16);
+        const int ot = n_in / 16, n_local = n_in % 16;
+        const int mb = m / 16, m_local = m % 16;
+        const int n = out_n0 + n_in;
+        if (m >= M || n >= out_width) continue;
+        const int src = ((n_local / 4) * 16 + m_local) * 4 + (n_local % 4);
+        float v;
+        if (EPI == EPI_SWIGLU) {
+            float g = 0.f, u = 0.f;
+#pragma unroll
+            for (int w = 0; w < GV_WAVES; ++w) {
+                g += red[w][(2 * ot) * MB + mb][src];
+                u += red[w][(2 * ot + 1) * MB + mb][src];
+            }
+            v = g / (1.0f + expf(-g)) * u;
+        } else {
+            v = 0.f;
+#pragma unroll
+            for (int w = 0; w < GV_WAVES; ++w) v += red[w][ot * MB + mb][src];
+        }
+        st(y + static_cast<size_t>(m) * out_width + n, v);
+    }
+}
+
+template <typename T, typename TOUT, int MB, int EPI>
+static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream) {
+    const int out_width = (EPI == EPI_SWIGLU) ? I : N;
+    const int tiles = (out_width + 15) / 16;
+    auto run = [&](auto nt_tag) {
+        constexpr int NTc = decltype(nt_tag)::value;
+        constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
+        const int grid = (tiles + NOUT - 1) / NOUT;
+        skinny_gemm_kernel<T, TOUT, MB, NTc, EPI><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I);
+    };
+    // NT * MB fragments of partial sums share 64 KB of LDS: at most 8
+    if constexpr (MB <= 2) {
+        if (NT >= 4) { run(std::integral_constant<int, 4>{}); return NI_LAUNCH_RESULT(); }
+    }
+    if constexpr (EPI == EPI_SWIGLU) {
+        run(std::integral_constant<int, 2>{});
+    } else {
+        if (NT >= 2) run(std::integral_constant<int, 2>{});
+        else run(std::integral_constant<int, 1>{});
+    }
+    return NI_LAUNCH_RESULT();
+}
+
+template <typename T, typename TOUT, int EPI>
+static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream) {
+    if (M <= 16) return launch_nt<T, TOUT, 1, EPI>(x, W, y, M, N, K, I, NT, stream);
+    if (M <= 32) return launch_nt<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream);
+    return launch_nt<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, stream);
+}
+
+// epilogue: 0 store in the input type, 1 store float32, 2 SwiGLU (W is [2I, K], y is [M, I]).
+// K must be a multiple of 16 bytes' worth of elements x 2 (bf16: 16, f32: 8); M <= 64.
+NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N, int K, int epilogue, int tiles_per_group,
+                             int dtype, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 64) return -1;
+    const int el = dtype == 0 ? 8 : 16;
+    if (K % el != 0) return -2;
+    const int I = N / 2;
+    if (epilogue == 2 && (N % 2)) return -3;
+    if (dtype == 0) {
+        if (epilogue == 2) return launch_mb<float, float, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, stream);
+        return launch_mb<float, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, stream);
+    }
+    if (epilogue == 2) return launch_mb<bf16_t, bf16_t, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, stream);
+    if (epilogue == 1) return launch_mb<bf16_t, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, stream);
+    return launch_mb<bf16_t, bf16_t, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, stream);
+}

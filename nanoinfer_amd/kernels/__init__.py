@@ -45,6 +45,10 @@ def sampling_lib() -> ctypes.CDLL:
     return _load(_build.SAMPLING)
 
 
+def skinny_lib() -> ctypes.CDLL:
+    return _load(_build.SKINNY)
+
+
 def attention_lib(head_dim: int) -> ctypes.CDLL:
     return _load(_build.attention_target(head_dim))
 
@@ -263,13 +267,69 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
 
 # ------------------------------------------------------------------ matrix product (library)
 
-def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``x . weight^T`` with ``weight`` stored [out, in]; float32 inputs are multiplied in true
-    float32 (the reduced-precision matrix modes of the library are switched off at import)."""
+SKINNY_MAX_ROWS = 64
+
+
+def skinny_ok(M: int, K: int, dtype: torch.dtype) -> bool:
+    """Whether the hand-written skinny product takes this shape: at most 64 rows, rows of W that
+    split into whole 32-byte lane loads."""
+    return 0 < M <= SKINNY_MAX_ROWS and K % (8 if dtype == torch.float32 else 16) == 0
+
+
+def _tiles_per_group(n_out: int) -> int:
+    tiles = (n_out + 15) // 16
+    return 4 if tiles >= 2048 else (2 if tiles >= 512 else 1)
+
+
+def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, swiglu: bool = False) -> torch.Tensor:
+    """``x . weight^T`` for at most 64 rows of ``x``, streaming ``weight`` once (MFMA).  ``out``
+    may be float32 for bfloat16 inputs.  With ``swiglu`` the weight is a stacked [2I, K] matrix
+    (gate rows, then up rows) and ``out`` [M, I] receives ``silu(gate) * up``."""
+    M, Kd = x.shape
+    N = weight.shape[0]
+    _gpu(x, "x")
+    _gpu(weight, "weight", x.dtype)
+    _need(weight.shape[1] == Kd, f"skinny_gemm: {tuple(x.shape)} x {tuple(weight.shape)}^T")
+    _need(skinny_ok(M, Kd, x.dtype), f"skinny_gemm does not take M={M}, K={Kd} in {x.dtype}")
+    if swiglu:
+        _need(N % 2 == 0, "a stacked gate/up matrix needs an even number of rows")
+        _gpu(out, "out", x.dtype, (M, N // 2))
+        epi = 2
+    else:
+        _need(out.dtype in (x.dtype, torch.float32), f"out must be {x.dtype} or float32")
+        _gpu(out, "out", None, (M, N))
+        epi = 1 if (out.dtype == torch.float32 and x.dtype != torch.float32) else 0
+    _check(skinny_lib().ni_skinny_gemm(_ptr(x), _ptr(weight), _ptr(out), M, N, Kd, epi,
+                                       _tiles_per_group(N // 2 if swiglu else N), dtype_code(x.dtype), _stream()),
+           "skinny_gemm")
+    return out
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``x . weight^T`` with ``weight`` stored [out, in].  Few rows go to the hand-written skinny
+    product; many rows to the library (rocBLAS/hipBLASLt), where float32 inputs are multiplied in
+    true float32 (the reduced-precision matrix modes of the library are switched off at import).
+    ``out_dtype`` float32 keeps the float32 accumulators of a bfloat16 product."""
     _need(x.is_cuda and weight.is_cuda, "linear needs GPU tensors")
     _need(x.dtype == weight.dtype, f"linear: activation {x.dtype} and weight {weight.dtype} differ")
-    _need(x.shape[-1] == weight.shape[1], f"linear: {tuple(x.shape)} x {tuple(weight.shape)}^T")
-    return torch.matmul(x, weight.t(), out=out)
+    _need(x.dim() == 2 and x.shape[1] == weight.shape[1], f"linear: {tuple(x.shape)} x {tuple(weight.shape)}^T")
+    out_dtype = out_dtype or x.dtype
+    if skinny_ok(x.shape[0], x.shape[1], x.dtype):
+        out = torch.empty(x.shape[0], weight.shape[0], dtype=out_dtype, device=x.device)
+        return skinny_gemm(x, weight, out)
+    if out_dtype != x.dtype:
+        return torch.mm(x, weight.t(), out_dtype=out_dtype)
+    return torch.matmul(x, weight.t())
+
+
+def linear_swiglu(x: torch.Tensor, weight_gate_up: torch.Tensor) -> torch.Tensor:
+    """``silu(x . Wg^T) * (x . Wu^T)`` for the stacked matrix [Wg; Wu]: fused into the product for
+    few rows, product then the SwiGLU kernel for many."""
+    inter = weight_gate_up.shape[0] // 2
+    out = torch.empty(x.shape[0], inter, dtype=x.dtype, device=x.device)
+    if skinny_ok(x.shape[0], x.shape[1], x.dtype):
+        return skinny_gemm(x, weight_gate_up, out, swiglu=True)
+    return swiglu(torch.matmul(x, weight_gate_up.t()), out)
 
 
 def require_gpu() -> torch.device:

@@ -219,10 +219,7 @@ class SwiGLU(Part):
         self.w_down = rt.matrix(names["down"], weights["down"])
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        gu = K.linear(x, self.w_gate_up)
-        act = torch.empty(x.shape[0], self.intermediate_size, dtype=x.dtype, device=x.device)
-        K.swiglu(gu, act)
-        return K.linear(act, self.w_down)
+        return K.linear(K.linear_swiglu(x, self.w_gate_up), self.w_down)
 
 
 # ------------------------------------------------------------------ block
@@ -279,6 +276,4 @@ class LinearHead(Part):
         self.weight = rt.matrix(spec.weights["weight"], weights["weight"])
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        if x.dtype == torch.float32:
-            return K.linear(x, self.weight)
-        return torch.mm(x, self.weight.t(), out_dtype=torch.float32)
+        return K.linear(x, self.weight, out_dtype=torch.float32)

@@ -342,3 +342,42 @@ def test_sampling_closed_forms(K):
     assert set(got) <= top5 and len(set(got)) > 1
     again = sample_rows(K, logits, [1.0] * 64, [5] * 64, [1.0] * 64, [1.0] * 64, [[]] * 64, us)
     assert again == got
+
+
+# ------------------------------------------------------------------ skinny matrix product
+
+def _skinny_case(Kmod, dtype, M, N, Kd):
+    g = torch.Generator().manual_seed(M * 1000 + N + Kd)
+    x = torch.randn(M, Kd, generator=g).to(DT[dtype])
+    w = (torch.randn(N, Kd, generator=g) / math.sqrt(Kd)).to(DT[dtype])
+    want = x.double() @ w.double().t()
+    if not Kmod.skinny_ok(M, Kd, DT[dtype]):
+        with pytest.raises(Kmod.KernelError):
+            Kmod.skinny_gemm(dev(x), dev(w), torch.empty(M, N, device="cuda", dtype=DT[dtype]))
+        return
+    out = Kmod.skinny_gemm(dev(x), dev(w), torch.empty(M, N, device="cuda", dtype=DT[dtype]))
+    assert rel(out, want) < KTOL[dtype], "store"
+    out32 = Kmod.skinny_gemm(dev(x), dev(w), torch.empty(M, N, device="cuda", dtype=torch.float32))
+    assert rel(out32, want) < 3e-6, "float32 out"
+    if N % 2 == 0:
+        act = Kmod.skinny_gemm(dev(x), dev(w), torch.empty(M, N // 2, device="cuda", dtype=DT[dtype]), swiglu=True)
+        assert rel(act, P.swiglu(want[:, :N // 2], want[:, N // 2:])) < KTOL[dtype], "swiglu"
+    assert rel(Kmod.linear(dev(x), dev(w)), want) < KTOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("M,N,Kd", [(1, 16, 16), (5, 50, 64), (16, 1000, 192), (17, 778, 2048), (40, 2064, 528),
+                                    (64, 96, 8192), (8, 128256, 64), (3, 33, 48), (33, 40000, 256), (2, 34, 24)])
+def test_skinny_product(K, dtype, M, N, Kd):
+    _skinny_case(K, dtype, M, N, Kd)
+
+
+def test_skinny_product_reference_vector(K):
+    # test/test_cuda_kernel/test_matmul_kernel.cpp:30-99: ones x 0.5 with K = 128 gives 64
+    out = K.skinny_gemm(torch.ones(3, 128, device="cuda"), torch.full((7, 128), 0.5, device="cuda"),
+                        torch.empty(3, 7, device="cuda"))
+    assert torch.all(out == 64.0)
+    # many rows go to the library, in true float32
+    g = torch.Generator().manual_seed(0)
+    x, w = torch.randn(300, 1024, generator=g), torch.randn(512, 1024, generator=g) / 32
+    assert rel(K.linear(dev(x), dev(w)), x.double() @ w.double().t()) < 3e-6
