@@ -42,6 +42,13 @@ class Model:
                 raise ValueError(f"block {run.block} reads cache {run.cache} before any block has written it")
         self.max_positions = spec.max_positions
 
+    def graph_safe(self) -> bool:
+        """Whether a step of this model may be recorded into a HIP graph: every part says of itself
+        that its launches depend on device data only (``graph_safe``), never on the host lists."""
+        parts = [self.embedding, self.final_norm, self.head] + list(self.blocks)
+        return all(getattr(p, "graph_safe", False) is True or (callable(getattr(p, "graph_safe", None)) and p.graph_safe())
+                   for p in parts)
+
     def cache_needs(self) -> Dict[int, CacheNeed]:
         return dict(self._needs)
 

@@ -51,9 +51,11 @@ class StepContext:
     per cache group a block table [B, pages] and a slot mapping [T].  Host lists, one entry per
     sequence of the step, in batch order: ``requests``, ``q_start`` (first row of its portion),
     ``q_len``, ``context_len`` (tokens in the cache after this step), ``state_slot``.
+    ``max_context`` bounds every context length of the step; in a step that is recorded into a
+    HIP graph it is a rounded-up bound, and the host lists must not steer the computation.
     """
 
-    def __init__(self, device: torch.device):
+    def __init__(self, device: torch.device, scratch_owner=None, recording: bool = False):
         self.device = device
         self.n_tokens = 0
         self.n_seqs = 0
@@ -69,31 +71,48 @@ class StepContext:
         self.seq_of_token: torch.Tensor = None
         self.logit_rows: Optional[torch.Tensor] = None
         self.groups: List[GroupView] = []
-        self._workspace: Optional[torch.Tensor] = None
-        self._workspace_owner = None
+        self.recording = recording
+        self._scratch_owner = scratch_owner
+        self._scratch: Optional[torch.Tensor] = None
 
     def workspace(self, n_floats: int) -> torch.Tensor:
         """Float32 scratch that lives until the next request for scratch (one user at a time)."""
-        owner = self._workspace_owner
-        ws = owner._scratch if owner is not None else self._workspace
-        if ws is None or ws.numel() < n_floats:
-            ws = torch.empty(max(n_floats, 1 << 16), dtype=torch.float32, device=self.device)
-            if owner is not None:
-                owner._scratch = ws
-            else:
-                self._workspace = ws
-        return ws
+        if self.recording or self._scratch_owner is None:
+            # a recorded step keeps its scratch in the graph's own memory
+            if self._scratch is None or self._scratch.numel() < n_floats:
+                self._scratch = torch.empty(n_floats, dtype=torch.float32, device=self.device)
+            return self._scratch
+        owner = self._scratch_owner
+        if owner._scratch is None or owner._scratch.numel() < n_floats:
+            owner._scratch = torch.empty(max(n_floats, 1 << 16), dtype=torch.float32, device=self.device)
+        return owner._scratch
+
+
+@dataclass
+class _RecordedStep:
+    """A decode step of fixed shape recorded into a HIP graph, with the buffers it reads and writes."""
+
+    graph: "torch.cuda.CUDAGraph"
+    meta: torch.Tensor            # int32, device: every integer table of the step, fixed layout
+    staging: torch.Tensor         # the same, pinned host memory
+    logits: torch.Tensor
+    ctx: StepContext
+    copied: "torch.cuda.Event" = None    # the last upload of the tables has left the staging buffer
 
 
 class ModelRunner:
     """A model, its cache, and the step function over both.
 
     ``max_tokens`` is the number of tokens the page pools hold (rounded up to whole pages);
-    ``max_requests`` the number of requests that may be live at once.
+    ``max_requests`` the number of requests that may be live at once.  With ``use_graphs`` a step
+    that consists of single tokens only (decoding) is recorded once per shape into a HIP graph and
+    replayed afterwards: the launches of a whole step then cost one call.
     """
 
+    GRAPH_MAX_BATCH = 64
+
     def __init__(self, model_dir: str, dtype: str = "bfloat16", page_size: int = 16, max_tokens: int = 4096,
-                 max_requests: int = 64, device: Optional[torch.device] = None):
+                 max_requests: int = 64, device: Optional[torch.device] = None, use_graphs: bool = True):
         self.device = device or K.require_gpu()
         torch_dtype = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
                        "float32": torch.float32, "fp32": torch.float32}.get(dtype)
@@ -114,6 +133,13 @@ class ModelRunner:
         self.eos_token_ids = tuple(self.spec.eos_token_ids)
         self._done: Dict[Hashable, int] = {}   # tokens of each live request already in the cache
         self._scratch: Optional[torch.Tensor] = None
+        self._init_graphs(use_graphs)
+
+    def _init_graphs(self, use_graphs: bool) -> None:
+        import os
+        self.use_graphs = bool(use_graphs) and self.model.graph_safe() and not os.environ.get("NANOINFER_NO_GRAPHS")
+        self._recorded: Dict[tuple, _RecordedStep] = {}
+        self._unrecordable = set()
 
     # ---------------------------------------------------------------- bookkeeping
     def computed_tokens(self, request: Hashable) -> int:
@@ -128,14 +154,7 @@ class ModelRunner:
         return self.cache.can_reserve(request, self._done.get(request, 0) + n_new)
 
     # ---------------------------------------------------------------- the step
-    def _build_context(self, entries: List[StepEntry]) -> StepContext:
-        ctx = StepContext(self.device)
-        ctx._workspace_owner = self
-        ps = self.page_size
-        token_ids: List[int] = []
-        positions: List[int] = []
-        seq_of_token: List[int] = []
-        logit_rows: List[int] = []
+    def _check_and_reserve(self, entries: List[StepEntry]) -> None:
         seen = set()
         for e in entries:
             if e.request in seen:
@@ -163,6 +182,16 @@ class ModelRunner:
         for request, total in totals:
             if not self.cache.reserve(request, total):
                 raise StepError(f"reserving {total} tokens for request {request!r} failed after the check passed")
+
+    def _describe(self, entries: List[StepEntry], ctx: StepContext, table_width: Optional[int] = None):
+        """Fill the host side of ``ctx`` and return every integer table of the step as one flat
+        list, with the places of its parts: [token ids | positions | sequence of token | logit rows |
+        per group: slot mapping, block table]."""
+        ps = self.page_size
+        token_ids: List[int] = []
+        positions: List[int] = []
+        seq_of_token: List[int] = []
+        logit_rows: List[int] = []
         row = 0
         for si, e in enumerate(entries):
             n = len(e.tokens)
@@ -181,13 +210,11 @@ class ModelRunner:
         ctx.n_seqs = len(entries)
         ctx.max_context = max(ctx.context_len)
         ctx.max_q_len = max(ctx.q_len)
-        T, B, R = row, len(entries), len(logit_rows)
-        # one upload for all integer tables
         flat: List[int] = token_ids + positions + seq_of_token + logit_rows
-        group_meta = []
+        layout = []
         for g in self.cache.groups:
             tables = [g.tables[e.request] for e in entries]
-            width = max(len(t) for t in tables)
+            width = table_width or max(len(t) for t in tables)
             slot_mapping: List[int] = []
             for e, table in zip(entries, tables):
                 done = self._done.get(e.request, 0)
@@ -202,16 +229,18 @@ class ModelRunner:
             for t in tables:
                 flat.extend(t)
                 flat.extend([-1] * (width - len(t)))
-            group_meta.append((off_slot, off_table, width))
-        dev = torch.tensor(flat, dtype=torch.int32).to(self.device, non_blocking=False)
+            layout.append((off_slot, off_table, width))
+        return flat, layout, len(logit_rows)
+
+    def _bind(self, ctx: StepContext, dev: torch.Tensor, layout, n_rows: int) -> None:
+        T, B = ctx.n_tokens, ctx.n_seqs
         ctx.token_ids = dev[0:T]
         ctx.positions = dev[T:2 * T]
         ctx.seq_of_token = dev[2 * T:3 * T]
-        ctx.logit_rows = dev[3 * T:3 * T + R] if R else None
-        for (off_slot, off_table, width) in group_meta:
-            ctx.groups.append(GroupView(block_table=dev[off_table:off_table + B * width].view(B, width),
-                                        slot_mapping=dev[off_slot:off_slot + T], page_size=ps))
-        return ctx
+        ctx.logit_rows = dev[3 * T:3 * T + n_rows] if n_rows else None
+        ctx.groups = [GroupView(block_table=dev[off_table:off_table + B * width].view(B, width),
+                                slot_mapping=dev[off_slot:off_slot + T], page_size=self.page_size)
+                      for (off_slot, off_table, width) in layout]
 
     def _layer_cache(self, ctx: StepContext):
         cache = self.cache
@@ -232,6 +261,69 @@ class ModelRunner:
 
         return get
 
+    # ---------------------------------------------------------------- recorded decode steps
+    def _graph_shape(self, entries: List[StepEntry]):
+        """Key of the recorded step that can run these entries, or None when they must run eagerly:
+        single tokens only, each wanting its logits; table width and context bound rounded up to
+        powers of two so that few recordings serve a growing context."""
+        if not self.use_graphs or not 0 < len(entries) <= self.GRAPH_MAX_BATCH:
+            return None
+        if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
+            return None
+        longest = max(self._done.get(e.request, 0) for e in entries) + 1
+        pages = max(16, 1 << (self.cache.pages_for(longest) - 1).bit_length())
+        bound = max(256, 1 << (longest - 1).bit_length())
+        key = (len(entries), pages, bound)
+        return None if key in self._unrecordable else key
+
+    def _record(self, key, entries: List[StepEntry]) -> Optional[_RecordedStep]:
+        B, pages, bound = key
+        ctx = StepContext(self.device, recording=True)
+        flat, layout, n_rows = self._describe(entries, ctx, table_width=pages)
+        ctx.max_context = bound
+        staging = torch.tensor(flat, dtype=torch.int32).pin_memory()
+        meta = staging.to(self.device)
+        self._bind(ctx, meta, layout, n_rows)
+        calls_before = K.library_calls()
+        # run the step once the ordinary way first: code objects get loaded and buffers sized outside
+        # the recording.  Running a decode step twice is harmless: it writes the same keys, values
+        # and logits again.
+        warm = StepContext(self.device, scratch_owner=self)
+        flat_w, layout_w, rows_w = self._describe(entries, warm)
+        self._bind(warm, torch.tensor(flat_w, dtype=torch.int32).to(self.device), layout_w, rows_w)
+        self.model.forward(warm, self._layer_cache(warm))
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(ctx, self._layer_cache(ctx))
+        if K.library_calls() != calls_before:
+            # a library routine ran inside: its nodes are not ours to vouch for, so this shape runs eagerly
+            self._unrecordable.add(key)
+            return None
+        rec = _RecordedStep(graph, meta, staging, logits, ctx, torch.cuda.Event())
+        rec.copied.record()
+        self._recorded[key] = rec
+        return rec
+
+    def _replay(self, key, entries: List[StepEntry]) -> Optional[torch.Tensor]:
+        rec = self._recorded.get(key)
+        if rec is None:
+            rec = self._record(key, entries)
+            if rec is None:
+                return None
+            # the recording itself ran nothing: fall through to the first replay
+        ctx = StepContext(self.device)
+        flat, _, _ = self._describe(entries, ctx, table_width=key[1])
+        if len(flat) != rec.staging.numel():
+            raise StepError("a recorded step was asked to run another shape")
+        rec.copied.synchronize()          # the previous upload must have read the staging buffer
+        rec.staging.copy_(torch.tensor(flat, dtype=torch.int32))
+        rec.meta.copy_(rec.staging, non_blocking=True)
+        rec.copied.record()
+        rec.graph.replay()
+        self._last_context_len = ctx.context_len
+        return rec.logits.clone()         # the graph's own buffer is overwritten by its next replay
+
     def step(self, entries: Sequence[StepEntry], end: Iterable[Hashable] = ()) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits ``[wanted, vocab]`` on the device, rows in the
         order of the entries and of each entry's ``want`` (None when nothing is wanted).  Requests
@@ -239,9 +331,21 @@ class ModelRunner:
         entries = list(entries)
         logits = None
         if entries:
-            ctx = self._build_context(entries)
-            logits = self.model.forward(ctx, self._layer_cache(ctx))
-            for e, total in zip(entries, ctx.context_len):
+            self._check_and_reserve(entries)
+            key = self._graph_shape(entries)
+            totals = None
+            if key is not None:
+                logits = self._replay(key, entries)
+                if logits is not None:
+                    totals = self._last_context_len
+            if totals is None:
+                ctx = StepContext(self.device, scratch_owner=self)
+                flat, layout, n_rows = self._describe(entries, ctx)
+                dev = torch.tensor(flat, dtype=torch.int32).to(self.device, non_blocking=False)
+                self._bind(ctx, dev, layout, n_rows)
+                logits = self.model.forward(ctx, self._layer_cache(ctx))
+                totals = ctx.context_len
+            for e, total in zip(entries, totals):
                 self._done[e.request] = total
                 self.cache.release_passed(e.request, total)
         for r in end:

@@ -268,6 +268,13 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
 # ------------------------------------------------------------------ matrix product (library)
 
 SKINNY_MAX_ROWS = 64
+_library_calls = 0
+
+
+def library_calls() -> int:
+    """How many matrix products went to the library so far (a recorded step must contain none)."""
+    return _library_calls
+
 
 
 def skinny_ok(M: int, K: int, dtype: torch.dtype) -> bool:
@@ -317,6 +324,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
     if skinny_ok(x.shape[0], x.shape[1], x.dtype):
         out = torch.empty(x.shape[0], weight.shape[0], dtype=out_dtype, device=x.device)
         return skinny_gemm(x, weight, out)
+    global _library_calls
+    _library_calls += 1
     if out_dtype != x.dtype:
         return torch.mm(x, weight.t(), out_dtype=out_dtype)
     return torch.matmul(x, weight.t())
@@ -329,6 +338,8 @@ def linear_swiglu(x: torch.Tensor, weight_gate_up: torch.Tensor) -> torch.Tensor
     out = torch.empty(x.shape[0], inter, dtype=x.dtype, device=x.device)
     if skinny_ok(x.shape[0], x.shape[1], x.dtype):
         return skinny_gemm(x, weight_gate_up, out, swiglu=True)
+    global _library_calls
+    _library_calls += 1
     return swiglu(torch.matmul(x, weight_gate_up.t()), out)
 
 

@@ -89,6 +89,9 @@ class Part:
 
     family = ""
     kind = ""
+    # True when a part's launches depend only on device data and on the sizes of the step, so that
+    # a step may be recorded once and replayed; a part that reads the step's host lists says False
+    graph_safe = False
 
     @classmethod
     def weight_requests(cls, spec: PartSpec) -> List[WeightRequest]:

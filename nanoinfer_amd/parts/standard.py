@@ -35,6 +35,8 @@ class TableEmbedding(Part):
     """``h[t] = E[id[t]]``, no scaling (src/op/embedding.cpp:14-70, kernel embedding_kernel.cu:30-48).
     params: vocab_size, hidden_size.  weights: weight [vocab, hidden]."""
 
+    graph_safe = True
+
     @classmethod
     def weight_requests(cls, spec):
         return [WeightRequest(spec.weights["weight"], (spec.params["vocab_size"], spec.params["hidden_size"]))]
@@ -56,6 +58,8 @@ class TableEmbedding(Part):
 class RMSNorm(Part):
     """``x * rsqrt(mean(x^2) + eps) * w`` in float32 (src/op/rmsnorm.cpp:14-69, rmsnorm_kernel.cu:50-103).
     params: size, eps.  weights: weight [size]."""
+
+    graph_safe = True
 
     @classmethod
     def weight_requests(cls, spec):
@@ -102,6 +106,8 @@ class RotaryPosition(Part):
     """Rotation of pairs by ``pos * f_p``.  params: rotary_dim, theta, scaling (dict or None),
     max_positions.  One table per distinct set of constants is shared by all layers."""
 
+    graph_safe = True
+
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
         p = spec.params
@@ -125,6 +131,8 @@ class RotaryPosition(Part):
 class NoPosition(Part):
     """No position encoding: keys and queries are used as projected."""
 
+    graph_safe = True
+
     max_positions = None
 
     def tables(self):
@@ -143,6 +151,8 @@ class Attention(Part):
     The three input projections are stacked into one matrix at load, so one product feeds the
     rotation-and-cache-write kernel directly.
     """
+
+    graph_safe = True
 
     @classmethod
     def weight_requests(cls, spec):
@@ -201,6 +211,8 @@ class SwiGLU(Part):
     params: hidden_size, intermediate_size.  weights: gate [I, d], up [I, d], down [d, I].
     gate and up are stacked so one product yields both halves."""
 
+    graph_safe = True
+
     @classmethod
     def weight_requests(cls, spec):
         p, w = spec.params, spec.weights
@@ -250,6 +262,9 @@ class PreNormBlock:
     def cache_need(self) -> CacheNeed:
         return self.mixer.cache_need()
 
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe is True for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn))
+
     def forward(self, h, pending, ctx, cache: LayerCache):
         x = self.mixer_norm.forward(h, pending)
         a = self.mixer.forward(x, ctx, cache)
@@ -265,6 +280,8 @@ class LinearHead(Part):
     """``logits = x . W^T`` in float32 output (src/model/llama.cpp:383-386).  params: vocab_size,
     hidden_size.  weights: weight [vocab, hidden]; a tied head names the embedding's tensor and
     shares its device buffer."""
+
+    graph_safe = True
 
     @classmethod
     def weight_requests(cls, spec):

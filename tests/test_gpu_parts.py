@@ -131,6 +131,7 @@ class SpecRunner:
         r.cache = KVCacheManager(r.model.cache_needs(), page_size, max_tokens // page_size, 4, dtype=DT[dtype], device=r.device)
         r.vocab_size, r.max_positions, r.eos_token_ids = spec.vocab_size, r.model.max_positions, ()
         r._done, r._scratch = {}, None
+        r._init_graphs(True)
         return r
 
 

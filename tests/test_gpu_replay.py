@@ -264,3 +264,55 @@ def test_trace_run_program(dtype, tmp_path):
                 row += 1
             held[r] = base + len(t)
     compare(got, requests, folder, dtype, "trace_run mixed")
+
+
+# ------------------------------------------------------------------ recorded (HIP graph) decode steps
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_decode_steps_equal_eager_ones(dtype):
+    """Decode steps are recorded once per shape and replayed.  Every replay is checked against a
+    runner that records nothing, with eager work (prompt portions of other requests, requests
+    coming and going, a changing batch size) and synchronisations between the replays."""
+    from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
+    name = "B"
+    folder = model_folder(name)
+    vocab = ALL[name]["vocab_size"]
+    recorded = ModelRunner(folder, dtype=dtype, page_size=8, max_tokens=1024, max_requests=4)
+    eager = ModelRunner(folder, dtype=dtype, page_size=8, max_tokens=1024, max_requests=4, use_graphs=False)
+    assert recorded.use_graphs and not eager.use_graphs
+    reqs = {f"g{i}": random_tokens(vocab, n, 300 + i) for i, n in enumerate((150, 90, 120))}
+    done = {k: 0 for k in reqs}
+    got = {}
+
+    def both(entries, end=()):
+        a = recorded.step([StepEntry(*e) for e in entries], end=end)
+        b = eager.step([StepEntry(*e) for e in entries], end=end)
+        torch.cuda.synchronize()
+        assert (a is None) == (b is None)
+        if a is not None:
+            assert float((a - b).abs().max()) <= TOL[dtype] * float(b.abs().max()) * 0.1
+            row = 0
+            for rid, toks, want in entries:
+                for w in want:
+                    got[(rid, done[rid] + w)] = a[row].clone()
+                    row += 1
+        for rid, toks, _ in entries:
+            done[rid] += len(toks)
+
+    def dec(rid):
+        return (rid, [reqs[rid][done[rid]]], [0])
+
+    both([("g0", list(reqs["g0"][:40]), [39])])
+    for _ in range(30):
+        both([dec("g0")])                                        # batch 1, replayed
+    both([("g1", list(reqs["g1"][:33]), []), dec("g0")])          # eager: a prompt portion beside a token
+    for _ in range(25):
+        both([dec("g0"), dec("g1")])                              # batch 2
+    both([("g2", list(reqs["g2"][:64]), [0, 63])])
+    for i in range(30):
+        both([dec("g1"), dec("g2"), dec("g0")] if i % 3 else [dec("g2"), dec("g0")])
+    while done["g1"] < len(reqs["g1"]):
+        both([dec("g1")], end=["g1"] if done["g1"] == len(reqs["g1"]) - 1 else ())
+    both([dec("g0"), dec("g2")])
+    assert len(recorded._recorded) >= 3 and not eager._recorded
+    compare(got, reqs, folder, dtype, "recorded decode")
