@@ -7,7 +7,11 @@
 // 64/LPK whole rows per access, which are adjacent in a pool laid out
 // [page, kv_head, slot_in_page, head_dim].  Every lane group keeps a running (max, sum, output)
 // of its own for each query head; they are merged across the wave by shuffles, across waves
-// through LDS and across splits by a second kernel.  Softmax and both products are float32.
+// through LDS, and across splits by a second, small kernel (letting the last workgroup of a split
+// range do it needs device-wide fences, which cost more on this chip of eight L2 caches than the
+// second launch does).
+// Softmax and both products are float32; the bfloat16 instantiation takes exponentials with the
+// hardware's exp2, the float32 one with the accurate library routine.
 //
 // Formula (reference: src/op/kernels/cuda/paged_attention_kernel.cu:111-199 for one token,
 // src/op/kernels/cuda/prefill_attention_kernel.cu:66-141 for a chunk): the query at position P
@@ -34,17 +38,24 @@ template <typename T> struct Lanes {
     static constexpr int KPI = ATT_THREADS / LPK;  // keys per workgroup iteration
 };
 
-__device__ __forceinline__ float scale_of(float m, float m_new) { return m == -INFINITY ? 0.f : expf(m - m_new); }
+// "minus infinity" that stays finite under subtraction: exp(NEG - x) is 0, never NaN
+#define NEG_BIG (-1.0e30f)
+
+template <bool FAST> __device__ __forceinline__ float ex(float x) {
+    if constexpr (FAST) return __expf(x);
+    else return expf(x);
+}
 
 template <typename T>
 __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ kpool, const T* __restrict__ vpool,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ seq_of_token,
-    const int32_t* __restrict__ positions, T* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int H, int KVH, int page_size, int window, float scale, int nsplit) {
+    const int32_t* __restrict__ positions, T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+    int H, int KVH, int page_size, int window, float scale, int nsplit) {
     using L = Lanes<T>;
     constexpr int LPK = L::LPK, EPL = L::EPL, KPI = L::KPI, HD = HEAD_DIM;
     constexpr int WAVES = ATT_THREADS / WAVE;
+    constexpr bool FAST = sizeof(T) == 2;
 
     const int t = blockIdx.x;
     const int G = H / KVH;
@@ -84,43 +95,64 @@ __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
     float m[GT], l[GT], acc[GT][EPL];
 #pragma unroll
     for (int i = 0; i < GT; ++i) {
-        m[i] = -INFINITY;
+        m[i] = NEG_BIG;
         l[i] = 0.f;
 #pragma unroll
         for (int e = 0; e < EPL; ++e) acc[i][e] = 0.f;
     }
 
+    // U keys per lane group and trip: their table entries are fetched first, then all their rows,
+    // then the arithmetic.  The running maximum moves once per trip, so a trip costs one
+    // rescaling of the output and U + 1 exponentials per head.
+    constexpr int U = EPL <= 8 ? 4 : 2;
+    const int page_shift = (page_size & (page_size - 1)) == 0 ? __ffs(page_size) - 1 : -1;
     const int iters = (k1 > k0) ? (k1 - k0 + KPI - 1) / KPI : 0;
-    for (int it = 0; it < iters; ++it) {
-        const int j = k0 + it * KPI + kslot;
-        const bool valid = j < k1;
-        float kk[EPL], vv[EPL];
-        if (valid) {
-            const int page = table[j / page_size];
-            const int off = j % page_size;
-            const size_t base = ((static_cast<size_t>(page) * KVH + g) * page_size + off) * HD + sub * EPL;
-            VecIO<T, EPL>::load(kpool + base, kk);
-            VecIO<T, EPL>::load(vpool + base, vv);
-        } else {
+    for (int it = 0; it < iters; it += U) {
+        bool valid[U];
+        size_t base[U];
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) { kk[e] = 0.f; vv[e] = 0.f; }
+        for (int u = 0; u < U; ++u) {
+            const int j = k0 + (it + u) * KPI + kslot;
+            valid[u] = j < k1;
+            const int jj = valid[u] ? j : k0;       // a key of this sequence in any case: the address stays legal
+            const int lp = page_shift >= 0 ? (jj >> page_shift) : jj / page_size;
+            const int off = page_shift >= 0 ? (jj & (page_size - 1)) : jj % page_size;
+            const int page = table[lp];
+            base[u] = ((static_cast<size_t>(page) * KVH + g) * page_size + off) * HD + sub * EPL;
+        }
+        float kk[U][EPL], vv[U][EPL];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            VecIO<T, EPL>::load(kpool + base[u], kk[u]);
+            VecIO<T, EPL>::load(vpool + base[u], vv[u]);
         }
 #pragma unroll
         for (int i = 0; i < GT; ++i) {
-            float s = 0.f;
+            float sc[U];
+            float m_new = m[i];
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) s += qreg[i][e] * kk[e];
+            for (int u = 0; u < U; ++u) {
+                float d = 0.f;
 #pragma unroll
-            for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, WAVE);
-            if (valid) {
-                const float m_new = fmaxf(m[i], s);
-                const float corr = scale_of(m[i], m_new);
-                const float p = expf(s - m_new);
-                l[i] = l[i] * corr + p;
+                for (int e = 0; e < EPL; ++e) d += qreg[i][e] * kk[u][e];
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) acc[i][e] = acc[i][e] * corr + p * vv[e];
-                m[i] = m_new;
+                for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, WAVE);
+                sc[u] = d;
+                if (valid[u]) m_new = fmaxf(m_new, d);
             }
+            const float corr = ex<FAST>(m[i] - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) acc[i][e] *= corr;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const float p = valid[u] ? ex<FAST>(sc[u] - m_new) : 0.f;
+                psum += p;
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) acc[i][e] += p * vv[u][e];
+            }
+            l[i] = l[i] * corr + psum;
+            m[i] = m_new;
         }
     }
 
@@ -132,8 +164,8 @@ __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
             const float m_o = __shfl_xor(m[i], o, WAVE);
             const float l_o = __shfl_xor(l[i], o, WAVE);
             const float m_new = fmaxf(m[i], m_o);
-            const float a = scale_of(m[i], m_new);
-            const float b = scale_of(m_o, m_new);
+            const float a = ex<FAST>(m[i] - m_new);
+            const float b = ex<FAST>(m_o - m_new);
             l[i] = l[i] * a + l_o * b;
 #pragma unroll
             for (int e = 0; e < EPL; ++e) {
@@ -168,9 +200,9 @@ __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
         float Lsum = 0.f, O = 0.f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
-            const float sc = scale_of(sm_m[w][i], M);
-            Lsum += sm_l[w][i] * sc;
-            O += sm_acc[w][i][dim] * sc;
+            const float f = ex<FAST>(sm_m[w][i] - M);
+            Lsum += sm_l[w][i] * f;
+            O += sm_acc[w][i][dim] * f;
         }
         const int h = h0 + i;
         if (nsplit == 1) {
@@ -187,16 +219,18 @@ __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
 template <typename T>
 __global__ void merge_splits_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                     T* __restrict__ out, int H, int nsplit) {
+    constexpr bool FAST = sizeof(T) == 2;
     const int t = blockIdx.x, h = blockIdx.y;
     const size_t p0 = (static_cast<size_t>(t) * H + h) * nsplit;
-    float M = -INFINITY;
+    float M = NEG_BIG;
     for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[(p0 + s) * 2]);
     for (int dim = threadIdx.x; dim < HEAD_DIM; dim += blockDim.x) {
         float Lsum = 0.f, O = 0.f;
+#pragma unroll 4
         for (int s = 0; s < nsplit; ++s) {
-            const float sc = scale_of(part_ml[(p0 + s) * 2], M);
-            Lsum += part_ml[(p0 + s) * 2 + 1] * sc;
-            O += part_o[(p0 + s) * HEAD_DIM + dim] * sc;
+            const float f = ex<FAST>(part_ml[(p0 + s) * 2] - M);
+            Lsum += part_ml[(p0 + s) * 2 + 1] * f;
+            O += part_o[(p0 + s) * HEAD_DIM + dim] * f;
         }
         st(out + static_cast<size_t>(t) * H * HEAD_DIM + static_cast<size_t>(h) * HEAD_DIM + dim, O / Lsum);
     }
@@ -205,15 +239,15 @@ __global__ void merge_splits_kernel(const float* __restrict__ part_o, const floa
 template <typename T>
 static int launch(const void* q, int q_stride, const void* kpool, const void* vpool, const void* block_table,
                   int table_stride, const void* seq_of_token, const void* positions, void* out, void* part_o,
-                  void* part_ml, int T_tokens, int H, int KVH, int page_size, int window, float scale, int nsplit,
-                  hipStream_t stream) {
+                  void* part_ml, int T_tokens, int H, int KVH, int page_size, int window, float scale,
+                  int nsplit, hipStream_t stream) {
     const int G = H / KVH;
     const int chunks = (G + GT - 1) / GT;
     dim3 grid(T_tokens, KVH * chunks, nsplit);
     token_attention_kernel<T><<<grid, ATT_THREADS, 0, stream>>>(
         (const T*)q, q_stride, (const T*)kpool, (const T*)vpool, (const int32_t*)block_table, table_stride,
-        (const int32_t*)seq_of_token, (const int32_t*)positions, (T*)out, (float*)part_o, (float*)part_ml, H, KVH,
-        page_size, window, scale, nsplit);
+        (const int32_t*)seq_of_token, (const int32_t*)positions, (T*)out, (float*)part_o, (float*)part_ml,
+        H, KVH, page_size, window, scale, nsplit);
     int err = NI_LAUNCH_RESULT();
     if (err || nsplit == 1) return err;
     merge_splits_kernel<T><<<dim3(T_tokens, H), 64, 0, stream>>>((const float*)part_o, (const float*)part_ml, (T*)out,
@@ -222,15 +256,17 @@ static int launch(const void* q, int q_stride, const void* kpool, const void* vp
 }
 
 NI_EXPORT int ni_attention_head_dim() { return HEAD_DIM; }
+NI_EXPORT int ni_attention_heads_per_group() { return GT; }
 
 // part_o: float [T, H, nsplit, HEAD_DIM], part_ml: float [T, H, nsplit, 2]; unused when nsplit == 1.
 NI_EXPORT int ni_token_attention(const void* q, int q_stride, const void* kpool, const void* vpool,
                                  const void* block_table, int table_stride, const void* seq_of_token,
-                                 const void* positions, void* out, void* part_o, void* part_ml, int T_tokens, int H,
-                                 int KVH, int page_size, int window, float scale, int nsplit, int dtype,
-                                 hipStream_t stream) {
+                                 const void* positions, void* out, void* part_o, void* part_ml,
+                                 int T_tokens, int H, int KVH, int page_size, int window, float scale, int nsplit,
+                                 int dtype, hipStream_t stream) {
     if (T_tokens <= 0) return 0;
     if (H % KVH != 0 || nsplit < 1 || nsplit > 65535 || page_size < 1) return -1;
+    if (nsplit > 1 && (!part_o || !part_ml)) return -2;
     if (dtype == 0)
         return launch<float>(q, q_stride, kpool, vpool, block_table, table_stride, seq_of_token, positions, out,
                              part_o, part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, stream);

@@ -28,10 +28,56 @@ __global__ void embedding_kernel(const int32_t* __restrict__ ids, const T* __res
 // Without `rows` the sum is written back to h (the residual stream moves on) and out has T rows.
 // With `rows` (a gather before the output head) h is left alone and out row r comes from h[rows[r]].
 // Formula: src/op/kernels/cuda/rmsnorm_kernel.cu:50-103 of the reference.
-template <typename TP, typename TO>
+// Rows of up to NV * blockDim elements are held in registers: every load of the row is issued
+// before anything waits, and the row is read from memory once.
+template <typename TP, typename TO, int NV>
 __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TP* __restrict__ pending,
                                    const float* __restrict__ w, TO* __restrict__ out,
                                    const int32_t* __restrict__ rows, int d, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
+    float* hrow = h + src * d;
+    const TP* prow = pending ? pending + src * d : nullptr;
+    float v[NV], wv[NV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        v[j] = i < d ? hrow[i] : 0.f;
+        wv[j] = i < d ? w[i] : 0.f;
+    }
+    if (prow) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int i = threadIdx.x + j * blockDim.x;
+            if (i < d) v[j] += ld(prow + i);
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) ss += v[j] * v[j];
+    if (!rows && prow) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int i = threadIdx.x + j * blockDim.x;
+            if (i < d) hrow[i] = v[j];
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(d) + eps);
+    TO* orow = out + static_cast<size_t>(r) * d;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        if (i < d) st(orow + i, (v[j] * inv) * wv[j]);
+    }
+}
+
+// Rows of any width: two passes over memory.
+template <typename TP, typename TO>
+__global__ void add_rmsnorm_wide_kernel(float* __restrict__ h, const TP* __restrict__ pending,
+                                        const float* __restrict__ w, TO* __restrict__ out,
+                                        const int32_t* __restrict__ rows, int d, float eps) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
@@ -169,16 +215,27 @@ NI_EXPORT int ni_embedding(const void* ids, const void* table, void* out, int T,
     return NI_LAUNCH_RESULT();
 }
 
+template <typename TP, typename TO>
+static void launch_add_rmsnorm(float* h, const TP* pending, const float* w, TO* out, const int32_t* rows, int n_rows,
+                               int d, float eps, hipStream_t stream) {
+    constexpr int NV = 8;
+    if (d <= NV * 1024) {
+        const int threads = d <= NV * 64 ? 64 : d <= NV * 128 ? 128 : d <= NV * 256 ? 256 : d <= NV * 512 ? 512 : 1024;
+        add_rmsnorm_kernel<TP, TO, NV><<<n_rows, threads, 0, stream>>>(h, pending, w, out, rows, d, eps);
+    } else {
+        add_rmsnorm_wide_kernel<TP, TO><<<n_rows, 1024, 0, stream>>>(h, pending, w, out, rows, d, eps);
+    }
+}
+
 NI_EXPORT int ni_add_rmsnorm(void* h, const void* pending, const void* w, void* out, const void* rows,
                              int n_rows, int d, float eps, int dtype, hipStream_t stream) {
     if (n_rows <= 0) return 0;
-    const int threads = d >= 1024 ? 256 : (d >= 256 ? 128 : 64);
     if (dtype == 0)
-        add_rmsnorm_kernel<float, float><<<n_rows, threads, 0, stream>>>(
-            (float*)h, (const float*)pending, (const float*)w, (float*)out, (const int32_t*)rows, d, eps);
+        launch_add_rmsnorm<float, float>((float*)h, (const float*)pending, (const float*)w, (float*)out,
+                                         (const int32_t*)rows, n_rows, d, eps, stream);
     else
-        add_rmsnorm_kernel<bf16_t, bf16_t><<<n_rows, threads, 0, stream>>>(
-            (float*)h, (const bf16_t*)pending, (const float*)w, (bf16_t*)out, (const int32_t*)rows, d, eps);
+        launch_add_rmsnorm<bf16_t, bf16_t>((float*)h, (const bf16_t*)pending, (const float*)w, (bf16_t*)out,
+                                           (const int32_t*)rows, n_rows, d, eps, stream);
     return NI_LAUNCH_RESULT();
 }
 

@@ -46,13 +46,64 @@ __device__ int block_argmax(const float* __restrict__ row, int V, float* out_max
     return idx;
 }
 
-__global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(const float* __restrict__ logits, int32_t* __restrict__ out,
-                                                               int V) {
-    __shared__ float s_val[SAMPLE_WAVES];
-    __shared__ int s_idx[SAMPLE_WAVES];
-    float mx;
-    int idx = block_argmax(logits + static_cast<size_t>(blockIdx.x) * V, V, &mx, s_val, s_idx);
-    if (threadIdx.x == 0) out[blockIdx.x] = idx;
+// Stage one: ARGMAX_PARTS workgroups share a row, each finds the best of its slice (float4 loads
+// when the row allows).  Stage two: one wavefront per row picks among the parts.
+#define ARGMAX_PARTS 32
+#define ARGMAX_THREADS 256
+
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_part_kernel(const float* __restrict__ logits, float* __restrict__ part_val,
+                                                                    int32_t* __restrict__ part_idx, int V) {
+    __shared__ float s_val[ARGMAX_THREADS / WAVE];
+    __shared__ int s_idx[ARGMAX_THREADS / WAVE];
+    const int r = blockIdx.x, part = blockIdx.y;
+    const float* row = logits + static_cast<size_t>(r) * V;
+    const int per = ((V + ARGMAX_PARTS - 1) / ARGMAX_PARTS + 3) & ~3;      // a multiple of 4 elements
+    const int lo = part * per, hi = min(V, lo + per);
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    if ((V & 3) == 0) {         // rows are 16-byte aligned: four logits a load
+        for (int i = lo + threadIdx.x * 4; i < hi; i += ARGMAX_THREADS * 4) {
+            const float4 v = *reinterpret_cast<const float4*>(row + i);
+            better(best, idx, v.x, i);
+            better(best, idx, v.y, i + 1);
+            better(best, idx, v.z, i + 2);
+            better(best, idx, v.w, i + 3);
+        }
+    } else {
+        for (int i = lo + threadIdx.x; i < hi; i += ARGMAX_THREADS) better(best, idx, row[i], i);
+    }
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+        float v2 = __shfl_xor(best, off, WAVE);
+        int i2 = __shfl_xor(idx, off, WAVE);
+        better(best, idx, v2, i2);
+    }
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    if (lane == 0) { s_val[wave] = best; s_idx[wave] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < ARGMAX_THREADS / WAVE; ++w) better(best, idx, s_val[w], s_idx[w]);
+        part_val[r * ARGMAX_PARTS + part] = best;
+        part_idx[r * ARGMAX_PARTS + part] = idx;
+    }
+}
+
+__global__ void argmax_final_kernel(const float* __restrict__ part_val, const int32_t* __restrict__ part_idx,
+                                    int32_t* __restrict__ out) {
+    const int r = blockIdx.x;
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    if (threadIdx.x < ARGMAX_PARTS) {
+        best = part_val[r * ARGMAX_PARTS + threadIdx.x];
+        idx = part_idx[r * ARGMAX_PARTS + threadIdx.x];
+    }
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+        float v2 = __shfl_xor(best, off, WAVE);
+        int i2 = __shfl_xor(idx, off, WAVE);
+        better(best, idx, v2, i2);
+    }
+    if (threadIdx.x == 0) out[r] = idx == 0x7fffffff ? 0 : idx;    // a row of NaN: the first token
 }
 
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
@@ -210,9 +261,14 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     if (tid == 0) out[r] = s_pick != 0x7fffffff ? s_pick : (s_last >= 0 ? s_last : best);
 }
 
-NI_EXPORT int ni_argmax(const void* logits, void* out, int R, int V, hipStream_t stream) {
+// part_val: float [R, 32], part_idx: int32 [R, 32] scratch
+NI_EXPORT int ni_argmax(const void* logits, void* out, void* part_val, void* part_idx, int R, int V, hipStream_t stream) {
     if (R <= 0) return 0;
-    argmax_kernel<<<R, SAMPLE_THREADS, 0, stream>>>((const float*)logits, (int32_t*)out, V);
+    argmax_part_kernel<<<dim3(R, ARGMAX_PARTS), ARGMAX_THREADS, 0, stream>>>((const float*)logits, (float*)part_val,
+                                                                             (int32_t*)part_idx, V);
+    int err = NI_LAUNCH_RESULT();
+    if (err) return err;
+    argmax_final_kernel<<<R, WAVE, 0, stream>>>((const float*)part_val, (const int32_t*)part_idx, (int32_t*)out);
     return NI_LAUNCH_RESULT();
 }
 

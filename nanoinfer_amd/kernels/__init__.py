@@ -243,7 +243,9 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
     if out is None:
         out = torch.empty(R, dtype=torch.int32, device=logits.device)
     _gpu(out, "out", torch.int32, (R,))
-    _check(sampling_lib().ni_argmax(_ptr(logits), _ptr(out), R, V, _stream()), "argmax")
+    part_val = torch.empty(R, 32, dtype=torch.float32, device=logits.device)
+    part_idx = torch.empty(R, 32, dtype=torch.int32, device=logits.device)
+    _check(sampling_lib().ni_argmax(_ptr(logits), _ptr(out), _ptr(part_val), _ptr(part_idx), R, V, _stream()), "argmax")
     return out
 
 
