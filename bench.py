@@ -79,6 +79,8 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (named in config)")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
+                    help="run one phase only (for profiling; prints no result line)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
@@ -154,6 +156,13 @@ def main() -> int:
             runner.release(i)
         return dt / steps, mean_ctx
 
+    if args.phase == "prefill":
+        log(f"prefill of {PROMPT_LEN}: {measure_prefill() * 1e3:.2f} ms")
+        return 0
+    if args.phase == "decode":
+        step_s, _ = measure_decode(args.batch, args.steps, args.warmup)
+        log(f"decode batch {args.batch}: {step_s * 1e3:.3f} ms a step")
+        return 0
     log("prefill ...")
     prefill_s = measure_prefill()
     log(f"prefill of {PROMPT_LEN}: {prefill_s * 1e3:.2f} ms")
