@@ -94,12 +94,14 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-    // two pieces per trip, all their loads issued before the first multiply, to keep enough bytes in flight
+    // PT pieces per trip, all their loads issued before the first multiply, to keep enough bytes in
+    // flight; the wavefront covers pieces [first + wave * per_wave, ...) of its K range in order.
+    constexpr int PT = (NT * MB <= 2) ? 4 : 2;
     const int pieces = (K + CH - 1) / CH;
-    for (int c = wave; c < pieces; c += 2 * GV_WAVES) {
-        Piece<T> xb[2][MB], wa[2][NT];
+    for (int c = wave; c < pieces; c += PT * GV_WAVES) {
+        Piece<T> xb[PT][MB], wa[PT][NT];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < PT; ++u) {
             const int k = (c + u * GV_WAVES) * CH + kg * EL;
             const bool kok = k < K;                  // K is a multiple of EL: a lane's 32 bytes are all in or all out
 #pragma unroll
@@ -112,7 +114,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
             }
         }
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+        for (int u = 0; u < PT; ++u)
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
