@@ -12,7 +12,10 @@
 // both operands is all that is required.  Partial sums meet in LDS.
 //
 // Epilogues: store (compute type or float32), or SwiGLU over paired tiles (tile 2j from the gate
-// rows, tile 2j+1 from the up rows of a stacked [2I, K] matrix): out[m, n] = silu(g) * u.
+// rows, tile 2j+1 from the up rows of a stacked [2I, K] matrix): out[m, n] = silu(g) * u; or
+// rotation + cache write for a stacked [q; k; v] matrix: a workgroup owns the two tiles of one
+// head that hold the partners (j, j + hd/2) of a rotation, turns them by the angle of the row's
+// position, and stores query heads to a buffer, key and value heads straight into their pages.
 // float32 inputs are multiplied in true float32 (no reduced-precision MFMA).
 #include <type_traits>
 
@@ -57,11 +60,23 @@ template <> struct Piece<float> {
     }
 };
 
-enum { EPI_STORE = 0, EPI_SWIGLU = 1 };
+enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_ROPE = 2 };
+
+// What the rotation epilogue needs beside the product.
+struct RopeArgs {
+    const int32_t* positions;      // [M]
+    const float* cos_t;            // [max_pos, hd/2]
+    const float* sin_t;
+    const int32_t* slot_mapping;   // [M] page * page_size + slot, or null: keys and values are not stored
+    void* kpool;                   // [pages, KVH, page_size, hd]
+    void* vpool;
+    int H, KVH, hd, page_size;
+};
 
 template <typename T, typename TOUT, int MB, int NT, int EPI>
 __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __restrict__ x, const T* __restrict__ W,
-                                                                 TOUT* __restrict__ y, int M, int N, int K, int I) {
+                                                                 TOUT* __restrict__ y, int M, int N, int K, int I,
+                                                                 RopeArgs rope) {
     constexpr int EL = Piece<T>::ELEMS;
     constexpr int CH = 4 * EL;                       // k elements in a 128-byte piece of a row
     const int tid = threadIdx.x;
@@ -75,7 +90,11 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
     const T* wrow[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        const int col0 = (EPI == EPI_SWIGLU) ? (wg * (NT / 2) + nt / 2) * 16 : (wg * NT + nt) * 16;
+        int col0 = (EPI == EPI_SWIGLU) ? (wg * (NT / 2) + nt / 2) * 16 : (wg * NT + nt) * 16;
+        if (EPI == EPI_ROPE) {      // workgroup = (head, pair of tiles): dims [16 p, 16 p + 16) and the same + hd/2
+            const int per_head = rope.hd / 32;
+            col0 = (wg / per_head) * rope.hd + (wg % per_head) * 16 + nt * (rope.hd / 2);
+        }
         const int shift = (EPI == EPI_SWIGLU && (nt % 2)) ? I : 0;      // odd tiles of a pair come from the up rows
         wrow[nt] = W + static_cast<size_t>(min(col0 + r, n_limit - 1) + shift) * K;
     }
@@ -132,6 +151,51 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
     __syncthreads();
 
     // D[n_local][m_local] of a tile sits at lane = (n_local / 4) * 16 + m_local, register n_local % 4
+    if constexpr (EPI == EPI_ROPE) {
+        const int per_head = rope.hd / 32;
+        const int head = wg / per_head;                 // among H query, KVH key, KVH value heads
+        const int j0 = (wg % per_head) * 16;            // first of this workgroup's 16 pairs
+        const int half = rope.hd / 2;
+        for (int item = tid; item < MB * 16 * 16; item += GV_THREADS) {
+            const int n_local = item % 16;
+            const int m = item / 16;
+            if (m >= M) continue;
+            const int mb = m / 16, m_local = m % 16;
+            const int src = ((n_local / 4) * 16 + m_local) * 4 + (n_local % 4);
+            float x0 = 0.f, x1 = 0.f;
+#pragma unroll
+            for (int w = 0; w < GV_WAVES; ++w) {
+                x0 += red[w][0 * MB + mb][src];
+                x1 += red[w][1 * MB + mb][src];
+            }
+            const int j = j0 + n_local;
+            if (head < rope.H + rope.KVH) {             // queries and keys turn, values do not
+                const int pos = rope.positions[m];
+                const float c = rope.cos_t[static_cast<size_t>(pos) * half + j];
+                const float sn = rope.sin_t[static_cast<size_t>(pos) * half + j];
+                const float y0 = x0 * c - x1 * sn;
+                const float y1 = x0 * sn + x1 * c;
+                x0 = y0; x1 = y1;
+            }
+            if (head < rope.H) {
+                TOUT* dst = y + static_cast<size_t>(m) * rope.H * rope.hd + static_cast<size_t>(head) * rope.hd;
+                st(dst + j, x0);
+                st(dst + j + half, x1);
+            } else if (rope.slot_mapping) {
+                const int slot = rope.slot_mapping[m];
+                if (slot >= 0) {
+                    const bool is_k = head < rope.H + rope.KVH;
+                    const int g = is_k ? head - rope.H : head - rope.H - rope.KVH;
+                    TOUT* pool = static_cast<TOUT*>(is_k ? rope.kpool : rope.vpool);
+                    TOUT* dst = pool + ((static_cast<size_t>(slot / rope.page_size) * rope.KVH + g) * rope.page_size +
+                                        slot % rope.page_size) * rope.hd;
+                    st(dst + j, x0);
+                    st(dst + j + half, x1);
+                }
+            }
+        }
+        return;
+    }
     constexpr int NOUT = (EPI == EPI_SWIGLU) ? NT / 2 : NT;      // output tiles of the workgroup
     const int out_n0 = wg * NOUT * 16;
     const int out_width = (EPI == EPI_SWIGLU) ? I : N;
@@ -162,20 +226,21 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
 }
 
 template <typename T, typename TOUT, int MB, int EPI>
-static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream) {
+static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream,
+                     RopeArgs rope = RopeArgs{}) {
     const int out_width = (EPI == EPI_SWIGLU) ? I : N;
     const int tiles = (out_width + 15) / 16;
     auto run = [&](auto nt_tag) {
         constexpr int NTc = decltype(nt_tag)::value;
         constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
         const int grid = (tiles + NOUT - 1) / NOUT;
-        skinny_gemm_kernel<T, TOUT, MB, NTc, EPI><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I);
+        skinny_gemm_kernel<T, TOUT, MB, NTc, EPI><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope);
     };
     // NT * MB fragments of partial sums share 64 KB of LDS: at most 8
-    if constexpr (MB <= 2) {
+    if constexpr (MB <= 2 && EPI != EPI_ROPE) {
         if (NT >= 4) { run(std::integral_constant<int, 4>{}); return NI_LAUNCH_RESULT(); }
     }
-    if constexpr (EPI == EPI_SWIGLU) {
+    if constexpr (EPI == EPI_SWIGLU || EPI == EPI_ROPE) {
         run(std::integral_constant<int, 2>{});
     } else {
         if (NT >= 2) run(std::integral_constant<int, 2>{});
@@ -185,10 +250,11 @@ static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K,
 }
 
 template <typename T, typename TOUT, int EPI>
-static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream) {
-    if (M <= 16) return launch_nt<T, TOUT, 1, EPI>(x, W, y, M, N, K, I, NT, stream);
-    if (M <= 32) return launch_nt<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream);
-    return launch_nt<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, stream);
+static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream,
+                     RopeArgs rope = RopeArgs{}) {
+    if (M <= 16) return launch_nt<T, TOUT, 1, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
+    if (M <= 32) return launch_nt<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
+    return launch_nt<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
 }
 
 // epilogue: 0 store in the input type, 1 store float32, 2 SwiGLU (W is [2I, K], y is [M, I]).
@@ -208,4 +274,22 @@ NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N
     if (epilogue == 2) return launch_mb<bf16_t, bf16_t, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, stream);
     if (epilogue == 1) return launch_mb<bf16_t, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, stream);
     return launch_mb<bf16_t, bf16_t, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, stream);
+}
+
+// Product with the stacked [q; k; v] matrix ((H + 2 KVH) * hd rows), rotation of query and key
+// heads by the rows' positions, queries to q_out [M, H * hd], keys and values into the pools at
+// slot_mapping (null: not stored).  hd must be a multiple of 32 and fully rotated.
+NI_EXPORT int ni_skinny_qkv_rope(const void* x, const void* W, void* q_out, const void* positions, const void* cos_t,
+                                 const void* sin_t, const void* slot_mapping, void* kpool, void* vpool, int M, int K,
+                                 int H, int KVH, int hd, int page_size, int dtype, hipStream_t stream) {
+    if (M <= 0) return 0;
+    if (M > 64) return -1;
+    if (K % (dtype == 0 ? 8 : 16) != 0) return -2;
+    if (hd % 32 != 0 || H <= 0 || KVH <= 0 || page_size < 1) return -3;
+    RopeArgs rope{(const int32_t*)positions, (const float*)cos_t, (const float*)sin_t, (const int32_t*)slot_mapping,
+                  kpool, vpool, H, KVH, hd, page_size};
+    const int N = (H + 2 * KVH) * hd;
+    // launch_nt sizes the grid from the output width: one workgroup per two tiles
+    if (dtype == 0) return launch_mb<float, float, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, stream, rope);
+    return launch_mb<bf16_t, bf16_t, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, stream, rope);
 }

@@ -314,6 +314,39 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, swiglu
     return out
 
 
+def qkv_rope_ok(M: int, K: int, hd: int, rotary_dim: int, dtype: torch.dtype) -> bool:
+    """Whether the product with a stacked [q; k; v] matrix can rotate and store in its epilogue:
+    few rows, a head size that splits into pairs of 16-wide tiles, the whole head rotated."""
+    return skinny_ok(M, K, dtype) and hd % 32 == 0 and rotary_dim == hd
+
+
+def skinny_qkv_rope(x: torch.Tensor, w_qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor,
+                    sin: torch.Tensor, slot_mapping: Optional[torch.Tensor], kpool: Optional[torch.Tensor],
+                    vpool: Optional[torch.Tensor], H: int, KVH: int, hd: int) -> torch.Tensor:
+    """``x . w_qkv^T`` for few rows with rotation and cache write fused in: returns the rotated
+    queries [M, H*hd]; rotated keys and plain values go straight into the pools at ``slot_mapping``."""
+    M, Kd = x.shape
+    _gpu(x, "x")
+    _gpu(w_qkv, "w_qkv", x.dtype, ((H + 2 * KVH) * hd, Kd))
+    _need(qkv_rope_ok(M, Kd, hd, 2 * cos.shape[1], x.dtype), f"skinny_qkv_rope does not take M={M}, K={Kd}, hd={hd}")
+    _gpu(positions, "positions", torch.int32, (M,))
+    _gpu(cos, "cos", torch.float32)
+    _gpu(sin, "sin", torch.float32, cos.shape)
+    page_size = 1
+    if slot_mapping is not None:
+        _gpu(slot_mapping, "slot_mapping", torch.int32, (M,))
+        _gpu(kpool, "kpool", x.dtype)
+        _gpu(vpool, "vpool", x.dtype, kpool.shape)
+        _need(kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd,
+              f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
+        page_size = kpool.shape[2]
+    q = torch.empty(M, H * hd, dtype=x.dtype, device=x.device)
+    _check(skinny_lib().ni_skinny_qkv_rope(_ptr(x), _ptr(w_qkv), _ptr(q), _ptr(positions), _ptr(cos), _ptr(sin),
+                                           _ptr(slot_mapping), _ptr(kpool), _ptr(vpool), M, Kd, H, KVH, hd,
+                                           page_size, dtype_code(x.dtype), _stream()), "skinny_qkv_rope")
+    return q
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """``x . weight^T`` with ``weight`` stored [out, in].  Few rows go to the hand-written skinny
     product; many rows to the library (rocBLAS/hipBLASLt), where float32 inputs are multiplied in

@@ -189,11 +189,16 @@ class Attention(Part):
 
     def forward(self, x: torch.Tensor, ctx, cache: LayerCache) -> torch.Tensor:
         T = x.shape[0]
-        qkv = K.linear(x, self.w_qkv)
         tables = self.position.tables()
         cos, sin = tables if tables is not None else (None, None)
-        K.rope_kv_write(qkv, ctx.positions, cos, sin, cache.slot_mapping if cache.writes else None,
-                        cache.kpool, cache.vpool, self.H, self.KVH, self.hd)
+        slots = cache.slot_mapping if cache.writes else None
+        if cos is not None and K.qkv_rope_ok(T, x.shape[1], self.hd, 2 * cos.shape[1], x.dtype):
+            # few rows: rotation and cache write ride on the product's epilogue
+            qkv = K.skinny_qkv_rope(x, self.w_qkv, ctx.positions, cos, sin, slots, cache.kpool, cache.vpool,
+                                    self.H, self.KVH, self.hd)
+        else:
+            qkv = K.linear(x, self.w_qkv)
+            K.rope_kv_write(qkv, ctx.positions, cos, sin, slots, cache.kpool, cache.vpool, self.H, self.KVH, self.hd)
         out = torch.empty(T, self.H * self.hd, dtype=x.dtype, device=x.device)
         max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window)
         nsplit = K.choose_splits(T, self.KVH, self.H // self.KVH, max_keys)

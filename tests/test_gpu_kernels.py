@@ -381,3 +381,43 @@ def test_skinny_product_reference_vector(K):
     g = torch.Generator().manual_seed(0)
     x, w = torch.randn(300, 1024, generator=g), torch.randn(512, 1024, generator=g) / 32
     assert rel(K.linear(dev(x), dev(w)), x.double() @ w.double().t()) < 3e-6
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("M,H,KVH,hd,Kd,ps", [(1, 4, 2, 32, 64, 8), (8, 32, 8, 64, 2048, 16), (5, 6, 1, 32, 192, 8),
+                                             (40, 3, 3, 128, 96, 4), (64, 8, 2, 96, 256, 16)])
+def test_product_with_rotation_and_cache_write(K, dtype, M, H, KVH, hd, Kd, ps):
+    """The fused epilogue against the plain steps: product, rotation of pairs (j, j + hd/2), write by slot."""
+    g = torch.Generator().manual_seed(M + hd)
+    x = torch.randn(M, Kd, generator=g).to(DT[dtype])
+    w = (torch.randn((H + 2 * KVH) * hd, Kd, generator=g) / math.sqrt(Kd)).to(DT[dtype])
+    positions = torch.randint(0, 500, (M,), generator=g).to(torch.int32)
+    pages = -(-M // ps) + 2
+    slots = torch.tensor(random.Random(1).sample(range(pages * ps), M), dtype=torch.int32)
+    inv = P.rope_frequencies(hd, 10000.0, None)
+    cos, sin = K.rope_table(dev(torch.from_numpy(inv)), 512)
+    kpool = torch.full((pages, KVH, ps, hd), 7.0, dtype=DT[dtype], device="cuda")
+    vpool = torch.full((pages, KVH, ps, hd), 7.0, dtype=DT[dtype], device="cuda")
+    assert K.qkv_rope_ok(M, Kd, hd, hd, DT[dtype])
+    q = K.skinny_qkv_rope(dev(x), dev(w), dev(positions), cos, sin, dev(slots), kpool, vpool, H, KVH, hd)
+    qkv = x.double() @ w.double().t()
+    s, c = P.rope_tables(positions.tolist(), inv)
+    q_ref = plain_rotate_half(qkv[:, :H * hd].reshape(M, H, hd), s, c, hd)
+    k_ref = plain_rotate_half(qkv[:, H * hd:(H + KVH) * hd].reshape(M, KVH, hd), s, c, hd)
+    v_ref = qkv[:, (H + KVH) * hd:].reshape(M, KVH, hd)
+    assert rel(q.reshape(M, H, hd), q_ref) < KTOL[dtype]
+    kp, vp = kpool.cpu().double(), vpool.cpu().double()
+    touched = torch.zeros(pages, ps, dtype=torch.bool)
+    scale_k, scale_v = float(k_ref.abs().max()), float(v_ref.abs().max())
+    for t in range(M):
+        page, off = int(slots[t]) // ps, int(slots[t]) % ps
+        touched[page, off] = True
+        assert float((kp[page, :, off] - k_ref[t]).abs().max()) < KTOL[dtype] * scale_k
+        assert float((vp[page, :, off] - v_ref[t]).abs().max()) < KTOL[dtype] * scale_v
+    untouched = ~touched[:, None, :].expand(pages, KVH, ps)
+    assert bool((kp[untouched] == 7.0).all()) and bool((vp[untouched] == 7.0).all())
+    # without a slot mapping nothing is stored, the queries are the same
+    k2 = torch.full_like(kpool, 3.0)
+    q2 = K.skinny_qkv_rope(dev(x), dev(w), dev(positions), cos, sin, None, None, None, H, KVH, hd)
+    assert torch.equal(q2, q) and bool((k2 == 3.0).all())
+    assert not K.qkv_rope_ok(M, Kd, 48, 48, DT[dtype]) and not K.qkv_rope_ok(M, Kd, hd, hd // 2, DT[dtype])
