@@ -101,31 +101,38 @@ __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
         for (int e = 0; e < EPL; ++e) acc[i][e] = 0.f;
     }
 
-    // U keys per lane group and trip: their table entries are fetched first, then all their rows,
-    // then the arithmetic.  The running maximum moves once per trip, so a trip costs one
-    // rescaling of the output and U + 1 exponentials per head.
+    // U keys per lane group and trip.  The loop is pipelined by hand: while trip t is being
+    // multiplied, the rows of trip t+1 are in flight and the table entries of trip t+2 are being
+    // fetched, so the two dependent memory round trips of a trip (table, then rows) overlap with
+    // arithmetic instead of adding up trip after trip.  The running maximum moves once per trip:
+    // one rescaling of the output and U + 1 exponentials per head and trip.
     constexpr int U = EPL <= 8 ? 4 : 2;
     const int page_shift = (page_size & (page_size - 1)) == 0 ? __ffs(page_size) - 1 : -1;
     const int iters = (k1 > k0) ? (k1 - k0 + KPI - 1) / KPI : 0;
-    for (int it = 0; it < iters; it += U) {
-        bool valid[U];
-        size_t base[U];
+
+    struct Where { size_t base[U]; bool valid[U]; };
+    auto locate = [&](int it, Where& w) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int j = k0 + (it + u) * KPI + kslot;
-            valid[u] = j < k1;
-            const int jj = valid[u] ? j : k0;       // a key of this sequence in any case: the address stays legal
+            w.valid[u] = j < k1;
+            const int jj = w.valid[u] ? j : k0;     // a key of this sequence in any case: the address stays legal
             const int lp = page_shift >= 0 ? (jj >> page_shift) : jj / page_size;
             const int off = page_shift >= 0 ? (jj & (page_size - 1)) : jj % page_size;
             const int page = table[lp];
-            base[u] = ((static_cast<size_t>(page) * KVH + g) * page_size + off) * HD + sub * EPL;
+            w.base[u] = ((static_cast<size_t>(page) * KVH + g) * page_size + off) * HD + sub * EPL;
         }
-        float kk[U][EPL], vv[U][EPL];
+    };
+    struct Rows { RawRow<T, EPL> k[U], v[U]; bool valid[U]; };     // as loaded: converted when multiplied
+    auto fetch = [&](const Where& w, Rows& r) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            VecIO<T, EPL>::load(kpool + base[u], kk[u]);
-            VecIO<T, EPL>::load(vpool + base[u], vv[u]);
+            r.k[u].load(kpool + w.base[u]);
+            r.v[u].load(vpool + w.base[u]);
+            r.valid[u] = w.valid[u];
         }
+    };
+    auto multiply = [&](const Rows& r) {
 #pragma unroll
         for (int i = 0; i < GT; ++i) {
             float sc[U];
@@ -134,11 +141,11 @@ __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
             for (int u = 0; u < U; ++u) {
                 float d = 0.f;
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) d += qreg[i][e] * kk[u][e];
+                for (int e = 0; e < EPL; ++e) d += qreg[i][e] * r.k[u].get(e);
 #pragma unroll
                 for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, WAVE);
                 sc[u] = d;
-                if (valid[u]) m_new = fmaxf(m_new, d);
+                if (r.valid[u]) m_new = fmaxf(m_new, d);
             }
             const float corr = ex<FAST>(m[i] - m_new);
             float psum = 0.f;
@@ -146,14 +153,32 @@ __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
             for (int e = 0; e < EPL; ++e) acc[i][e] *= corr;
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const float p = valid[u] ? ex<FAST>(sc[u] - m_new) : 0.f;
+                const float p = r.valid[u] ? ex<FAST>(sc[u] - m_new) : 0.f;
                 psum += p;
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) acc[i][e] += p * vv[u][e];
+                for (int e = 0; e < EPL; ++e) acc[i][e] += p * r.v[u].get(e);
             }
             l[i] = l[i] * corr + psum;
             m[i] = m_new;
         }
+    };
+
+    // two trips per turn of the loop, A and B, each with a place of its own in registers
+    Where wa, wb;
+    Rows ra, rb;
+    if (iters > 0) {
+        locate(0, wa);
+        if (iters > U) locate(U, wb);
+        fetch(wa, ra);
+    }
+    for (int it = 0; it < iters; it += 2 * U) {
+        const bool has_b = it + U < iters, has_a2 = it + 2 * U < iters, has_b2 = it + 3 * U < iters;
+        if (has_b) fetch(wb, rb);
+        if (has_a2) locate(it + 2 * U, wa);
+        multiply(ra);
+        if (has_a2) fetch(wa, ra);
+        if (has_b2) locate(it + 3 * U, wb);
+        if (has_b) multiply(rb);
     }
 
     // merge the lane groups of a wave (lanes with equal `sub`)

@@ -1,0 +1,264 @@
+// Attention of prompt portions over the paged key/value cache on the matrix cores of gfx950.
+// bfloat16 only; compiled once per head size (-DHEAD_DIM=n, a multiple of 32 up to 256).
+//
+// A workgroup of four wavefronts owns one tile of consecutive tokens of one sequence and the
+// query heads of one kv head (HPT of them at a time).  A wavefront owns 16 "rows": TPT = 16/HPT
+// tokens times HPT heads, all reading the same keys and values.  Keys are walked 32 at a time:
+//
+//   S^T[key, row]  = K[key, :] . Q[row, :]       v_mfma_f32_16x16x32_bf16, K rows straight from
+//                                                 global memory as the A operand, Q as B
+//   softmax        float32, online: every lane holds 8 scores of ONE row (its column of S^T),
+//                  so the maximum needs two shuffles and the rescaling of the output none
+//   O^T[dim, row] += V^T[dim, key] . P^T[key, row]   the scores of a lane are already laid out
+//                  as the B operand; V^T comes from a tile of V that the workgroup stages in LDS
+//
+// Computing the transposes is what makes P need no data movement between the two products: the
+// k index of an MFMA is only a label, and a lane's eight scores (keys kg*4+i of both 16-key
+// halves) are given the labels kg*8+j on both operands.
+//
+// Formula as in the token-at-a-time kernel (reference: src/op/kernels/cuda/prefill_attention_kernel.cu:66-141,
+// 422-455): the query at position P reads keys max(0, P+1-window)..P, scores are scaled by `scale`,
+// softmax subtracts the maximum, divides by the plain sum; probabilities are rounded to bfloat16
+// for the second product, sums stay float32.
+#include "common.h"
+
+#ifndef HEAD_DIM
+#error "HEAD_DIM must be defined"
+#endif
+static_assert(HEAD_DIM % 32 == 0 && HEAD_DIM >= 32 && HEAD_DIM <= 256, "head size: multiple of 32, at most 256");
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+#define MA_WAVES 4
+#define MA_THREADS (MA_WAVES * WAVE)
+#define KSTEP 32
+#define NEG_BIG (-1.0e30f)
+#define VPAD 8   // elements of padding per staged row of V: the four key groups of a read fall on different banks
+
+struct QTile { int32_t seq, row0, ntok, pos0; };   // tokens row0..row0+ntok-1 of the batch, positions pos0..
+
+template <int HPT>
+__global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
+    const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
+    const int32_t* __restrict__ block_table, int table_stride, const QTile* __restrict__ tiles,
+    bf16_t* __restrict__ out, int H, int KVH, int page_size, int window, float scale) {
+    constexpr int HD = HEAD_DIM;
+    constexpr int TPT = 16 / HPT;            // tokens of a wavefront
+    constexpr int KK = HD / 32;              // k steps of the first product
+    constexpr int DT = HD / 16;              // 16-wide tiles of the head dimension in the output
+    constexpr int VROW = HD + VPAD;
+    __shared__ __attribute__((aligned(16))) uint16_t vs[2][KSTEP][VROW];
+
+    const QTile tile = tiles[blockIdx.x];
+    const int G = H / KVH;
+    const int chunks = (G + HPT - 1) / HPT;
+    const int g = blockIdx.y / chunks;
+    const int chunk = blockIdx.y % chunks;
+
+    const int tid = threadIdx.x;
+    const int wave = tid / WAVE, lane = tid % WAVE;
+    const int r = lane % 16, kg = lane / 16;
+
+    // this lane's row: one (token, head) pair
+    const int tt = wave * TPT + r / HPT;                 // token within the tile
+    const int hh = chunk * HPT + r % HPT;                // head within the group
+    const bool row_ok = tt < tile.ntok && hh < G;
+    const int head = g * G + hh;
+    const int pos = tile.pos0 + tt;
+    const int row_lo = (row_ok && window > 0) ? max(0, pos + 1 - window) : 0;
+
+    // key range of the workgroup (uniform), walked in steps of 32 from a multiple of 32
+    const int kend = tile.pos0 + tile.ntok;
+    const int kbeg = (window > 0 ? max(0, tile.pos0 + 1 - window) : 0) / KSTEP * KSTEP;
+    const int nsteps = (kend - kbeg + KSTEP - 1) / KSTEP;
+    // last position any row of this wavefront has: steps beyond it are skipped by the wavefront
+    const int wave_tok_hi = min(tile.ntok, (wave + 1) * TPT) - 1;
+    const bool wave_ok = wave * TPT < tile.ntok;
+    const int wave_pmax = tile.pos0 + wave_tok_hi;
+
+    const int32_t* table = block_table + static_cast<size_t>(tile.seq) * table_stride;
+    const int page_shift = (page_size & (page_size - 1)) == 0 ? __ffs(page_size) - 1 : -1;
+    auto row_address = [&](int key) -> size_t {       // offset of key's row for kv head g, key clamped into the sequence
+        const int kc = min(key, kend - 1);
+        const int lp = page_shift >= 0 ? (kc >> page_shift) : kc / page_size;
+        const int off = page_shift >= 0 ? (kc & (page_size - 1)) : kc % page_size;
+        return ((static_cast<size_t>(table[lp]) * KVH + g) * page_size + off) * HD;
+    };
+
+    // Q as the B operand: lane (row r, group kg) holds dims kk*32 + kg*8 .. +8
+    uint4 qf[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        if (row_ok)
+            qf[kk] = *reinterpret_cast<const uint4*>(q + static_cast<size_t>(tile.row0 + tt) * q_stride +
+                                                     static_cast<size_t>(head) * HD + kk * 32 + kg * 8);
+        else
+            qf[kk] = make_uint4(0, 0, 0, 0);
+    }
+
+    float m_run = NEG_BIG, l_run = 0.f;
+    floatx4_t o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    // staging of V: thread -> (key of the step, 8-dim chunk); HD/8 chunks a key
+    constexpr int CHUNKS = HD / 8;
+    constexpr int V_ITEMS = KSTEP * CHUNKS;
+    constexpr int V_PER_THREAD = (V_ITEMS + MA_THREADS - 1) / MA_THREADS;
+    uint4 vreg[V_PER_THREAD];
+    auto load_v = [&](int ks) {
+#pragma unroll
+        for (int i = 0; i < V_PER_THREAD; ++i) {
+            const int item = tid + i * MA_THREADS;
+            if (item < V_ITEMS) {
+                const int key = ks + item / CHUNKS;
+                vreg[i] = *reinterpret_cast<const uint4*>(vpool + row_address(key) + (item % CHUNKS) * 8);
+            }
+        }
+    };
+    auto store_v = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < V_PER_THREAD; ++i) {
+            const int item = tid + i * MA_THREADS;
+            if (item < V_ITEMS) *reinterpret_cast<uint4*>(&vs[buf][item / CHUNKS][(item % CHUNKS) * 8]) = vreg[i];
+        }
+    };
+    // K as the A operand: lane (key r of a 16-key half, group kg) holds dims kk*32 + kg*8 .. +8
+    uint4 kf[2][KK], kf_next[2][KK];
+    auto load_k = [&](int ks, uint4 (&dst)[2][KK]) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const size_t base = row_address(ks + t * 16 + r);
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) dst[t][kk] = *reinterpret_cast<const uint4*>(kpool + base + kk * 32 + kg * 8);
+        }
+    };
+
+    if (nsteps > 0) {
+        load_v(kbeg);
+        load_k(kbeg, kf);
+        store_v(0);
+    }
+    for (int s = 0; s < nsteps; ++s) {
+        const int ks = kbeg + s * KSTEP;
+        __syncthreads();                       // V of this step is in vs[s & 1]; nobody still reads the other buffer
+        const bool more = s + 1 < nsteps;
+        if (more) {
+            load_v(ks + KSTEP);
+            load_k(ks + KSTEP, kf_next);
+        }
+        if (wave_ok && ks <= wave_pmax) {
+            // S^T for the two 16-key halves
+            floatx4_t st[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                st[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk)
+                    st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[t][kk]),
+                                                                    __builtin_bit_cast(bf16x8_t, qf[kk]), st[t], 0, 0, 0);
+            }
+            // this lane: row r, keys ks + t*16 + kg*4 + i
+            float sc[8];
+            float mx = NEG_BIG;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = ks + t * 16 + kg * 4 + i;
+                    const bool ok = row_ok && key <= pos && key >= row_lo;
+                    const float v = ok ? st[t][i] * scale : NEG_BIG;
+                    sc[t * 4 + i] = v;
+                    mx = fmaxf(mx, v);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+            const float m_new = fmaxf(m_run, mx);
+            const float corr = __expf(m_run - m_new);
+            float psum = 0.f;
+            uint32_t pw[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float p0 = sc[2 * j] > 0.5f * NEG_BIG ? __expf(sc[2 * j] - m_new) : 0.f;
+                const float p1 = sc[2 * j + 1] > 0.5f * NEG_BIG ? __expf(sc[2 * j + 1] - m_new) : 0.f;
+                psum += p0 + p1;
+                pw[j] = static_cast<uint32_t>(f32_to_bf16_bits(p0)) | (static_cast<uint32_t>(f32_to_bf16_bits(p1)) << 16);
+            }
+            l_run = l_run * corr + psum;
+            m_run = m_new;
+            const uint4 pf = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+            // O^T += V^T . P^T : the A operand of lane (dim r of a 16-dim tile, group kg) is V[key_j][dim]
+            // for the same eight keys, in the same order, as the lane's scores
+            const uint16_t (*vb)[VROW] = vs[s & 1];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                uint32_t vw[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int j0 = 2 * j, j1 = 2 * j + 1;
+                    const int key0 = (j0 < 4 ? 0 : 16) + kg * 4 + (j0 & 3);
+                    const int key1 = (j1 < 4 ? 0 : 16) + kg * 4 + (j1 & 3);
+                    vw[j] = static_cast<uint32_t>(vb[key0][dt * 16 + r]) | (static_cast<uint32_t>(vb[key1][dt * 16 + r]) << 16);
+                }
+                const uint4 vf = make_uint4(vw[0], vw[1], vw[2], vw[3]);
+                o[dt] *= corr;
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vf),
+                                                                __builtin_bit_cast(bf16x8_t, pf), o[dt], 0, 0, 0);
+            }
+        }
+        if (more) {
+            store_v((s + 1) & 1);
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) kf[t][kk] = kf_next[t][kk];
+        }
+    }
+
+    // the sum of a row is spread over the four lanes that share it
+    l_run += __shfl_xor(l_run, 16, WAVE);
+    l_run += __shfl_xor(l_run, 32, WAVE);
+    if (row_ok && l_run > 0.f) {
+        const float inv = 1.0f / l_run;
+        bf16_t* dst = out + static_cast<size_t>(tile.row0 + tt) * H * HD + static_cast<size_t>(head) * HD;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            float v4[4] = {o[dt][0] * inv, o[dt][1] * inv, o[dt][2] * inv, o[dt][3] * inv};
+            VecIO<bf16_t, 4>::store(dst + dt * 16 + kg * 4, v4);
+        }
+    }
+}
+
+NI_EXPORT int ni_mfma_attention_head_dim() { return HEAD_DIM; }
+
+// Tokens of one tile for a model with `group` query heads per kv head.
+NI_EXPORT int ni_mfma_attention_tile_tokens(int group) {
+    const int hpt = group >= 16 ? 16 : group > 4 ? 8 : group > 2 ? 4 : group > 1 ? 2 : 1;
+    return MA_WAVES * (16 / hpt);
+}
+
+// tiles: QTile [n_tiles] built by the host from the portions of the step with the tile size above.
+NI_EXPORT int ni_mfma_attention(const void* q, int q_stride, const void* kpool, const void* vpool, const void* block_table,
+                                int table_stride, const void* tiles, int n_tiles, void* out, int H, int KVH,
+                                int page_size, int window, float scale, hipStream_t stream) {
+    if (n_tiles <= 0) return 0;
+    if (H % KVH != 0 || page_size < 1) return -1;
+    const int G = H / KVH;
+    const int hpt = G >= 16 ? 16 : G > 4 ? 8 : G > 2 ? 4 : G > 1 ? 2 : 1;
+    const int chunks = (G + hpt - 1) / hpt;
+    dim3 grid(n_tiles, KVH * chunks);
+#define MA_LAUNCH(HPT_)                                                                                              \
+    mfma_attention_kernel<HPT_><<<grid, MA_THREADS, 0, stream>>>(                                                  \
+        (const bf16_t*)q, q_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table,        \
+        table_stride, (const QTile*)tiles, (bf16_t*)out, H, KVH, page_size, window, scale)
+    switch (hpt) {
+        case 1: MA_LAUNCH(1); break;
+        case 2: MA_LAUNCH(2); break;
+        case 4: MA_LAUNCH(4); break;
+        case 8: MA_LAUNCH(8); break;
+        default: MA_LAUNCH(16); break;
+    }
+#undef MA_LAUNCH
+    return NI_LAUNCH_RESULT();
+}

@@ -123,6 +123,44 @@ template <int N> struct VecIO<bf16_t, N> {
     }
 };
 
+// N consecutive elements kept as loaded (no conversion yet), so that rows waiting in registers
+// for their turn cost as few registers as they cost bytes.
+template <typename T, int N> struct RawRow {
+    static constexpr int BYTES = N * sizeof(T);
+    static constexpr int WORDS = (BYTES + 3) / 4;
+    uint32_t w[WORDS];
+    __device__ __forceinline__ void load(const T* p) {
+        if constexpr (BYTES % 16 == 0) {
+#pragma unroll
+            for (int i = 0; i < BYTES / 16; ++i) {
+                const uint4 v = reinterpret_cast<const uint4*>(p)[i];
+                w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
+            }
+        } else if constexpr (BYTES % 8 == 0) {
+#pragma unroll
+            for (int i = 0; i < BYTES / 8; ++i) {
+                const uint2 v = reinterpret_cast<const uint2*>(p)[i];
+                w[2 * i] = v.x; w[2 * i + 1] = v.y;
+            }
+        } else if constexpr (BYTES % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < BYTES / 4; ++i) w[i] = reinterpret_cast<const uint32_t*>(p)[i];
+        } else {      // an odd number of 16-bit elements
+            const uint16_t* q = reinterpret_cast<const uint16_t*>(p);
+#pragma unroll
+            for (int i = 0; i < WORDS; ++i) {
+                const uint32_t lo = q[2 * i];
+                const uint32_t hi = (2 * i + 1 < N) ? q[2 * i + 1] : 0u;
+                w[i] = lo | (hi << 16);
+            }
+        }
+    }
+    __device__ __forceinline__ float get(int i) const {
+        if constexpr (sizeof(T) == 4) return __uint_as_float(w[i]);
+        else return __uint_as_float((i & 1) ? (w[i / 2] & 0xffff0000u) : (w[i / 2] << 16));
+    }
+};
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);

@@ -190,7 +190,7 @@ def choose_splits(n_tokens: int, kv_heads: int, group: int, max_keys: int) -> in
     fills the 256 compute units.  One piece never holds fewer than 256 keys."""
     chunks = (group + 3) // 4
     items = max(1, n_tokens * kv_heads * chunks)
-    want = max(1, 1024 // items)
+    want = max(1, 512 // items)
     return int(max(1, min(want, (max_keys + 255) // 256, 64)))
 
 
