@@ -19,7 +19,7 @@
 // Formula as in the token-at-a-time kernel (reference: src/op/kernels/cuda/prefill_attention_kernel.cu:66-141,
 // 422-455): the query at position P reads keys max(0, P+1-window)..P, scores are scaled by `scale`,
 // softmax subtracts the maximum, divides by the plain sum; probabilities are rounded to bfloat16
-// for the second product, sums stay float32.
+// for the second product and summed as rounded, in float32.
 #include "common.h"
 
 #ifndef HEAD_DIM
@@ -182,8 +182,11 @@ __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
             for (int j = 0; j < 4; ++j) {
                 const float p0 = sc[2 * j] > 0.5f * NEG_BIG ? __expf(sc[2 * j] - m_new) : 0.f;
                 const float p1 = sc[2 * j + 1] > 0.5f * NEG_BIG ? __expf(sc[2 * j + 1] - m_new) : 0.f;
-                psum += p0 + p1;
-                pw[j] = static_cast<uint32_t>(f32_to_bf16_bits(p0)) | (static_cast<uint32_t>(f32_to_bf16_bits(p1)) << 16);
+                // the sum is taken over the rounded weights, the ones the second product uses: the
+                // output is then an exact convex combination of values, whatever the rounding
+                const uint32_t b0 = f32_to_bf16_bits(p0), b1 = f32_to_bf16_bits(p1);
+                psum += __uint_as_float(b0 << 16) + __uint_as_float(b1 << 16);
+                pw[j] = b0 | (b1 << 16);
             }
             l_run = l_run * corr + psum;
             m_run = m_new;

@@ -74,6 +74,20 @@ class StepContext:
         self.recording = recording
         self._scratch_owner = scratch_owner
         self._scratch: Optional[torch.Tensor] = None
+        self._q_tiles: Dict[int, torch.Tensor] = {}
+
+    def q_tiles(self, tile_tokens: int) -> torch.Tensor:
+        """The portions of the step cut into tiles of at most ``tile_tokens`` tokens, int32 [n, 4]
+        rows of (sequence, first row, tokens, first position) on the device; built once per step
+        and tile size from the host lists (so not in a recorded step)."""
+        if self.recording:
+            raise StepError("tiles come from the host lists of a step and cannot be part of a recorded step")
+        t = self._q_tiles.get(tile_tokens)
+        if t is None:
+            flat = K.build_q_tiles(self.q_start, self.q_len, self.context_len, tile_tokens)
+            t = torch.tensor(flat, dtype=torch.int32).view(-1, 4).to(self.device)
+            self._q_tiles[tile_tokens] = t
+        return t
 
     def workspace(self, n_floats: int) -> torch.Tensor:
         """Float32 scratch that lives until the next request for scratch (one user at a time)."""

@@ -53,6 +53,10 @@ def attention_lib(head_dim: int) -> ctypes.CDLL:
     return _load(_build.attention_target(head_dim))
 
 
+def attention_mfma_lib(head_dim: int) -> ctypes.CDLL:
+    return _load(_build.attention_mfma_target(head_dim))
+
+
 def dtype_code(dtype: torch.dtype) -> int:
     try:
         return _DTYPE_CODE[dtype]
@@ -232,6 +236,52 @@ def token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
                                   _ptr(part_o), _ptr(part_ml), T, H, KVH, kpool.shape[2],
                                   int(window) if window else 0, ctypes.c_float(scale), nsplit,
                                   dtype_code(qkv.dtype), _stream()), "token_attention")
+    return out
+
+
+def mfma_attention_ok(dtype: torch.dtype, hd: int) -> bool:
+    """Whether the matrix-core attention kernel takes this type and head size."""
+    return dtype == torch.bfloat16 and hd % 32 == 0 and 32 <= hd <= 256
+
+
+def mfma_tile_tokens(hd: int, group: int) -> int:
+    """Tokens of one tile of the matrix-core attention kernel for ``group`` query heads per kv head."""
+    return int(attention_mfma_lib(hd).ni_mfma_attention_tile_tokens(int(group)))
+
+
+def build_q_tiles(q_start, q_len, context_len, tile_tokens: int):
+    """Cut the portions of a step (host lists: first row, length, context after the step) into
+    tiles of at most ``tile_tokens`` tokens: flat list of (sequence, first row, tokens, first position)."""
+    flat = []
+    for s, (row, n, total) in enumerate(zip(q_start, q_len, context_len)):
+        first = total - n
+        for t0 in range(0, n, tile_tokens):
+            flat.extend((s, row + t0, min(tile_tokens, n - t0), first + t0))
+    return flat
+
+
+def mfma_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
+                   tiles: torch.Tensor, out: torch.Tensor, H: int, KVH: int, hd: int, scale: float,
+                   window: Optional[int]) -> torch.Tensor:
+    """Attention of prompt portions on the matrix cores (bfloat16).  ``tiles`` is int32 [n, 4] from
+    :func:`build_q_tiles`; the pools already hold the keys and values of every position of the step."""
+    T = qkv.shape[0]
+    _gpu(qkv, "qkv", torch.bfloat16)
+    _need(mfma_attention_ok(qkv.dtype, hd), f"mfma_attention does not take {qkv.dtype} with head size {hd}")
+    _need(qkv.shape[1] >= H * hd and qkv.shape[1] % 8 == 0, "qkv is narrower than the query heads or its rows are unaligned")
+    _need(H % KVH == 0, f"{H} query heads do not divide into {KVH} kv heads")
+    _gpu(kpool, "kpool", torch.bfloat16)
+    _gpu(vpool, "vpool", torch.bfloat16, kpool.shape)
+    _need(kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd,
+          f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
+    _gpu(block_table, "block_table", torch.int32)
+    _gpu(tiles, "tiles", torch.int32)
+    _need(tiles.dim() == 2 and tiles.shape[1] == 4, "tiles must be [n, 4]")
+    _gpu(out, "out", torch.bfloat16, (T, H * hd))
+    _check(attention_mfma_lib(hd).ni_mfma_attention(_ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table),
+                                                    block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(out), H, KVH,
+                                                    kpool.shape[2], int(window) if window else 0, ctypes.c_float(scale),
+                                                    _stream()), "mfma_attention")
     return out
 
 

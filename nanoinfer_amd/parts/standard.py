@@ -153,6 +153,7 @@ class Attention(Part):
     """
 
     graph_safe = True
+    MFMA_MIN_PORTION = 8     # a step whose longest portion has this many tokens goes to the matrix-core kernel
 
     @classmethod
     def weight_requests(cls, spec):
@@ -200,6 +201,12 @@ class Attention(Part):
             qkv = K.linear(x, self.w_qkv)
             K.rope_kv_write(qkv, ctx.positions, cos, sin, slots, cache.kpool, cache.vpool, self.H, self.KVH, self.hd)
         out = torch.empty(T, self.H * self.hd, dtype=x.dtype, device=x.device)
+        if (not ctx.recording and ctx.max_q_len >= self.MFMA_MIN_PORTION and K.mfma_attention_ok(x.dtype, self.hd)):
+            # prompt portions: tiles of tokens on the matrix cores
+            tiles = ctx.q_tiles(K.mfma_tile_tokens(self.hd, self.H // self.KVH))
+            K.mfma_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, out, self.H, self.KVH, self.hd,
+                             self.scale, self.window)
+            return K.linear(out, self.w_o)
         max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window)
         nsplit = K.choose_splits(T, self.KVH, self.H // self.KVH, max_keys)
         ws = ctx.workspace(T * self.H * nsplit * (self.hd + 2)) if nsplit > 1 else None

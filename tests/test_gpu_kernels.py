@@ -154,7 +154,7 @@ def test_swiglu(K, dtype):
 
 # ------------------------------------------------------------------ attention over pages
 
-def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boost=None):
+def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boost=None, kernel="token"):
     """Sequences of ``lens`` keys each; the last ``q_lens`` of each are this step's queries.  The
     cache is filled through a shuffled block table; everything else in the pools is NaN so that a
     read outside a sequence's own keys poisons the result."""
@@ -178,8 +178,9 @@ def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boo
         if boost is not None:
             bb, key_at, query_at, factor = boost
             if bb == b:
-                k[key_at] *= factor
-                q[query_at] = k[key_at].repeat_interleave(H // KVH, 0) / factor * 4
+                # the inputs stay exactly representable in the compute type
+                k[key_at] = (k[key_at] * factor).to(DT[dtype]).float()
+                q[query_at] = (k[key_at].repeat_interleave(H // KVH, 0) / factor * 4).to(DT[dtype]).float()
         for p in range(pages_per[b]):
             table[b, p] = ids[at]
             lo, hi = p * ps, min(n, (p + 1) * ps)
@@ -198,9 +199,16 @@ def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boo
             row += 1
     out = torch.empty(T, H * hd, device="cuda", dtype=DT[dtype])
     ws = torch.empty(max(1, T * H * nsplit * (hd + 2)), device="cuda") if nsplit > 1 else None
-    K.token_attention(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table),
-                      dev(torch.tensor(seq_of, dtype=torch.int32)), dev(torch.tensor(positions, dtype=torch.int32)),
-                      out, H, KVH, hd, 1.0 / math.sqrt(hd), window, nsplit, ws)
+    if kernel == "mfma":
+        starts = [sum(q_lens[:b]) for b in range(B)]
+        flat = K.build_q_tiles(starts, q_lens, lens, K.mfma_tile_tokens(hd, H // KVH))
+        tiles = dev(torch.tensor(flat, dtype=torch.int32).view(-1, 4))
+        K.mfma_attention(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table), tiles, out,
+                         H, KVH, hd, 1.0 / math.sqrt(hd), window)
+    else:
+            K.token_attention(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table),
+                          dev(torch.tensor(seq_of, dtype=torch.int32)), dev(torch.tensor(positions, dtype=torch.int32)),
+                          out, H, KVH, hd, 1.0 / math.sqrt(hd), window, nsplit, ws)
     want = torch.cat([P.causal_attention(qs[b], ks[b], vs[b], range(n), window=window)[n - q_lens[b]:].reshape(q_lens[b], H * hd)
                       for b, n in enumerate(lens)])
     return out, want, (qs, ks, vs)
@@ -240,6 +248,35 @@ def test_attention_finds_a_far_key_among_hundreds(K, dtype):
             got = out.double().cpu().reshape(8, 64)
             expect = vs[0][key_at].double().repeat_interleave(4, 0)
             assert float((got - expect).abs().max()) < 0.05, key_at     # the one key took all the weight
+
+
+# ---- the matrix-core kernel for prompt portions (bfloat16)
+
+@pytest.mark.parametrize("H,KVH,hd,ps", [(4, 2, 32, 8), (6, 1, 32, 8), (32, 8, 64, 16), (16, 2, 128, 16), (2, 2, 256, 16),
+                                         (3, 3, 96, 4), (32, 1, 64, 16), (5, 5, 64, 5), (12, 4, 64, 16)])
+def test_mfma_attention_head_sizes_and_groups(K, H, KVH, hd, ps):
+    # whole prompts, portions that start in the middle of a sequence, single tokens beside them, tile edges
+    lens, q_lens = [1, 37, 130, 64, 200, 17], [1, 37, 2, 1, 77, 16]
+    out, want, _ = paged_case(K, "bfloat16", H, KVH, hd, ps, lens, q_lens, None, hd + H, 1, kernel="mfma")
+    assert not torch.isnan(out).any(), "a key outside the sequence's own pages took part"
+    assert rel(out, want) < KTOL["bfloat16"], (H, KVH, hd, ps)
+
+
+def test_mfma_attention_window_and_far_key(K):
+    for window in (1, 7, 16, 33, 100):
+        out, want, _ = paged_case(K, "bfloat16", 4, 2, 32, 8, [150, 9, 33], [150, 9, 2], window, window, 1, kernel="mfma")
+        assert not torch.isnan(out).any()
+        assert rel(out, want) < KTOL["bfloat16"], window
+    for key_at in (37, 16, 15, 0, 31, 32, 698):
+        out, want, (qs, ks, vs) = paged_case(K, "bfloat16", 8, 2, 64, 16, [700], [5], None, 9, 1,
+                                             boost=(0, key_at, 699, 6.0), kernel="mfma")
+        assert rel(out, want) < KTOL["bfloat16"]
+        got = out.double().cpu()[-1].reshape(8, 64)
+        expect = vs[0][key_at].double().repeat_interleave(4, 0)
+        assert float((got - expect).abs().max()) < 0.05, key_at
+    with pytest.raises(Exception):
+        K.attention_mfma_lib(48)
+    assert not K.mfma_attention_ok(torch.float32, 64) and not K.mfma_attention_ok(torch.bfloat16, 48)
 
 
 def test_attention_uniform_keys_reference_vector(K):
