@@ -298,3 +298,16 @@ NI_EXPORT int ni_token_attention(const void* q, int q_stride, const void* kpool,
     return launch<bf16_t>(q, q_stride, kpool, vpool, block_table, table_stride, seq_of_token, positions, out, part_o,
                           part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, stream);
 }
+
+// Merge of partial results in the layout above, for kernels of other libraries that split the keys.
+NI_EXPORT int ni_merge_splits(const void* part_o, const void* part_ml, void* out, int T_tokens, int H, int nsplit,
+                              int dtype, hipStream_t stream) {
+    if (T_tokens <= 0) return 0;
+    if (dtype == 0)
+        merge_splits_kernel<float><<<dim3(T_tokens, H), 64, 0, stream>>>((const float*)part_o, (const float*)part_ml,
+                                                                        (float*)out, H, nsplit);
+    else
+        merge_splits_kernel<bf16_t><<<dim3(T_tokens, H), 64, 0, stream>>>((const float*)part_o, (const float*)part_ml,
+                                                                         (bf16_t*)out, H, nsplit);
+    return NI_LAUNCH_RESULT();
+}

@@ -42,7 +42,8 @@ template <int HPT>
 __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int32_t* __restrict__ block_table, int table_stride, const QTile* __restrict__ tiles,
-    bf16_t* __restrict__ out, int H, int KVH, int page_size, int window, float scale) {
+    bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int H, int KVH, int page_size,
+    int window, float scale, int nsplit) {
     constexpr int HD = HEAD_DIM;
     constexpr int TPT = 16 / HPT;            // tokens of a wavefront
     constexpr int KK = HD / 32;              // k steps of the first product
@@ -71,7 +72,12 @@ __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
     // key range of the workgroup (uniform), walked in steps of 32 from a multiple of 32
     const int kend = tile.pos0 + tile.ntok;
     const int kbeg = (window > 0 ? max(0, tile.pos0 + 1 - window) : 0) / KSTEP * KSTEP;
-    const int nsteps = (kend - kbeg + KSTEP - 1) / KSTEP;
+    const int nsteps_all = (kend - kbeg + KSTEP - 1) / KSTEP;
+    // a split (blockIdx.z) takes a contiguous run of steps
+    const int per_split = (nsteps_all + nsplit - 1) / nsplit;
+    const int s_begin = blockIdx.z * per_split;
+    const int nsteps = max(0, min(nsteps_all, s_begin + per_split) - s_begin);
+    const int kfirst = kbeg + s_begin * KSTEP;
     // last position any row of this wavefront has: steps beyond it are skipped by the wavefront
     const int wave_tok_hi = min(tile.ntok, (wave + 1) * TPT) - 1;
     const bool wave_ok = wave * TPT < tile.ntok;
@@ -106,26 +112,24 @@ __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
     constexpr int CHUNKS = HD / 8;
     constexpr int V_ITEMS = KSTEP * CHUNKS;
     constexpr int V_PER_THREAD = (V_ITEMS + MA_THREADS - 1) / MA_THREADS;
-    uint4 vreg[V_PER_THREAD];
-    auto load_v = [&](int ks) {
+    auto load_v = [&](int ks, uint4 (&dst)[V_PER_THREAD]) {
 #pragma unroll
         for (int i = 0; i < V_PER_THREAD; ++i) {
             const int item = tid + i * MA_THREADS;
             if (item < V_ITEMS) {
                 const int key = ks + item / CHUNKS;
-                vreg[i] = *reinterpret_cast<const uint4*>(vpool + row_address(key) + (item % CHUNKS) * 8);
+                dst[i] = *reinterpret_cast<const uint4*>(vpool + row_address(key) + (item % CHUNKS) * 8);
             }
         }
     };
-    auto store_v = [&](int buf) {
+    auto store_v = [&](int buf, const uint4 (&src)[V_PER_THREAD]) {
 #pragma unroll
         for (int i = 0; i < V_PER_THREAD; ++i) {
             const int item = tid + i * MA_THREADS;
-            if (item < V_ITEMS) *reinterpret_cast<uint4*>(&vs[buf][item / CHUNKS][(item % CHUNKS) * 8]) = vreg[i];
+            if (item < V_ITEMS) *reinterpret_cast<uint4*>(&vs[buf][item / CHUNKS][(item % CHUNKS) * 8]) = src[i];
         }
     };
     // K as the A operand: lane (key r of a 16-key half, group kg) holds dims kk*32 + kg*8 .. +8
-    uint4 kf[2][KK], kf_next[2][KK];
     auto load_k = [&](int ks, uint4 (&dst)[2][KK]) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -135,18 +139,24 @@ __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
         }
     };
 
+    // Loads run two steps ahead of the arithmetic: while step s is multiplied, the rows of step
+    // s+1 are being written to LDS (they were asked for a step ago) and those of s+2 are asked for.
+    uint4 kf[2][KK], kf1[2][KK], kf2[2][KK];
+    uint4 v1[V_PER_THREAD], v2[V_PER_THREAD];
     if (nsteps > 0) {
-        load_v(kbeg);
-        load_k(kbeg, kf);
-        store_v(0);
+        load_k(kfirst, kf);
+        load_v(kfirst, v1);
+        if (nsteps > 1) load_k(kfirst + KSTEP, kf1);
+        store_v(0, v1);
+        if (nsteps > 1) load_v(kfirst + KSTEP, v1);
     }
     for (int s = 0; s < nsteps; ++s) {
-        const int ks = kbeg + s * KSTEP;
+        const int ks = kfirst + s * KSTEP;
         __syncthreads();                       // V of this step is in vs[s & 1]; nobody still reads the other buffer
-        const bool more = s + 1 < nsteps;
-        if (more) {
-            load_v(ks + KSTEP);
-            load_k(ks + KSTEP, kf_next);
+        const bool more = s + 1 < nsteps, more2 = s + 2 < nsteps;
+        if (more2) {
+            load_k(ks + 2 * KSTEP, kf2);
+            load_v(ks + 2 * KSTEP, v2);
         }
         if (wave_ok && ks <= wave_pmax) {
             // S^T for the two 16-key halves
@@ -211,17 +221,30 @@ __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
             }
         }
         if (more) {
-            store_v((s + 1) & 1);
+            store_v((s + 1) & 1, v1);
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) kf[t][kk] = kf_next[t][kk];
+                for (int kk = 0; kk < KK; ++kk) { kf[t][kk] = kf1[t][kk]; kf1[t][kk] = kf2[t][kk]; }
+#pragma unroll
+            for (int i = 0; i < V_PER_THREAD; ++i) v1[i] = v2[i];
         }
     }
 
     // the sum of a row is spread over the four lanes that share it
     l_run += __shfl_xor(l_run, 16, WAVE);
     l_run += __shfl_xor(l_run, 32, WAVE);
+    if (nsplit > 1) {
+        // partial (maximum, sum, unnormalised output) of this split, merged by a second kernel
+        if (row_ok) {
+            const size_t p = (static_cast<size_t>(tile.row0 + tt) * H + head) * nsplit + blockIdx.z;
+            if (kg == 0) { part_ml[p * 2] = m_run; part_ml[p * 2 + 1] = l_run; }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                *reinterpret_cast<float4*>(part_o + p * HD + dt * 16 + kg * 4) = make_float4(o[dt][0], o[dt][1], o[dt][2], o[dt][3]);
+        }
+        return;
+    }
     if (row_ok && l_run > 0.f) {
         const float inv = 1.0f / l_run;
         bf16_t* dst = out + static_cast<size_t>(tile.row0 + tt) * H * HD + static_cast<size_t>(head) * HD;
@@ -242,19 +265,24 @@ NI_EXPORT int ni_mfma_attention_tile_tokens(int group) {
 }
 
 // tiles: QTile [n_tiles] built by the host from the portions of the step with the tile size above.
+// With nsplit > 1 the key range of every tile is cut into nsplit runs; partial results go to part_o
+// (float [T, H, nsplit, HEAD_DIM]) and part_ml (float [T, H, nsplit, 2]) and `out` is left to the
+// merge kernel of the token-at-a-time library (same layout).
 NI_EXPORT int ni_mfma_attention(const void* q, int q_stride, const void* kpool, const void* vpool, const void* block_table,
-                                int table_stride, const void* tiles, int n_tiles, void* out, int H, int KVH,
-                                int page_size, int window, float scale, hipStream_t stream) {
+                                int table_stride, const void* tiles, int n_tiles, void* out, void* part_o, void* part_ml,
+                                int H, int KVH, int page_size, int window, float scale, int nsplit, hipStream_t stream) {
     if (n_tiles <= 0) return 0;
-    if (H % KVH != 0 || page_size < 1) return -1;
+    if (H % KVH != 0 || page_size < 1 || nsplit < 1 || nsplit > 64) return -1;
+    if (nsplit > 1 && (!part_o || !part_ml)) return -2;
     const int G = H / KVH;
     const int hpt = G >= 16 ? 16 : G > 4 ? 8 : G > 2 ? 4 : G > 1 ? 2 : 1;
     const int chunks = (G + hpt - 1) / hpt;
-    dim3 grid(n_tiles, KVH * chunks);
+    dim3 grid(n_tiles, KVH * chunks, nsplit);
 #define MA_LAUNCH(HPT_)                                                                                              \
     mfma_attention_kernel<HPT_><<<grid, MA_THREADS, 0, stream>>>(                                                  \
         (const bf16_t*)q, q_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table,        \
-        table_stride, (const QTile*)tiles, (bf16_t*)out, H, KVH, page_size, window, scale)
+        table_stride, (const QTile*)tiles, (bf16_t*)out, (float*)part_o, (float*)part_ml, H, KVH, page_size, window,  \
+        scale, nsplit)
     switch (hpt) {
         case 1: MA_LAUNCH(1); break;
         case 2: MA_LAUNCH(2); break;

@@ -260,11 +260,20 @@ def build_q_tiles(q_start, q_len, context_len, tile_tokens: int):
     return flat
 
 
+def mfma_splits(n_tiles: int, kv_heads: int, group: int, max_keys: int) -> int:
+    """Into how many runs the matrix-core kernel cuts the keys of every tile so that about a
+    thousand workgroups exist; a run is never shorter than 256 keys."""
+    hpt = 16 if group >= 16 else 8 if group > 4 else 4 if group > 2 else 2 if group > 1 else 1
+    items = max(1, n_tiles * kv_heads * ((group + hpt - 1) // hpt))
+    return int(max(1, min(1024 // items, max_keys // 256, 16)))
+
+
 def mfma_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                    tiles: torch.Tensor, out: torch.Tensor, H: int, KVH: int, hd: int, scale: float,
-                   window: Optional[int]) -> torch.Tensor:
+                   window: Optional[int], nsplit: int = 1, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of prompt portions on the matrix cores (bfloat16).  ``tiles`` is int32 [n, 4] from
-    :func:`build_q_tiles`; the pools already hold the keys and values of every position of the step."""
+    :func:`build_q_tiles`; the pools already hold the keys and values of every position of the step.
+    ``workspace`` (float32, ``T*H*nsplit*(hd+2)`` elements) is needed when ``nsplit > 1``."""
     T = qkv.shape[0]
     _gpu(qkv, "qkv", torch.bfloat16)
     _need(mfma_attention_ok(qkv.dtype, hd), f"mfma_attention does not take {qkv.dtype} with head size {hd}")
@@ -278,10 +287,23 @@ def mfma_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
     _gpu(tiles, "tiles", torch.int32)
     _need(tiles.dim() == 2 and tiles.shape[1] == 4, "tiles must be [n, 4]")
     _gpu(out, "out", torch.bfloat16, (T, H * hd))
+    part_o = part_ml = None
+    if nsplit > 1:
+        need = T * H * nsplit * (hd + 2)
+        _need(workspace is not None and workspace.dtype == torch.float32 and workspace.numel() >= need,
+              f"attention workspace of {need} floats needed for {nsplit} splits")
+        _gpu(workspace, "workspace")
+        flat = workspace.view(-1)
+        part_o = flat[: T * H * nsplit * hd]
+        part_ml = flat[T * H * nsplit * hd: need]
     _check(attention_mfma_lib(hd).ni_mfma_attention(_ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table),
-                                                    block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(out), H, KVH,
-                                                    kpool.shape[2], int(window) if window else 0, ctypes.c_float(scale),
+                                                    block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(out),
+                                                    _ptr(part_o), _ptr(part_ml), H, KVH, kpool.shape[2],
+                                                    int(window) if window else 0, ctypes.c_float(scale), nsplit,
                                                     _stream()), "mfma_attention")
+    if nsplit > 1:
+        _check(attention_lib(hd).ni_merge_splits(_ptr(part_o), _ptr(part_ml), _ptr(out), T, H, nsplit,
+                                                 dtype_code(out.dtype), _stream()), "merge_splits")
     return out
 
 

@@ -204,7 +204,7 @@ def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boo
         flat = K.build_q_tiles(starts, q_lens, lens, K.mfma_tile_tokens(hd, H // KVH))
         tiles = dev(torch.tensor(flat, dtype=torch.int32).view(-1, 4))
         K.mfma_attention(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table), tiles, out,
-                         H, KVH, hd, 1.0 / math.sqrt(hd), window)
+                         H, KVH, hd, 1.0 / math.sqrt(hd), window, nsplit, ws)
     else:
             K.token_attention(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table),
                           dev(torch.tensor(seq_of, dtype=torch.int32)), dev(torch.tensor(positions, dtype=torch.int32)),
@@ -257,9 +257,10 @@ def test_attention_finds_a_far_key_among_hundreds(K, dtype):
 def test_mfma_attention_head_sizes_and_groups(K, H, KVH, hd, ps):
     # whole prompts, portions that start in the middle of a sequence, single tokens beside them, tile edges
     lens, q_lens = [1, 37, 130, 64, 200, 17], [1, 37, 2, 1, 77, 16]
-    out, want, _ = paged_case(K, "bfloat16", H, KVH, hd, ps, lens, q_lens, None, hd + H, 1, kernel="mfma")
-    assert not torch.isnan(out).any(), "a key outside the sequence's own pages took part"
-    assert rel(out, want) < KTOL["bfloat16"], (H, KVH, hd, ps)
+    for nsplit in (1, 3):
+        out, want, _ = paged_case(K, "bfloat16", H, KVH, hd, ps, lens, q_lens, None, hd + H, nsplit, kernel="mfma")
+        assert not torch.isnan(out).any(), "a key outside the sequence's own pages took part"
+        assert rel(out, want) < KTOL["bfloat16"], (H, KVH, hd, ps, nsplit)
 
 
 def test_mfma_attention_window_and_far_key(K):
@@ -268,7 +269,7 @@ def test_mfma_attention_window_and_far_key(K):
         assert not torch.isnan(out).any()
         assert rel(out, want) < KTOL["bfloat16"], window
     for key_at in (37, 16, 15, 0, 31, 32, 698):
-        out, want, (qs, ks, vs) = paged_case(K, "bfloat16", 8, 2, 64, 16, [700], [5], None, 9, 1,
+        out, want, (qs, ks, vs) = paged_case(K, "bfloat16", 8, 2, 64, 16, [700], [5], None, 9, 1 + key_at % 4,
                                              boost=(0, key_at, 699, 6.0), kernel="mfma")
         assert rel(out, want) < KTOL["bfloat16"]
         got = out.double().cpu()[-1].reshape(8, 64)
