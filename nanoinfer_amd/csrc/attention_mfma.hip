@@ -139,24 +139,28 @@ __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
         }
     };
 
-    // Loads run two steps ahead of the arithmetic: while step s is multiplied, the rows of step
-    // s+1 are being written to LDS (they were asked for a step ago) and those of s+2 are asked for.
-    uint4 kf[2][KK], kf1[2][KK], kf2[2][KK];
-    uint4 v1[V_PER_THREAD], v2[V_PER_THREAD];
-    if (nsteps > 0) {
-        load_k(kfirst, kf);
-        load_v(kfirst, v1);
-        if (nsteps > 1) load_k(kfirst + KSTEP, kf1);
-        store_v(0, v1);
-        if (nsteps > 1) load_v(kfirst + KSTEP, v1);
+    // Loads run DEPTH - 1 steps ahead of the arithmetic: rows wait in registers (a ring, rotated
+    // every step) while older steps are multiplied, so a step costs its arithmetic, not a memory
+    // round trip.  V of step s+1 is written to LDS during step s, DEPTH - 2 steps after it was asked for.
+    constexpr int DEPTH = 4;
+    uint4 kf[DEPTH][2][KK];
+    uint4 vr[DEPTH][V_PER_THREAD];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        if (d < nsteps) {
+            if (wave_ok) load_k(kfirst + d * KSTEP, kf[d]);
+            load_v(kfirst + d * KSTEP, vr[d]);
+        }
     }
+    if (nsteps > 0) store_v(0, vr[0]);
     for (int s = 0; s < nsteps; ++s) {
         const int ks = kfirst + s * KSTEP;
         __syncthreads();                       // V of this step is in vs[s & 1]; nobody still reads the other buffer
-        const bool more = s + 1 < nsteps, more2 = s + 2 < nsteps;
-        if (more2) {
-            load_k(ks + 2 * KSTEP, kf2);
-            load_v(ks + 2 * KSTEP, v2);
+        const bool more = s + 1 < nsteps, ahead = s + DEPTH < nsteps;
+        uint4 k_new[2][KK], v_new[V_PER_THREAD];
+        if (ahead) {
+            if (wave_ok && ks + DEPTH * KSTEP <= wave_pmax) load_k(ks + DEPTH * KSTEP, k_new);   // only who will multiply them
+            load_v(ks + DEPTH * KSTEP, v_new);
         }
         if (wave_ok && ks <= wave_pmax) {
             // S^T for the two 16-key halves
@@ -166,7 +170,7 @@ __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
                 st[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int kk = 0; kk < KK; ++kk)
-                    st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[t][kk]),
+                    st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[0][t][kk]),
                                                                     __builtin_bit_cast(bf16x8_t, qf[kk]), st[t], 0, 0, 0);
             }
             // this lane: row r, keys ks + t*16 + kg*4 + i
@@ -220,15 +224,22 @@ __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
                                                                 __builtin_bit_cast(bf16x8_t, pf), o[dt], 0, 0, 0);
             }
         }
-        if (more) {
-            store_v((s + 1) & 1, v1);
+        if (more) store_v((s + 1) & 1, vr[1]);
+#pragma unroll
+        for (int d = 0; d + 1 < DEPTH; ++d) {
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) { kf[t][kk] = kf1[t][kk]; kf1[t][kk] = kf2[t][kk]; }
+                for (int kk = 0; kk < KK; ++kk) kf[d][t][kk] = kf[d + 1][t][kk];
 #pragma unroll
-            for (int i = 0; i < V_PER_THREAD; ++i) v1[i] = v2[i];
+            for (int i = 0; i < V_PER_THREAD; ++i) vr[d][i] = vr[d + 1][i];
         }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) kf[DEPTH - 1][t][kk] = k_new[t][kk];
+#pragma unroll
+        for (int i = 0; i < V_PER_THREAD; ++i) vr[DEPTH - 1][i] = v_new[i];
     }
 
     // the sum of a row is spread over the four lanes that share it
