@@ -11,6 +11,11 @@
 // instructions per piece.  The MFMA's k index is only a label, so the same lane-to-k mapping on
 // both operands is all that is required.  Partial sums meet in LDS.
 //
+// W comes either as stored, [N, K] row-major, or re-tiled once at load into the order this kernel
+// reads it: [tile of 16 rows][128-byte piece][lane][32 bytes], zero-padded to whole tiles and
+// pieces.  A wavefront's load is then 2 KB of consecutive memory instead of sixteen 128-byte
+// runs 2*K bytes apart, which is worth about a third on the [2048, 8192] matrix.
+//
 // Epilogues: store (compute type or float32), or SwiGLU over paired tiles (tile 2j from the gate
 // rows, tile 2j+1 from the up rows of a stacked [2I, K] matrix): out[m, n] = silu(g) * u; or
 // rotation + cache write for a stacked [q; k; v] matrix: a workgroup owns the two tiles of one
@@ -73,7 +78,7 @@ struct RopeArgs {
     int H, KVH, hd, page_size;
 };
 
-template <typename T, typename TOUT, int MB, int NT, int EPI>
+template <typename T, typename TOUT, int MB, int NT, int EPI, bool TILED>
 __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                                  TOUT* __restrict__ y, int M, int N, int K, int I,
                                                                  RopeArgs rope) {
@@ -96,7 +101,10 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
             col0 = (wg / per_head) * rope.hd + (wg % per_head) * 16 + nt * (rope.hd / 2);
         }
         const int shift = (EPI == EPI_SWIGLU && (nt % 2)) ? I : 0;      // odd tiles of a pair come from the up rows
-        wrow[nt] = W + static_cast<size_t>(min(col0 + r, n_limit - 1) + shift) * K;
+        if (TILED)      // first byte of this lane in piece 0 of the tile; the buffer is padded, nothing to clamp
+            wrow[nt] = W + static_cast<size_t>((col0 + shift) / 16) * ((K + CH - 1) / CH) * (WAVE * EL) + lane * EL;
+        else
+            wrow[nt] = W + static_cast<size_t>(min(col0 + r, n_limit - 1) + shift) * K;
     }
     const T* xrow[MB];
     bool xok[MB];
@@ -121,11 +129,16 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
         Piece<T> xb[PT][MB], wa[PT][NT];
 #pragma unroll
         for (int u = 0; u < PT; ++u) {
-            const int k = (c + u * GV_WAVES) * CH + kg * EL;
+            const int piece = c + u * GV_WAVES;
+            const int k = piece * CH + kg * EL;
             const bool kok = k < K;                  // K is a multiple of EL: a lane's 32 bytes are all in or all out
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                if (kok) wa[u][nt].load(wrow[nt] + k); else wa[u][nt].zero();
+                if (TILED) {
+                    if (piece < pieces) wa[u][nt].load(wrow[nt] + static_cast<size_t>(piece) * (WAVE * EL)); else wa[u][nt].zero();
+                } else {
+                    if (kok) wa[u][nt].load(wrow[nt] + k); else wa[u][nt].zero();
+                }
             }
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
@@ -226,15 +239,18 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
 }
 
 template <typename T, typename TOUT, int MB, int EPI>
-static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream,
-                     RopeArgs rope = RopeArgs{}) {
+static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, bool tiled,
+                     hipStream_t stream, RopeArgs rope = RopeArgs{}) {
     const int out_width = (EPI == EPI_SWIGLU) ? I : N;
     const int tiles = (out_width + 15) / 16;
     auto run = [&](auto nt_tag) {
         constexpr int NTc = decltype(nt_tag)::value;
         constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
         const int grid = (tiles + NOUT - 1) / NOUT;
-        skinny_gemm_kernel<T, TOUT, MB, NTc, EPI><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope);
+        if (tiled)
+            skinny_gemm_kernel<T, TOUT, MB, NTc, EPI, true><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope);
+        else
+            skinny_gemm_kernel<T, TOUT, MB, NTc, EPI, false><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope);
     };
     // NT * MB fragments of partial sums share 64 KB of LDS: at most 8
     if constexpr (MB <= 2 && EPI != EPI_ROPE) {
@@ -250,30 +266,32 @@ static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K,
 }
 
 template <typename T, typename TOUT, int EPI>
-static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream,
-                     RopeArgs rope = RopeArgs{}) {
-    if (M <= 16) return launch_nt<T, TOUT, 1, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
-    if (M <= 32) return launch_nt<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
-    return launch_nt<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
+static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, bool tiled,
+                     hipStream_t stream, RopeArgs rope = RopeArgs{}) {
+    if (M <= 16) return launch_nt<T, TOUT, 1, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
+    if (M <= 32) return launch_nt<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
+    return launch_nt<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
 }
 
 // epilogue: 0 store in the input type, 1 store float32, 2 SwiGLU (W is [2I, K], y is [M, I]).
 // K must be a multiple of 16 bytes' worth of elements x 2 (bf16: 16, f32: 8); M <= 64.
+// tiled: W is in the re-tiled order described at the top (swiglu then needs N/2 to be a multiple of 16).
 NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N, int K, int epilogue, int tiles_per_group,
-                             int dtype, hipStream_t stream) {
+                             int tiled, int dtype, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64) return -1;
     const int el = dtype == 0 ? 8 : 16;
     if (K % el != 0) return -2;
     const int I = N / 2;
     if (epilogue == 2 && (N % 2)) return -3;
+    if (epilogue == 2 && tiled && (I % 16)) return -4;
     if (dtype == 0) {
-        if (epilogue == 2) return launch_mb<float, float, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, stream);
-        return launch_mb<float, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, stream);
+        if (epilogue == 2) return launch_mb<float, float, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
+        return launch_mb<float, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
     }
-    if (epilogue == 2) return launch_mb<bf16_t, bf16_t, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, stream);
-    if (epilogue == 1) return launch_mb<bf16_t, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, stream);
-    return launch_mb<bf16_t, bf16_t, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, stream);
+    if (epilogue == 2) return launch_mb<bf16_t, bf16_t, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
+    if (epilogue == 1) return launch_mb<bf16_t, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
+    return launch_mb<bf16_t, bf16_t, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
 }
 
 // Product with the stacked [q; k; v] matrix ((H + 2 KVH) * hd rows), rotation of query and key
@@ -281,7 +299,7 @@ NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N
 // slot_mapping (null: not stored).  hd must be a multiple of 32 and fully rotated.
 NI_EXPORT int ni_skinny_qkv_rope(const void* x, const void* W, void* q_out, const void* positions, const void* cos_t,
                                  const void* sin_t, const void* slot_mapping, void* kpool, void* vpool, int M, int K,
-                                 int H, int KVH, int hd, int page_size, int dtype, hipStream_t stream) {
+                                 int H, int KVH, int hd, int page_size, int tiled, int dtype, hipStream_t stream) {
     if (M <= 0) return 0;
     if (M > 64) return -1;
     if (K % (dtype == 0 ? 8 : 16) != 0) return -2;
@@ -290,6 +308,6 @@ NI_EXPORT int ni_skinny_qkv_rope(const void* x, const void* W, void* q_out, cons
                   kpool, vpool, H, KVH, hd, page_size};
     const int N = (H + 2 * KVH) * hd;
     // launch_nt sizes the grid from the output width: one workgroup per two tiles
-    if (dtype == 0) return launch_mb<float, float, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, stream, rope);
-    return launch_mb<bf16_t, bf16_t, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, stream, rope);
+    if (dtype == 0) return launch_mb<float, float, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, tiled != 0, stream, rope);
+    return launch_mb<bf16_t, bf16_t, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, tiled != 0, stream, rope);
 }

@@ -342,6 +342,46 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
 # ------------------------------------------------------------------ matrix product (library)
 
 SKINNY_MAX_ROWS = 64
+
+
+def tile_weight(w: torch.Tensor) -> torch.Tensor:
+    """``w`` [N, K] re-laid for the skinny product: [tile of 16 rows][128-byte piece][lane][32 bytes]
+    with lane = 16 * (which 32 bytes of the piece) + (row in the tile), zero-padded to whole tiles
+    and pieces.  Flat, same type and device as ``w``."""
+    N, Kd = w.shape
+    el = 8 if w.dtype == torch.float32 else 16
+    ch = 4 * el
+    Np, Kp = (N + 15) // 16 * 16, (Kd + ch - 1) // ch * ch
+    if (Np, Kp) != (N, Kd):
+        padded = torch.zeros(Np, Kp, dtype=w.dtype, device=w.device)
+        padded[:N, :Kd] = w
+        w = padded
+    return w.view(Np // 16, 16, Kp // ch, 4, el).permute(0, 2, 3, 1, 4).contiguous().view(-1)
+
+
+class Weight:
+    """A matrix [out, in] as the products want it: ``rows`` as stored (for the library product of
+    many rows) and, optionally, ``tiles`` in the order the skinny product streams it."""
+
+    __slots__ = ("rows", "tiles")
+
+    def __init__(self, rows: torch.Tensor, tiled: bool = True):
+        self.rows = rows
+        self.tiles = tile_weight(rows) if tiled and rows.dtype in (torch.float32, torch.bfloat16) else None
+
+    @property
+    def shape(self):
+        return self.rows.shape
+
+    @property
+    def dtype(self):
+        return self.rows.dtype
+
+
+def _rows_and_tiles(weight):
+    if isinstance(weight, Weight):
+        return weight.rows, weight.tiles
+    return weight, None
 _library_calls = 0
 
 
@@ -367,11 +407,14 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, swiglu
     may be float32 for bfloat16 inputs.  With ``swiglu`` the weight is a stacked [2I, K] matrix
     (gate rows, then up rows) and ``out`` [M, I] receives ``silu(gate) * up``."""
     M, Kd = x.shape
+    weight, tiles = _rows_and_tiles(weight)
     N = weight.shape[0]
     _gpu(x, "x")
     _gpu(weight, "weight", x.dtype)
     _need(weight.shape[1] == Kd, f"skinny_gemm: {tuple(x.shape)} x {tuple(weight.shape)}^T")
     _need(skinny_ok(M, Kd, x.dtype), f"skinny_gemm does not take M={M}, K={Kd} in {x.dtype}")
+    if swiglu and tiles is not None and (N // 2) % 16:
+        tiles = None          # gate and up halves do not start on tile boundaries: stream the rows as stored
     if swiglu:
         _need(N % 2 == 0, "a stacked gate/up matrix needs an even number of rows")
         _gpu(out, "out", x.dtype, (M, N // 2))
@@ -380,9 +423,9 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, swiglu
         _need(out.dtype in (x.dtype, torch.float32), f"out must be {x.dtype} or float32")
         _gpu(out, "out", None, (M, N))
         epi = 1 if (out.dtype == torch.float32 and x.dtype != torch.float32) else 0
-    _check(skinny_lib().ni_skinny_gemm(_ptr(x), _ptr(weight), _ptr(out), M, N, Kd, epi,
-                                       _tiles_per_group(N // 2 if swiglu else N), dtype_code(x.dtype), _stream()),
-           "skinny_gemm")
+    _check(skinny_lib().ni_skinny_gemm(_ptr(x), _ptr(weight if tiles is None else tiles), _ptr(out), M, N, Kd, epi,
+                                       _tiles_per_group(N // 2 if swiglu else N), 0 if tiles is None else 1,
+                                       dtype_code(x.dtype), _stream()), "skinny_gemm")
     return out
 
 
@@ -398,6 +441,7 @@ def skinny_qkv_rope(x: torch.Tensor, w_qkv: torch.Tensor, positions: torch.Tenso
     """``x . w_qkv^T`` for few rows with rotation and cache write fused in: returns the rotated
     queries [M, H*hd]; rotated keys and plain values go straight into the pools at ``slot_mapping``."""
     M, Kd = x.shape
+    w_qkv, tiles = _rows_and_tiles(w_qkv)
     _gpu(x, "x")
     _gpu(w_qkv, "w_qkv", x.dtype, ((H + 2 * KVH) * hd, Kd))
     _need(qkv_rope_ok(M, Kd, hd, 2 * cos.shape[1], x.dtype), f"skinny_qkv_rope does not take M={M}, K={Kd}, hd={hd}")
@@ -413,9 +457,10 @@ def skinny_qkv_rope(x: torch.Tensor, w_qkv: torch.Tensor, positions: torch.Tenso
               f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
         page_size = kpool.shape[2]
     q = torch.empty(M, H * hd, dtype=x.dtype, device=x.device)
-    _check(skinny_lib().ni_skinny_qkv_rope(_ptr(x), _ptr(w_qkv), _ptr(q), _ptr(positions), _ptr(cos), _ptr(sin),
-                                           _ptr(slot_mapping), _ptr(kpool), _ptr(vpool), M, Kd, H, KVH, hd,
-                                           page_size, dtype_code(x.dtype), _stream()), "skinny_qkv_rope")
+    _check(skinny_lib().ni_skinny_qkv_rope(_ptr(x), _ptr(w_qkv if tiles is None else tiles), _ptr(q), _ptr(positions),
+                                           _ptr(cos), _ptr(sin), _ptr(slot_mapping), _ptr(kpool), _ptr(vpool), M, Kd,
+                                           H, KVH, hd, page_size, 0 if tiles is None else 1, dtype_code(x.dtype),
+                                           _stream()), "skinny_qkv_rope")
     return q
 
 
@@ -424,13 +469,15 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
     product; many rows to the library (rocBLAS/hipBLASLt), where float32 inputs are multiplied in
     true float32 (the reduced-precision matrix modes of the library are switched off at import).
     ``out_dtype`` float32 keeps the float32 accumulators of a bfloat16 product."""
-    _need(x.is_cuda and weight.is_cuda, "linear needs GPU tensors")
-    _need(x.dtype == weight.dtype, f"linear: activation {x.dtype} and weight {weight.dtype} differ")
-    _need(x.dim() == 2 and x.shape[1] == weight.shape[1], f"linear: {tuple(x.shape)} x {tuple(weight.shape)}^T")
+    rows, _ = _rows_and_tiles(weight)
+    _need(x.is_cuda and rows.is_cuda, "linear needs GPU tensors")
+    _need(x.dtype == rows.dtype, f"linear: activation {x.dtype} and weight {rows.dtype} differ")
+    _need(x.dim() == 2 and x.shape[1] == rows.shape[1], f"linear: {tuple(x.shape)} x {tuple(rows.shape)}^T")
     out_dtype = out_dtype or x.dtype
     if skinny_ok(x.shape[0], x.shape[1], x.dtype):
-        out = torch.empty(x.shape[0], weight.shape[0], dtype=out_dtype, device=x.device)
+        out = torch.empty(x.shape[0], rows.shape[0], dtype=out_dtype, device=x.device)
         return skinny_gemm(x, weight, out)
+    weight = rows
     global _library_calls
     _library_calls += 1
     if out_dtype != x.dtype:
@@ -447,7 +494,8 @@ def linear_swiglu(x: torch.Tensor, weight_gate_up: torch.Tensor) -> torch.Tensor
         return skinny_gemm(x, weight_gate_up, out, swiglu=True)
     global _library_calls
     _library_calls += 1
-    return swiglu(torch.matmul(x, weight_gate_up.t()), out)
+    rows, _ = _rows_and_tiles(weight_gate_up)
+    return swiglu(torch.matmul(x, rows.t()), out)
 
 
 def require_gpu() -> torch.device:

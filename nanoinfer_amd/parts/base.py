@@ -74,6 +74,18 @@ class Runtime:
             self.shared[key] = t
         return t
 
+    def weight(self, name: str, cpu: torch.Tensor, tiled: bool = True):
+        """A checkpoint matrix as a :class:`nanoinfer_amd.kernels.Weight`: its rows on the device in the
+        compute type (shared with :meth:`matrix`) plus, when ``tiled``, the copy that the skinny
+        product of decoding streams."""
+        from .. import kernels as K
+        key = ("weight", name, self.dtype, tiled)
+        w = self.shared.get(key)
+        if w is None:
+            w = K.Weight(self.matrix(name, cpu), tiled=tiled)
+            self.shared[key] = w
+        return w
+
     def vector32(self, name: str, cpu: torch.Tensor) -> torch.Tensor:
         """A one-dimensional parameter (a norm's weight) on the device, always float32."""
         key = ("vector", name)

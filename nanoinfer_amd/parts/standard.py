@@ -177,13 +177,9 @@ class Attention(Part):
         pos_spec: PartSpec = p["position"]
         self.position = get_part("position", pos_spec.kind)(pos_spec, {}, rt)
         names = spec.weights
-        fused_name = "|".join((names["q"], names["k"], names["v"]))
-        key = ("matrix", fused_name, rt.dtype)
-        if key not in rt.shared:
-            rt.shared[key] = torch.cat([weights["q"], weights["k"], weights["v"]], dim=0).to(
-                device=rt.device, dtype=rt.dtype).contiguous()
-        self.w_qkv = rt.shared[key]
-        self.w_o = rt.matrix(names["o"], weights["o"])
+        self.w_qkv = rt.weight("|".join((names["q"], names["k"], names["v"])),
+                               torch.cat([weights["q"], weights["k"], weights["v"]], dim=0))
+        self.w_o = rt.weight(names["o"], weights["o"])
 
     def cache_need(self) -> CacheNeed:
         return CacheNeed(kv=KVNeed(self.KVH, self.hd, self.window))
@@ -238,12 +234,8 @@ class SwiGLU(Part):
         super().__init__(spec, weights, rt)
         self.intermediate_size = int(spec.params["intermediate_size"])
         names = spec.weights
-        key = ("matrix", names["gate"] + "|" + names["up"], rt.dtype)
-        if key not in rt.shared:
-            rt.shared[key] = torch.cat([weights["gate"], weights["up"]], dim=0).to(
-                device=rt.device, dtype=rt.dtype).contiguous()
-        self.w_gate_up = rt.shared[key]
-        self.w_down = rt.matrix(names["down"], weights["down"])
+        self.w_gate_up = rt.weight(names["gate"] + "|" + names["up"], torch.cat([weights["gate"], weights["up"]], dim=0))
+        self.w_down = rt.weight(names["down"], weights["down"])
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         return K.linear(K.linear_swiglu(x, self.w_gate_up), self.w_down)
@@ -305,6 +297,7 @@ class LinearHead(Part):
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
         self.vocab_size = int(spec.params["vocab_size"])
+        # the large matrix is streamed as stored: re-tiling gains nothing at its size and would double it
         self.weight = rt.matrix(spec.weights["weight"], weights["weight"])
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:

@@ -401,6 +401,13 @@ def _skinny_case(Kmod, dtype, M, N, Kd):
         act = Kmod.skinny_gemm(dev(x), dev(w), torch.empty(M, N // 2, device="cuda", dtype=DT[dtype]), swiglu=True)
         assert rel(act, P.swiglu(want[:, :N // 2], want[:, N // 2:])) < KTOL[dtype], "swiglu"
     assert rel(Kmod.linear(dev(x), dev(w)), want) < KTOL[dtype]
+    # the re-tiled copy of the matrix gives the same sums in the same order
+    tiled = Kmod.Weight(dev(w))
+    assert tiled.tiles is not None and tiled.tiles.numel() >= w.numel()
+    assert torch.equal(Kmod.skinny_gemm(dev(x), tiled, torch.empty(M, N, device="cuda", dtype=DT[dtype])), out)
+    assert torch.equal(Kmod.skinny_gemm(dev(x), tiled, torch.empty(M, N, device="cuda", dtype=torch.float32)), out32)
+    if N % 2 == 0:
+        assert torch.equal(Kmod.skinny_gemm(dev(x), tiled, torch.empty(M, N // 2, device="cuda", dtype=DT[dtype]), swiglu=True), act)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -458,4 +465,8 @@ def test_product_with_rotation_and_cache_write(K, dtype, M, H, KVH, hd, Kd, ps):
     k2 = torch.full_like(kpool, 3.0)
     q2 = K.skinny_qkv_rope(dev(x), dev(w), dev(positions), cos, sin, None, None, None, H, KVH, hd)
     assert torch.equal(q2, q) and bool((k2 == 3.0).all())
+    # the re-tiled matrix: same queries, same pages
+    k3, v3 = torch.full_like(kpool, 7.0), torch.full_like(vpool, 7.0)
+    q3 = K.skinny_qkv_rope(dev(x), K.Weight(dev(w)), dev(positions), cos, sin, dev(slots), k3, v3, H, KVH, hd)
+    assert torch.equal(q3, q) and torch.equal(k3, kpool) and torch.equal(v3, vpool)
     assert not K.qkv_rope_ok(M, Kd, 48, 48, DT[dtype]) and not K.qkv_rope_ok(M, Kd, hd, hd // 2, DT[dtype])
