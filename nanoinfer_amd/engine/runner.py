@@ -316,14 +316,30 @@ class ModelRunner:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx, self._layer_cache(ctx))
-        if K.library_calls() != calls_before:
-            # a library routine ran inside: its nodes are not ours to vouch for, so this shape runs eagerly
+        if K.library_calls() != calls_before and not self._replays_faithfully(graph, logits, warm, entries):
+            # a library routine ran inside and its recorded nodes do not reproduce the eager result
+            # (some record memory-clearing nodes that misbehave on replay): this shape runs eagerly
             self._unrecordable.add(key)
             return None
         rec = _RecordedStep(graph, meta, staging, logits, ctx, torch.cuda.Event())
         rec.copied.record()
         self._recorded[key] = rec
         return rec
+
+    def _replays_faithfully(self, graph, logits, warm: StepContext, entries: List[StepEntry], rounds: int = 3) -> bool:
+        """Replay a fresh recording several times, with the same step run eagerly and a
+        synchronisation between the replays, and compare every replay with the eager logits.
+        A decode step may be run any number of times: it writes the same keys and values again."""
+        for _ in range(rounds):
+            graph.replay()
+            torch.cuda.synchronize()
+            got = logits.clone()
+            want = self.model.forward(warm, self._layer_cache(warm))
+            torch.cuda.synchronize()
+            scale = float(want.abs().max())
+            if not bool(torch.isfinite(got).all()) or float((got - want).abs().max()) > 1e-3 * max(scale, 1e-30):
+                return False
+        return True
 
     def _replay(self, key, entries: List[StepEntry]) -> Optional[torch.Tensor]:
         rec = self._recorded.get(key)

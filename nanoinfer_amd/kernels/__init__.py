@@ -341,7 +341,8 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
 
 # ------------------------------------------------------------------ matrix product (library)
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 64        # what the kernel takes
+SKINNY_BEST_ROWS = 16       # up to here it beats the library product on this chip (measured at the 1B sizes)
 
 
 def tile_weight(w: torch.Tensor) -> torch.Tensor:
@@ -474,7 +475,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
     _need(x.dtype == rows.dtype, f"linear: activation {x.dtype} and weight {rows.dtype} differ")
     _need(x.dim() == 2 and x.shape[1] == rows.shape[1], f"linear: {tuple(x.shape)} x {tuple(rows.shape)}^T")
     out_dtype = out_dtype or x.dtype
-    if skinny_ok(x.shape[0], x.shape[1], x.dtype):
+    if x.shape[0] <= SKINNY_BEST_ROWS and skinny_ok(x.shape[0], x.shape[1], x.dtype):
         out = torch.empty(x.shape[0], rows.shape[0], dtype=out_dtype, device=x.device)
         return skinny_gemm(x, weight, out)
     weight = rows
@@ -490,7 +491,7 @@ def linear_swiglu(x: torch.Tensor, weight_gate_up: torch.Tensor) -> torch.Tensor
     few rows, product then the SwiGLU kernel for many."""
     inter = weight_gate_up.shape[0] // 2
     out = torch.empty(x.shape[0], inter, dtype=x.dtype, device=x.device)
-    if skinny_ok(x.shape[0], x.shape[1], x.dtype):
+    if x.shape[0] <= SKINNY_BEST_ROWS and skinny_ok(x.shape[0], x.shape[1], x.dtype):
         return skinny_gemm(x, weight_gate_up, out, swiglu=True)
     global _library_calls
     _library_calls += 1

@@ -316,3 +316,27 @@ def test_recorded_decode_steps_equal_eager_ones(dtype):
     both([dec("g0"), dec("g2")])
     assert len(recorded._recorded) >= 3 and not eager._recorded
     compare(got, reqs, folder, dtype, "recorded decode")
+
+
+def test_recorded_steps_with_library_products_are_checked_before_use():
+    """More than 16 rows go to the library's matrix product.  A recording that contains one is
+    replayed against eager runs before it is trusted; whatever that check decides, the logits of
+    every step equal those of a runner that records nothing."""
+    from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
+    folder = model_folder("A", stored="bfloat16")
+    recorded = ModelRunner(folder, dtype="bfloat16", page_size=16, max_tokens=2048, max_requests=24)
+    eager = ModelRunner(folder, dtype="bfloat16", page_size=16, max_tokens=2048, max_requests=24, use_graphs=False)
+    n = 20
+    prompts = [list(random_tokens(256, 5 + i, 700 + i)) for i in range(n)]
+    for i, p in enumerate(prompts):
+        a = recorded.step([StepEntry(i, p, [len(p) - 1])])
+        b = eager.step([StepEntry(i, p, [len(p) - 1])])
+        assert float((a - b).abs().max()) <= 1e-3 * float(b.abs().max())
+    toks = [7 * i % 256 for i in range(n)]
+    for step in range(6):
+        a = recorded.step([StepEntry(i, [toks[i]], [0]) for i in range(n)])
+        b = eager.step([StepEntry(i, [toks[i]], [0]) for i in range(n)])
+        torch.cuda.synchronize()
+        assert float((a - b).abs().max()) <= 2e-3 * float(b.abs().max()), step
+        toks = a.argmax(-1).tolist()
+    assert len(recorded._recorded) + len(recorded._unrecordable) == 1
