@@ -5,8 +5,8 @@
 A step is one decode step of a batch of 8 requests whose prompts of 2,048 random tokens are in
 the cache (context limit 4,096): the step function runs the 8 new tokens as one batch, the
 argmax kernel picks the next ones, and they come back to the host, as in generation.  ``value``
-is decoded tokens per second.  The same line carries the prefill of one 2,048-token prompt (in
-portions of 512, as the configuration says), the decode step's fraction of the HBM roofline, and
+is decoded tokens per second.  The same line carries the prefill of one 2,048-token prompt (one
+portion, the engine's default; ``--prefill-chunk`` cuts it), the decode step's fraction of the HBM roofline, and
 decode at batch 1 and 64.  Peaks are MI355X's published ones: HBM 8 TB/s, dense bf16 MFMA
 2.5 PFLOP/s, fp32 157.3 TFLOP/s.  The reference publishes no numbers for this model, so
 ``vs_baseline`` is null.
@@ -38,7 +38,7 @@ LLAMA_1B = {
 FULL_LAYERS = 16
 PROMPT_LEN = 2048
 CONTEXT_LEN = 4096
-PREFILL_CHUNK = 512
+PREFILL_CHUNK = 2048      # the engine's default portion: the whole prompt in one step
 BLOCK_SIZE = 16
 HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
@@ -78,6 +78,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--prefill-chunk", type=int, default=PREFILL_CHUNK, help="tokens of a prompt portion in the prefill measurement")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
                     help="run one phase only (for profiling; prints no result line)")
@@ -115,15 +116,17 @@ def main() -> int:
         return [rng.randrange(V) for _ in range(PROMPT_LEN)]
 
     def measure_prefill():
-        """One prompt of 2,048 tokens in portions of 512; the last portion yields the first token."""
+        """One prompt of 2,048 tokens; the last portion yields the first token."""
         times = []
+        chunk = args.prefill_chunk
         for rep in range(3):
             toks = prompt()
             torch.cuda.synchronize()
             t = time.perf_counter()
-            for s in range(0, PROMPT_LEN, PREFILL_CHUNK):
-                last = s + PREFILL_CHUNK >= PROMPT_LEN
-                logits = runner.step([StepEntry("p", toks[s:s + PREFILL_CHUNK], [PREFILL_CHUNK - 1] if last else [])])
+            for s in range(0, PROMPT_LEN, chunk):
+                part = toks[s:s + chunk]
+                last = s + chunk >= PROMPT_LEN
+                logits = runner.step([StepEntry("p", part, [len(part) - 1] if last else [])])
             K.argmax(logits).tolist()
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t)
@@ -198,7 +201,7 @@ def main() -> int:
             "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
             "tied_embeddings": True, "global_batch": args.batch, "prompt_len": PROMPT_LEN,
             "seq_len": CONTEXT_LEN, "decode_context_mean": round(mean_ctx, 1), "kv_block_size": BLOCK_SIZE,
-            "prefill_chunk": PREFILL_CHUNK, "parallelism": "single-gpu",
+            "prefill_chunk": args.prefill_chunk, "parallelism": "single-gpu",
         },
         "prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(flops / prefill_s / FLOP_PEAK[args.dtype], 4)},

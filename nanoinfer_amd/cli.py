@@ -42,7 +42,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--ignore-eos", action="store_true", help="generate --max-tokens tokens whatever is sampled")
     ap.add_argument("--max-batch-size", type=int, default=8)
     ap.add_argument("--max-sequences", type=int, default=16)
-    ap.add_argument("--prefill-chunk-size", type=int, default=512)
+    ap.add_argument("--prefill-chunk-size", type=int, default=2048)
     ap.add_argument("--max-num-batched-tokens", type=int, default=2048)
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--num-cache-blocks", type=int, default=1024)

@@ -46,12 +46,12 @@ template <bool FAST> __device__ __forceinline__ float ex(float x) {
     else return expf(x);
 }
 
-template <typename T>
+template <typename T, bool POW2>
 __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ kpool, const T* __restrict__ vpool,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ positions, T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
-    int H, int KVH, int page_size, int window, float scale, int nsplit) {
+    int H, int KVH, int page_size, int page_shift, int window, float scale, int nsplit) {
     using L = Lanes<T>;
     constexpr int LPK = L::LPK, EPL = L::EPL, KPI = L::KPI, HD = HEAD_DIM;
     constexpr int WAVES = ATT_THREADS / WAVE;
@@ -102,25 +102,32 @@ __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
     }
 
     // U keys per lane group and trip.  The loop is pipelined by hand: while trip t is being
-    // multiplied, the rows of trip t+1 are in flight and the table entries of trip t+2 are being
-    // fetched, so the two dependent memory round trips of a trip (table, then rows) overlap with
-    // arithmetic instead of adding up trip after trip.  The running maximum moves once per trip:
-    // one rescaling of the output and U + 1 exponentials per head and trip.
+    // multiplied, the rows of trip t+1 are in flight and the addresses of trip t+2 are being
+    // worked out.  The running maximum moves once per trip: one rescaling of the output and
+    // U + 1 exponentials per head and trip.
     constexpr int U = EPL <= 8 ? 4 : 2;
-    const int page_shift = (page_size & (page_size - 1)) == 0 ? __ffs(page_size) - 1 : -1;
-    const int iters = (k1 > k0) ? (k1 - k0 + KPI - 1) / KPI : 0;
+    auto page_of = [&](int j) { return POW2 ? (j >> page_shift) : j / page_size; };
+    auto slot_of = [&](int j) { return POW2 ? (j & (page_size - 1)) : j % page_size; };
+
+    // The block table of the key range is copied to LDS, a segment of TBL_MAX pages at a time
+    // (one segment, unless the range is very long).  A table entry read from global memory
+    // inside the loop would have to be waited for before the rows it points to can be asked
+    // for, and that wait, being in order, would also drain every row load still in flight: one
+    // full memory round trip per trip, whatever is prefetched.  With the table in LDS the row
+    // loads of a trip depend on no other load, and stay in flight across the arithmetic.
+    constexpr int TBL_MAX = 1024;
+    __shared__ int32_t tbl[TBL_MAX];
+    int s0 = k0, s1 = k0, lp0 = 0;     // keys s0..s1-1 are the current segment, its first page is lp0
 
     struct Where { size_t base[U]; bool valid[U]; };
     auto locate = [&](int it, Where& w) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int j = k0 + (it + u) * KPI + kslot;
-            w.valid[u] = j < k1;
-            const int jj = w.valid[u] ? j : k0;     // a key of this sequence in any case: the address stays legal
-            const int lp = page_shift >= 0 ? (jj >> page_shift) : jj / page_size;
-            const int off = page_shift >= 0 ? (jj & (page_size - 1)) : jj % page_size;
-            const int page = table[lp];
-            w.base[u] = ((static_cast<size_t>(page) * KVH + g) * page_size + off) * HD + sub * EPL;
+            const int j = s0 + (it + u) * KPI + kslot;
+            w.valid[u] = j < s1;
+            const int jj = w.valid[u] ? j : s0;     // a key of this segment in any case: the address stays legal
+            const int page = tbl[page_of(jj) - lp0];
+            w.base[u] = ((static_cast<size_t>(page) * KVH + g) * page_size + slot_of(jj)) * HD + sub * EPL;
         }
     };
     struct Rows { RawRow<T, EPL> k[U], v[U]; bool valid[U]; };     // as loaded: converted when multiplied
@@ -163,22 +170,31 @@ __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
         }
     };
 
-    // two trips per turn of the loop, A and B, each with a place of its own in registers
-    Where wa, wb;
-    Rows ra, rb;
-    if (iters > 0) {
+    while (s1 < k1) {
+        s0 = s1;
+        lp0 = page_of(s0);
+        s1 = min(k1, (lp0 + TBL_MAX) * page_size);
+        __syncthreads();               // nobody still reads the previous segment's entries
+        for (int i = tid; i <= page_of(s1 - 1) - lp0; i += ATT_THREADS) tbl[i] = table[lp0 + i];
+        __syncthreads();
+        const int iters = (s1 - s0 + KPI - 1) / KPI;
+
+        // Two trips per turn of the loop, A and B, each with a place of its own in registers.
+        // Rows past the end of the segment are loaded from a legal address and not used, so
+        // that the loads are never under a branch.
+        Where wa, wb;
+        Rows ra, rb;
         locate(0, wa);
-        if (iters > U) locate(U, wb);
+        locate(U, wb);
         fetch(wa, ra);
-    }
-    for (int it = 0; it < iters; it += 2 * U) {
-        const bool has_b = it + U < iters, has_a2 = it + 2 * U < iters, has_b2 = it + 3 * U < iters;
-        if (has_b) fetch(wb, rb);
-        if (has_a2) locate(it + 2 * U, wa);
-        multiply(ra);
-        if (has_a2) fetch(wa, ra);
-        if (has_b2) locate(it + 3 * U, wb);
-        if (has_b) multiply(rb);
+        for (int it = 0; it < iters; it += 2 * U) {
+            fetch(wb, rb);
+            locate(it + 2 * U, wa);
+            multiply(ra);
+            fetch(wa, ra);
+            locate(it + 3 * U, wb);
+            if (it + U < iters) multiply(rb);
+        }
     }
 
     // merge the lane groups of a wave (lanes with equal `sub`)
@@ -269,10 +285,15 @@ static int launch(const void* q, int q_stride, const void* kpool, const void* vp
     const int G = H / KVH;
     const int chunks = (G + GT - 1) / GT;
     dim3 grid(T_tokens, KVH * chunks, nsplit);
-    token_attention_kernel<T><<<grid, ATT_THREADS, 0, stream>>>(
+    // a page size that is a power of two gets shifts and masks, any other divisions
+    const bool pow2 = (page_size & (page_size - 1)) == 0;
+    int page_shift = 0;
+    while (pow2 && (1 << page_shift) < page_size) ++page_shift;
+    auto kernel = pow2 ? token_attention_kernel<T, true> : token_attention_kernel<T, false>;
+    kernel<<<grid, ATT_THREADS, 0, stream>>>(
         (const T*)q, q_stride, (const T*)kpool, (const T*)vpool, (const int32_t*)block_table, table_stride,
         (const int32_t*)seq_of_token, (const int32_t*)positions, (T*)out, (float*)part_o, (float*)part_ml,
-        H, KVH, page_size, window, scale, nsplit);
+        H, KVH, page_size, page_shift, window, scale, nsplit);
     int err = NI_LAUNCH_RESULT();
     if (err || nsplit == 1) return err;
     merge_splits_kernel<T><<<dim3(T_tokens, H), 64, 0, stream>>>((const float*)part_o, (const float*)part_ml, (T*)out,

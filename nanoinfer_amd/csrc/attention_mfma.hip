@@ -30,26 +30,26 @@ static_assert(HEAD_DIM % 32 == 0 && HEAD_DIM >= 32 && HEAD_DIM <= 256, "head siz
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
-#define MA_WAVES 4
-#define MA_THREADS (MA_WAVES * WAVE)
 #define KSTEP 32
+#define MA_WAVES 4
 #define NEG_BIG (-1.0e30f)
-#define VPAD 8   // elements of padding per staged row of V: the four key groups of a read fall on different banks
+#define VPAD 8   // elements of padding per staged row of V^T: the sixteen rows of a 16-byte read fall on different banks
 
 struct QTile { int32_t seq, row0, ntok, pos0; };   // tokens row0..row0+ntok-1 of the batch, positions pos0..
 
-template <int HPT>
-__global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
+template <int HPT, bool POW2>
+__global__ __launch_bounds__(MA_WAVES * WAVE) void mfma_attention_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int32_t* __restrict__ block_table, int table_stride, const QTile* __restrict__ tiles,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int H, int KVH, int page_size,
-    int window, float scale, int nsplit) {
+    int page_shift, int window, float scale, int nsplit) {
     constexpr int HD = HEAD_DIM;
+    constexpr int MA_THREADS = MA_WAVES * WAVE;
     constexpr int TPT = 16 / HPT;            // tokens of a wavefront
     constexpr int KK = HD / 32;              // k steps of the first product
     constexpr int DT = HD / 16;              // 16-wide tiles of the head dimension in the output
-    constexpr int VROW = HD + VPAD;
-    __shared__ __attribute__((aligned(16))) uint16_t vs[2][KSTEP][VROW];
+    constexpr int VROW = KSTEP + VPAD;
+    __shared__ __attribute__((aligned(16))) uint16_t vs[2][HD][VROW];      // V^T of a step: [dim][key, in the lanes' order]
 
     const QTile tile = tiles[blockIdx.x];
     const int G = H / KVH;
@@ -84,12 +84,19 @@ __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
     const int wave_pmax = tile.pos0 + wave_tok_hi;
 
     const int32_t* table = block_table + static_cast<size_t>(tile.seq) * table_stride;
-    const int page_shift = (page_size & (page_size - 1)) == 0 ? __ffs(page_size) - 1 : -1;
-    auto row_address = [&](int key) -> size_t {       // offset of key's row for kv head g, key clamped into the sequence
-        const int kc = min(key, kend - 1);
-        const int lp = page_shift >= 0 ? (kc >> page_shift) : kc / page_size;
-        const int off = page_shift >= 0 ? (kc & (page_size - 1)) : kc % page_size;
-        return ((static_cast<size_t>(table[lp]) * KVH + g) * page_size + off) * HD;
+    auto page_of = [&](int key) { return POW2 ? (key >> page_shift) : key / page_size; };
+    auto slot_of = [&](int key) { return POW2 ? (key & (page_size - 1)) : key % page_size; };
+    // The block table of the workgroup's keys is copied to LDS, a segment of TBL_MAX pages at a
+    // time (one segment, unless the key range is very long): an entry read from global memory
+    // inside the loop would have to be waited for before its rows can be asked for, and that
+    // wait, being in order, would drain every row load still in flight.
+    constexpr int TBL_MAX = 1024;
+    __shared__ int32_t tbl[TBL_MAX];
+    int key_lo = 0, key_hi = 0, lp0 = 0;              // keys of the current segment, and its first page
+    auto row_address = [&](int key) -> size_t {       // offset of key's row for kv head g, key clamped into the segment
+        const int kc = min(max(key, key_lo), key_hi);
+        const int page = tbl[page_of(kc) - lp0];
+        return ((static_cast<size_t>(max(page, 0)) * KVH + g) * page_size + slot_of(kc)) * HD;
     };
 
     // Q as the B operand: lane (row r, group kg) holds dims kk*32 + kg*8 .. +8
@@ -108,7 +115,10 @@ __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-    // staging of V: thread -> (key of the step, 8-dim chunk); HD/8 chunks a key
+    // Staging of V: a thread loads 8 dims of one key (16 bytes) and writes them to LDS transposed,
+    // at the column where the lanes of the second product expect that key: lane group kg reads
+    // the eight keys {t*16 + kg*4 + i} as one 16-byte row piece [kg*8 + t*4 + i].  A wavefront
+    // covers all 32 keys and two 8-dim chunks, which spreads its 2-byte writes over the banks.
     constexpr int CHUNKS = HD / 8;
     constexpr int V_ITEMS = KSTEP * CHUNKS;
     constexpr int V_PER_THREAD = (V_ITEMS + MA_THREADS - 1) / MA_THREADS;
@@ -116,17 +126,22 @@ __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
 #pragma unroll
         for (int i = 0; i < V_PER_THREAD; ++i) {
             const int item = tid + i * MA_THREADS;
-            if (item < V_ITEMS) {
-                const int key = ks + item / CHUNKS;
-                dst[i] = *reinterpret_cast<const uint4*>(vpool + row_address(key) + (item % CHUNKS) * 8);
-            }
+            if (item < V_ITEMS)
+                dst[i] = *reinterpret_cast<const uint4*>(vpool + row_address(ks + item % KSTEP) + (item / KSTEP) * 8);
         }
     };
     auto store_v = [&](int buf, const uint4 (&src)[V_PER_THREAD]) {
 #pragma unroll
         for (int i = 0; i < V_PER_THREAD; ++i) {
             const int item = tid + i * MA_THREADS;
-            if (item < V_ITEMS) *reinterpret_cast<uint4*>(&vs[buf][item / CHUNKS][(item % CHUNKS) * 8]) = src[i];
+            if (item < V_ITEMS) {
+                const int key = item % KSTEP, dim0 = (item / KSTEP) * 8;
+                const int col = ((key % 16) / 4) * 8 + (key / 16) * 4 + key % 4;
+                const uint32_t w[4] = {src[i].x, src[i].y, src[i].z, src[i].w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    vs[buf][dim0 + e][col] = static_cast<uint16_t>(e & 1 ? w[e / 2] >> 16 : w[e / 2] & 0xffffu);
+            }
         }
     };
     // K as the A operand: lane (key r of a 16-key half, group kg) holds dims kk*32 + kg*8 .. +8
@@ -145,101 +160,103 @@ __global__ __launch_bounds__(MA_THREADS) void mfma_attention_kernel(
     constexpr int DEPTH = 4;
     uint4 kf[DEPTH][2][KK];
     uint4 vr[DEPTH][V_PER_THREAD];
+    for (int seg0 = 0; seg0 < nsteps;) {
+        key_lo = kfirst + seg0 * KSTEP;
+        lp0 = page_of(key_lo);
+        const int seg_steps = min(nsteps - seg0, ((lp0 + TBL_MAX) * page_size - key_lo) / KSTEP);
+        key_hi = min(key_lo + seg_steps * KSTEP, kend) - 1;
+        __syncthreads();                   // nobody still reads the previous segment's table or V tiles
+        for (int i = tid; i <= page_of(key_hi) - lp0; i += MA_THREADS) tbl[i] = table[lp0 + i];
+        __syncthreads();
+        // rows past the end of the segment are read from its last key and not used: no load is under a branch
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-        if (d < nsteps) {
-            if (wave_ok) load_k(kfirst + d * KSTEP, kf[d]);
-            load_v(kfirst + d * KSTEP, vr[d]);
+        for (int d = 0; d < DEPTH; ++d) {
+            load_k(key_lo + d * KSTEP, kf[d]);
+            load_v(key_lo + d * KSTEP, vr[d]);
         }
-    }
-    if (nsteps > 0) store_v(0, vr[0]);
-    for (int s = 0; s < nsteps; ++s) {
-        const int ks = kfirst + s * KSTEP;
-        __syncthreads();                       // V of this step is in vs[s & 1]; nobody still reads the other buffer
-        const bool more = s + 1 < nsteps, ahead = s + DEPTH < nsteps;
-        uint4 k_new[2][KK], v_new[V_PER_THREAD];
-        if (ahead) {
-            if (wave_ok && ks + DEPTH * KSTEP <= wave_pmax) load_k(ks + DEPTH * KSTEP, k_new);   // only who will multiply them
+        store_v(0, vr[0]);
+        for (int s = 0; s < seg_steps; ++s) {
+            const int ks = key_lo + s * KSTEP;
+            // V of this step is in vs[s & 1]; nobody still reads the other buffer.  Only LDS is ordered
+            // here: a full barrier would also wait for every row load that is in flight for later steps.
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+            uint4 k_new[2][KK], v_new[V_PER_THREAD];
+            load_k(ks + DEPTH * KSTEP, k_new);
             load_v(ks + DEPTH * KSTEP, v_new);
-        }
-        if (wave_ok && ks <= wave_pmax) {
-            // S^T for the two 16-key halves
-            floatx4_t st[2];
+            if (wave_ok && ks <= wave_pmax) {
+                // S^T for the two 16-key halves
+                floatx4_t st[2];
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                st[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+                for (int t = 0; t < 2; ++t) {
+                    st[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk)
-                    st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[0][t][kk]),
-                                                                    __builtin_bit_cast(bf16x8_t, qf[kk]), st[t], 0, 0, 0);
-            }
-            // this lane: row r, keys ks + t*16 + kg*4 + i
-            float sc[8];
-            float mx = NEG_BIG;
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int key = ks + t * 16 + kg * 4 + i;
-                    const bool ok = row_ok && key <= pos && key >= row_lo;
-                    const float v = ok ? st[t][i] * scale : NEG_BIG;
-                    sc[t * 4 + i] = v;
-                    mx = fmaxf(mx, v);
+                    for (int kk = 0; kk < KK; ++kk)
+                        st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[0][t][kk]),
+                                                                        __builtin_bit_cast(bf16x8_t, qf[kk]), st[t], 0, 0, 0);
                 }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-            const float m_new = fmaxf(m_run, mx);
-            const float corr = __expf(m_run - m_new);
-            float psum = 0.f;
-            uint32_t pw[4];
+                // this lane: row r, keys ks + t*16 + kg*4 + i
+                float sc[8];
+                float mx = NEG_BIG;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float p0 = sc[2 * j] > 0.5f * NEG_BIG ? __expf(sc[2 * j] - m_new) : 0.f;
-                const float p1 = sc[2 * j + 1] > 0.5f * NEG_BIG ? __expf(sc[2 * j + 1] - m_new) : 0.f;
-                // the sum is taken over the rounded weights, the ones the second product uses: the
-                // output is then an exact convex combination of values, whatever the rounding
-                const uint32_t b0 = f32_to_bf16_bits(p0), b1 = f32_to_bf16_bits(p1);
-                psum += __uint_as_float(b0 << 16) + __uint_as_float(b1 << 16);
-                pw[j] = b0 | (b1 << 16);
-            }
-            l_run = l_run * corr + psum;
-            m_run = m_new;
-            const uint4 pf = make_uint4(pw[0], pw[1], pw[2], pw[3]);
-            // O^T += V^T . P^T : the A operand of lane (dim r of a 16-dim tile, group kg) is V[key_j][dim]
-            // for the same eight keys, in the same order, as the lane's scores
-            const uint16_t (*vb)[VROW] = vs[s & 1];
+                for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                uint32_t vw[4];
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = ks + t * 16 + kg * 4 + i;
+                        const bool ok = row_ok && key <= pos && key >= row_lo;
+                        const float v = ok ? st[t][i] * scale : NEG_BIG;
+                        sc[t * 4 + i] = v;
+                        mx = fmaxf(mx, v);
+                    }
+                mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+                const float m_new = fmaxf(m_run, mx);
+                const float corr = __expf(m_run - m_new);
+                float psum = 0.f;
+                uint32_t pw[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int j0 = 2 * j, j1 = 2 * j + 1;
-                    const int key0 = (j0 < 4 ? 0 : 16) + kg * 4 + (j0 & 3);
-                    const int key1 = (j1 < 4 ? 0 : 16) + kg * 4 + (j1 & 3);
-                    vw[j] = static_cast<uint32_t>(vb[key0][dt * 16 + r]) | (static_cast<uint32_t>(vb[key1][dt * 16 + r]) << 16);
+                    const float p0 = sc[2 * j] > 0.5f * NEG_BIG ? __expf(sc[2 * j] - m_new) : 0.f;
+                    const float p1 = sc[2 * j + 1] > 0.5f * NEG_BIG ? __expf(sc[2 * j + 1] - m_new) : 0.f;
+                    // the sum is taken over the rounded weights, the ones the second product uses: the
+                    // output is then an exact convex combination of values, whatever the rounding
+                    const uint32_t b0 = f32_to_bf16_bits(p0), b1 = f32_to_bf16_bits(p1);
+                    psum += __uint_as_float(b0 << 16) + __uint_as_float(b1 << 16);
+                    pw[j] = b0 | (b1 << 16);
                 }
-                const uint4 vf = make_uint4(vw[0], vw[1], vw[2], vw[3]);
-                o[dt] *= corr;
-                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vf),
-                                                                __builtin_bit_cast(bf16x8_t, pf), o[dt], 0, 0, 0);
-            }
-        }
-        if (more) store_v((s + 1) & 1, vr[1]);
+                l_run = l_run * corr + psum;
+                m_run = m_new;
+                const uint4 pf = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+                // O^T += V^T . P^T : the A operand of lane (dim r of a 16-dim tile, group kg) is V[key_j][dim]
+                // for the same eight keys, in the same order, as the lane's scores
+                const uint16_t (*vb)[VROW] = vs[s & 1];
 #pragma unroll
-        for (int d = 0; d + 1 < DEPTH; ++d) {
+                for (int dt = 0; dt < DT; ++dt) {
+                    const uint4 vf = *reinterpret_cast<const uint4*>(&vb[dt * 16 + r][kg * 8]);
+                    o[dt] *= corr;
+                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vf),
+                                                                    __builtin_bit_cast(bf16x8_t, pf), o[dt], 0, 0, 0);
+                }
+            }
+            store_v((s + 1) & 1, vr[1]);
+#pragma unroll
+            for (int d = 0; d + 1 < DEPTH; ++d) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int kk = 0; kk < KK; ++kk) kf[d][t][kk] = kf[d + 1][t][kk];
+#pragma unroll
+                for (int i = 0; i < V_PER_THREAD; ++i) vr[d][i] = vr[d + 1][i];
+            }
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) kf[d][t][kk] = kf[d + 1][t][kk];
+                for (int kk = 0; kk < KK; ++kk) kf[DEPTH - 1][t][kk] = k_new[t][kk];
 #pragma unroll
-            for (int i = 0; i < V_PER_THREAD; ++i) vr[d][i] = vr[d + 1][i];
+            for (int i = 0; i < V_PER_THREAD; ++i) vr[DEPTH - 1][i] = v_new[i];
         }
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int kk = 0; kk < KK; ++kk) kf[DEPTH - 1][t][kk] = k_new[t][kk];
-#pragma unroll
-        for (int i = 0; i < V_PER_THREAD; ++i) vr[DEPTH - 1][i] = v_new[i];
+        seg0 += seg_steps;
     }
 
     // the sum of a row is spread over the four lanes that share it
@@ -288,12 +305,19 @@ NI_EXPORT int ni_mfma_attention(const void* q, int q_stride, const void* kpool, 
     const int G = H / KVH;
     const int hpt = G >= 16 ? 16 : G > 4 ? 8 : G > 2 ? 4 : G > 1 ? 2 : 1;
     const int chunks = (G + hpt - 1) / hpt;
+    // a page size that is a power of two gets shifts and masks, any other divisions
+    const bool pow2 = (page_size & (page_size - 1)) == 0;
+    int page_shift = 0;
+    while (pow2 && (1 << page_shift) < page_size) ++page_shift;
     dim3 grid(n_tiles, KVH * chunks, nsplit);
-#define MA_LAUNCH(HPT_)                                                                                              \
-    mfma_attention_kernel<HPT_><<<grid, MA_THREADS, 0, stream>>>(                                                  \
-        (const bf16_t*)q, q_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table,        \
-        table_stride, (const QTile*)tiles, (bf16_t*)out, (float*)part_o, (float*)part_ml, H, KVH, page_size, window,  \
-        scale, nsplit)
+#define MA_LAUNCH(HPT_)                                                                                             \
+    {                                                                                                               \
+        auto kernel = pow2 ? mfma_attention_kernel<HPT_, true> : mfma_attention_kernel<HPT_, false>;               \
+        kernel<<<grid, MA_WAVES * WAVE, 0, stream>>>(                                                               \
+            (const bf16_t*)q, q_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table,   \
+            table_stride, (const QTile*)tiles, (bf16_t*)out, (float*)part_o, (float*)part_ml, H, KVH, page_size,   \
+            page_shift, window, scale, nsplit);                                                                     \
+    }
     switch (hpt) {
         case 1: MA_LAUNCH(1); break;
         case 2: MA_LAUNCH(2); break;

@@ -70,7 +70,7 @@ def library_path(name: str, sources: List[str], defines: Optional[Dict[str, obje
     for d in _lib_dirs():
         try:
             os.makedirs(d, exist_ok=True)
-            probe = os.path.join(d, f".w{os.getpid()}")
+            probe = os.path.join(d, f".w{os.getpid()}-{threading.get_ident()}")
             with open(probe, "w"):
                 pass
             os.remove(probe)
@@ -81,7 +81,7 @@ def library_path(name: str, sources: List[str], defines: Optional[Dict[str, obje
     if out_dir is None:
         raise BuildError(f"no writable folder for compiled kernels among {_lib_dirs()}")
     out = os.path.join(out_dir, fname)
-    tmp = out + f".tmp{os.getpid()}"
+    tmp = out + f".tmp{os.getpid()}-{threading.get_ident()}"
     cmd = [find_hipcc()] + FLAGS + [f"-D{k}={v}" for k, v in sorted(defines.items())] + \
           [f"-I{HERE}"] + [os.path.join(HERE, s) for s in sources] + ["-o", tmp]
     env = dict(os.environ)

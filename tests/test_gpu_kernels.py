@@ -250,6 +250,22 @@ def test_attention_finds_a_far_key_among_hundreds(K, dtype):
             assert float((got - expect).abs().max()) < 0.05, key_at     # the one key took all the weight
 
 
+@pytest.mark.parametrize("kernel", ["token", "mfma"])
+def test_attention_block_table_longer_than_one_segment(K, kernel):
+    """The kernels keep 1,024 entries of a block table in LDS at a time.  With pages of one or
+    three slots a range of 2,500 keys needs several such segments; a boosted key is placed in the
+    first, at the seam and in the last, so that a segment read through the wrong entries shows."""
+    n = 2500
+    for ps, key_at in ((1, 5), (1, 1023), (1, 1024), (1, 2499), (3, 3071 % n), (3, 1)):
+        out, want, (qs, ks, vs) = paged_case(K, "bfloat16", 4, 2, 64, ps, [n, 40], [3, 2], None, ps + key_at, 1,
+                                             boost=(0, key_at, n - 1, 6.0), kernel=kernel)
+        assert not torch.isnan(out).any()
+        assert rel(out, want) < KTOL["bfloat16"], (ps, key_at)
+        got = out.double().cpu()[2].reshape(4, 64)
+        expect = vs[0][key_at].double().repeat_interleave(2, 0)
+        assert float((got - expect).abs().max()) < 0.05, (ps, key_at)
+
+
 # ---- the matrix-core kernel for prompt portions (bfloat16)
 
 @pytest.mark.parametrize("H,KVH,hd,ps", [(4, 2, 32, 8), (6, 1, 32, 8), (32, 8, 64, 16), (16, 2, 128, 16), (2, 2, 256, 16),
