@@ -2,7 +2,9 @@
 // Compiled once per head size (-DHEAD_DIM=n, a multiple of 16 up to 256).
 //
 // A work item is (query token, kv head, chunk of the query heads that share it, split of the
-// key range).  The 256 threads of a workgroup are arranged as key slots x dimension lanes:
+// key range).  The threads of a workgroup (256, or 512 when there are few work items: then one
+// workgroup walks a whole key range with eight wavefronts and no second kernel has to merge
+// splits) are arranged as key slots x dimension lanes:
 // LPK consecutive lanes hold one key row between them (EPL dims each), so a wavefront reads
 // 64/LPK whole rows per access, which are adjacent in a pool laid out
 // [page, kv_head, slot_in_page, head_dim].  Every lane group keeps a running (max, sum, output)
@@ -26,7 +28,8 @@
 #endif
 static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256, "head size: multiple of 16, at most 256");
 
-#define ATT_THREADS 256
+#define ATT_THREADS 256        // threads of a workgroup, narrow form
+#define ATT_THREADS_WIDE 512   // wide form
 #define GT 4  // query heads handled together by one workgroup
 
 template <typename T> struct Lanes {
@@ -35,7 +38,6 @@ template <typename T> struct Lanes {
     static constexpr int LPK = want <= 1 ? 1 : want <= 2 ? 2 : want <= 4 ? 4 : want <= 8 ? 8 : 16;
     static constexpr int EPL = HEAD_DIM / LPK;
     static_assert(LPK * EPL == HEAD_DIM, "lanes x elements must cover a head");
-    static constexpr int KPI = ATT_THREADS / LPK;  // keys per workgroup iteration
 };
 
 // "minus infinity" that stays finite under subtraction: exp(NEG - x) is 0, never NaN
@@ -46,15 +48,16 @@ template <bool FAST> __device__ __forceinline__ float ex(float x) {
     else return expf(x);
 }
 
-template <typename T, bool POW2>
-__global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
+template <typename T, bool POW2, int THREADS>
+__global__ __launch_bounds__(THREADS) void token_attention_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ kpool, const T* __restrict__ vpool,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ positions, T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     int H, int KVH, int page_size, int page_shift, int window, float scale, int nsplit) {
     using L = Lanes<T>;
-    constexpr int LPK = L::LPK, EPL = L::EPL, KPI = L::KPI, HD = HEAD_DIM;
-    constexpr int WAVES = ATT_THREADS / WAVE;
+    constexpr int LPK = L::LPK, EPL = L::EPL, HD = HEAD_DIM;
+    constexpr int KPI = THREADS / LPK;           // keys per workgroup iteration
+    constexpr int WAVES = THREADS / WAVE;
     constexpr bool FAST = sizeof(T) == 2;
 
     const int t = blockIdx.x;
@@ -175,7 +178,7 @@ __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
         lp0 = page_of(s0);
         s1 = min(k1, (lp0 + TBL_MAX) * page_size);
         __syncthreads();               // nobody still reads the previous segment's entries
-        for (int i = tid; i <= page_of(s1 - 1) - lp0; i += ATT_THREADS) tbl[i] = table[lp0 + i];
+        for (int i = tid; i <= page_of(s1 - 1) - lp0; i += THREADS) tbl[i] = table[lp0 + i];
         __syncthreads();
         const int iters = (s1 - s0 + KPI - 1) / KPI;
 
@@ -232,7 +235,7 @@ __global__ __launch_bounds__(ATT_THREADS) void token_attention_kernel(
     }
     __syncthreads();
 
-    for (int idx = tid; idx < gc * HD; idx += ATT_THREADS) {
+    for (int idx = tid; idx < gc * HD; idx += THREADS) {
         const int i = idx / HD;
         const int dim = idx % HD;
         float M = sm_m[0][i];
@@ -281,7 +284,7 @@ template <typename T>
 static int launch(const void* q, int q_stride, const void* kpool, const void* vpool, const void* block_table,
                   int table_stride, const void* seq_of_token, const void* positions, void* out, void* part_o,
                   void* part_ml, int T_tokens, int H, int KVH, int page_size, int window, float scale,
-                  int nsplit, hipStream_t stream) {
+                  int nsplit, bool wide, hipStream_t stream) {
     const int G = H / KVH;
     const int chunks = (G + GT - 1) / GT;
     dim3 grid(T_tokens, KVH * chunks, nsplit);
@@ -289,11 +292,18 @@ static int launch(const void* q, int q_stride, const void* kpool, const void* vp
     const bool pow2 = (page_size & (page_size - 1)) == 0;
     int page_shift = 0;
     while (pow2 && (1 << page_shift) < page_size) ++page_shift;
-    auto kernel = pow2 ? token_attention_kernel<T, true> : token_attention_kernel<T, false>;
-    kernel<<<grid, ATT_THREADS, 0, stream>>>(
-        (const T*)q, q_stride, (const T*)kpool, (const T*)vpool, (const int32_t*)block_table, table_stride,
-        (const int32_t*)seq_of_token, (const int32_t*)positions, (T*)out, (float*)part_o, (float*)part_ml,
-        H, KVH, page_size, page_shift, window, scale, nsplit);
+#define TA_ARGS                                                                                                    \
+    (const T*)q, q_stride, (const T*)kpool, (const T*)vpool, (const int32_t*)block_table, table_stride,            \
+        (const int32_t*)seq_of_token, (const int32_t*)positions, (T*)out, (float*)part_o, (float*)part_ml, H, KVH, \
+        page_size, page_shift, window, scale, nsplit
+    if (wide) {
+        auto kernel = pow2 ? token_attention_kernel<T, true, ATT_THREADS_WIDE> : token_attention_kernel<T, false, ATT_THREADS_WIDE>;
+        kernel<<<grid, ATT_THREADS_WIDE, 0, stream>>>(TA_ARGS);
+    } else {
+        auto kernel = pow2 ? token_attention_kernel<T, true, ATT_THREADS> : token_attention_kernel<T, false, ATT_THREADS>;
+        kernel<<<grid, ATT_THREADS, 0, stream>>>(TA_ARGS);
+    }
+#undef TA_ARGS
     int err = NI_LAUNCH_RESULT();
     if (err || nsplit == 1) return err;
     merge_splits_kernel<T><<<dim3(T_tokens, H), 64, 0, stream>>>((const float*)part_o, (const float*)part_ml, (T*)out,
@@ -305,19 +315,20 @@ NI_EXPORT int ni_attention_head_dim() { return HEAD_DIM; }
 NI_EXPORT int ni_attention_heads_per_group() { return GT; }
 
 // part_o: float [T, H, nsplit, HEAD_DIM], part_ml: float [T, H, nsplit, 2]; unused when nsplit == 1.
+// wide != 0 asks for workgroups of 512 threads instead of 256.
 NI_EXPORT int ni_token_attention(const void* q, int q_stride, const void* kpool, const void* vpool,
                                  const void* block_table, int table_stride, const void* seq_of_token,
                                  const void* positions, void* out, void* part_o, void* part_ml,
                                  int T_tokens, int H, int KVH, int page_size, int window, float scale, int nsplit,
-                                 int dtype, hipStream_t stream) {
+                                 int wide, int dtype, hipStream_t stream) {
     if (T_tokens <= 0) return 0;
     if (H % KVH != 0 || nsplit < 1 || nsplit > 65535 || page_size < 1) return -1;
     if (nsplit > 1 && (!part_o || !part_ml)) return -2;
     if (dtype == 0)
         return launch<float>(q, q_stride, kpool, vpool, block_table, table_stride, seq_of_token, positions, out,
-                             part_o, part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, stream);
+                             part_o, part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, wide != 0, stream);
     return launch<bf16_t>(q, q_stride, kpool, vpool, block_table, table_stride, seq_of_token, positions, out, part_o,
-                          part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, stream);
+                          part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, wide != 0, stream);
 }
 
 // Merge of partial results in the layout above, for kernels of other libraries that split the keys.

@@ -23,6 +23,14 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
     return static_cast<uint16_t>(u >> 16);
 }
 
+// Two floats to two bfloat16 in one word (first argument in the low half) by the hardware's
+// conversion, which rounds to nearest even like the routine above.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    typedef __bf16 bf16x2_hw __attribute__((ext_vector_type(2)));
+    typedef float floatx2_hw __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2_hw{lo, hi}, bf16x2_hw));
+}
+
 template <typename T> struct Elem;
 template <> struct Elem<float> {
     static __device__ __forceinline__ float load(const float* p) { return *p; }

@@ -198,16 +198,7 @@ def choose_splits(n_tokens: int, kv_heads: int, group: int, max_keys: int) -> in
     return int(max(1, min(want, (max_keys + 255) // 256, 64)))
 
 
-def token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
-                    seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, H: int, KVH: int,
-                    hd: int, scale: float, window: Optional[int], nsplit: int,
-                    workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Attention of every token of ``qkv`` over the paged cache of its sequence.
-
-    ``qkv`` is [T, >= H*hd] with the (rotated) query heads first; the pools already hold the keys
-    and values of all positions up to each token's own.  ``workspace`` (float32, at least
-    ``T*H*nsplit*(hd+2)`` elements) is needed when ``nsplit > 1``.
-    """
+def _token_attention_checks(qkv, kpool, vpool, block_table, seq_of_token, positions, out, H, KVH, hd, nsplit, workspace):
     T = qkv.shape[0]
     _gpu(qkv, "qkv")
     _need(qkv.shape[1] >= H * hd, "qkv is narrower than the query heads")
@@ -230,12 +221,58 @@ def token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
         flat = workspace.view(-1)
         part_o = flat[: T * H * nsplit * hd]
         part_ml = flat[T * H * nsplit * hd: need]
+    return T, part_o, part_ml
+
+
+def token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
+                    seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, H: int, KVH: int,
+                    hd: int, scale: float, window: Optional[int], nsplit: int,
+                    workspace: Optional[torch.Tensor] = None, wide: bool = False) -> torch.Tensor:
+    """Attention of every token of ``qkv`` over the paged cache of its sequence.
+
+    ``qkv`` is [T, >= H*hd] with the (rotated) query heads first; the pools already hold the keys
+    and values of all positions up to each token's own.  ``workspace`` (float32, at least
+    ``T*H*nsplit*(hd+2)`` elements) is needed when ``nsplit > 1``.  ``wide`` asks for workgroups
+    of 512 threads instead of 256.
+    """
+    T, part_o, part_ml = _token_attention_checks(qkv, kpool, vpool, block_table, seq_of_token, positions, out,
+                                                 H, KVH, hd, nsplit, workspace)
     lib = attention_lib(hd)
     _check(lib.ni_token_attention(_ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table),
                                   block_table.shape[1], _ptr(seq_of_token), _ptr(positions), _ptr(out),
                                   _ptr(part_o), _ptr(part_ml), T, H, KVH, kpool.shape[2],
-                                  int(window) if window else 0, ctypes.c_float(scale), nsplit,
+                                  int(window) if window else 0, ctypes.c_float(scale), nsplit, int(bool(wide)),
                                   dtype_code(qkv.dtype), _stream()), "token_attention")
+    return out
+
+
+def mfma_token_splits(n_tokens: int, kv_heads: int, group: int, max_keys: int) -> int:
+    """Into how many runs the matrix-core kernel for single tokens cuts every key range: enough
+    for about one workgroup per compute unit, a run never shorter than 256 keys (measured at
+    batches 1 to 64 and contexts of 2,100 and 8,200 keys)."""
+    items = max(1, n_tokens * kv_heads * ((group + 15) // 16))
+    return int(max(1, min(256 // items, max_keys // 256, 64)))
+
+
+def mfma_token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
+                         seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, H: int, KVH: int,
+                         hd: int, scale: float, window: Optional[int], nsplit: int,
+                         workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """:func:`token_attention` on the matrix cores (bfloat16, head sizes that :func:`mfma_attention_ok`
+    takes): the query heads of a kv head are the rows of the products, the wavefronts of a
+    workgroup share out the keys."""
+    _need(mfma_attention_ok(qkv.dtype, hd), f"mfma_token_attention does not take {qkv.dtype} with head size {hd}")
+    _need(qkv.shape[1] % 8 == 0, "rows of qkv are not aligned to 16 bytes")
+    T, part_o, part_ml = _token_attention_checks(qkv, kpool, vpool, block_table, seq_of_token, positions, out,
+                                                 H, KVH, hd, nsplit, workspace)
+    _need(kpool.numel() // hd < 2 ** 32, "the matrix-core attention kernels number the rows of a pool in 32 bits")
+    _check(attention_mfma_lib(hd).ni_mfma_token_attention(
+        _ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table), block_table.shape[1],
+        _ptr(seq_of_token), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), T, H, KVH, kpool.shape[2],
+        int(window) if window else 0, ctypes.c_float(scale), nsplit, _stream()), "mfma_token_attention")
+    if nsplit > 1:
+        _check(attention_lib(hd).ni_merge_splits(_ptr(part_o), _ptr(part_ml), _ptr(out), T, H, nsplit,
+                                                 dtype_code(out.dtype), _stream()), "merge_splits")
     return out
 
 
@@ -283,6 +320,7 @@ def mfma_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
     _gpu(vpool, "vpool", torch.bfloat16, kpool.shape)
     _need(kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd,
           f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
+    _need(kpool.numel() // hd < 2 ** 32, "the matrix-core attention kernels number the rows of a pool in 32 bits")
     _gpu(block_table, "block_table", torch.int32)
     _gpu(tiles, "tiles", torch.int32)
     _need(tiles.dim() == 2 and tiles.shape[1] == 4, "tiles must be [n, 4]")

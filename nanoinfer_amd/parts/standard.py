@@ -206,11 +206,15 @@ class Attention(Part):
             K.mfma_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, out, self.H, self.KVH, self.hd,
                              self.scale, self.window, nsplit, ws)
             return K.linear(out, self.w_o)
+        # single tokens and short portions, token by token
         max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window)
-        nsplit = K.choose_splits(T, self.KVH, self.H // self.KVH, max_keys)
+        on_matrix_cores = K.mfma_attention_ok(x.dtype, self.hd)
+        choose = K.mfma_token_splits if on_matrix_cores else K.choose_splits
+        nsplit = choose(T, self.KVH, self.H // self.KVH, max_keys)
         ws = ctx.workspace(T * self.H * nsplit * (self.hd + 2)) if nsplit > 1 else None
-        K.token_attention(qkv, cache.kpool, cache.vpool, cache.block_table, ctx.seq_of_token, ctx.positions, out,
-                          self.H, self.KVH, self.hd, self.scale, self.window, nsplit, ws)
+        attend = K.mfma_token_attention if on_matrix_cores else K.token_attention
+        attend(qkv, cache.kpool, cache.vpool, cache.block_table, ctx.seq_of_token, ctx.positions, out,
+               self.H, self.KVH, self.hd, self.scale, self.window, nsplit, ws)
         return K.linear(out, self.w_o)
 
 

@@ -1,5 +1,6 @@
 """Each HIP kernel alone against its plain reference, at sizes other than the engine's tests use:
 widths and vocabularies that are no power of two, head sizes in steps of 16, odd page sizes."""
+import functools
 import math
 import random
 
@@ -206,9 +207,11 @@ def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boo
         K.mfma_attention(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table), tiles, out,
                          H, KVH, hd, 1.0 / math.sqrt(hd), window, nsplit, ws)
     else:
-            K.token_attention(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table),
-                          dev(torch.tensor(seq_of, dtype=torch.int32)), dev(torch.tensor(positions, dtype=torch.int32)),
-                          out, H, KVH, hd, 1.0 / math.sqrt(hd), window, nsplit, ws)
+        fn = {"token": K.token_attention, "token_wide": functools.partial(K.token_attention, wide=True),
+              "mfma_token": K.mfma_token_attention}[kernel]
+        fn(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table),
+           dev(torch.tensor(seq_of, dtype=torch.int32)), dev(torch.tensor(positions, dtype=torch.int32)),
+           out, H, KVH, hd, 1.0 / math.sqrt(hd), window, nsplit, ws)
     want = torch.cat([P.causal_attention(qs[b], ks[b], vs[b], range(n), window=window)[n - q_lens[b]:].reshape(q_lens[b], H * hd)
                       for b, n in enumerate(lens)])
     return out, want, (qs, ks, vs)
@@ -219,10 +222,10 @@ def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boo
                                          (8, 2, 96, 4), (2, 1, 112, 16), (16, 2, 128, 16), (2, 2, 256, 16)])
 def test_attention_head_sizes_and_groups(K, dtype, H, KVH, hd, ps):
     lens, q_lens = [1, 37, 130, 64], [1, 37, 2, 1]
-    for nsplit in (1, 3):
-        out, want, _ = paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, None, hd + nsplit, nsplit)
+    for nsplit, kernel in ((1, "token"), (3, "token"), (1, "token_wide"), (2, "token_wide")):
+        out, want, _ = paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, None, hd + nsplit, nsplit, kernel=kernel)
         assert not torch.isnan(out).any(), "a key outside the sequence's own pages was read"
-        assert rel(out, want) < KTOL[dtype], (H, KVH, hd, ps, nsplit)
+        assert rel(out, want) < KTOL[dtype], (H, KVH, hd, ps, nsplit, kernel)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -250,7 +253,7 @@ def test_attention_finds_a_far_key_among_hundreds(K, dtype):
             assert float((got - expect).abs().max()) < 0.05, key_at     # the one key took all the weight
 
 
-@pytest.mark.parametrize("kernel", ["token", "mfma"])
+@pytest.mark.parametrize("kernel", ["token", "mfma", "mfma_token"])
 def test_attention_block_table_longer_than_one_segment(K, kernel):
     """The kernels keep 1,024 entries of a block table in LDS at a time.  With pages of one or
     three slots a range of 2,500 keys needs several such segments; a boosted key is placed in the
@@ -277,6 +280,31 @@ def test_mfma_attention_head_sizes_and_groups(K, H, KVH, hd, ps):
         out, want, _ = paged_case(K, "bfloat16", H, KVH, hd, ps, lens, q_lens, None, hd + H, nsplit, kernel="mfma")
         assert not torch.isnan(out).any(), "a key outside the sequence's own pages took part"
         assert rel(out, want) < KTOL["bfloat16"], (H, KVH, hd, ps, nsplit)
+
+
+@pytest.mark.parametrize("H,KVH,hd,ps", [(4, 2, 32, 8), (6, 1, 32, 8), (32, 8, 64, 16), (16, 2, 128, 16), (2, 2, 256, 16),
+                                         (3, 3, 96, 4), (40, 2, 64, 16), (5, 5, 64, 5), (12, 4, 160, 16)])
+def test_mfma_token_attention_head_sizes_and_groups(K, H, KVH, hd, ps):
+    # the kernel for single tokens: rows are the query heads of a kv head (20 of them: two chunks of 16)
+    lens, q_lens = [1, 37, 130, 64, 300, 33], [1, 37, 2, 1, 3, 1]
+    for nsplit in (1, 3):
+        out, want, _ = paged_case(K, "bfloat16", H, KVH, hd, ps, lens, q_lens, None, hd + H, nsplit, kernel="mfma_token")
+        assert not torch.isnan(out).any(), "a key outside the sequence's own pages took part"
+        assert rel(out, want) < KTOL["bfloat16"], (H, KVH, hd, ps, nsplit)
+
+
+def test_mfma_token_attention_window_and_far_key(K):
+    for window in (1, 7, 16, 33, 100):
+        out, want, _ = paged_case(K, "bfloat16", 4, 2, 32, 8, [150, 9, 33], [150, 9, 2], window, window, 1, kernel="mfma_token")
+        assert not torch.isnan(out).any()
+        assert rel(out, want) < KTOL["bfloat16"], window
+    for key_at in (37, 16, 15, 0, 31, 32, 127, 128, 698):
+        out, want, (qs, ks, vs) = paged_case(K, "bfloat16", 8, 2, 64, 16, [700], [1], None, 9, 1 + key_at % 4,
+                                             boost=(0, key_at, 699, 6.0), kernel="mfma_token")
+        assert rel(out, want) < KTOL["bfloat16"]
+        got = out.double().cpu()[-1].reshape(8, 64)
+        expect = vs[0][key_at].double().repeat_interleave(4, 0)
+        assert float((got - expect).abs().max()) < 0.05, key_at
 
 
 def test_mfma_attention_window_and_far_key(K):
