@@ -21,6 +21,16 @@
 // rotation + cache write for a stacked [q; k; v] matrix: a workgroup owns the two tiles of one
 // head that hold the partners (j, j + hd/2) of a rotation, turns them by the angle of the row's
 // position, and stores query heads to a buffer, key and value heads straight into their pages.
+// or addition into the float32 residual stream (h[m, n] += the product, in place: a workgroup
+// reads and writes only its own columns).
+//
+// A second kernel serves the decode step proper: at most 16 rows and re-tiled weights.  It keeps two
+// trips in registers (one multiplied while the other's loads are under way), and can take, instead
+// of x, the float32 residual stream h [M, K] with the weights and eps of an RMSNorm: every
+// workgroup then normalises the rows itself (sums of squares over the wavefronts' K slices, met in
+// LDS) while its first pieces of W are already on their way, and keeps the normalised operand in
+// registers (K up to XP * 8 pieces).  With that prologue and the residual epilogue a block of a
+// decoder needs no kernel of its own for the residual sum or the norm.
 // float32 inputs are multiplied in true float32 (no reduced-precision MFMA).
 #include <type_traits>
 
@@ -41,6 +51,10 @@ template <> struct Piece<bf16_t> {
         hi = reinterpret_cast<const uint4*>(p)[1];
     }
     __device__ __forceinline__ void zero() { lo = make_uint4(0, 0, 0, 0); hi = lo; }
+    __device__ __forceinline__ void from_floats(const float (&f)[16]) {
+        lo = make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7]));
+        hi = make_uint4(pack_bf16x2(f[8], f[9]), pack_bf16x2(f[10], f[11]), pack_bf16x2(f[12], f[13]), pack_bf16x2(f[14], f[15]));
+    }
     static __device__ __forceinline__ floatx4_t mma(const Piece& a, const Piece& b, floatx4_t c) {
         c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a.lo), __builtin_bit_cast(bf16x8_t, b.lo), c, 0, 0, 0);
         c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a.hi), __builtin_bit_cast(bf16x8_t, b.hi), c, 0, 0, 0);
@@ -58,6 +72,10 @@ template <> struct Piece<float> {
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[i] = 0.f;
     }
+    __device__ __forceinline__ void from_floats(const float (&f)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = f[i];
+    }
     static __device__ __forceinline__ floatx4_t mma(const Piece& a, const Piece& b, floatx4_t c) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[i], b.v[i], c, 0, 0, 0);
@@ -65,7 +83,14 @@ template <> struct Piece<float> {
     }
 };
 
-enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_ROPE = 2 };
+enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_ROPE = 2, EPI_RESIDUAL = 3 };
+
+// The normalising prologue's inputs.
+struct NormArgs {
+    const float* h;        // [M, K] residual stream
+    const float* weight;   // [K]
+    float eps;
+};
 
 // What the rotation epilogue needs beside the product.
 struct RopeArgs {
@@ -78,81 +103,14 @@ struct RopeArgs {
     int H, KVH, hd, page_size;
 };
 
-template <typename T, typename TOUT, int MB, int NT, int EPI, bool TILED>
-__global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __restrict__ x, const T* __restrict__ W,
-                                                                 TOUT* __restrict__ y, int M, int N, int K, int I,
-                                                                 RopeArgs rope) {
-    constexpr int EL = Piece<T>::ELEMS;
-    constexpr int CH = 4 * EL;                       // k elements in a 128-byte piece of a row
+// What follows the main loop of both kernels: the wavefronts' partial sums meet in LDS and the
+// epilogue stores them.
+template <typename T, typename TOUT, int MB, int NT, int EPI>
+__device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TOUT* __restrict__ y, int M, int N, int I,
+                                              const RopeArgs& rope) {
     const int tid = threadIdx.x;
     const int wave = tid / WAVE, lane = tid % WAVE;
-    const int r = lane % 16, kg = lane / 16;
     const int wg = blockIdx.x;
-
-    // weight row that this lane reads in each tile; tiles may hang over the edge of the matrix, then
-    // the row index is clamped (never read past W) and the result is not stored
-    const int n_limit = (EPI == EPI_SWIGLU) ? I : N;
-    const T* wrow[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        int col0 = (EPI == EPI_SWIGLU) ? (wg * (NT / 2) + nt / 2) * 16 : (wg * NT + nt) * 16;
-        if (EPI == EPI_ROPE) {      // workgroup = (head, pair of tiles): dims [16 p, 16 p + 16) and the same + hd/2
-            const int per_head = rope.hd / 32;
-            col0 = (wg / per_head) * rope.hd + (wg % per_head) * 16 + nt * (rope.hd / 2);
-        }
-        const int shift = (EPI == EPI_SWIGLU && (nt % 2)) ? I : 0;      // odd tiles of a pair come from the up rows
-        if (TILED)      // first byte of this lane in piece 0 of the tile; the buffer is padded, nothing to clamp
-            wrow[nt] = W + static_cast<size_t>((col0 + shift) / 16) * ((K + CH - 1) / CH) * (WAVE * EL) + lane * EL;
-        else
-            wrow[nt] = W + static_cast<size_t>(min(col0 + r, n_limit - 1) + shift) * K;
-    }
-    const T* xrow[MB];
-    bool xok[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-        const int m = mb * 16 + r;
-        xok[mb] = m < M;
-        xrow[mb] = x + static_cast<size_t>(min(m, M - 1)) * K;
-    }
-
-    floatx4_t acc[NT][MB];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-
-    // PT pieces per trip, all their loads issued before the first multiply, to keep enough bytes in
-    // flight; the wavefront covers pieces [first + wave * per_wave, ...) of its K range in order.
-    constexpr int PT = (NT * MB <= 2) ? 4 : 2;
-    const int pieces = (K + CH - 1) / CH;
-    for (int c = wave; c < pieces; c += PT * GV_WAVES) {
-        Piece<T> xb[PT][MB], wa[PT][NT];
-#pragma unroll
-        for (int u = 0; u < PT; ++u) {
-            const int piece = c + u * GV_WAVES;
-            const int k = piece * CH + kg * EL;
-            const bool kok = k < K;                  // K is a multiple of EL: a lane's 32 bytes are all in or all out
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                if (TILED) {
-                    if (piece < pieces) wa[u][nt].load(wrow[nt] + static_cast<size_t>(piece) * (WAVE * EL)); else wa[u][nt].zero();
-                } else {
-                    if (kok) wa[u][nt].load(wrow[nt] + k); else wa[u][nt].zero();
-                }
-            }
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb) {
-                if (kok && xok[mb]) xb[u][mb].load(xrow[mb] + k); else xb[u][mb].zero();
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < PT; ++u)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = Piece<T>::mma(wa[u][nt], xb[u][mb], acc[nt][mb]);
-    }
-
     // partial sums of the wavefronts meet in LDS: red[wave][tile][lane * 4 + i]
     __shared__ float red[GV_WAVES][NT * MB][WAVE * 4];
 #pragma unroll
@@ -234,8 +192,220 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
 #pragma unroll
             for (int w = 0; w < GV_WAVES; ++w) v += red[w][ot * MB + mb][src];
         }
-        st(y + static_cast<size_t>(m) * out_width + n, v);
+        TOUT* dst = y + static_cast<size_t>(m) * out_width + n;
+        if constexpr (EPI == EPI_RESIDUAL) *dst += v;      // float32 residual stream, this workgroup's own columns
+        else st(dst, v);
     }
+}
+
+template <typename T, typename TOUT, int MB, int NT, int EPI, bool TILED>
+__global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __restrict__ x, const T* __restrict__ W,
+                                                                 TOUT* __restrict__ y, int M, int N, int K, int I,
+                                                                 RopeArgs rope) {
+    constexpr int EL = Piece<T>::ELEMS;
+    constexpr int CH = 4 * EL;                       // k elements in a 128-byte piece of a row
+    const int tid = threadIdx.x;
+    const int wave = tid / WAVE, lane = tid % WAVE;
+    const int r = lane % 16, kg = lane / 16;
+    const int wg = blockIdx.x;
+
+    // weight row that this lane reads in each tile; tiles may hang over the edge of the matrix, then
+    // the row index is clamped (never read past W) and the result is not stored
+    const int n_limit = (EPI == EPI_SWIGLU) ? I : N;
+    const T* wrow[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        int col0 = (EPI == EPI_SWIGLU) ? (wg * (NT / 2) + nt / 2) * 16 : (wg * NT + nt) * 16;
+        if (EPI == EPI_ROPE) {      // workgroup = (head, pair of tiles): dims [16 p, 16 p + 16) and the same + hd/2
+            const int per_head = rope.hd / 32;
+            col0 = (wg / per_head) * rope.hd + (wg % per_head) * 16 + nt * (rope.hd / 2);
+        }
+        const int shift = (EPI == EPI_SWIGLU && (nt % 2)) ? I : 0;      // odd tiles of a pair come from the up rows
+        if (TILED)      // first byte of this lane in piece 0 of the tile; a tile past the matrix reads the last one and stores nothing
+            wrow[nt] = W + static_cast<size_t>(min((col0 + shift) / 16, (N + 15) / 16 - 1)) * ((K + CH - 1) / CH) * (WAVE * EL) + lane * EL;
+        else
+            wrow[nt] = W + static_cast<size_t>(min(col0 + r, n_limit - 1) + shift) * K;
+    }
+    const T* xrow[MB];
+    bool xok[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = mb * 16 + r;
+        xok[mb] = m < M;
+        xrow[mb] = x + static_cast<size_t>(min(m, M - 1)) * K;
+    }
+
+    floatx4_t acc[NT][MB];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    // PT pieces per trip, all their loads issued before the first multiply, to keep enough bytes in
+    // flight; the wavefront covers pieces [first + wave * per_wave, ...) of its K range in order.
+    constexpr int PT = (NT * MB <= 2) ? 4 : 2;
+    const int pieces = (K + CH - 1) / CH;
+    for (int c = wave; c < pieces; c += PT * GV_WAVES) {
+        Piece<T> xb[PT][MB], wa[PT][NT];
+#pragma unroll
+        for (int u = 0; u < PT; ++u) {
+            const int piece = c + u * GV_WAVES;
+            const int k = piece * CH + kg * EL;
+            const bool kok = k < K;                  // K is a multiple of EL: a lane's 32 bytes are all in or all out
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                if (TILED) {
+                    if (piece < pieces) wa[u][nt].load(wrow[nt] + static_cast<size_t>(piece) * (WAVE * EL)); else wa[u][nt].zero();
+                } else {
+                    if (kok) wa[u][nt].load(wrow[nt] + k); else wa[u][nt].zero();
+                }
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                if (kok && xok[mb]) xb[u][mb].load(xrow[mb] + k); else xb[u][mb].zero();
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < PT; ++u)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = Piece<T>::mma(wa[u][nt], xb[u][mb], acc[nt][mb]);
+    }
+
+    skinny_finish<T, TOUT, MB, NT, EPI>(acc, y, M, N, I, rope);
+}
+
+// The decode step's kernel: at most 16 rows, W re-tiled (and zero-padded to whole pieces, so a lane
+// past the end of a row multiplies by zero whatever it read of x).  XP == 0: x is given.
+// XP > 0: x = RMSNorm(h) with the wavefront's XP pieces of the normalised row kept in registers.
+template <typename T, typename TOUT, int NT, int EPI, int XP>
+__global__ __launch_bounds__(GV_THREADS) void skinny_decode_kernel(const T* __restrict__ x, const T* __restrict__ W,
+                                                                   TOUT* __restrict__ y, int M, int N, int K, int I,
+                                                                   RopeArgs rope, NormArgs norm) {
+    constexpr int EL = Piece<T>::ELEMS;
+    constexpr int CH = 4 * EL;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;      // the same in every lane: say so
+    const int r = lane % 16, kg = lane / 16;
+    const int wg = blockIdx.x;
+    const int pieces = (K + CH - 1) / CH;
+
+    const T* wrow[NT];      // first byte of this lane in piece 0 of each tile
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        int col0 = (EPI == EPI_SWIGLU) ? (wg * (NT / 2) + nt / 2) * 16 : (wg * NT + nt) * 16;
+        if (EPI == EPI_ROPE) {
+            const int per_head = rope.hd / 32;
+            col0 = (wg / per_head) * rope.hd + (wg % per_head) * 16 + nt * (rope.hd / 2);
+        }
+        const int shift = (EPI == EPI_SWIGLU && (nt % 2)) ? I : 0;
+        const int limit = (N + 15) / 16 - 1;         // a workgroup's last tiles may lie past the matrix: read the last one, store nothing
+        wrow[nt] = W + static_cast<size_t>(min((col0 + shift) / 16, limit)) * pieces * (WAVE * EL) + lane * EL;
+    }
+
+    floatx4_t acc[NT][1];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[nt][0] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    // PT pieces per trip; trip t of a wavefront covers pieces wave + (t * PT + u) * 8.  Two trips are
+    // in registers at a time, in two fixed sets (A and B): one is multiplied while the other's loads
+    // are under way.
+    constexpr int PT = NT <= 2 ? 4 : 2;
+    constexpr int STRIDE = PT * GV_WAVES;
+    auto load_w = [&](int c, Piece<T> (&wa)[PT][NT]) {
+#pragma unroll
+        for (int u = 0; u < PT; ++u) {
+            const int piece = min(c + u * GV_WAVES, pieces - 1);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) wa[u][nt].load(wrow[nt] + static_cast<size_t>(piece) * (WAVE * EL));
+        }
+    };
+    auto multiply = [&](int c, const Piece<T> (&wa)[PT][NT], const Piece<T> (&xb)[PT][1]) {
+#pragma unroll
+        for (int u = 0; u < PT; ++u) {
+            if (c + u * GV_WAVES < pieces) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) acc[nt][0] = Piece<T>::mma(wa[u][nt], xb[u][0], acc[nt][0]);
+            }
+        }
+    };
+
+    Piece<T> wa_a[PT][NT], wa_b[PT][NT];
+    load_w(wave, wa_a);
+    const int row = min(r, M - 1);       // columns of rows that do not exist are computed from the last row and not stored
+    if constexpr (XP > 0) {
+        // Normalising prologue, while the first pieces of W are on their way: this lane's elements of
+        // its row of h for every piece of the wavefront, the sum of their squares, the row's total over
+        // lanes and wavefronts, then (h * inv) * weight rounded to the operand type.
+        constexpr int TRIPS = XP / PT;
+        static_assert(XP % PT == 0, "whole trips");
+        const float* hrow = norm.h + static_cast<size_t>(row) * K;
+        constexpr bool KEEP = XP * EL <= 64;        // the row's elements wait in registers, or are read a second time
+        float hv[KEEP ? XP : 1][EL];
+        float ss = 0.f;
+#pragma unroll
+        for (int p = 0; p < XP; ++p) {
+            const int k = (wave + p * GV_WAVES) * CH + kg * EL;
+            const int kc = min(k, K - EL);
+            float part = 0.f;
+#pragma unroll
+            for (int e = 0; e < EL; e += 4) {
+                const float4 v = *reinterpret_cast<const float4*>(hrow + kc + e);
+                if constexpr (KEEP) { hv[p][e] = v.x; hv[p][e + 1] = v.y; hv[p][e + 2] = v.z; hv[p][e + 3] = v.w; }
+                part += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+            }
+            ss += k < K ? part : 0.f;
+        }
+        ss += __shfl_xor(ss, 16, WAVE);
+        ss += __shfl_xor(ss, 32, WAVE);
+        __shared__ float ssum[GV_WAVES][16];
+        if (kg == 0) ssum[wave][r] = ss;
+        __syncthreads();
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < GV_WAVES; ++w) total += ssum[w][r];
+        const float inv = 1.0f / sqrtf(total / static_cast<float>(K) + norm.eps);
+        Piece<T> xn[TRIPS][PT][1];
+#pragma unroll
+        for (int p = 0; p < XP; ++p) {
+            const int kc = min((wave + p * GV_WAVES) * CH + kg * EL, K - EL);
+            float f[EL];
+#pragma unroll
+            for (int e = 0; e < EL; e += 4) {
+                const float4 wv = *reinterpret_cast<const float4*>(norm.weight + kc + e);
+                float4 v;
+                if constexpr (KEEP) v = make_float4(hv[p][e], hv[p][e + 1], hv[p][e + 2], hv[p][e + 3]);
+                else v = *reinterpret_cast<const float4*>(hrow + kc + e);
+                f[e] = (v.x * inv) * wv.x; f[e + 1] = (v.y * inv) * wv.y;
+                f[e + 2] = (v.z * inv) * wv.z; f[e + 3] = (v.w * inv) * wv.w;
+            }
+            xn[p / PT][p % PT][0].from_floats(f);
+        }
+#pragma unroll
+        for (int t = 0; t < TRIPS; t += 2) {
+            const int c = wave + t * STRIDE;
+            if (t + 1 < TRIPS && c + STRIDE < pieces) load_w(c + STRIDE, wa_b);
+            multiply(c, wa_a, xn[t]);
+            if (t + 2 < TRIPS && c + 2 * STRIDE < pieces) load_w(c + 2 * STRIDE, wa_a);
+            if (t + 1 < TRIPS) multiply(c + STRIDE, wa_b, xn[t + 1 < TRIPS ? t + 1 : t]);
+        }
+    } else {
+        const T* xrow = x + static_cast<size_t>(row) * K;
+        auto load_x = [&](int c, Piece<T> (&xb)[PT][1]) {
+#pragma unroll
+            for (int u = 0; u < PT; ++u) xb[u][0].load(xrow + min((c + u * GV_WAVES) * CH + kg * EL, K - EL));
+        };
+        Piece<T> xb_a[PT][1], xb_b[PT][1];
+        load_x(wave, xb_a);
+        for (int c = wave; c < pieces; c += 2 * STRIDE) {
+            if (c + STRIDE < pieces) { load_w(c + STRIDE, wa_b); load_x(c + STRIDE, xb_b); }
+            multiply(c, wa_a, xb_a);
+            if (c + 2 * STRIDE < pieces) { load_w(c + 2 * STRIDE, wa_a); load_x(c + 2 * STRIDE, xb_a); }
+            multiply(c + STRIDE, wa_b, xb_b);
+        }
+    }
+    skinny_finish<T, TOUT, 1, NT, EPI>(acc, y, M, N, I, rope);
 }
 
 template <typename T, typename TOUT, int MB, int EPI>
@@ -265,15 +435,67 @@ static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K,
     return NI_LAUNCH_RESULT();
 }
 
+// The decode kernel: NT as launch_nt chooses it.  XP: pieces per wavefront of the normalising prologue, 0 without.
+template <typename T, typename TOUT, int EPI, int XP>
+static int launch_decode(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream,
+                         RopeArgs rope = RopeArgs{}, NormArgs norm = NormArgs{}) {
+    const int out_width = (EPI == EPI_SWIGLU) ? I : N;
+    const int tiles = (out_width + 15) / 16;
+    auto run = [&](auto nt_tag) {
+        constexpr int NTc = decltype(nt_tag)::value;
+        constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
+        const int grid = (tiles + NOUT - 1) / NOUT;
+        skinny_decode_kernel<T, TOUT, NTc, EPI, XP><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm);
+    };
+    if constexpr (EPI != EPI_ROPE) {
+        if (NT >= 4) { run(std::integral_constant<int, 4>{}); return NI_LAUNCH_RESULT(); }
+    }
+    if constexpr (EPI == EPI_SWIGLU || EPI == EPI_ROPE) {
+        run(std::integral_constant<int, 2>{});
+    } else {
+        if (NT >= 2) run(std::integral_constant<int, 2>{});
+        else run(std::integral_constant<int, 1>{});
+    }
+    return NI_LAUNCH_RESULT();
+}
+
 template <typename T, typename TOUT, int EPI>
 static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, bool tiled,
                      hipStream_t stream, RopeArgs rope = RopeArgs{}) {
-    if (M <= 16) return launch_nt<T, TOUT, 1, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
-    if (M <= 32) return launch_nt<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
-    return launch_nt<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
+    if (M <= 16 && tiled) return launch_decode<T, TOUT, EPI, 0>(x, W, y, M, N, K, I, NT, stream, rope);
+    if constexpr (EPI == EPI_RESIDUAL) {
+        return -7;      // the residual epilogue exists in the decode kernel only
+    } else {
+        if (M <= 16) return launch_nt<T, TOUT, 1, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
+        if (M <= 32) return launch_nt<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
+        return launch_nt<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
+    }
 }
 
-// epilogue: 0 store in the input type, 1 store float32, 2 SwiGLU (W is [2I, K], y is [M, I]).
+// Pieces of 128 bytes that one wavefront holds of a row of K elements, rounded up to what the
+// normalising prologue is compiled for, or 0 if the row is too long for it: the normalised row
+// has to fit the registers beside two trips of W (bfloat16: K <= 2048, float32: K <= 2048).
+template <typename T>
+static int prologue_pieces(int K) {
+    constexpr int CH = 4 * Piece<T>::ELEMS;
+    const int per_wave = ((K + CH - 1) / CH + GV_WAVES - 1) / GV_WAVES;
+    if (per_wave <= 4) return 4;
+    return (std::is_same<T, float>::value && per_wave <= 8) ? 8 : 0;
+}
+
+template <typename T, int EPI>
+static int launch_normed(const NormArgs& norm, const void* W, void* y, int M, int N, int K, int I, int NT,
+                         hipStream_t stream, RopeArgs rope = RopeArgs{}) {
+    const int xp = prologue_pieces<T>(K);
+    if (xp == 4) return launch_decode<T, T, EPI, 4>(nullptr, W, y, M, N, K, I, NT, stream, rope, norm);
+    if constexpr (std::is_same<T, float>::value) {
+        if (xp == 8) return launch_decode<T, T, EPI, 8>(nullptr, W, y, M, N, K, I, NT, stream, rope, norm);
+    }
+    return -5;
+}
+
+// epilogue: 0 store in the input type, 1 store float32, 2 SwiGLU (W is [2I, K], y is [M, I]),
+// 3 add into y, the float32 residual stream [M, N] (M <= 16, tiled W).
 // K must be a multiple of 16 bytes' worth of elements x 2 (bf16: 16, f32: 8); M <= 64.
 // tiled: W is in the re-tiled order described at the top (swiglu then needs N/2 to be a multiple of 16).
 NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N, int K, int epilogue, int tiles_per_group,
@@ -286,20 +508,48 @@ NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N
     if (epilogue == 2 && (N % 2)) return -3;
     if (epilogue == 2 && tiled && (I % 16)) return -4;
     if (dtype == 0) {
+        if (epilogue == 3) return launch_mb<float, float, EPI_RESIDUAL>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
         if (epilogue == 2) return launch_mb<float, float, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
         return launch_mb<float, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
     }
+    if (epilogue == 3) return launch_mb<bf16_t, float, EPI_RESIDUAL>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
     if (epilogue == 2) return launch_mb<bf16_t, bf16_t, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
     if (epilogue == 1) return launch_mb<bf16_t, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
     return launch_mb<bf16_t, bf16_t, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
 }
 
+// Whether the normalising prologue takes M rows of K elements of this type (1) or not (0).
+NI_EXPORT int ni_skinny_prologue_ok(int M, int K, int dtype) {
+    if (M < 1 || M > 16 || K % (dtype == 0 ? 8 : 16) != 0) return 0;
+    return (dtype == 0 ? prologue_pieces<float>(K) : prologue_pieces<bf16_t>(K)) != 0;
+}
+
+// The same product on RMSNorm(h) instead of a given x: h float32 [M <= 16, K], norm_weight float32 [K],
+// W re-tiled.  epilogue 0 (store in the compute type) or 2 (SwiGLU).
+NI_EXPORT int ni_skinny_gemm_normed(const void* h, const void* norm_weight, float eps, const void* W, void* y, int M, int N,
+                                    int K, int epilogue, int tiles_per_group, int dtype, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (!ni_skinny_prologue_ok(M, K, dtype)) return -5;
+    if (epilogue != 0 && epilogue != 2) return -6;
+    const int I = N / 2;
+    if (epilogue == 2 && ((N % 2) || (I % 16))) return -4;
+    const NormArgs norm{(const float*)h, (const float*)norm_weight, eps};
+    if (dtype == 0) {
+        if (epilogue == 2) return launch_normed<float, EPI_SWIGLU>(norm, W, y, M, N, K, I, tiles_per_group, stream);
+        return launch_normed<float, EPI_STORE>(norm, W, y, M, N, K, I, tiles_per_group, stream);
+    }
+    if (epilogue == 2) return launch_normed<bf16_t, EPI_SWIGLU>(norm, W, y, M, N, K, I, tiles_per_group, stream);
+    return launch_normed<bf16_t, EPI_STORE>(norm, W, y, M, N, K, I, tiles_per_group, stream);
+}
+
 // Product with the stacked [q; k; v] matrix ((H + 2 KVH) * hd rows), rotation of query and key
 // heads by the rows' positions, queries to q_out [M, H * hd], keys and values into the pools at
 // slot_mapping (null: not stored).  hd must be a multiple of 32 and fully rotated.
-NI_EXPORT int ni_skinny_qkv_rope(const void* x, const void* W, void* q_out, const void* positions, const void* cos_t,
-                                 const void* sin_t, const void* slot_mapping, void* kpool, void* vpool, int M, int K,
-                                 int H, int KVH, int hd, int page_size, int tiled, int dtype, hipStream_t stream) {
+// With x null the product is taken on RMSNorm(h): h float32 [M <= 16, K], norm_weight [K], W re-tiled.
+NI_EXPORT int ni_skinny_qkv_rope(const void* x, const void* h, const void* norm_weight, float eps, const void* W,
+                                 void* q_out, const void* positions, const void* cos_t, const void* sin_t,
+                                 const void* slot_mapping, void* kpool, void* vpool, int M, int K, int H, int KVH, int hd,
+                                 int page_size, int tiled, int dtype, hipStream_t stream) {
     if (M <= 0) return 0;
     if (M > 64) return -1;
     if (K % (dtype == 0 ? 8 : 16) != 0) return -2;
@@ -307,7 +557,13 @@ NI_EXPORT int ni_skinny_qkv_rope(const void* x, const void* W, void* q_out, cons
     RopeArgs rope{(const int32_t*)positions, (const float*)cos_t, (const float*)sin_t, (const int32_t*)slot_mapping,
                   kpool, vpool, H, KVH, hd, page_size};
     const int N = (H + 2 * KVH) * hd;
-    // launch_nt sizes the grid from the output width: one workgroup per two tiles
+    // the grid is sized from the output width: one workgroup per two tiles
+    if (!x) {
+        if (!h || !norm_weight || !tiled || !ni_skinny_prologue_ok(M, K, dtype)) return -5;
+        const NormArgs norm{(const float*)h, (const float*)norm_weight, eps};
+        if (dtype == 0) return launch_normed<float, EPI_ROPE>(norm, W, q_out, M, N, K, 0, 2, stream, rope);
+        return launch_normed<bf16_t, EPI_ROPE>(norm, W, q_out, M, N, K, 0, 2, stream, rope);
+    }
     if (dtype == 0) return launch_mb<float, float, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, tiled != 0, stream, rope);
     return launch_mb<bf16_t, bf16_t, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, tiled != 0, stream, rope);
 }

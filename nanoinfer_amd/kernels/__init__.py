@@ -8,6 +8,7 @@ rocBLAS/hipBLASLt), as the reference takes them from cuBLAS (src/op/kernels/cuda
 from __future__ import annotations
 
 import ctypes
+import functools
 import math
 from typing import Dict, Optional
 
@@ -381,6 +382,7 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
 
 SKINNY_MAX_ROWS = 64        # what the kernel takes
 SKINNY_BEST_ROWS = 16       # up to here it beats the library product on this chip (measured at the 1B sizes)
+FUSE_NORMS = True           # residual sums and norms ride on the skinny products of a decode step where they can
 
 
 def tile_weight(w: torch.Tensor) -> torch.Tensor:
@@ -441,30 +443,90 @@ def _tiles_per_group(n_out: int) -> int:
     return 4 if tiles >= 2048 else (2 if tiles >= 512 else 1)
 
 
-def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, swiglu: bool = False) -> torch.Tensor:
+class NormedInput:
+    """The input of a product given as the float32 residual stream ``h`` [M, K] together with the
+    weight and eps of the RMSNorm that stands before the product: the skinny product normalises the
+    rows in its prologue instead of a kernel of its own (:func:`norm_prologue_ok` says when)."""
+
+    __slots__ = ("h", "weight", "eps", "dtype")
+
+    def __init__(self, h: torch.Tensor, weight: torch.Tensor, eps: float, dtype: torch.dtype):
+        self.h, self.weight, self.eps, self.dtype = h, weight, float(eps), dtype
+
+    @property
+    def shape(self):
+        return self.h.shape
+
+    @property
+    def device(self):
+        return self.h.device
+
+
+@functools.lru_cache(maxsize=None)
+def _prologue_sizes_ok(M: int, K: int, code: int) -> bool:
+    return bool(skinny_lib().ni_skinny_prologue_ok(M, K, code))
+
+
+def norm_prologue_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
+    """Whether the skinny product can take RMSNorm(h) for its input: at most 16 rows, a re-tiled
+    matrix, rows short enough for the normalised operand to stay in registers."""
+    return (isinstance(weight, Weight) and weight.tiles is not None and dtype in _DTYPE_CODE
+            and _prologue_sizes_ok(int(M), int(K), dtype_code(dtype)))
+
+
+def residual_epilogue_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
+    """Whether the skinny product can add its result straight into the float32 residual stream."""
+    return (isinstance(weight, Weight) and weight.tiles is not None and 0 < M <= SKINNY_BEST_ROWS
+            and skinny_ok(M, K, dtype))
+
+
+def _check_normed(x: NormedInput, Kd: int) -> None:
+    _gpu(x.h, "h", torch.float32)
+    _need(x.h.dim() == 2 and x.h.shape[1] == Kd, f"normed input {tuple(x.h.shape)} against K={Kd}")
+    _gpu(x.weight, "norm weight", torch.float32, (Kd,))
+
+
+def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bool = False) -> torch.Tensor:
     """``x . weight^T`` for at most 64 rows of ``x``, streaming ``weight`` once (MFMA).  ``out``
     may be float32 for bfloat16 inputs.  With ``swiglu`` the weight is a stacked [2I, K] matrix
-    (gate rows, then up rows) and ``out`` [M, I] receives ``silu(gate) * up``."""
+    (gate rows, then up rows) and ``out`` [M, I] receives ``silu(gate) * up``.  With ``residual``
+    ``out`` is the float32 residual stream [M, N] and the product is added into it.  ``x`` may be a
+    :class:`NormedInput`."""
+    normed = isinstance(x, NormedInput)
     M, Kd = x.shape
-    weight, tiles = _rows_and_tiles(weight)
-    N = weight.shape[0]
-    _gpu(x, "x")
-    _gpu(weight, "weight", x.dtype)
-    _need(weight.shape[1] == Kd, f"skinny_gemm: {tuple(x.shape)} x {tuple(weight.shape)}^T")
-    _need(skinny_ok(M, Kd, x.dtype), f"skinny_gemm does not take M={M}, K={Kd} in {x.dtype}")
+    dtype = x.dtype
+    rows, tiles = _rows_and_tiles(weight)
+    N = rows.shape[0]
+    _gpu(rows, "weight", dtype)
+    _need(rows.shape[1] == Kd, f"skinny_gemm: {tuple(x.shape)} x {tuple(rows.shape)}^T")
+    _need(skinny_ok(M, Kd, dtype), f"skinny_gemm does not take M={M}, K={Kd} in {dtype}")
     if swiglu and tiles is not None and (N // 2) % 16:
         tiles = None          # gate and up halves do not start on tile boundaries: stream the rows as stored
     if swiglu:
         _need(N % 2 == 0, "a stacked gate/up matrix needs an even number of rows")
-        _gpu(out, "out", x.dtype, (M, N // 2))
+        _need(not residual, "swiglu and residual exclude each other")
+        _gpu(out, "out", dtype, (M, N // 2))
         epi = 2
+    elif residual:
+        _need(tiles is not None and M <= 16, "the residual epilogue needs a re-tiled matrix and at most 16 rows")
+        _gpu(out, "out", torch.float32, (M, N))
+        epi = 3
     else:
-        _need(out.dtype in (x.dtype, torch.float32), f"out must be {x.dtype} or float32")
+        _need(out.dtype in (dtype, torch.float32), f"out must be {dtype} or float32")
         _gpu(out, "out", None, (M, N))
-        epi = 1 if (out.dtype == torch.float32 and x.dtype != torch.float32) else 0
-    _check(skinny_lib().ni_skinny_gemm(_ptr(x), _ptr(weight if tiles is None else tiles), _ptr(out), M, N, Kd, epi,
-                                       _tiles_per_group(N // 2 if swiglu else N), 0 if tiles is None else 1,
-                                       dtype_code(x.dtype), _stream()), "skinny_gemm")
+        epi = 1 if (out.dtype == torch.float32 and dtype != torch.float32) else 0
+    per_group = _tiles_per_group(N // 2 if swiglu else N)
+    if normed:
+        _need(tiles is not None and norm_prologue_ok(M, Kd, dtype, weight) and epi in (0, 2),
+              f"the normalising prologue does not take M={M}, K={Kd} in {dtype} with this matrix and epilogue")
+        _check_normed(x, Kd)
+        _check(skinny_lib().ni_skinny_gemm_normed(_ptr(x.h), _ptr(x.weight), ctypes.c_float(x.eps), _ptr(tiles), _ptr(out),
+                                                  M, N, Kd, epi, per_group, dtype_code(dtype), _stream()),
+               "skinny_gemm_normed")
+        return out
+    _gpu(x, "x")
+    _check(skinny_lib().ni_skinny_gemm(_ptr(x), _ptr(rows if tiles is None else tiles), _ptr(out), M, N, Kd, epi,
+                                       per_group, 0 if tiles is None else 1, dtype_code(dtype), _stream()), "skinny_gemm")
     return out
 
 
@@ -474,44 +536,66 @@ def qkv_rope_ok(M: int, K: int, hd: int, rotary_dim: int, dtype: torch.dtype) ->
     return skinny_ok(M, K, dtype) and hd % 32 == 0 and rotary_dim == hd
 
 
-def skinny_qkv_rope(x: torch.Tensor, w_qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor,
+def skinny_qkv_rope(x, w_qkv, positions: torch.Tensor, cos: torch.Tensor,
                     sin: torch.Tensor, slot_mapping: Optional[torch.Tensor], kpool: Optional[torch.Tensor],
                     vpool: Optional[torch.Tensor], H: int, KVH: int, hd: int) -> torch.Tensor:
     """``x . w_qkv^T`` for few rows with rotation and cache write fused in: returns the rotated
-    queries [M, H*hd]; rotated keys and plain values go straight into the pools at ``slot_mapping``."""
+    queries [M, H*hd]; rotated keys and plain values go straight into the pools at ``slot_mapping``.
+    ``x`` may be a :class:`NormedInput`."""
+    normed = isinstance(x, NormedInput)
     M, Kd = x.shape
-    w_qkv, tiles = _rows_and_tiles(w_qkv)
-    _gpu(x, "x")
-    _gpu(w_qkv, "w_qkv", x.dtype, ((H + 2 * KVH) * hd, Kd))
-    _need(qkv_rope_ok(M, Kd, hd, 2 * cos.shape[1], x.dtype), f"skinny_qkv_rope does not take M={M}, K={Kd}, hd={hd}")
+    dtype = x.dtype
+    rows, tiles = _rows_and_tiles(w_qkv)
+    _gpu(rows, "w_qkv", dtype, ((H + 2 * KVH) * hd, Kd))
+    _need(qkv_rope_ok(M, Kd, hd, 2 * cos.shape[1], dtype), f"skinny_qkv_rope does not take M={M}, K={Kd}, hd={hd}")
     _gpu(positions, "positions", torch.int32, (M,))
     _gpu(cos, "cos", torch.float32)
     _gpu(sin, "sin", torch.float32, cos.shape)
     page_size = 1
     if slot_mapping is not None:
         _gpu(slot_mapping, "slot_mapping", torch.int32, (M,))
-        _gpu(kpool, "kpool", x.dtype)
-        _gpu(vpool, "vpool", x.dtype, kpool.shape)
+        _gpu(kpool, "kpool", dtype)
+        _gpu(vpool, "vpool", dtype, kpool.shape)
         _need(kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd,
               f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
         page_size = kpool.shape[2]
-    q = torch.empty(M, H * hd, dtype=x.dtype, device=x.device)
-    _check(skinny_lib().ni_skinny_qkv_rope(_ptr(x), _ptr(w_qkv if tiles is None else tiles), _ptr(q), _ptr(positions),
-                                           _ptr(cos), _ptr(sin), _ptr(slot_mapping), _ptr(kpool), _ptr(vpool), M, Kd,
-                                           H, KVH, hd, page_size, 0 if tiles is None else 1, dtype_code(x.dtype),
-                                           _stream()), "skinny_qkv_rope")
+    if normed:
+        _need(norm_prologue_ok(M, Kd, dtype, w_qkv), f"the normalising prologue does not take M={M}, K={Kd} in {dtype}")
+        _check_normed(x, Kd)
+        x_ptr, h_ptr, nw_ptr, eps = None, _ptr(x.h), _ptr(x.weight), x.eps
+        device = x.h.device
+    else:
+        _gpu(x, "x")
+        x_ptr, h_ptr, nw_ptr, eps = _ptr(x), None, None, 0.0
+        device = x.device
+    q = torch.empty(M, H * hd, dtype=dtype, device=device)
+    _check(skinny_lib().ni_skinny_qkv_rope(x_ptr, h_ptr, nw_ptr, ctypes.c_float(eps), _ptr(rows if tiles is None else tiles),
+                                           _ptr(q), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping), _ptr(kpool),
+                                           _ptr(vpool), M, Kd, H, KVH, hd, page_size, 0 if tiles is None else 1,
+                                           dtype_code(dtype), _stream()), "skinny_qkv_rope")
     return q
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optional[torch.Tensor] = None):
     """``x . weight^T`` with ``weight`` stored [out, in].  Few rows go to the hand-written skinny
     product; many rows to the library (rocBLAS/hipBLASLt), where float32 inputs are multiplied in
     true float32 (the reduced-precision matrix modes of the library are switched off at import).
-    ``out_dtype`` float32 keeps the float32 accumulators of a bfloat16 product."""
+    ``out_dtype`` float32 keeps the float32 accumulators of a bfloat16 product.  ``x`` may be a
+    :class:`NormedInput` where :func:`norm_prologue_ok` holds.  With ``residual`` (the float32
+    residual stream, where :func:`residual_epilogue_ok` holds) the product is added into it and
+    nothing is returned."""
     rows, _ = _rows_and_tiles(weight)
+    if isinstance(x, NormedInput):
+        _need(residual is None, "a normed input and a residual output in one product are not compiled")
+        out = torch.empty(x.shape[0], rows.shape[0], dtype=x.dtype, device=x.device)
+        return skinny_gemm(x, weight, out)
     _need(x.is_cuda and rows.is_cuda, "linear needs GPU tensors")
     _need(x.dtype == rows.dtype, f"linear: activation {x.dtype} and weight {rows.dtype} differ")
     _need(x.dim() == 2 and x.shape[1] == rows.shape[1], f"linear: {tuple(x.shape)} x {tuple(rows.shape)}^T")
+    if residual is not None:
+        _need(residual_epilogue_ok(x.shape[0], x.shape[1], x.dtype, weight), "the residual epilogue does not take this product")
+        skinny_gemm(x, weight, residual, residual=True)
+        return None
     out_dtype = out_dtype or x.dtype
     if x.shape[0] <= SKINNY_BEST_ROWS and skinny_ok(x.shape[0], x.shape[1], x.dtype):
         out = torch.empty(x.shape[0], rows.shape[0], dtype=out_dtype, device=x.device)
@@ -524,12 +608,12 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
     return torch.matmul(x, weight.t())
 
 
-def linear_swiglu(x: torch.Tensor, weight_gate_up: torch.Tensor) -> torch.Tensor:
+def linear_swiglu(x, weight_gate_up) -> torch.Tensor:
     """``silu(x . Wg^T) * (x . Wu^T)`` for the stacked matrix [Wg; Wu]: fused into the product for
-    few rows, product then the SwiGLU kernel for many."""
+    few rows, product then the SwiGLU kernel for many.  ``x`` may be a :class:`NormedInput`."""
     inter = weight_gate_up.shape[0] // 2
     out = torch.empty(x.shape[0], inter, dtype=x.dtype, device=x.device)
-    if x.shape[0] <= SKINNY_BEST_ROWS and skinny_ok(x.shape[0], x.shape[1], x.dtype):
+    if isinstance(x, NormedInput) or (x.shape[0] <= SKINNY_BEST_ROWS and skinny_ok(x.shape[0], x.shape[1], x.dtype)):
         return skinny_gemm(x, weight_gate_up, out, swiglu=True)
     global _library_calls
     _library_calls += 1

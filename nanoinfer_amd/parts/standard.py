@@ -76,6 +76,10 @@ class RMSNorm(Part):
         out = torch.empty(n, self.size, dtype=self.rt.dtype, device=self.rt.device)
         return K.add_rmsnorm(h, pending, self.weight, self.eps, out, rows)
 
+    def as_prologue(self, h: torch.Tensor):
+        """This norm of ``h`` (nothing pending) as an input that a product can normalise itself."""
+        return K.NormedInput(h, self.weight, self.eps, self.rt.dtype)
+
 
 # ------------------------------------------------------------------ position
 
@@ -184,7 +188,18 @@ class Attention(Part):
     def cache_need(self) -> CacheNeed:
         return CacheNeed(kv=KVNeed(self.KVH, self.hd, self.window))
 
-    def forward(self, x: torch.Tensor, ctx, cache: LayerCache) -> torch.Tensor:
+    def takes_normed(self, T: int) -> bool:
+        """Whether ``forward`` takes the norm before it as a prologue of its first product for T tokens."""
+        tables = self.position.tables()
+        d = self.w_qkv.shape[1]
+        return (K.FUSE_NORMS and tables is not None and K.qkv_rope_ok(T, d, self.hd, 2 * tables[0].shape[1], self.rt.dtype)
+                and K.norm_prologue_ok(T, d, self.rt.dtype, self.w_qkv))
+
+    def adds_residual(self, T: int) -> bool:
+        """Whether ``forward`` can add its output straight into the residual stream for T tokens."""
+        return K.FUSE_NORMS and K.residual_epilogue_ok(T, self.H * self.hd, self.rt.dtype, self.w_o)
+
+    def forward(self, x, ctx, cache: LayerCache, residual: Optional[torch.Tensor] = None):
         T = x.shape[0]
         tables = self.position.tables()
         cos, sin = tables if tables is not None else (None, None)
@@ -205,7 +220,7 @@ class Attention(Part):
             ws = ctx.workspace(T * self.H * nsplit * (self.hd + 2)) if nsplit > 1 else None
             K.mfma_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, out, self.H, self.KVH, self.hd,
                              self.scale, self.window, nsplit, ws)
-            return K.linear(out, self.w_o)
+            return K.linear(out, self.w_o, residual=residual)
         # single tokens and short portions, token by token
         max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window)
         on_matrix_cores = K.mfma_attention_ok(x.dtype, self.hd)
@@ -215,7 +230,7 @@ class Attention(Part):
         attend = K.mfma_token_attention if on_matrix_cores else K.token_attention
         attend(qkv, cache.kpool, cache.vpool, cache.block_table, ctx.seq_of_token, ctx.positions, out,
                self.H, self.KVH, self.hd, self.scale, self.window, nsplit, ws)
-        return K.linear(out, self.w_o)
+        return K.linear(out, self.w_o, residual=residual)
 
 
 # ------------------------------------------------------------------ feed-forward
@@ -241,8 +256,16 @@ class SwiGLU(Part):
         self.w_gate_up = rt.weight(names["gate"] + "|" + names["up"], torch.cat([weights["gate"], weights["up"]], dim=0))
         self.w_down = rt.weight(names["down"], weights["down"])
 
-    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        return K.linear(K.linear_swiglu(x, self.w_gate_up), self.w_down)
+    def takes_normed(self, T: int) -> bool:
+        d = self.w_gate_up.shape[1]
+        return (K.FUSE_NORMS and self.intermediate_size % 16 == 0
+                and K.norm_prologue_ok(T, d, self.rt.dtype, self.w_gate_up))
+
+    def adds_residual(self, T: int) -> bool:
+        return K.FUSE_NORMS and K.residual_epilogue_ok(T, self.intermediate_size, self.rt.dtype, self.w_down)
+
+    def forward(self, x, ctx, residual: Optional[torch.Tensor] = None):
+        return K.linear(K.linear_swiglu(x, self.w_gate_up), self.w_down, residual=residual)
 
 
 # ------------------------------------------------------------------ block
@@ -252,7 +275,11 @@ class PreNormBlock:
     """``h += mixer(norm1(h)); h += ffn(norm2(h))`` (src/model/llama.cpp:324-379).
 
     The residual stream ``h`` is float32.  The last addend is handed on as ``pending`` and is
-    summed into ``h`` by the next norm, in float32, in the same pass that normalises.
+    summed into ``h`` by the next norm, in float32, in the same pass that normalises.  Two optional
+    abilities of a mixer or feed-forward shorten this for steps of few tokens: ``adds_residual(T)``
+    (its last product adds into ``h`` itself: nothing is pending) and ``takes_normed(T)`` (its first
+    product normalises ``h`` itself, given the norm's ``as_prologue(h)``).  A part without them is
+    run the plain way.
     """
 
     family = "block"
@@ -276,11 +303,30 @@ class PreNormBlock:
     def graph_safe(self) -> bool:
         return all(p.graph_safe is True for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn))
 
+    @staticmethod
+    def _normed_input(norm, part, h, pending):
+        """What ``part`` is given for ``norm(h + pending)``: the norm as a prologue where both sides can, else its output."""
+        T = h.shape[0]
+        takes = getattr(part, "takes_normed", None)
+        prologue = getattr(norm, "as_prologue", None)
+        if pending is None and takes is not None and prologue is not None and takes(T):
+            return prologue(h)
+        return norm.forward(h, pending)
+
     def forward(self, h, pending, ctx, cache: LayerCache):
-        x = self.mixer_norm.forward(h, pending)
-        a = self.mixer.forward(x, ctx, cache)
-        x = self.ffn_norm.forward(h, a)
-        f = self.ffn.forward(x, ctx)
+        T = h.shape[0]
+        x = self._normed_input(self.mixer_norm, self.mixer, h, pending)
+        adds = getattr(self.mixer, "adds_residual", None)
+        if adds is not None and adds(T):
+            a = self.mixer.forward(x, ctx, cache, residual=h)
+        else:
+            a = self.mixer.forward(x, ctx, cache)
+        x = self._normed_input(self.ffn_norm, self.ffn, h, a)
+        adds = getattr(self.ffn, "adds_residual", None)
+        if adds is not None and adds(T):
+            f = self.ffn.forward(x, ctx, residual=h)
+        else:
+            f = self.ffn.forward(x, ctx)
         return h, f
 
 

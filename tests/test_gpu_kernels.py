@@ -461,6 +461,54 @@ def test_skinny_product(K, dtype, M, N, Kd):
     _skinny_case(K, dtype, M, N, Kd)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("M,N,Kd", [(1, 32, 64), (5, 50, 192), (16, 1000, 528), (8, 4096, 2048), (3, 778, 1024), (16, 96, 48),
+                                    (2, 64, 4096)])
+def test_skinny_product_with_norm_prologue_and_residual_epilogue(K, dtype, M, N, Kd):
+    """RMSNorm(h) as the input of a product (store and SwiGLU epilogues), and a product added into
+    the residual stream, against the plain steps in float64.  Row widths that are no multiple of a
+    128-byte piece (528, 48) put the zero padding of the re-tiled matrix to work."""
+    g = torch.Generator().manual_seed(M * 77 + N + Kd)
+    h = torch.randn(M, Kd, generator=g) * 3
+    nw = 1 + 0.1 * torch.randn(Kd, generator=g)
+    eps = 2e-6
+    w = (torch.randn(N, Kd, generator=g) / math.sqrt(Kd)).to(DT[dtype])
+    W = K.Weight(dev(w))
+    xn = P.rmsnorm(h.double(), nw, eps)
+    ok = K.norm_prologue_ok(M, Kd, DT[dtype], W)
+    assert ok == (Kd <= 2048), "rows up to 2,048 elements are taken"
+    assert not K.norm_prologue_ok(17, Kd, DT[dtype], W) and not K.norm_prologue_ok(M, Kd, DT[dtype], dev(w))
+    normed = K.NormedInput(dev(h), dev(nw), eps, DT[dtype])
+    if not ok:      # refused with a reason, never run
+        with pytest.raises(K.KernelError):
+            K.skinny_gemm(normed, W, torch.empty(M, N, device="cuda", dtype=DT[dtype]))
+        return
+    # the operand is rounded to the compute type after the norm, as the separate kernel rounds its output
+    xr = xn.to(DT[dtype]).double()
+    want = xr @ w.double().t()
+    out = K.skinny_gemm(normed, W, torch.empty(M, N, device="cuda", dtype=DT[dtype]))
+    assert rel(out, want) < KTOL[dtype], "normed, store"
+    assert rel(K.linear(normed, W), want) < KTOL[dtype]
+    if N % 32 == 0:
+        act = K.skinny_gemm(normed, W, torch.empty(M, N // 2, device="cuda", dtype=DT[dtype]), swiglu=True)
+        assert rel(act, P.swiglu(want[:, :N // 2], want[:, N // 2:])) < KTOL[dtype], "normed, swiglu"
+        assert rel(K.linear_swiglu(normed, W), P.swiglu(want[:, :N // 2], want[:, N // 2:])) < KTOL[dtype]
+    # the same numbers as norm kernel + product, up to the order of the sum of squares
+    x_sep = K.add_rmsnorm(dev(h.clone()), None, dev(nw), eps, torch.empty(M, Kd, device="cuda", dtype=DT[dtype]))
+    sep = K.skinny_gemm(x_sep, W, torch.empty(M, N, device="cuda", dtype=DT[dtype]))
+    assert rel(out, sep.double().cpu()) < KTOL[dtype]
+    # residual epilogue: stream += x . W^T, in float32, other columns and rows untouched
+    x = torch.randn(M, Kd, generator=g).to(DT[dtype])
+    stream = torch.randn(M + 2, N, generator=g)
+    buf = dev(stream.clone())
+    assert K.residual_epilogue_ok(M, Kd, DT[dtype], W) and not K.residual_epilogue_ok(M, Kd, DT[dtype], dev(w))
+    assert K.linear(dev(x), W, residual=buf[:M]) is None
+    assert rel(buf[:M], stream[:M].double() + x.double() @ w.double().t()) < 3e-6
+    assert torch.equal(buf[M:].cpu(), stream[M:])
+    with pytest.raises(K.KernelError):
+        K.skinny_gemm(normed, dev(w), torch.empty(M, N, device="cuda", dtype=DT[dtype]))       # needs the re-tiled matrix
+
+
 def test_skinny_product_reference_vector(K):
     # test/test_cuda_kernel/test_matmul_kernel.cpp:30-99: ones x 0.5 with K = 128 gives 64
     out = K.skinny_gemm(torch.ones(3, 128, device="cuda"), torch.full((7, 128), 0.5, device="cuda"),
@@ -489,6 +537,19 @@ def test_product_with_rotation_and_cache_write(K, dtype, M, H, KVH, hd, Kd, ps):
     vpool = torch.full((pages, KVH, ps, hd), 7.0, dtype=DT[dtype], device="cuda")
     assert K.qkv_rope_ok(M, Kd, hd, hd, DT[dtype])
     q = K.skinny_qkv_rope(dev(x), dev(w), dev(positions), cos, sin, dev(slots), kpool, vpool, H, KVH, hd)
+    W = K.Weight(dev(w))
+    if K.norm_prologue_ok(M, Kd, DT[dtype], W):
+        # the same product taken on RMSNorm(h): queries and pages as from the norm kernel's output
+        h = torch.randn(M, Kd, generator=g) * 2
+        nw = 1 + 0.1 * torch.randn(Kd, generator=g)
+        x_sep = K.add_rmsnorm(dev(h.clone()), None, dev(nw), 1e-5, torch.empty(M, Kd, device="cuda", dtype=DT[dtype]))
+        kp1, vp1 = torch.zeros_like(kpool), torch.zeros_like(vpool)
+        q1 = K.skinny_qkv_rope(x_sep, W, dev(positions), cos, sin, dev(slots), kp1, vp1, H, KVH, hd)
+        kp2, vp2 = torch.zeros_like(kpool), torch.zeros_like(vpool)
+        q2 = K.skinny_qkv_rope(K.NormedInput(dev(h), dev(nw), 1e-5, DT[dtype]), W, dev(positions), cos, sin, dev(slots),
+                               kp2, vp2, H, KVH, hd)
+        for got, want_t in ((q2, q1), (kp2, kp1), (vp2, vp1)):
+            assert rel(got, want_t.double().cpu()) < KTOL[dtype]
     qkv = x.double() @ w.double().t()
     s, c = P.rope_tables(positions.tolist(), inv)
     q_ref = plain_rotate_half(qkv[:, :H * hd].reshape(M, H, hd), s, c, hd)
