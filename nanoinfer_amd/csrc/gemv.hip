@@ -332,30 +332,47 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_decode_kernel(const T* __re
     };
 
     Piece<T> wa_a[PT][NT], wa_b[PT][NT];
-    load_w(wave, wa_a);
     const int row = min(r, M - 1);       // columns of rows that do not exist are computed from the last row and not stored
     if constexpr (XP > 0) {
-        // Normalising prologue, while the first pieces of W are on their way: this lane's elements of
-        // its row of h for every piece of the wavefront, the sum of their squares, the row's total over
-        // lanes and wavefronts, then (h * inv) * weight rounded to the operand type.
+        // Normalising prologue: this lane's elements of its row of h for every piece of the wavefront
+        // and the norm's weights at the same places are asked for first, the first trip of W right
+        // behind them.  Loads come back in the order they were issued, so the small ones (cache hits)
+        // arrive while W is still on its way from HBM, and the sum of squares, its meeting over lanes
+        // and wavefronts in LDS and the rounding of (h * weight) * inv to the operand type all happen
+        // under the shadow of W.  Lanes whose row does not exist load and compute nothing.
         constexpr int TRIPS = XP / PT;
         static_assert(XP % PT == 0, "whole trips");
         const float* hrow = norm.h + static_cast<size_t>(row) * K;
+        const bool live = r < M;
         constexpr bool KEEP = XP * EL <= 64;        // the row's elements wait in registers, or are read a second time
-        float hv[KEEP ? XP : 1][EL];
-        float ss = 0.f;
+        float4 hraw[XP][EL / 4], wraw[KEEP ? XP : 1][EL / 4];
+        if (live) {
 #pragma unroll
-        for (int p = 0; p < XP; ++p) {
-            const int k = (wave + p * GV_WAVES) * CH + kg * EL;
-            const int kc = min(k, K - EL);
-            float part = 0.f;
+            for (int p = 0; p < XP; ++p) {
+                const int kc = min((wave + p * GV_WAVES) * CH + kg * EL, K - EL);
 #pragma unroll
-            for (int e = 0; e < EL; e += 4) {
-                const float4 v = *reinterpret_cast<const float4*>(hrow + kc + e);
-                if constexpr (KEEP) { hv[p][e] = v.x; hv[p][e + 1] = v.y; hv[p][e + 2] = v.z; hv[p][e + 3] = v.w; }
-                part += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+                for (int e = 0; e < EL / 4; ++e) {
+                    hraw[p][e] = *reinterpret_cast<const float4*>(hrow + kc + 4 * e);
+                    if constexpr (KEEP) wraw[p][e] = *reinterpret_cast<const float4*>(norm.weight + kc + 4 * e);
+                }
             }
-            ss += k < K ? part : 0.f;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(wave, wa_a);
+        __builtin_amdgcn_sched_barrier(0);
+        float ss = 0.f;
+        if (live) {
+#pragma unroll
+            for (int p = 0; p < XP; ++p) {
+                const int k = (wave + p * GV_WAVES) * CH + kg * EL;
+                float part = 0.f;
+#pragma unroll
+                for (int e = 0; e < EL / 4; ++e) {
+                    const float4 v = hraw[p][e];
+                    part += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+                }
+                ss += k < K ? part : 0.f;
+            }
         }
         ss += __shfl_xor(ss, 16, WAVE);
         ss += __shfl_xor(ss, 32, WAVE);
@@ -369,16 +386,19 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_decode_kernel(const T* __re
         Piece<T> xn[TRIPS][PT][1];
 #pragma unroll
         for (int p = 0; p < XP; ++p) {
-            const int kc = min((wave + p * GV_WAVES) * CH + kg * EL, K - EL);
             float f[EL];
+            const int kc = min((wave + p * GV_WAVES) * CH + kg * EL, K - EL);
 #pragma unroll
-            for (int e = 0; e < EL; e += 4) {
-                const float4 wv = *reinterpret_cast<const float4*>(norm.weight + kc + e);
-                float4 v;
-                if constexpr (KEEP) v = make_float4(hv[p][e], hv[p][e + 1], hv[p][e + 2], hv[p][e + 3]);
-                else v = *reinterpret_cast<const float4*>(hrow + kc + e);
-                f[e] = (v.x * inv) * wv.x; f[e + 1] = (v.y * inv) * wv.y;
-                f[e + 2] = (v.z * inv) * wv.z; f[e + 3] = (v.w * inv) * wv.w;
+            for (int e = 0; e < EL / 4; ++e) {
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f), wv = v;
+                if constexpr (KEEP) {
+                    if (live) { v = hraw[p][e]; wv = wraw[p][e]; }
+                } else if (live) {
+                    v = *reinterpret_cast<const float4*>(hrow + kc + 4 * e);
+                    wv = *reinterpret_cast<const float4*>(norm.weight + kc + 4 * e);
+                }
+                f[4 * e] = (v.x * inv) * wv.x; f[4 * e + 1] = (v.y * inv) * wv.y;
+                f[4 * e + 2] = (v.z * inv) * wv.z; f[4 * e + 3] = (v.w * inv) * wv.w;
             }
             xn[p / PT][p % PT][0].from_floats(f);
         }
@@ -391,6 +411,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_decode_kernel(const T* __re
             if (t + 1 < TRIPS) multiply(c + STRIDE, wa_b, xn[t + 1 < TRIPS ? t + 1 : t]);
         }
     } else {
+        load_w(wave, wa_a);
         const T* xrow = x + static_cast<size_t>(row) * K;
         auto load_x = [&](int c, Piece<T> (&xb)[PT][1]) {
 #pragma unroll
