@@ -105,14 +105,14 @@ struct RopeArgs {
 
 // What follows the main loop of both kernels: the wavefronts' partial sums meet in LDS and the
 // epilogue stores them.
-template <typename T, typename TOUT, int MB, int NT, int EPI>
+template <typename T, typename TOUT, int MB, int NT, int EPI, int WV = GV_WAVES>
 __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TOUT* __restrict__ y, int M, int N, int I,
                                               const RopeArgs& rope) {
     const int tid = threadIdx.x;
     const int wave = tid / WAVE, lane = tid % WAVE;
     const int wg = blockIdx.x;
     // partial sums of the wavefronts meet in LDS: red[wave][tile][lane * 4 + i]
-    __shared__ float red[GV_WAVES][NT * MB][WAVE * 4];
+    __shared__ float red[WV][NT * MB][WAVE * 4];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -127,7 +127,7 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
         const int head = wg / per_head;                 // among H query, KVH key, KVH value heads
         const int j0 = (wg % per_head) * 16;            // first of this workgroup's 16 pairs
         const int half = rope.hd / 2;
-        for (int item = tid; item < MB * 16 * 16; item += GV_THREADS) {
+        for (int item = tid; item < MB * 16 * 16; item += WV * WAVE) {
             const int n_local = item % 16;
             const int m = item / 16;
             if (m >= M) continue;
@@ -135,7 +135,7 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
             const int src = ((n_local / 4) * 16 + m_local) * 4 + (n_local % 4);
             float x0 = 0.f, x1 = 0.f;
 #pragma unroll
-            for (int w = 0; w < GV_WAVES; ++w) {
+            for (int w = 0; w < WV; ++w) {
                 x0 += red[w][0 * MB + mb][src];
                 x1 += red[w][1 * MB + mb][src];
             }
@@ -170,7 +170,7 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
     constexpr int NOUT = (EPI == EPI_SWIGLU) ? NT / 2 : NT;      // output tiles of the workgroup
     const int out_n0 = wg * NOUT * 16;
     const int out_width = (EPI == EPI_SWIGLU) ? I : N;
-    for (int item = tid; item < MB * 16 * NOUT * 16; item += GV_THREADS) {
+    for (int item = tid; item < MB * 16 * NOUT * 16; item += WV * WAVE) {
         const int n_in = item % (NOUT * 16);
         const int m = item / (NOUT * 16);
         const int ot = n_in / 16, n_local = n_in % 16;
@@ -182,7 +182,7 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
         if (EPI == EPI_SWIGLU) {
             float g = 0.f, u = 0.f;
 #pragma unroll
-            for (int w = 0; w < GV_WAVES; ++w) {
+            for (int w = 0; w < WV; ++w) {
                 g += red[w][(2 * ot) * MB + mb][src];
                 u += red[w][(2 * ot + 1) * MB + mb][src];
             }
@@ -190,7 +190,7 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
         } else {
             v = 0.f;
 #pragma unroll
-            for (int w = 0; w < GV_WAVES; ++w) v += red[w][ot * MB + mb][src];
+            for (int w = 0; w < WV; ++w) v += red[w][ot * MB + mb][src];
         }
         TOUT* dst = y + static_cast<size_t>(m) * out_width + n;
         if constexpr (EPI == EPI_RESIDUAL) *dst += v;      // float32 residual stream, this workgroup's own columns
@@ -279,8 +279,10 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
 // The decode step's kernel: at most 16 rows, W re-tiled (and zero-padded to whole pieces, so a lane
 // past the end of a row multiplies by zero whatever it read of x).  XP == 0: x is given.
 // XP > 0: x = RMSNorm(h) with the wavefront's XP pieces of the normalised row kept in registers.
-template <typename T, typename TOUT, int NT, int EPI, int XP>
-__global__ __launch_bounds__(GV_THREADS) void skinny_decode_kernel(const T* __restrict__ x, const T* __restrict__ W,
+// WV wavefronts split K: 8, or 16 for a matrix of few tiles and long rows, whose workgroups are too
+// few to fill the chip and have to keep more loads in flight each.
+template <typename T, typename TOUT, int NT, int EPI, int XP, int WV>
+__global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                                    TOUT* __restrict__ y, int M, int N, int K, int I,
                                                                    RopeArgs rope, NormArgs norm) {
     constexpr int EL = Piece<T>::ELEMS;
@@ -311,12 +313,12 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_decode_kernel(const T* __re
     // PT pieces per trip; trip t of a wavefront covers pieces wave + (t * PT + u) * 8.  Two trips are
     // in registers at a time, in two fixed sets (A and B): one is multiplied while the other's loads
     // are under way.
-    constexpr int PT = NT <= 2 ? 4 : 2;
-    constexpr int STRIDE = PT * GV_WAVES;
+    constexpr int PT = (NT <= 2 && WV <= 8) ? 4 : 2;      // sixteen wavefronts have half the registers each
+    constexpr int STRIDE = PT * WV;
     auto load_w = [&](int c, Piece<T> (&wa)[PT][NT]) {
 #pragma unroll
         for (int u = 0; u < PT; ++u) {
-            const int piece = min(c + u * GV_WAVES, pieces - 1);
+            const int piece = min(c + u * WV, pieces - 1);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) wa[u][nt].load(wrow[nt] + static_cast<size_t>(piece) * (WAVE * EL));
         }
@@ -324,7 +326,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_decode_kernel(const T* __re
     auto multiply = [&](int c, const Piece<T> (&wa)[PT][NT], const Piece<T> (&xb)[PT][1]) {
 #pragma unroll
         for (int u = 0; u < PT; ++u) {
-            if (c + u * GV_WAVES < pieces) {
+            if (c + u * WV < pieces) {
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) acc[nt][0] = Piece<T>::mma(wa[u][nt], xb[u][0], acc[nt][0]);
             }
@@ -349,7 +351,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_decode_kernel(const T* __re
         if (live) {
 #pragma unroll
             for (int p = 0; p < XP; ++p) {
-                const int kc = min((wave + p * GV_WAVES) * CH + kg * EL, K - EL);
+                const int kc = min((wave + p * WV) * CH + kg * EL, K - EL);
 #pragma unroll
                 for (int e = 0; e < EL / 4; ++e) {
                     hraw[p][e] = *reinterpret_cast<const float4*>(hrow + kc + 4 * e);
@@ -364,7 +366,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_decode_kernel(const T* __re
         if (live) {
 #pragma unroll
             for (int p = 0; p < XP; ++p) {
-                const int k = (wave + p * GV_WAVES) * CH + kg * EL;
+                const int k = (wave + p * WV) * CH + kg * EL;
                 float part = 0.f;
 #pragma unroll
                 for (int e = 0; e < EL / 4; ++e) {
@@ -376,18 +378,18 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_decode_kernel(const T* __re
         }
         ss += __shfl_xor(ss, 16, WAVE);
         ss += __shfl_xor(ss, 32, WAVE);
-        __shared__ float ssum[GV_WAVES][16];
+        __shared__ float ssum[WV][16];
         if (kg == 0) ssum[wave][r] = ss;
         __syncthreads();
         float total = 0.f;
 #pragma unroll
-        for (int w = 0; w < GV_WAVES; ++w) total += ssum[w][r];
+        for (int w = 0; w < WV; ++w) total += ssum[w][r];
         const float inv = 1.0f / sqrtf(total / static_cast<float>(K) + norm.eps);
         Piece<T> xn[TRIPS][PT][1];
 #pragma unroll
         for (int p = 0; p < XP; ++p) {
             float f[EL];
-            const int kc = min((wave + p * GV_WAVES) * CH + kg * EL, K - EL);
+            const int kc = min((wave + p * WV) * CH + kg * EL, K - EL);
 #pragma unroll
             for (int e = 0; e < EL / 4; ++e) {
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f), wv = v;
@@ -415,7 +417,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_decode_kernel(const T* __re
         const T* xrow = x + static_cast<size_t>(row) * K;
         auto load_x = [&](int c, Piece<T> (&xb)[PT][1]) {
 #pragma unroll
-            for (int u = 0; u < PT; ++u) xb[u][0].load(xrow + min((c + u * GV_WAVES) * CH + kg * EL, K - EL));
+            for (int u = 0; u < PT; ++u) xb[u][0].load(xrow + min((c + u * WV) * CH + kg * EL, K - EL));
         };
         Piece<T> xb_a[PT][1], xb_b[PT][1];
         load_x(wave, xb_a);
@@ -426,7 +428,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_decode_kernel(const T* __re
             multiply(c + STRIDE, wa_b, xb_b);
         }
     }
-    skinny_finish<T, TOUT, 1, NT, EPI>(acc, y, M, N, I, rope);
+    skinny_finish<T, TOUT, 1, NT, EPI, WV>(acc, y, M, N, I, rope);
 }
 
 template <typename T, typename TOUT, int MB, int EPI>
@@ -466,7 +468,14 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
         constexpr int NTc = decltype(nt_tag)::value;
         constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
         const int grid = (tiles + NOUT - 1) / NOUT;
-        skinny_decode_kernel<T, TOUT, NTc, EPI, XP><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm);
+        if constexpr (XP == 0 && NTc == 1) {
+            // fewer workgroups than compute units and rows of 4,096 elements or more: sixteen wavefronts each
+            if (grid <= 160 && K >= 4096) {
+                skinny_decode_kernel<T, TOUT, NTc, EPI, XP, 16><<<grid, 16 * WAVE, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm);
+                return;
+            }
+        }
+        skinny_decode_kernel<T, TOUT, NTc, EPI, XP, GV_WAVES><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm);
     };
     if constexpr (EPI != EPI_ROPE) {
         if (NT >= 4) { run(std::integral_constant<int, 4>{}); return NI_LAUNCH_RESULT(); }
