@@ -85,7 +85,11 @@ class StepContext:
         t = self._q_tiles.get(tile_tokens)
         if t is None:
             flat = K.build_q_tiles(self.q_start, self.q_len, self.context_len, tile_tokens)
-            t = torch.tensor(flat, dtype=torch.int32).view(-1, 4).to(self.device)
+            upload = getattr(self._scratch_owner, "_upload", None)
+            if upload is not None:       # through the runner's pinned buffers: the host does not wait for the GPU
+                t = upload(flat).view(-1, 4)
+            else:
+                t = torch.tensor(flat, dtype=torch.int32).view(-1, 4).to(self.device)
             self._q_tiles[tile_tokens] = t
         return t
 
@@ -157,6 +161,27 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and self.model.graph_safe() and not os.environ.get("NANOINFER_NO_GRAPHS")
         self._recorded: Dict[tuple, _RecordedStep] = {}
         self._unrecordable = set()
+        self._staging = [(None, None)] * 3     # pinned host buffers for the tables of eager steps, and their uploads' events
+        self._staging_turn = 0
+
+    def _upload(self, flat: List[int]) -> torch.Tensor:
+        """The integer tables of an eager step on the device.  They go through one of a few pinned
+        host buffers used in turn, so that the copy is asynchronous and the host can prepare and
+        launch a step while the one before it still runs."""
+        n = len(flat)
+        i = self._staging_turn = (self._staging_turn + 1) % len(self._staging)
+        buf, done = self._staging[i]
+        if done is not None:
+            done.synchronize()            # the upload that last used this buffer has read it
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(n, 4096, 2 * (buf.numel() if buf is not None else 0)), dtype=torch.int32).pin_memory()
+        buf[:n] = torch.tensor(flat, dtype=torch.int32)
+        dev = torch.empty(n, dtype=torch.int32, device=self.device)
+        dev.copy_(buf[:n], non_blocking=True)
+        done = done or torch.cuda.Event()
+        done.record()
+        self._staging[i] = (buf, done)
+        return dev
 
     # ---------------------------------------------------------------- bookkeeping
     def computed_tokens(self, request: Hashable) -> int:
@@ -407,8 +432,7 @@ class ModelRunner:
             if totals is None:
                 ctx = StepContext(self.device, scratch_owner=self)
                 flat, layout, n_rows = self._describe(entries, ctx)
-                dev = torch.tensor(flat, dtype=torch.int32).to(self.device, non_blocking=False)
-                self._bind(ctx, dev, layout, n_rows)
+                self._bind(ctx, self._upload(flat), layout, n_rows)
                 logits = self.model.forward(ctx, self._layer_cache(ctx))
                 totals = ctx.context_len
             for e, total in zip(entries, totals):

@@ -69,7 +69,14 @@ def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> ctypes.c_void_p:
+    """The current stream of the current device as the kernels' launch argument (the raw handle is
+    asked for directly: building a Stream object costs more than a small kernel's launch)."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
@@ -79,12 +86,15 @@ def _need(cond: bool, msg: str) -> None:
 
 
 def _gpu(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
-    _need(t.is_cuda, f"{name} must live on the GPU (no CPU fallback exists)")
-    _need(t.is_contiguous(), f"{name} must be contiguous")
-    if dtype is not None:
-        _need(t.dtype == dtype, f"{name} must be {dtype}, is {t.dtype}")
-    if shape is not None:
-        _need(tuple(t.shape) == tuple(shape), f"{name} must have shape {tuple(shape)}, has {tuple(t.shape)}")
+    """Host-side check of one kernel operand; the message is built only when the check fails."""
+    if not t.is_cuda:
+        raise KernelError(f"{name} must live on the GPU (no CPU fallback exists)")
+    if not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, is {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name} must have shape {tuple(shape)}, has {tuple(t.shape)}")
 
 
 def _check(err: int, what: str) -> None:
@@ -153,17 +163,19 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[torc
     rot = 0
     if cos is not None:
         rot = 2 * cos.shape[1]
-        _need(rot <= hd, f"rotary size {rot} exceeds the head size {hd}")
+        if not (rot <= hd):
+            raise KernelError(f"rotary size {rot} exceeds the head size {hd}")
         _gpu(cos, "cos", torch.float32)
         _gpu(sin, "sin", torch.float32, cos.shape)
     page_size = 1
     if slot_mapping is not None:
         _gpu(slot_mapping, "slot_mapping", torch.int32, (T,))
-        _need(kpool is not None and vpool is not None, "a slot mapping needs both pools")
+        if not (kpool is not None and vpool is not None):
+            raise KernelError("a slot mapping needs both pools")
         _gpu(kpool, "kpool", qkv.dtype)
         _gpu(vpool, "vpool", qkv.dtype, kpool.shape)
-        _need(kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd,
-              f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
+        if not (kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd):
+            raise KernelError(f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
         page_size = kpool.shape[2]
     _check(core().ni_rope_kv_write(_ptr(qkv), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
                                    _ptr(kpool), _ptr(vpool), T, H, KVH, hd, rot, page_size,
@@ -173,7 +185,8 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[torc
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """``out = silu(gate_up[:, :I]) * gate_up[:, I:]``."""
     T, two_i = gate_up.shape
-    _need(two_i % 2 == 0, "gate_up needs an even width")
+    if not (two_i % 2 == 0):
+        raise KernelError("gate_up needs an even width")
     _gpu(gate_up, "gate_up")
     _gpu(out, "out", gate_up.dtype, (T, two_i // 2))
     _check(core().ni_swiglu(_ptr(gate_up), _ptr(out), T, two_i // 2, dtype_code(gate_up.dtype), _stream()), "swiglu")
@@ -202,22 +215,25 @@ def choose_splits(n_tokens: int, kv_heads: int, group: int, max_keys: int) -> in
 def _token_attention_checks(qkv, kpool, vpool, block_table, seq_of_token, positions, out, H, KVH, hd, nsplit, workspace):
     T = qkv.shape[0]
     _gpu(qkv, "qkv")
-    _need(qkv.shape[1] >= H * hd, "qkv is narrower than the query heads")
-    _need(H % KVH == 0, f"{H} query heads do not divide into {KVH} kv heads")
+    if not (qkv.shape[1] >= H * hd):
+        raise KernelError("qkv is narrower than the query heads")
+    if not (H % KVH == 0):
+        raise KernelError(f"{H} query heads do not divide into {KVH} kv heads")
     _gpu(kpool, "kpool", qkv.dtype)
     _gpu(vpool, "vpool", qkv.dtype, kpool.shape)
-    _need(kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd,
-          f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
+    if not (kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd):
+        raise KernelError(f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
     _gpu(block_table, "block_table", torch.int32)
-    _need(block_table.dim() == 2, "block_table must be [sequences, pages]")
+    if not (block_table.dim() == 2):
+        raise KernelError("block_table must be [sequences, pages]")
     _gpu(seq_of_token, "seq_of_token", torch.int32, (T,))
     _gpu(positions, "positions", torch.int32, (T,))
     _gpu(out, "out", qkv.dtype, (T, H * hd))
     part_o = part_ml = None
     if nsplit > 1:
         need = T * H * nsplit * (hd + 2)
-        _need(workspace is not None and workspace.dtype == torch.float32 and workspace.numel() >= need,
-              f"attention workspace of {need} floats needed for {nsplit} splits")
+        if not (workspace is not None and workspace.dtype == torch.float32 and workspace.numel() >= need):
+            raise KernelError(f"attention workspace of {need} floats needed for {nsplit} splits")
         _gpu(workspace, "workspace")
         flat = workspace.view(-1)
         part_o = flat[: T * H * nsplit * hd]
@@ -262,11 +278,14 @@ def mfma_token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Te
     """:func:`token_attention` on the matrix cores (bfloat16, head sizes that :func:`mfma_attention_ok`
     takes): the query heads of a kv head are the rows of the products, the wavefronts of a
     workgroup share out the keys."""
-    _need(mfma_attention_ok(qkv.dtype, hd), f"mfma_token_attention does not take {qkv.dtype} with head size {hd}")
-    _need(qkv.shape[1] % 8 == 0, "rows of qkv are not aligned to 16 bytes")
+    if not (mfma_attention_ok(qkv.dtype, hd)):
+        raise KernelError(f"mfma_token_attention does not take {qkv.dtype} with head size {hd}")
+    if not (qkv.shape[1] % 8 == 0):
+        raise KernelError("rows of qkv are not aligned to 16 bytes")
     T, part_o, part_ml = _token_attention_checks(qkv, kpool, vpool, block_table, seq_of_token, positions, out,
                                                  H, KVH, hd, nsplit, workspace)
-    _need(kpool.numel() // hd < 2 ** 32, "the matrix-core attention kernels number the rows of a pool in 32 bits")
+    if not (kpool.numel() // hd < 2 ** 32):
+        raise KernelError("the matrix-core attention kernels number the rows of a pool in 32 bits")
     _check(attention_mfma_lib(hd).ni_mfma_token_attention(
         _ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table), block_table.shape[1],
         _ptr(seq_of_token), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), T, H, KVH, kpool.shape[2],
@@ -316,23 +335,28 @@ def mfma_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
     ``workspace`` (float32, ``T*H*nsplit*(hd+2)`` elements) is needed when ``nsplit > 1``."""
     T = qkv.shape[0]
     _gpu(qkv, "qkv", torch.bfloat16)
-    _need(mfma_attention_ok(qkv.dtype, hd), f"mfma_attention does not take {qkv.dtype} with head size {hd}")
-    _need(qkv.shape[1] >= H * hd and qkv.shape[1] % 8 == 0, "qkv is narrower than the query heads or its rows are unaligned")
-    _need(H % KVH == 0, f"{H} query heads do not divide into {KVH} kv heads")
+    if not (mfma_attention_ok(qkv.dtype, hd)):
+        raise KernelError(f"mfma_attention does not take {qkv.dtype} with head size {hd}")
+    if not (qkv.shape[1] >= H * hd and qkv.shape[1] % 8 == 0):
+        raise KernelError("qkv is narrower than the query heads or its rows are unaligned")
+    if not (H % KVH == 0):
+        raise KernelError(f"{H} query heads do not divide into {KVH} kv heads")
     _gpu(kpool, "kpool", torch.bfloat16)
     _gpu(vpool, "vpool", torch.bfloat16, kpool.shape)
-    _need(kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd,
-          f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
-    _need(kpool.numel() // hd < 2 ** 32, "the matrix-core attention kernels number the rows of a pool in 32 bits")
+    if not (kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd):
+        raise KernelError(f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
+    if not (kpool.numel() // hd < 2 ** 32):
+        raise KernelError("the matrix-core attention kernels number the rows of a pool in 32 bits")
     _gpu(block_table, "block_table", torch.int32)
     _gpu(tiles, "tiles", torch.int32)
-    _need(tiles.dim() == 2 and tiles.shape[1] == 4, "tiles must be [n, 4]")
+    if not (tiles.dim() == 2 and tiles.shape[1] == 4):
+        raise KernelError("tiles must be [n, 4]")
     _gpu(out, "out", torch.bfloat16, (T, H * hd))
     part_o = part_ml = None
     if nsplit > 1:
         need = T * H * nsplit * (hd + 2)
-        _need(workspace is not None and workspace.dtype == torch.float32 and workspace.numel() >= need,
-              f"attention workspace of {need} floats needed for {nsplit} splits")
+        if not (workspace is not None and workspace.dtype == torch.float32 and workspace.numel() >= need):
+            raise KernelError(f"attention workspace of {need} floats needed for {nsplit} splits")
         _gpu(workspace, "workspace")
         flat = workspace.view(-1)
         part_o = flat[: T * H * nsplit * hd]
@@ -406,10 +430,11 @@ class Weight:
     """A matrix [out, in] as the products want it: ``rows`` as stored (for the library product of
     many rows) and, optionally, ``tiles`` in the order the skinny product streams it."""
 
-    __slots__ = ("rows", "tiles")
+    __slots__ = ("rows", "tiles", "rows_t")
 
     def __init__(self, rows: torch.Tensor, tiled: bool = True):
         self.rows = rows
+        self.rows_t = rows.t()        # the view the library product takes, made once
         self.tiles = tile_weight(rows) if tiled and rows.dtype in (torch.float32, torch.bfloat16) else None
 
     @property
@@ -484,7 +509,8 @@ def residual_epilogue_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
 
 def _check_normed(x: NormedInput, Kd: int) -> None:
     _gpu(x.h, "h", torch.float32)
-    _need(x.h.dim() == 2 and x.h.shape[1] == Kd, f"normed input {tuple(x.h.shape)} against K={Kd}")
+    if not (x.h.dim() == 2 and x.h.shape[1] == Kd):
+        raise KernelError(f"normed input {tuple(x.h.shape)} against K={Kd}")
     _gpu(x.weight, "norm weight", torch.float32, (Kd,))
 
 
@@ -500,27 +526,33 @@ def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bo
     rows, tiles = _rows_and_tiles(weight)
     N = rows.shape[0]
     _gpu(rows, "weight", dtype)
-    _need(rows.shape[1] == Kd, f"skinny_gemm: {tuple(x.shape)} x {tuple(rows.shape)}^T")
-    _need(skinny_ok(M, Kd, dtype), f"skinny_gemm does not take M={M}, K={Kd} in {dtype}")
+    if not (rows.shape[1] == Kd):
+        raise KernelError(f"skinny_gemm: {tuple(x.shape)} x {tuple(rows.shape)}^T")
+    if not (skinny_ok(M, Kd, dtype)):
+        raise KernelError(f"skinny_gemm does not take M={M}, K={Kd} in {dtype}")
     if swiglu and tiles is not None and (N // 2) % 16:
         tiles = None          # gate and up halves do not start on tile boundaries: stream the rows as stored
     if swiglu:
-        _need(N % 2 == 0, "a stacked gate/up matrix needs an even number of rows")
-        _need(not residual, "swiglu and residual exclude each other")
+        if not (N % 2 == 0):
+            raise KernelError("a stacked gate/up matrix needs an even number of rows")
+        if not (not residual):
+            raise KernelError("swiglu and residual exclude each other")
         _gpu(out, "out", dtype, (M, N // 2))
         epi = 2
     elif residual:
-        _need(tiles is not None and M <= 16, "the residual epilogue needs a re-tiled matrix and at most 16 rows")
+        if not (tiles is not None and M <= 16):
+            raise KernelError("the residual epilogue needs a re-tiled matrix and at most 16 rows")
         _gpu(out, "out", torch.float32, (M, N))
         epi = 3
     else:
-        _need(out.dtype in (dtype, torch.float32), f"out must be {dtype} or float32")
+        if not (out.dtype in (dtype, torch.float32)):
+            raise KernelError(f"out must be {dtype} or float32")
         _gpu(out, "out", None, (M, N))
         epi = 1 if (out.dtype == torch.float32 and dtype != torch.float32) else 0
     per_group = _tiles_per_group(N // 2 if swiglu else N)
     if normed:
-        _need(tiles is not None and norm_prologue_ok(M, Kd, dtype, weight) and epi in (0, 2),
-              f"the normalising prologue does not take M={M}, K={Kd} in {dtype} with this matrix and epilogue")
+        if not (tiles is not None and norm_prologue_ok(M, Kd, dtype, weight) and epi in (0, 2)):
+            raise KernelError(f"the normalising prologue does not take M={M}, K={Kd} in {dtype} with this matrix and epilogue")
         _check_normed(x, Kd)
         _check(skinny_lib().ni_skinny_gemm_normed(_ptr(x.h), _ptr(x.weight), ctypes.c_float(x.eps), _ptr(tiles), _ptr(out),
                                                   M, N, Kd, epi, per_group, dtype_code(dtype), _stream()),
@@ -549,7 +581,8 @@ def skinny_qkv_rope(x, w_qkv, positions: torch.Tensor, cos: torch.Tensor,
     dtype = x.dtype
     rows, tiles = _rows_and_tiles(w_qkv)
     _gpu(rows, "w_qkv", dtype, ((H + 2 * KVH) * hd, Kd))
-    _need(qkv_rope_ok(M, Kd, hd, 2 * cos.shape[1], dtype), f"skinny_qkv_rope does not take M={M}, K={Kd}, hd={hd}")
+    if not (qkv_rope_ok(M, Kd, hd, 2 * cos.shape[1], dtype)):
+        raise KernelError(f"skinny_qkv_rope does not take M={M}, K={Kd}, hd={hd}")
     _gpu(positions, "positions", torch.int32, (M,))
     _gpu(cos, "cos", torch.float32)
     _gpu(sin, "sin", torch.float32, cos.shape)
@@ -558,11 +591,12 @@ def skinny_qkv_rope(x, w_qkv, positions: torch.Tensor, cos: torch.Tensor,
         _gpu(slot_mapping, "slot_mapping", torch.int32, (M,))
         _gpu(kpool, "kpool", dtype)
         _gpu(vpool, "vpool", dtype, kpool.shape)
-        _need(kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd,
-              f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
+        if not (kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd):
+            raise KernelError(f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
         page_size = kpool.shape[2]
     if normed:
-        _need(norm_prologue_ok(M, Kd, dtype, w_qkv), f"the normalising prologue does not take M={M}, K={Kd} in {dtype}")
+        if not (norm_prologue_ok(M, Kd, dtype, w_qkv)):
+            raise KernelError(f"the normalising prologue does not take M={M}, K={Kd} in {dtype}")
         _check_normed(x, Kd)
         x_ptr, h_ptr, nw_ptr, eps = None, _ptr(x.h), _ptr(x.weight), x.eps
         device = x.h.device
@@ -588,26 +622,31 @@ def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optiona
     nothing is returned."""
     rows, _ = _rows_and_tiles(weight)
     if isinstance(x, NormedInput):
-        _need(residual is None, "a normed input and a residual output in one product are not compiled")
+        if not (residual is None):
+            raise KernelError("a normed input and a residual output in one product are not compiled")
         out = torch.empty(x.shape[0], rows.shape[0], dtype=x.dtype, device=x.device)
         return skinny_gemm(x, weight, out)
-    _need(x.is_cuda and rows.is_cuda, "linear needs GPU tensors")
-    _need(x.dtype == rows.dtype, f"linear: activation {x.dtype} and weight {rows.dtype} differ")
-    _need(x.dim() == 2 and x.shape[1] == rows.shape[1], f"linear: {tuple(x.shape)} x {tuple(rows.shape)}^T")
+    if not (x.is_cuda and rows.is_cuda):
+        raise KernelError("linear needs GPU tensors")
+    if not (x.dtype == rows.dtype):
+        raise KernelError(f"linear: activation {x.dtype} and weight {rows.dtype} differ")
+    if not (x.dim() == 2 and x.shape[1] == rows.shape[1]):
+        raise KernelError(f"linear: {tuple(x.shape)} x {tuple(rows.shape)}^T")
     if residual is not None:
-        _need(residual_epilogue_ok(x.shape[0], x.shape[1], x.dtype, weight), "the residual epilogue does not take this product")
+        if not (residual_epilogue_ok(x.shape[0], x.shape[1], x.dtype, weight)):
+            raise KernelError("the residual epilogue does not take this product")
         skinny_gemm(x, weight, residual, residual=True)
         return None
     out_dtype = out_dtype or x.dtype
     if x.shape[0] <= SKINNY_BEST_ROWS and skinny_ok(x.shape[0], x.shape[1], x.dtype):
         out = torch.empty(x.shape[0], rows.shape[0], dtype=out_dtype, device=x.device)
         return skinny_gemm(x, weight, out)
-    weight = rows
+    rows_t = weight.rows_t if isinstance(weight, Weight) else rows.t()
     global _library_calls
     _library_calls += 1
     if out_dtype != x.dtype:
-        return torch.mm(x, weight.t(), out_dtype=out_dtype)
-    return torch.matmul(x, weight.t())
+        return torch.mm(x, rows_t, out_dtype=out_dtype)
+    return torch.mm(x, rows_t)
 
 
 def linear_swiglu(x, weight_gate_up) -> torch.Tensor:
@@ -619,8 +658,8 @@ def linear_swiglu(x, weight_gate_up) -> torch.Tensor:
         return skinny_gemm(x, weight_gate_up, out, swiglu=True)
     global _library_calls
     _library_calls += 1
-    rows, _ = _rows_and_tiles(weight_gate_up)
-    return swiglu(torch.matmul(x, rows.t()), out)
+    rows_t = weight_gate_up.rows_t if isinstance(weight_gate_up, Weight) else weight_gate_up.t()
+    return swiglu(torch.mm(x, rows_t), out)
 
 
 def require_gpu() -> torch.device:
