@@ -1,0 +1,49 @@
+"""The layer sizes of the Llama 3 family (two layers each, random weights) through the engine's
+step function against the plain implementation: a prompt in one portion and in two, then single
+tokens one by one (recorded steps), in float32 and bfloat16.  These are the hidden widths, head
+sizes and groups at which the kernels' other code paths run: head size 128, rows of 3,072 and
+4,096 elements (too long for the norm prologue in bfloat16, so the separate norm kernel runs),
+three query heads per kv head, an intermediate size of 14,336, the family's vocabulary."""
+import pytest
+import torch
+
+from gpu_common import assert_close, model_folder, plain_logits, random_tokens
+from tiny_configs import ALL
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["1B", "3B", "8B"])
+def test_family_layer_sizes(name, dtype):
+    from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
+
+    folder = model_folder(name, stored="bfloat16" if dtype == "bfloat16" else "float32")
+    vocab = ALL[name]["vocab_size"]
+    a = random_tokens(vocab, 75, 11)
+    b = random_tokens(vocab, 41, 12)
+    runner = ModelRunner(folder, dtype=dtype, page_size=16, max_tokens=256, max_requests=4)
+    got_a, got_b = {}, {}
+    # a: 60 tokens as one portion; b: 20 + 13 tokens in two steps, the second beside single tokens of a
+    out = runner.step([StepEntry("a", a[:60], list(range(60))), StepEntry("b", b[:20], [0, 19])])
+    for i in range(60):
+        got_a[i] = out[i]
+    got_b[0], got_b[19] = out[60], out[61]
+    out = runner.step([StepEntry("a", [a[60]], [0]), StepEntry("b", b[20:33], list(range(13)))])
+    got_a[60] = out[0]
+    for i in range(13):
+        got_b[20 + i] = out[1 + i]
+    # then both one token at a time, in the same batch: recorded decode steps
+    for i in range(8):
+        out = runner.step([StepEntry("a", [a[61 + i]], [0]), StepEntry("b", [b[33 + i]], [0])])
+        got_a[61 + i], got_b[33 + i] = out[0].clone(), out[1].clone()
+    # a alone to its end
+    for i in range(69, 75):
+        out = runner.step([StepEntry("a", [a[i]], [0])])
+        got_a[i] = out[0].clone()
+    runner.release("a"), runner.release("b")
+    runner.cache.check()
+    for tokens, got, rid in ((a, got_a, "a"), (b[:41], got_b, "b")):
+        want = plain_logits(folder, tuple(tokens), dtype)
+        idx = sorted(got)
+        assert_close(torch.stack([got[i] for i in idx]), want[idx], dtype, f"{name} {dtype} request {rid}")

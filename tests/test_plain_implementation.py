@@ -9,7 +9,7 @@ import torch
 import torch.nn.functional as F
 
 import plain_llama as P
-from tiny_configs import ALL, TINY_A, TINY_B
+from tiny_configs import TINY, TINY_A, TINY_B
 
 F64 = torch.float64
 
@@ -263,12 +263,12 @@ def vectorised_forward(config, tensors, tokens):
     return F.linear(h, head)
 
 
-@pytest.mark.parametrize("name", sorted(ALL))
+@pytest.mark.parametrize("name", sorted(TINY))
 def test_whole_model_two_ways(name, tmp_path):
     import nanoinfer_amd  # noqa: F401
     from nanoinfer_amd.weights.loader import make_random_model
 
-    make_random_model(str(tmp_path), ALL[name], seed=5, dtype="float32")
+    make_random_model(str(tmp_path), TINY[name], seed=5, dtype="float32")
     config, tensors = P.read_model_folder(str(tmp_path))
     g = torch.Generator().manual_seed(9)
     tokens = torch.randint(0, config["vocab_size"], (23,), generator=g).tolist()

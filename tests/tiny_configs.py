@@ -31,4 +31,27 @@ TINY_C = {
     "max_position_embeddings": 640, "tie_word_embeddings": True, "hidden_act": "silu",
 }
 
-ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+
+
+def _family(hidden, heads, kv_heads, head_dim, inter, vocab, factor, tied):
+    return {
+        "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+        "hidden_size": hidden, "num_hidden_layers": 2, "num_attention_heads": heads, "num_key_value_heads": kv_heads,
+        "head_dim": head_dim, "intermediate_size": inter, "vocab_size": vocab, "rms_norm_eps": 1e-5,
+        "rope_theta": 500000.0,
+        "rope_scaling": {"rope_type": "llama3", "factor": factor, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                         "original_max_position_embeddings": 8192},
+        "max_position_embeddings": 131072, "tie_word_embeddings": tied, "hidden_act": "silu",
+        "bos_token_id": 128000, "eos_token_id": 128001,
+    }
+
+
+# The layer sizes of the Llama 3 family (3.2 1B, 3.2 3B, 3.1 8B), two layers each: the widths, head
+# sizes and groups that the kernels meet in use.  1B keeps the family's vocabulary; the other two
+# a smaller, odd one, to keep the files small.
+FAMILY_1B = _family(2048, 32, 8, 64, 8192, 128256, 32.0, True)
+FAMILY_3B = _family(3072, 24, 8, 128, 8192, 16033, 32.0, True)
+FAMILY_8B = _family(4096, 32, 8, 128, 14336, 16033, 8.0, False)
+
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+ALL = {**TINY, "1B": FAMILY_1B, "3B": FAMILY_3B, "8B": FAMILY_8B}
