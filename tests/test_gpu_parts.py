@@ -1,6 +1,7 @@
 """Each part alone, built from a spec as the model builds it, against the plain functions; the
-order of layers as data; and a toy mixer with state of its own that is registered, built and
-stepped from here, without a change to the framework's files."""
+order of layers as data; and toy parts that are registered, built and stepped from here without a
+change to the framework's files: a mixer with state of its own, a feed-forward with routing beside
+a dense one, another position encoding."""
 import math
 
 import pytest
@@ -84,10 +85,15 @@ def test_position_part_shares_one_table():
 
 # ------------------------------------------------------------------ a model from a spec written here
 
-def tiny_spec(mixer_kinds, order, d=64, H=4, KVH=2, hd=16, I=96, V=128, window=None, position="rope", state_size=None):
+def tiny_spec(mixer_kinds, order, d=64, H=4, KVH=2, hd=16, I=96, V=128, window=None, position="rope", state_size=None,
+              ffn_kinds=None, experts=3):
     from nanoinfer_amd.config.spec import BlockSpec, LayerRun, ModelSpec, PartSpec
-    pos = PartSpec("rope", {"rotary_dim": hd, "theta": 10000.0, "scaling": None, "max_positions": 256}) \
-        if position == "rope" else PartSpec("none")
+    if position == "rope":
+        pos = PartSpec("rope", {"rotary_dim": hd, "theta": 10000.0, "scaling": None, "max_positions": 256})
+    elif position == "none":
+        pos = PartSpec("none")
+    else:       # a position encoding registered by a test: the same constants, its own kind
+        pos = PartSpec(position, {"rotary_dim": hd, "theta": 10000.0, "max_positions": 256})
     blocks = []
     for i, kind in enumerate(mixer_kinds):
         pre = f"L{i}."
@@ -97,10 +103,14 @@ def tiny_spec(mixer_kinds, order, d=64, H=4, KVH=2, hd=16, I=96, V=128, window=N
                              {"q": pre + "q", "k": pre + "k", "v": pre + "v", "o": pre + "o"})
         else:
             mixer = PartSpec(kind, {"hidden_size": d, "state_size": state_size}, {"inp": pre + "inp", "out": pre + "out"})
+        if ffn_kinds is None or ffn_kinds[i] == "swiglu":
+            ffn = PartSpec("swiglu", {"hidden_size": d, "intermediate_size": I},
+                           {"gate": pre + "g", "up": pre + "u", "down": pre + "d"})
+        else:
+            ffn = PartSpec(ffn_kinds[i], {"hidden_size": d, "intermediate_size": I, "experts": experts},
+                           {"router": pre + "router", "w1": pre + "w1", "w2": pre + "w2"})
         blocks.append(BlockSpec("prenorm", PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": pre + "n1"}), mixer,
-                                PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": pre + "n2"}),
-                                PartSpec("swiglu", {"hidden_size": d, "intermediate_size": I},
-                                         {"gate": pre + "g", "up": pre + "u", "down": pre + "d"})))
+                                PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": pre + "n2"}), ffn))
     return ModelSpec(V, d, 256, PartSpec("table", {"vocab_size": V, "hidden_size": d}, {"weight": "emb"}), blocks,
                      [LayerRun(*o) for o in order], PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": "nf"}),
                      PartSpec("linear", {"vocab_size": V, "hidden_size": d}, {"weight": "emb"}))
@@ -135,7 +145,7 @@ class SpecRunner:
         return r
 
 
-def plain_spec_forward(spec, tensors, tokens, extra_mixers=None):
+def plain_spec_forward(spec, tensors, tokens, extra_mixers=None, extra_ffns=None, extra_positions=None):
     """The plain implementation applied to a spec: same functions, parts chosen by the spec."""
     T = len(tokens)
     t64 = {k: v.double() for k, v in tensors.items()}
@@ -158,6 +168,11 @@ def plain_spec_forward(spec, tensors, tokens, extra_mixers=None):
                 q = P.rope_interleaved(q, s, c)
                 if run.writes_cache:
                     k = P.rope_interleaved(k, s, c)
+            elif p["position"].kind != "none":
+                s, c = extra_positions[p["position"].kind](T, p["position"].params)
+                q = P.rope_interleaved(q, s, c)
+                if run.writes_cache:
+                    k = P.rope_interleaved(k, s, c)
             if run.writes_cache:
                 kv[run.cache] = (k, v)
             k, v = kv[run.cache]
@@ -167,7 +182,10 @@ def plain_spec_forward(spec, tensors, tokens, extra_mixers=None):
         h = h + a
         x = P.rmsnorm(h, t64[b.ffn_norm.weights["weight"]], b.ffn_norm.params["eps"])
         f = b.ffn
-        h = h + P.linear(P.swiglu(P.linear(x, t64[f.weights["gate"]]), P.linear(x, t64[f.weights["up"]])), t64[f.weights["down"]])
+        if f.kind == "swiglu":
+            h = h + P.linear(P.swiglu(P.linear(x, t64[f.weights["gate"]]), P.linear(x, t64[f.weights["up"]])), t64[f.weights["down"]])
+        else:
+            h = h + extra_ffns[f.kind](x, t64, f)
     return P.linear(P.rmsnorm(h, t64[spec.final_norm.weights["weight"]], spec.final_norm.params["eps"]),
                     t64[spec.head.weights["weight"]])
 
@@ -310,3 +328,138 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped():
     assert rel(out, want["r"]) < TOL["float32"]
     runner.cache.check()
     assert runner.cache.slots.num_free == 4
+
+
+# ------------------------------------------------------------------ a toy feed-forward with routing
+
+def register_toy_routed_ffn():
+    from nanoinfer_amd.parts.base import Part, WeightRequest
+    from nanoinfer_amd.registry import register_part
+
+    @register_part("feed_forward", "toy_routed")
+    class ToyRoutedFeedForward(Part):
+        """Every token goes to the one expert whose router logit (float32) is largest and is scaled by
+        the softmax weight of that logit: y = p_e * W2_e relu(W1_e x).  Library tensor operations: it
+        shows that a feed-forward with routing fits the interface, it is no product kernel."""
+
+        @classmethod
+        def weight_requests(cls, spec):
+            d, i, e = spec.params["hidden_size"], spec.params["intermediate_size"], spec.params["experts"]
+            return [WeightRequest(spec.weights["router"], (e, d)), WeightRequest(spec.weights["w1"], (e * i, d)),
+                    WeightRequest(spec.weights["w2"], (e * d, i))]
+
+        def __init__(self, spec, weights, rt):
+            super().__init__(spec, weights, rt)
+            p = spec.params
+            self.d, self.i, self.e = p["hidden_size"], p["intermediate_size"], p["experts"]
+            self.router = rt.vector32(spec.weights["router"], weights["router"].reshape(-1)).view(self.e, self.d)
+            self.w1 = rt.matrix(spec.weights["w1"], weights["w1"]).view(self.e, self.i, self.d)
+            self.w2 = rt.matrix(spec.weights["w2"], weights["w2"]).view(self.e, self.d, self.i)
+
+        def forward(self, x, ctx):
+            logits = x.float() @ self.router.t()
+            prob = torch.softmax(logits, dim=-1)
+            choice = logits.argmax(dim=-1)
+            y = torch.zeros(x.shape[0], self.d, dtype=torch.float32, device=x.device)
+            for e in range(self.e):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    hidden = torch.relu(x[rows] @ self.w1[e].t())
+                    y[rows] = (hidden @ self.w2[e].t()).float() * prob[rows, e:e + 1]
+            return y.to(x.dtype)
+
+    return ToyRoutedFeedForward
+
+
+def plain_routed(x, t64, f):
+    p = f.params
+    d, i, e = p["hidden_size"], p["intermediate_size"], p["experts"]
+    router, w1, w2 = t64[f.weights["router"]], t64[f.weights["w1"]].view(e, i, d), t64[f.weights["w2"]].view(e, d, i)
+    logits = P.linear(x, router)
+    prob = torch.softmax(logits, dim=-1)
+    rows = []
+    for t in range(x.shape[0]):
+        c = int(logits[t].argmax())
+        rows.append(P.linear(torch.relu(P.linear(x[t:t + 1], w1[c])), w2[c])[0] * prob[t, c])
+    return torch.stack(rows)
+
+
+def test_toy_feed_forward_with_routing_beside_a_dense_one():
+    """One model whose first layer has a routed feed-forward defined here and whose second has the
+    framework's dense one: chosen per layer by the spec, stepped in portions and token by token
+    through the framework's step function without a change to its files."""
+    register_toy_routed_ffn()
+    spec = tiny_spec(["attention", "attention"], [(0, 0), (1, 1)], ffn_kinds=["toy_routed", "swiglu"], experts=3)
+    tensors = random_tensors(spec, 9)
+    tensors["L0.router"] = tensors["L0.router"] * 8          # decided choices: no token sits on a tie
+    tokens = list(random_tokens(128, 50, 4))
+    want = plain_spec_forward(spec, tensors, tokens, extra_ffns={"toy_routed": plain_routed})
+    choices = P.linear(P.rmsnorm(P.embedding(tensors["emb"].double(), tokens), tensors["L0.n1"].double(), 1e-5),
+                       tensors["L0.router"].double()).argmax(-1)
+    runner = SpecRunner(spec, tensors, "float32")
+    assert not runner.use_graphs                           # a part that does not declare itself graph-safe keeps the steps eager
+    for sizes in ([50], [9, 2, 1, 1, 17, 1]):
+        got = step_in_portions(runner, tokens, sizes)
+        assert rel(got, want) < TOL["float32"], sizes
+    assert len(set(choices.tolist())) >= 2                  # the tokens do go to different experts
+    runner.cache.check()
+
+
+# ------------------------------------------------------------------ a toy position encoding
+
+def register_toy_position():
+    from nanoinfer_amd.parts.base import Part
+    from nanoinfer_amd.registry import register_part
+
+    @register_part("position", "toy_sqrt")
+    class SquareRootPosition(Part):
+        """Rotation by sqrt(pos) * f_p instead of pos * f_p: another position encoding of the rotating
+        kind, given to the attention part as tables of its own."""
+
+        graph_safe = True
+
+        def __init__(self, spec, weights, rt):
+            super().__init__(spec, weights, rt)
+            p = spec.params
+            self.max_positions = int(p["max_positions"])
+            half = p["rotary_dim"] // 2
+            freq = torch.tensor([p["theta"] ** (-2.0 * j / p["rotary_dim"]) for j in range(half)], dtype=torch.float64)
+            angle = torch.arange(self.max_positions, dtype=torch.float64).sqrt()[:, None] * freq[None]
+            self.cos = angle.cos().float().to(rt.device).contiguous()
+            self.sin = angle.sin().float().to(rt.device).contiguous()
+
+        def tables(self):
+            return self.cos, self.sin
+
+    return SquareRootPosition
+
+
+def plain_sqrt_tables(T, params):
+    half = params["rotary_dim"] // 2
+    freq = torch.tensor([params["theta"] ** (-2.0 * j / params["rotary_dim"]) for j in range(half)], dtype=torch.float64)
+    angle = torch.arange(T, dtype=torch.float64).sqrt()[:, None] * freq[None]
+    return angle.sin(), angle.cos()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_position_encoding_feeds_the_attention_part(dtype):
+    """A position encoding registered here (angles sqrt(pos) * f) drives the framework's attention
+    part, its fused rotation epilogue and its recorded decode steps unchanged: only tables differ."""
+    from nanoinfer_amd.engine.runner import StepEntry
+    register_toy_position()
+    spec = tiny_spec(["attention", "attention"], [(0, 0), (1, 1)], hd=32, H=2, KVH=1, position="toy_sqrt")
+    tensors = random_tensors(spec, 12)
+    if dtype == "bfloat16":
+        tensors = {k: (v.to(torch.bfloat16).float() if v.dim() == 2 else v) for k, v in tensors.items()}
+    tokens = list(random_tokens(128, 40, 5))
+    want = plain_spec_forward(spec, tensors, tokens, extra_positions={"toy_sqrt": plain_sqrt_tables})
+    runner = SpecRunner(spec, tensors, dtype)
+    assert runner.use_graphs
+    outs = [runner.step([StepEntry("s", tokens[:25], list(range(25)))])]
+    for t in tokens[25:]:
+        outs.append(runner.step([StepEntry("s", [t], [0])]).clone())
+    runner.release("s")
+    assert rel(torch.cat(outs), want) < TOL[dtype]
+    # and it is no rope in disguise: the framework's own rotation gives other logits
+    other = tiny_spec(["attention", "attention"], [(0, 0), (1, 1)], hd=32, H=2, KVH=1, position="rope")
+    assert rel(plain_spec_forward(other, tensors, tokens), want) > 10 * TOL[dtype]
