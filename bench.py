@@ -72,6 +72,19 @@ def prefill_flops(cfg: dict, tokens: int) -> float:
     return linear + attention + 2.0 * V * d
 
 
+def config_record(cfg: dict, layers: int, batch: int, mean_ctx: float, prefill_chunk: int) -> dict:
+    """Every size of the measured configuration, flat (nothing nested, at most 20 keys)."""
+    return {
+        "model": "llama-3.2-1b-shape", "layers": layers, "layers_full_model": FULL_LAYERS,
+        "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
+        "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+        "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
+        "tied_embeddings": True, "global_batch": batch, "prompt_len": PROMPT_LEN,
+        "seq_len": CONTEXT_LEN, "decode_context_mean": round(mean_ctx, 1), "kv_block_size": BLOCK_SIZE,
+        "prefill_chunk": prefill_chunk, "parallelism": "single-gpu",
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -197,15 +210,7 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": args.dtype,
         "data": "synthetic: random weights (seed 0), uniform random token ids",
-        "config": {
-            "model": "llama-3.2-1b-shape", "layers": args.layers, "layers_full_model": FULL_LAYERS,
-            "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
-            "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
-            "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
-            "tied_embeddings": True, "global_batch": args.batch, "prompt_len": PROMPT_LEN,
-            "seq_len": CONTEXT_LEN, "decode_context_mean": round(mean_ctx, 1), "kv_block_size": BLOCK_SIZE,
-            "prefill_chunk": args.prefill_chunk, "parallelism": "single-gpu",
-        },
+        "config": config_record(cfg, args.layers, args.batch, mean_ctx, args.prefill_chunk),
         "prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(flops / prefill_s / FLOP_PEAK[args.dtype], 4)},
         "prefill_one_portion": {"value": round(PROMPT_LEN / whole_s, 1), "tokens": PROMPT_LEN, "ms": round(whole_s * 1e3, 3),
