@@ -281,7 +281,12 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
 // XP > 0: x = RMSNorm(h) with the wavefront's XP pieces of the normalised row kept in registers.
 // WV wavefronts split K: 8, or 16 for a matrix of few tiles and long rows, whose workgroups are too
 // few to fill the chip and have to keep more loads in flight each.
-template <typename T, typename TOUT, int NT, int EPI, int XP, int WV>
+// SR > 0 (with XP > 0): the prologue is staged through LDS for up to SR rows.  A vector load costs
+// the texture path the same time whatever it fetches, and the operand layout spreads a row over
+// few lanes: read in that layout, h and the norm's weights take twice the load instructions of W
+// itself.  Staged, the workgroup reads every element once with full loads, normalises, rounds, and
+// leaves the rows in LDS, from where the lanes pick their operands.
+template <typename T, typename TOUT, int NT, int EPI, int XP, int WV, int SR>
 __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                                    TOUT* __restrict__ y, int M, int N, int K, int I,
                                                                    RopeArgs rope, NormArgs norm) {
@@ -344,65 +349,135 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
         // under the shadow of W.  Lanes whose row does not exist load and compute nothing.
         constexpr int TRIPS = XP / PT;
         static_assert(XP % PT == 0, "whole trips");
-        const float* hrow = norm.h + static_cast<size_t>(row) * K;
-        const bool live = r < M;
-        constexpr bool KEEP = XP * EL <= 64;        // the row's elements wait in registers, or are read a second time
-        float4 hraw[XP][EL / 4], wraw[KEEP ? XP : 1][EL / 4];
-        if (live) {
+        Piece<T> xn[TRIPS][PT][1];
+        if constexpr (SR > 0) {
+            constexpr int THREADS = WV * WAVE;
+            constexpr int KMAX = XP * WV * CH;                 // elements of a row that the compiled size covers
+            constexpr int QPT = (KMAX / 4 + THREADS - 1) / THREADS;      // groups of four columns per thread
+            constexpr int XROW = KMAX + 16 / sizeof(T);        // 16 bytes of padding: rows start on different banks
+            __shared__ __attribute__((aligned(16))) T xs[SR][XROW];
+            __shared__ float ssum[WV][SR];
+            __shared__ float sinv[SR];
+            float4 hv[SR][QPT], wv[QPT];
+#pragma unroll
+            for (int q = 0; q < QPT; ++q) {
+                const int k = 4 * (tid + q * THREADS);
+                const bool in = k < K;
+                wv[q] = in ? *reinterpret_cast<const float4*>(norm.weight + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int m = 0; m < SR; ++m)
+                    hv[m][q] = (m < M && in) ? *reinterpret_cast<const float4*>(norm.h + static_cast<size_t>(m) * K + k)
+                                             : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+            // loads come back in the order they went out: the few of the prologue first, W right behind
+            __builtin_amdgcn_sched_barrier(0);
+            load_w(wave, wa_a);
+            __builtin_amdgcn_sched_barrier(0);
+            // all SR rows go through the same straight code (rows that do not exist are zeros): the
+            // reductions of the rows then overlap instead of waiting for one another behind branches
+            float ss[SR];
+#pragma unroll
+            for (int m = 0; m < SR; ++m) {
+                ss[m] = 0.f;
+#pragma unroll
+                for (int q = 0; q < QPT; ++q)
+                    ss[m] += hv[m][q].x * hv[m][q].x + hv[m][q].y * hv[m][q].y + hv[m][q].z * hv[m][q].z + hv[m][q].w * hv[m][q].w;
+            }
+#pragma unroll
+            for (int off = WAVE / 2; off > 0; off >>= 1)
+#pragma unroll
+                for (int m = 0; m < SR; ++m) ss[m] += __shfl_xor(ss[m], off, WAVE);
+            if (lane < SR) {
+                float mine = ss[0];
+#pragma unroll
+                for (int m = 1; m < SR; ++m) mine = lane == m ? ss[m] : mine;
+                ssum[wave][lane] = mine;
+            }
+            __syncthreads();
+            if (tid < SR) {
+                float total = 0.f;
+#pragma unroll
+                for (int w = 0; w < WV; ++w) total += ssum[w][tid];
+                sinv[tid] = 1.0f / sqrtf(total / static_cast<float>(K) + norm.eps);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int q = 0; q < QPT; ++q) {
+                const int k = 4 * (tid + q * THREADS);
+                if (k < K) {
+#pragma unroll
+                    for (int m = 0; m < SR; ++m) {
+                        const float inv = sinv[m];
+                        const float f[4] = {(hv[m][q].x * inv) * wv[q].x, (hv[m][q].y * inv) * wv[q].y,
+                                            (hv[m][q].z * inv) * wv[q].z, (hv[m][q].w * inv) * wv[q].w};
+                        VecIO<T, 4>::store(&xs[m][k], f);
+                    }
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int p = 0; p < XP; ++p)
+                xn[p / PT][p % PT][0].load(&xs[row][min((wave + p * WV) * CH + kg * EL, K - EL)]);
+        } else {
+            const float* hrow = norm.h + static_cast<size_t>(row) * K;
+            const bool live = r < M;
+            constexpr bool KEEP = XP * EL <= 64;        // the row's elements wait in registers, or are read a second time
+            float4 hraw[XP][EL / 4], wraw[KEEP ? XP : 1][EL / 4];
+            if (live) {
+#pragma unroll
+                for (int p = 0; p < XP; ++p) {
+                    const int kc = min((wave + p * WV) * CH + kg * EL, K - EL);
+#pragma unroll
+                    for (int e = 0; e < EL / 4; ++e) {
+                        hraw[p][e] = *reinterpret_cast<const float4*>(hrow + kc + 4 * e);
+                        if constexpr (KEEP) wraw[p][e] = *reinterpret_cast<const float4*>(norm.weight + kc + 4 * e);
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            load_w(wave, wa_a);
+            __builtin_amdgcn_sched_barrier(0);
+            float ss = 0.f;
+            if (live) {
+#pragma unroll
+                for (int p = 0; p < XP; ++p) {
+                    const int k = (wave + p * WV) * CH + kg * EL;
+                    float part = 0.f;
+#pragma unroll
+                    for (int e = 0; e < EL / 4; ++e) {
+                        const float4 v = hraw[p][e];
+                        part += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+                    }
+                    ss += k < K ? part : 0.f;
+                }
+            }
+            ss += __shfl_xor(ss, 16, WAVE);
+            ss += __shfl_xor(ss, 32, WAVE);
+            __shared__ float ssum[WV][16];
+            if (kg == 0) ssum[wave][r] = ss;
+            __syncthreads();
+            float total = 0.f;
+#pragma unroll
+            for (int w = 0; w < WV; ++w) total += ssum[w][r];
+            const float inv = 1.0f / sqrtf(total / static_cast<float>(K) + norm.eps);
 #pragma unroll
             for (int p = 0; p < XP; ++p) {
+                float f[EL];
                 const int kc = min((wave + p * WV) * CH + kg * EL, K - EL);
 #pragma unroll
                 for (int e = 0; e < EL / 4; ++e) {
-                    hraw[p][e] = *reinterpret_cast<const float4*>(hrow + kc + 4 * e);
-                    if constexpr (KEEP) wraw[p][e] = *reinterpret_cast<const float4*>(norm.weight + kc + 4 * e);
+                    float4 v = make_float4(0.f, 0.f, 0.f, 0.f), wv = v;
+                    if constexpr (KEEP) {
+                        if (live) { v = hraw[p][e]; wv = wraw[p][e]; }
+                    } else if (live) {
+                        v = *reinterpret_cast<const float4*>(hrow + kc + 4 * e);
+                        wv = *reinterpret_cast<const float4*>(norm.weight + kc + 4 * e);
+                    }
+                    f[4 * e] = (v.x * inv) * wv.x; f[4 * e + 1] = (v.y * inv) * wv.y;
+                    f[4 * e + 2] = (v.z * inv) * wv.z; f[4 * e + 3] = (v.w * inv) * wv.w;
                 }
+                xn[p / PT][p % PT][0].from_floats(f);
             }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        load_w(wave, wa_a);
-        __builtin_amdgcn_sched_barrier(0);
-        float ss = 0.f;
-        if (live) {
-#pragma unroll
-            for (int p = 0; p < XP; ++p) {
-                const int k = (wave + p * WV) * CH + kg * EL;
-                float part = 0.f;
-#pragma unroll
-                for (int e = 0; e < EL / 4; ++e) {
-                    const float4 v = hraw[p][e];
-                    part += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-                }
-                ss += k < K ? part : 0.f;
-            }
-        }
-        ss += __shfl_xor(ss, 16, WAVE);
-        ss += __shfl_xor(ss, 32, WAVE);
-        __shared__ float ssum[WV][16];
-        if (kg == 0) ssum[wave][r] = ss;
-        __syncthreads();
-        float total = 0.f;
-#pragma unroll
-        for (int w = 0; w < WV; ++w) total += ssum[w][r];
-        const float inv = 1.0f / sqrtf(total / static_cast<float>(K) + norm.eps);
-        Piece<T> xn[TRIPS][PT][1];
-#pragma unroll
-        for (int p = 0; p < XP; ++p) {
-            float f[EL];
-            const int kc = min((wave + p * WV) * CH + kg * EL, K - EL);
-#pragma unroll
-            for (int e = 0; e < EL / 4; ++e) {
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f), wv = v;
-                if constexpr (KEEP) {
-                    if (live) { v = hraw[p][e]; wv = wraw[p][e]; }
-                } else if (live) {
-                    v = *reinterpret_cast<const float4*>(hrow + kc + 4 * e);
-                    wv = *reinterpret_cast<const float4*>(norm.weight + kc + 4 * e);
-                }
-                f[4 * e] = (v.x * inv) * wv.x; f[4 * e + 1] = (v.y * inv) * wv.y;
-                f[4 * e + 2] = (v.z * inv) * wv.z; f[4 * e + 3] = (v.w * inv) * wv.w;
-            }
-            xn[p / PT][p % PT][0].from_floats(f);
         }
 #pragma unroll
         for (int t = 0; t < TRIPS; t += 2) {
@@ -471,11 +546,22 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
         if constexpr (XP == 0 && NTc == 1) {
             // fewer workgroups than compute units and rows of 4,096 elements or more: sixteen wavefronts each
             if (grid <= 160 && K >= 4096) {
-                skinny_decode_kernel<T, TOUT, NTc, EPI, XP, 16><<<grid, 16 * WAVE, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm);
+                skinny_decode_kernel<T, TOUT, NTc, EPI, XP, 16, 0><<<grid, 16 * WAVE, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm);
                 return;
             }
         }
-        skinny_decode_kernel<T, TOUT, NTc, EPI, XP, GV_WAVES><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm);
+        if constexpr (XP == 4 && NTc <= 2) {
+            // up to eight rows: the prologue staged through LDS (its rows and the partial sums both fit),
+            // compiled for 1, 4 and 8 rows
+#define NI_STAGED(SR_)                                                                                                   \
+    skinny_decode_kernel<T, TOUT, NTc, EPI, XP, GV_WAVES, SR_><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, \
+                                                                                                 (TOUT*)y, M, N, K, I, rope, norm)
+            if (M == 1) { NI_STAGED(1); return; }
+            if (M <= 4) { NI_STAGED(4); return; }
+            if (M <= 8) { NI_STAGED(8); return; }
+#undef NI_STAGED
+        }
+        skinny_decode_kernel<T, TOUT, NTc, EPI, XP, GV_WAVES, 0><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm);
     };
     if constexpr (EPI != EPI_ROPE) {
         if (NT >= 4) { run(std::integral_constant<int, 4>{}); return NI_LAUNCH_RESULT(); }
