@@ -70,10 +70,58 @@ def _as_stored(t: torch.Tensor) -> torch.Tensor:
     raise WeightFileError(f"tensor type {t.dtype} cannot be used")
 
 
+INDEX_NAME = "model.safetensors.index.json"
+
+
+class _Checkpoint:
+    """The tensors of a model folder by name: one ``model.safetensors``, or the shards that
+    ``model.safetensors.index.json`` names (its ``weight_map``: tensor name -> file name)."""
+
+    def __init__(self, folder: str):
+        single = os.path.join(folder, "model.safetensors")
+        index = os.path.join(folder, INDEX_NAME)
+        self.files: Dict[str, SafetensorsFile] = {}
+        self.where: Dict[str, str] = {}
+        if os.path.isfile(single) or not os.path.isfile(index):
+            self.path = single
+            f = self.files[single] = SafetensorsFile(single)
+            self.where = {n: single for n in f.names()}
+            return
+        self.path = index
+        try:
+            with open(index) as fh:
+                weight_map = json.load(fh)["weight_map"]
+        except (OSError, ValueError, KeyError) as e:
+            raise WeightFileError(f"{index}: not a shard index with a weight_map ({e})") from None
+        for name, shard in weight_map.items():
+            path = os.path.join(folder, str(shard))
+            if path not in self.files:
+                self.files[path] = SafetensorsFile(path)
+            self.where[name] = path
+        listed = set(weight_map)
+        for path, f in self.files.items():
+            for n in f.names():
+                if n not in listed:
+                    self.where.setdefault(n, path)      # a tensor the index forgot is still "unexpected", not lost
+        absent = sorted(n for n, path in self.where.items() if n not in self.files[path].names())
+        if absent:
+            raise WeightFileError(f"{index}: tensors named in the index are not in their shards: {absent}")
+
+    def names(self):
+        return self.where.keys()
+
+    def shape(self, name: str):
+        return self.files[self.where[name]].shape(name)
+
+    def tensor(self, name: str) -> torch.Tensor:
+        return self.files[self.where[name]].tensor(name)
+
+
 def load_tensors(folder: str, spec: ModelSpec) -> Dict[str, torch.Tensor]:
-    """The tensors ``spec`` needs from ``folder/model.safetensors`` (CPU views of the mapped file)."""
-    path = os.path.join(folder, "model.safetensors")
-    f = SafetensorsFile(path)
+    """The tensors ``spec`` needs from the checkpoint in ``folder`` (CPU views of the mapped files):
+    ``model.safetensors``, or the shards listed in ``model.safetensors.index.json``."""
+    f = _Checkpoint(folder)
+    path = f.path
     want = expected_tensors(spec)
     have = set(f.names())
     missing = sorted(n for n in want if n not in have)
@@ -89,11 +137,29 @@ def load_tensors(folder: str, spec: ModelSpec) -> Dict[str, torch.Tensor]:
     return {n: _as_stored(f.tensor(n)) for n in want}
 
 
-def write_model_folder(folder: str, config_json: Dict[str, Any], tensors: Dict[str, torch.Tensor]) -> str:
+def write_model_folder(folder: str, config_json: Dict[str, Any], tensors: Dict[str, torch.Tensor],
+                       shards: int = 1) -> str:
+    """``config.json`` and the checkpoint: one ``model.safetensors``, or ``shards`` files and their index."""
     os.makedirs(folder, exist_ok=True)
     with open(os.path.join(folder, "config.json"), "w") as fh:
         json.dump(config_json, fh, indent=2)
-    write_safetensors(os.path.join(folder, "model.safetensors"), tensors, {"format": "pt"})
+    if shards <= 1:
+        write_safetensors(os.path.join(folder, "model.safetensors"), tensors, {"format": "pt"})
+        return folder
+    names = list(tensors)
+    per = -(-len(names) // shards)
+    weight_map, total = {}, 0
+    for i in range(shards):
+        part = {n: tensors[n] for n in names[i * per:(i + 1) * per]}
+        if not part:
+            continue
+        fname = f"model-{i + 1:05d}-of-{shards:05d}.safetensors"
+        write_safetensors(os.path.join(folder, fname), part, {"format": "pt"})
+        for n, t in part.items():
+            weight_map[n] = fname
+            total += t.numel() * t.element_size()
+    with open(os.path.join(folder, INDEX_NAME), "w") as fh:
+        json.dump({"metadata": {"total_size": total}, "weight_map": weight_map}, fh, indent=2)
     return folder
 
 
@@ -101,7 +167,7 @@ _TORCH_DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": to
 
 
 def make_random_model(folder: str, config_json: Dict[str, Any], seed: int, dtype: str = "bfloat16",
-                      **init) -> str:
+                      shards: int = 1, **init) -> str:
     """Random-weights mode: write ``config.json`` and ``model.safetensors`` for the architecture
     that ``config_json`` names, from a seed.  ``dtype`` is the type the matrices are stored in."""
     if dtype not in _TORCH_DTYPES:
@@ -111,7 +177,7 @@ def make_random_model(folder: str, config_json: Dict[str, Any], seed: int, dtype
     tensors = arch.random_weights(cfg, seed, dtype=_TORCH_DTYPES[dtype], **init)
     out = dict(cfg.to_dict())
     out["torch_dtype"] = "bfloat16" if _TORCH_DTYPES[dtype] == torch.bfloat16 else "float32"
-    return write_model_folder(folder, out, tensors)
+    return write_model_folder(folder, out, tensors, shards=shards)
 
 
 def read_model_folder(folder: str):

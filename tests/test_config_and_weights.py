@@ -233,3 +233,37 @@ def test_tied_head_stored_twice_is_accepted_only_if_equal(tmp_path):
     with pytest.raises(WeightMismatchError) as e:
         load_tensors(bad, spec)
     assert e.value.unexpected == ["lm_head.weight"]
+
+
+def test_sharded_checkpoint_is_read_through_its_index(tmp_path):
+    one = make_random_model(str(tmp_path / "one"), TINY_B, seed=4, dtype="bfloat16")
+    three = make_random_model(str(tmp_path / "three"), TINY_B, seed=4, dtype="bfloat16", shards=3)
+    assert not os.path.exists(os.path.join(three, "model.safetensors"))
+    index = json.load(open(os.path.join(three, "model.safetensors.index.json")))
+    assert len(set(index["weight_map"].values())) == 3
+    _, _, spec = read_model_folder(three)
+    a, b = load_tensors(one, spec), load_tensors(three, spec)
+    assert sorted(a) == sorted(b) and all(torch.equal(a[n], b[n]) for n in a)
+    # the same single error over all shards: a tensor gone from its shard's index entry, an extra one in a shard
+    del index["weight_map"]["model.norm.weight"]
+    shard = os.path.join(three, index["weight_map"]["model.layers.0.mlp.up_proj.weight"])
+    tensors = dict(SafetensorsFile(shard).items())
+    del tensors["model.layers.0.mlp.up_proj.weight"]
+    tensors["stray.weight"] = torch.zeros(3)
+    from nanoinfer_amd.weights.safetensors_io import write_safetensors
+    write_safetensors(shard, tensors, {"format": "pt"})
+    del index["weight_map"]["model.layers.0.mlp.up_proj.weight"]
+    json.dump(index, open(os.path.join(three, "model.safetensors.index.json"), "w"))
+    with pytest.raises(WeightMismatchError) as e:
+        load_tensors(three, spec)
+    assert e.value.missing == ["model.layers.0.mlp.up_proj.weight"] and e.value.unexpected == ["stray.weight"]
+    # an index that names a tensor its shard does not hold, and an index that is no index
+    index["weight_map"]["model.layers.0.mlp.up_proj.weight"] = os.path.basename(shard)
+    json.dump(index, open(os.path.join(three, "model.safetensors.index.json"), "w"))
+    with pytest.raises(Exception) as e:
+        load_tensors(three, spec)
+    assert "not in their shards" in str(e.value)
+    open(os.path.join(three, "model.safetensors.index.json"), "w").write("{}")
+    with pytest.raises(Exception) as e:
+        load_tensors(three, spec)
+    assert "weight_map" in str(e.value)
