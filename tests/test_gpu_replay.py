@@ -190,6 +190,20 @@ def test_mixed_requests_on_few_pages(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,page", [("B", 12), ("C", 5), ("A", 1)])
+def test_pages_whose_size_is_no_power_of_two(name, page, dtype):
+    """The mixed trace again with pages of 12, 5 and 1 slots: page and slot of a position come from
+    a division, not a shift, in the cache books and in every kernel that walks a block table."""
+    folder = model_folder(name)
+    vocab = ALL[name]["vocab_size"]
+    requests = {f"p{i}": random_tokens(vocab, n, 900 + i) for i, n in enumerate([37, 70, 9, 25, 61])}
+    steps = mixed(requests, seed=5)
+    got, reused = run_in_process(folder, dtype, page, steps, max_live_tokens(steps, requests, page))
+    assert reused
+    compare(got, requests, folder, dtype, f"{name} pages of {page}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(dtype):
     """A short prompt, then some four hundred tokens one at a time: positions far beyond the prompt,
     many page boundaries, the split key range of the decode path."""
