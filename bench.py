@@ -4,7 +4,7 @@
 
 A step is one decode step of a batch of 8 requests whose prompts of 2,048 random tokens are in
 the cache (context limit 4,096): the step function runs the 8 new tokens as one batch, the
-argmax kernel picks the next ones, and they come back to the host, as in generation.  ``value``
+argmax kernels pick the next ones, and they come back to the host, as in greedy generation.  ``value``
 is decoded tokens per second.  The same line carries the prefill of one 2,048-token prompt in
 portions of 512 (``prefill``; ``--prefill-chunk`` changes the cut) and in one portion, the engine's
 default (``prefill_one_portion``), the decode step's fraction of the HBM roofline, and
@@ -157,7 +157,7 @@ def main() -> int:
 
         def one_step(toks):
             logits = runner.step([StepEntry(i, [t], [0]) for i, t in zip(ids, toks)])
-            return K.argmax(logits).tolist()
+            return runner.greedy_tokens(logits)      # as the engine's sampler asks for the tokens of greedy requests
 
         for _ in range(warmup):
             tokens = one_step(tokens)

@@ -99,7 +99,8 @@ class Engine:
         sampled: Dict[int, int] = {}
         if sampling:
             ids = self.sampler.sample(logits, [r.params for r in sampling], [r.generated for r in sampling],
-                                      [len(r.generated) for r in sampling])
+                                      [len(r.generated) for r in sampling],
+                                      greedy=getattr(self.runner, "greedy_tokens", None))
             sampled = {r.request_id: int(t) for r, t in zip(sampling, ids)}
         self.num_steps += 1
         return self.scheduler.commit(batch, sampled)

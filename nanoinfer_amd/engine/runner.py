@@ -119,6 +119,8 @@ class _RecordedStep:
     layout: list = None                  # per group (offset of slot mapping, offset of table, table width)
     order: tuple = ()                    # requests of the last replay, in batch order
     pages_written: list = None           # per group, per sequence: table entries already in the staging buffer
+    greedy: torch.Tensor = None          # int32, pinned host: argmax of every row of the logits, copied by the graph itself
+    replayed: "torch.cuda.Event" = None  # the last replay has finished (and with it the copy into ``greedy``)
 
 
 class ModelRunner:
@@ -163,6 +165,7 @@ class ModelRunner:
         self._unrecordable = set()
         self._staging = [(None, None)] * 3     # pinned host buffers for the tables of eager steps, and their uploads' events
         self._staging_turn = 0
+        self._greedy_of = None                 # (logits returned by the last recorded step, its recording)
 
     def _upload(self, flat: List[int]) -> torch.Tensor:
         """The integer tables of an eager step on the device.  They go through one of a few pinned
@@ -182,6 +185,16 @@ class ModelRunner:
         done.record()
         self._staging[i] = (buf, done)
         return dev
+
+    def greedy_tokens(self, logits: torch.Tensor) -> List[int]:
+        """The index of the largest logit of every row (lowest index on ties).  For the logits of a
+        recorded step the recording has already computed them and copied them to the host."""
+        held = self._greedy_of
+        if held is not None and held[0] is logits:
+            rec = held[1]
+            rec.replayed.synchronize()
+            return rec.greedy.tolist()
+        return K.argmax(logits).tolist()
 
     # ---------------------------------------------------------------- bookkeeping
     def computed_tokens(self, request: Hashable) -> int:
@@ -336,17 +349,22 @@ class ModelRunner:
         warm = StepContext(self.device, scratch_owner=self)
         flat_w, layout_w, rows_w = self._describe(entries, warm)
         self._bind(warm, torch.tensor(flat_w, dtype=torch.int32).to(self.device), layout_w, rows_w)
-        self.model.forward(warm, self._layer_cache(warm))
+        K.argmax(self.model.forward(warm, self._layer_cache(warm)))
         torch.cuda.synchronize()
+        greedy = torch.empty(n_rows, dtype=torch.int32).pin_memory()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx, self._layer_cache(ctx))
+            # greedy decoding needs only this: the recording picks the largest logit of every row
+            # and brings the ids to the host itself, so that no launch stands between step and token
+            greedy.copy_(K.argmax(logits), non_blocking=True)
         if K.library_calls() != calls_before and not self._replays_faithfully(graph, logits, warm, entries):
             # a library routine ran inside and its recorded nodes do not reproduce the eager result
             # (some record memory-clearing nodes that misbehave on replay): this shape runs eagerly
             self._unrecordable.add(key)
             return None
         rec = _RecordedStep(graph, meta, staging, logits, ctx, torch.cuda.Event())
+        rec.greedy, rec.replayed = greedy, torch.cuda.Event()
         rec.copied.record()
         self._recorded[key] = rec
         return rec
@@ -412,8 +430,11 @@ class ModelRunner:
         rec.meta.copy_(rec.staging, non_blocking=True)
         rec.copied.record()
         rec.graph.replay()
+        rec.replayed.record()
         self._last_context_len = totals
-        return rec.logits.clone()         # the graph's own buffer is overwritten by its next replay
+        out = rec.logits.clone()          # the graph's own buffer is overwritten by its next replay
+        self._greedy_of = (out, rec)
+        return out
 
     def step(self, entries: Sequence[StepEntry], end: Iterable[Hashable] = ()) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits ``[wanted, vocab]`` on the device, rows in the
@@ -421,6 +442,7 @@ class ModelRunner:
         named in ``end`` give back what they hold after the step."""
         entries = list(entries)
         logits = None
+        self._greedy_of = None
         if entries:
             self._check_and_reserve(entries)
             key = self._graph_shape(entries)

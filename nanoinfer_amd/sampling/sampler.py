@@ -41,13 +41,15 @@ class Sampler:
         self.device = device or K.require_gpu()
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams],
-               generated: Sequence[Sequence[int]], counters: Sequence[int]) -> List[int]:
+               generated: Sequence[Sequence[int]], counters: Sequence[int], greedy=None) -> List[int]:
+        """One token id per row of ``logits``.  ``greedy`` (optional) is a function from logits to
+        the argmax of every row, for a caller that may hold them already."""
         R, V = logits.shape
         if not (len(params) == len(generated) == len(counters) == R):
             raise ValueError(f"{R} rows of logits need {R} parameter sets, token lists and counters")
         plain_greedy = all(p.use_greedy() and not p.use_repetition_penalty() for p in params)
         if plain_greedy:
-            return K.argmax(logits).tolist()
+            return greedy(logits) if greedy is not None else K.argmax(logits).tolist()
         pen_ids: List[int] = []
         pen_off = [0]
         for p, g in zip(params, generated):

@@ -287,6 +287,7 @@ def test_recorded_decode_steps_equal_eager_ones(dtype):
     """Decode steps are recorded once per shape and replayed.  Every replay is checked against a
     runner that records nothing, with eager work (prompt portions of other requests, requests
     coming and going, a changing batch size) and synchronisations between the replays."""
+    from nanoinfer_amd import kernels as K
     from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
     name = "B"
     folder = model_folder(name)
@@ -305,6 +306,10 @@ def test_recorded_decode_steps_equal_eager_ones(dtype):
         assert (a is None) == (b is None)
         if a is not None:
             assert float((a - b).abs().max()) <= TOL[dtype] * float(b.abs().max()) * 0.1
+            # the tokens a recording brings to the host itself are the argmax of the logits it returns,
+            # replay after replay (asked for twice: the answer is kept until the next step)
+            assert recorded.greedy_tokens(a) == K.argmax(a).tolist() == recorded.greedy_tokens(a)
+            assert eager.greedy_tokens(b) == K.argmax(b).tolist()
             row = 0
             for rid, toks, want in entries:
                 for w in want:

@@ -51,7 +51,7 @@ class FakeRunner:
 
 
 class ArgmaxSampler:
-    def sample(self, logits, params, generated, counters):
+    def sample(self, logits, params, generated, counters, greedy=None):
         assert len(params) == len(generated) == len(counters) == logits.shape[0]
         return logits.argmax(dim=-1).tolist()
 
