@@ -200,6 +200,44 @@ class KVCacheManager:
         self._tokens[request] = total_tokens
         return True
 
+    def reserve_all(self, wanted) -> bool:
+        """:meth:`reserve` for several ``(request, total_tokens)`` pairs at once, all or nothing,
+        with one pass over the books (the common case of a decode step: no request needs a page)."""
+        wanted = list(wanted)
+        tokens = self._tokens
+        page = self.page_size
+        new = [r for r, _ in wanted if r not in tokens]
+        if len(new) > self.slots.num_free:
+            return False
+        needs = []
+        for g in self.groups:
+            tables = g.tables
+            per = []
+            total_new = 0
+            for r, t in wanted:
+                held = tokens.get(r)
+                if held is not None and t < held:
+                    raise CacheError(f"request {r!r} holds {held} tokens, cannot shrink to {t}")
+                n = (t + page - 1) // page - len(tables.get(r, ()))
+                if n > 0:
+                    per.append((r, n))
+                    total_new += n
+            if not g.pages.can_allocate(total_new):
+                return False
+            needs.append(per)
+        for r in new:
+            slot = self.slots.take(r)
+            for cid, t in self.state.items():
+                t[slot].zero_()
+            for g in self.groups:
+                g.tables[r] = []
+        for g, per in zip(self.groups, needs):
+            for r, n in per:
+                g.tables[r].extend(g.pages.allocate(n))
+        for r, t in wanted:
+            tokens[r] = t
+        return True
+
     def release_passed(self, request: Hashable, next_position: int) -> int:
         """Give back the pages of windowed groups that no query at ``next_position`` or later can
         read.  Their table entries become -1.  Returns how many pages were freed."""

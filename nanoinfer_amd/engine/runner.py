@@ -234,12 +234,9 @@ class ModelRunner:
                                 f"end at {self.model.max_positions}")
         # reserve for all entries, or for none
         totals = [(e.request, self._done.get(e.request, 0) + len(e.tokens)) for e in entries]
-        if not self.cache.can_reserve_all(totals):
+        if not self.cache.reserve_all(totals):
             raise OutOfPages(f"the step needs more pages or state slots than are free "
                              f"({self.cache.min_free_pages()} pages, {self.cache.slots.num_free} slots free)")
-        for request, total in totals:
-            if not self.cache.reserve(request, total):
-                raise StepError(f"reserving {total} tokens for request {request!r} failed after the check passed")
 
     def _describe(self, entries: List[StepEntry], ctx: StepContext, table_width: Optional[int] = None):
         """Fill the host side of ``ctx`` and return every integer table of the step as one flat

@@ -82,6 +82,22 @@ def test_can_reserve_all_counts_the_whole_step():
     m.check()
 
 
+def test_reserve_all_is_all_or_nothing_and_equals_single_reservations():
+    a = KVCacheManager(full(), page_size=4, num_pages=6, max_requests=3)
+    b = KVCacheManager(full(), page_size=4, num_pages=6, max_requests=3)
+    assert a.reserve_all([("x", 5), ("y", 9)]) and b.reserve("x", 5) and b.reserve("y", 9)
+    assert a.block_table(0, "x") == b.block_table(0, "x") and a.block_table(0, "y") == b.block_table(0, "y")
+    before = (a.free_pages(), a.block_table(0, "x")[:], a.slots.num_free)
+    assert not a.reserve_all([("x", 8), ("y", 12), ("z", 5)])           # one page short: nobody gets anything
+    assert (a.free_pages(), a.block_table(0, "x"), a.slots.num_free) == before and "z" not in a.live_requests()
+    assert a.reserve_all([("x", 8), ("y", 12)]) and a.free_pages() == 1   # x already has its 2 pages, y takes 1 more
+    assert a.reserve_all([("x", 8), ("y", 12)]) and a.free_pages() == 1   # nothing new to take: a decode step inside a page
+    with pytest.raises(CacheError):
+        a.reserve_all([("x", 3)])                                         # a request does not shrink
+    assert not a.reserve_all([("p", 1), ("q", 1)])                        # one state slot left, two newcomers
+    a.check()
+
+
 def test_groups_by_need_have_pages_of_their_own():
     needs = {0: CacheNeed(kv=KVNeed(2, 16)), 1: CacheNeed(kv=KVNeed(2, 16, window=8)),
              2: CacheNeed(kv=KVNeed(2, 16)), 3: CacheNeed(kv=KVNeed(1, 32)),
@@ -141,6 +157,20 @@ def test_random_orders_keep_the_books(seed):
                 m.release_passed(rid, want)
             else:
                 assert [g.pages.num_free for g in m.groups] == before and not m.has(rid)
+        elif op < 0.45 and live:
+            # a whole step at once: some live requests grow, a newcomer may join; all or nothing
+            step = {rid: live[rid] + rng.randint(0, ps + 1) for rid in rng.sample(list(live), rng.randint(1, len(live)))}
+            if rng.random() < 0.3:
+                step[next_id] = rng.randint(1, 2 * ps)
+                next_id += 1
+            before = ([g.pages.num_free for g in m.groups], {r: m.num_tokens(r) for r in live})
+            if m.reserve_all(list(step.items())):
+                for rid, want in step.items():
+                    live[rid] = want
+                    m.release_passed(rid, want)
+            else:
+                assert ([g.pages.num_free for g in m.groups], {r: m.num_tokens(r) for r in live}) == before
+                assert all(m.has(r) == (r in live) for r in step)
         elif op < 0.75 and live:
             rid = rng.choice(list(live))
             want = live[rid] + rng.randint(1, 2 * ps)

@@ -146,9 +146,12 @@ def test_rope_quarter_turn_vector(K):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_swiglu(K, dtype):
     g = torch.Generator().manual_seed(1)
-    gu = (torch.randn(7, 2 * 137, generator=g) * 3).to(DT[dtype])
-    out = K.swiglu(dev(gu), torch.empty(7, 137, device="cuda", dtype=DT[dtype]))
-    assert rel(out, P.swiglu(gu[:, :137].double(), gu[:, 137:].double())) < KTOL[dtype]
+    for width in (137, 136, 140, 4096):          # one element at a time, 16-byte vectors of either type, a long row
+        gu = (torch.randn(7, 2 * width, generator=g) * 3).to(DT[dtype])
+        gu[0, :4] = torch.tensor([-100.0, 100.0, -30.0, 0.0]).to(DT[dtype])     # the exponential overflows and underflows
+        out = K.swiglu(dev(gu), torch.empty(7, width, device="cuda", dtype=DT[dtype]))
+        assert bool(torch.isfinite(out).all())
+        assert rel(out, P.swiglu(gu[:, :width].double(), gu[:, width:].double())) < KTOL[dtype], width
     one = K.swiglu(torch.ones(1, 2, device="cuda"), torch.empty(1, 1, device="cuda"))
     assert abs(float(one) - 0.7310586) < 1e-6                          # test/test_op/test_layer_swiglu.cpp:65-108
 
