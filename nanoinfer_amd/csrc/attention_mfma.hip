@@ -99,7 +99,10 @@ __global__ __launch_bounds__(MA_WAVES * WAVE) void mfma_attention_kernel(
     constexpr int VROW = KSTEP + VPAD;
     __shared__ __attribute__((aligned(16))) uint16_t vs[2][HD][VROW];      // V^T of a step: [dim][key, in the lanes' order]
 
-    const QTile tile = tiles[blockIdx.x];
+    // the tiles of a portion come in the order of their positions, and a later tile has more keys to
+    // walk: the workgroups take them last first, so that the long ones start early and the short ones
+    // fill the end of the launch
+    const QTile tile = tiles[gridDim.x - 1 - blockIdx.x];
     const int G = H / KVH;
     const int chunks = (G + HPT - 1) / HPT;
     const int g = blockIdx.y / chunks;
