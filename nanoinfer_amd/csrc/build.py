@@ -123,7 +123,7 @@ def library_path(name: str, sources: List[str], defines: Optional[Dict[str, obje
 CORE = ("ni_ops", ["ops.hip"], {})
 SAMPLING = ("ni_sampling", ["sampling.hip"], {})
 SKINNY = ("ni_skinny_gemm", ["gemv.hip"], {})
-COMMON_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)
+COMMON_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 256)
 
 
 def attention_target(head_dim: int):
