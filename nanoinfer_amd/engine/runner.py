@@ -75,15 +75,18 @@ class StepContext:
         self._scratch_owner = scratch_owner
         self._scratch: Optional[torch.Tensor] = None
         self._q_tiles: Dict[int, torch.Tensor] = {}
+        self.tile_sizes_asked = set()
 
-    def q_tiles(self, tile_tokens: int) -> torch.Tensor:
+    def q_tiles(self, tile_tokens: int) -> Optional[torch.Tensor]:
         """The portions of the step cut into tiles of at most ``tile_tokens`` tokens, int32 [n, 4]
         rows of (sequence, first row, tokens, first position) on the device; built once per step
-        and tile size from the host lists (so not in a recorded step)."""
-        if self.recording:
-            raise StepError("tiles come from the host lists of a step and cannot be part of a recorded step")
+        and tile size from the host lists.  A recorded step has the tables it was recorded with
+        (the runner refills them before every replay) and no others: None then."""
         t = self._q_tiles.get(tile_tokens)
         if t is None:
+            self.tile_sizes_asked.add(tile_tokens)
+            if self.recording:
+                return None
             flat = K.build_q_tiles(self.q_start, self.q_len, self.context_len, tile_tokens)
             upload = getattr(self._scratch_owner, "_upload", None)
             if upload is not None:       # through the runner's pinned buffers: the host does not wait for the GPU
@@ -119,6 +122,7 @@ class _RecordedStep:
     layout: list = None                  # per group (offset of slot mapping, offset of table, table width)
     order: tuple = ()                    # requests of the last replay, in batch order
     pages_written: list = None           # per group, per sequence: table entries already in the staging buffer
+    tiles: dict = None                   # tile size -> (offset in the tables, number of tiles), for recorded prompt portions
     greedy: torch.Tensor = None          # int32, pinned host: argmax of every row of the logits, copied by the graph itself
     replayed: "torch.cuda.Event" = None  # the last replay has finished (and with it the copy into ``greedy``)
 
@@ -128,11 +132,14 @@ class ModelRunner:
 
     ``max_tokens`` is the number of tokens the page pools hold (rounded up to whole pages);
     ``max_requests`` the number of requests that may be live at once.  With ``use_graphs`` a step
-    that consists of single tokens only (decoding) is recorded once per shape into a HIP graph and
-    replayed afterwards: the launches of a whole step then cost one call.
+    that consists of single tokens only (decoding), or of one prompt portion of 64 tokens or more,
+    is recorded once per shape into a HIP graph and replayed afterwards: the launches of a whole
+    step then cost one call.
     """
 
     GRAPH_MAX_BATCH = 64
+    GRAPH_MIN_PORTION = 64        # a shorter prompt portion is not worth a recording
+    GRAPH_MAX_PORTIONS = 24       # recordings of prompt portions kept (each holds its activations)
 
     def __init__(self, model_dir: str, dtype: str = "bfloat16", page_size: int = 16, max_tokens: int = 4096,
                  max_requests: int = 64, device: Optional[torch.device] = None, use_graphs: bool = True):
@@ -318,83 +325,138 @@ class ModelRunner:
 
     # ---------------------------------------------------------------- recorded decode steps
     def _graph_shape(self, entries: List[StepEntry]):
-        """Key of the recorded step that can run these entries, or None when they must run eagerly:
-        single tokens only, each wanting its logits; table width and context bound rounded up to
+        """Key of the recorded step that can run these entries, or None when they must run eagerly.
+        Two kinds are recorded: single tokens only, each wanting its logits (``("d", batch, ...)``),
+        and one prompt portion alone that wants nothing or the logits of its last token
+        (``("p", tokens, ..., wanted rows)``).  Table width and context bound are rounded up to
         powers of two so that few recordings serve a growing context."""
         if not self.use_graphs or not 0 < len(entries) <= self.GRAPH_MAX_BATCH:
             return None
-        if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
-            return None
-        longest = max(self._done.get(e.request, 0) for e in entries) + 1
+        first = entries[0]
+        n = len(first.tokens)
+        if len(entries) == 1 and n >= self.GRAPH_MIN_PORTION:
+            want = list(first.want)
+            if want and want != [n - 1]:
+                return None
+            longest = self._done.get(first.request, 0) + n
+            kind, size, rows = "p", n, len(want)
+        else:
+            if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
+                return None
+            longest = max(self._done.get(e.request, 0) for e in entries) + 1
+            kind, size, rows = "d", len(entries), len(entries)
         pages = max(16, 1 << (self.cache.pages_for(longest) - 1).bit_length())
         bound = max(256, 1 << (longest - 1).bit_length())
-        key = (len(entries), pages, bound)
-        return None if key in self._unrecordable else key
+        key = (kind, size, pages, bound, rows)
+        if key in self._unrecordable:
+            return None
+        if kind == "p" and key not in self._recorded and \
+                sum(1 for k in self._recorded if k[0] == "p") >= self.GRAPH_MAX_PORTIONS:
+            return None
+        return key
+
+    def _tables_of(self, entries: List[StepEntry], ctx: StepContext, width: int, tile_sizes):
+        """Every integer table of a recorded step as one flat list: those of :meth:`_describe`, then
+        the attention tiles of each tile size the model asked for."""
+        flat, layout, n_rows = self._describe(entries, ctx, table_width=width)
+        tiles = {}
+        for ts in sorted(tile_sizes):
+            rows = K.build_q_tiles(ctx.q_start, ctx.q_len, ctx.context_len, ts)
+            tiles[ts] = (len(flat), len(rows) // 4)        # where they start, how many
+            flat.extend(rows)
+        return flat, layout, n_rows, tiles
 
     def _record(self, key, entries: List[StepEntry]) -> Optional[_RecordedStep]:
-        B, pages, bound = key
+        kind, size, pages, bound, _ = key
+        calls_before = K.library_calls()
+        # run the step once the ordinary way first: code objects get loaded and buffers sized outside
+        # the recording, and the model says which attention tiles it wants.  Running a step twice is
+        # harmless: it writes the same keys, values and logits again.
+        warm = StepContext(self.device, scratch_owner=self)
+        flat_w, layout_w, rows_w = self._describe(entries, warm)
+        self._bind(warm, torch.tensor(flat_w, dtype=torch.int32).to(self.device), layout_w, rows_w)
+        warm_logits = self.model.forward(warm, self._layer_cache(warm))
+        if warm_logits is not None:
+            K.argmax(warm_logits)
+        torch.cuda.synchronize()
         ctx = StepContext(self.device, recording=True)
-        flat, layout, n_rows = self._describe(entries, ctx, table_width=pages)
+        flat, layout, n_rows, tiles = self._tables_of(entries, ctx, pages, warm.tile_sizes_asked)
         ctx.max_context = bound
         staging = torch.tensor(flat, dtype=torch.int32).pin_memory()
         meta = staging.to(self.device)
         self._bind(ctx, meta, layout, n_rows)
-        calls_before = K.library_calls()
-        # run the step once the ordinary way first: code objects get loaded and buffers sized outside
-        # the recording.  Running a decode step twice is harmless: it writes the same keys, values
-        # and logits again.
-        warm = StepContext(self.device, scratch_owner=self)
-        flat_w, layout_w, rows_w = self._describe(entries, warm)
-        self._bind(warm, torch.tensor(flat_w, dtype=torch.int32).to(self.device), layout_w, rows_w)
-        K.argmax(self.model.forward(warm, self._layer_cache(warm)))
-        torch.cuda.synchronize()
-        greedy = torch.empty(n_rows, dtype=torch.int32).pin_memory()
+        for ts, (off, count) in tiles.items():
+            ctx._q_tiles[ts] = meta[off:off + 4 * count].view(-1, 4)
+        greedy = torch.empty(max(n_rows, 1), dtype=torch.int32).pin_memory()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx, self._layer_cache(ctx))
-            # greedy decoding needs only this: the recording picks the largest logit of every row
-            # and brings the ids to the host itself, so that no launch stands between step and token
-            greedy.copy_(K.argmax(logits), non_blocking=True)
+            if logits is not None:
+                # greedy decoding needs only this: the recording picks the largest logit of every row
+                # and brings the ids to the host itself, so that no launch stands between step and token
+                greedy.copy_(K.argmax(logits), non_blocking=True)
+        if ctx.tile_sizes_asked - set(tiles):
+            self._unrecordable.add(key)       # the recorded run asked for tiles the eager run did not: not the same step
+            return None
         if K.library_calls() != calls_before and not self._replays_faithfully(graph, logits, warm, entries):
             # a library routine ran inside and its recorded nodes do not reproduce the eager result
             # (some record memory-clearing nodes that misbehave on replay): this shape runs eagerly
             self._unrecordable.add(key)
             return None
         rec = _RecordedStep(graph, meta, staging, logits, ctx, torch.cuda.Event())
-        rec.greedy, rec.replayed = greedy, torch.cuda.Event()
+        rec.greedy, rec.replayed, rec.tiles = greedy, torch.cuda.Event(), tiles
         rec.copied.record()
         self._recorded[key] = rec
         return rec
 
+    def _written_rows(self, ctx: StepContext) -> torch.Tensor:
+        """The keys and values that a step has written, of every cache, gathered into one tensor:
+        all that a step which returns no logits leaves behind."""
+        parts = []
+        ps = self.page_size
+        for gi, g in enumerate(self.cache.groups):
+            slots = ctx.groups[gi].slot_mapping.long()
+            pages, offs = slots // ps, slots % ps
+            for cid in g.cache_ids:
+                parts.append(g.kpools[cid][pages, :, offs].float().reshape(-1))
+                parts.append(g.vpools[cid][pages, :, offs].float().reshape(-1))
+        return torch.cat(parts) if parts else torch.zeros(1, device=self.device)
+
     def _replays_faithfully(self, graph, logits, warm: StepContext, entries: List[StepEntry], rounds: int = 3) -> bool:
         """Replay a fresh recording several times, with the same step run eagerly and a
-        synchronisation between the replays, and compare every replay with the eager logits.
-        A decode step may be run any number of times: it writes the same keys and values again."""
+        synchronisation between the replays, and compare every replay with the eager run: the
+        logits, or for a step that returns none the keys and values it wrote.  A step may be run any
+        number of times: it writes the same keys and values again."""
         for _ in range(rounds):
             graph.replay()
             torch.cuda.synchronize()
-            got = logits.clone()
+            got = logits.clone() if logits is not None else self._written_rows(warm)
             want = self.model.forward(warm, self._layer_cache(warm))
+            if logits is None:
+                want = self._written_rows(warm)
             torch.cuda.synchronize()
             scale = float(want.abs().max())
             if not bool(torch.isfinite(got).all()) or float((got - want).abs().max()) > 1e-3 * max(scale, 1e-30):
                 return False
         return True
 
-    def _replay(self, key, entries: List[StepEntry]) -> Optional[torch.Tensor]:
+    def _replay(self, key, entries: List[StepEntry]) -> bool:
+        """Run the entries through the recording of their shape (made now if there is none).  False:
+        this shape cannot be recorded and the step has not run.  The logits are left in
+        ``self._replayed_logits``."""
         rec = self._recorded.get(key)
         if rec is None:
             rec = self._record(key, entries)
             if rec is None:
-                return None
+                return False
             # the recording itself ran nothing: fall through to the first replay
         rec.copied.synchronize()          # the previous upload must have read the staging buffer
-        B, width, _ = key
+        kind, B, width = key[0], key[1], key[2]
         ps = self.page_size
         st = rec.staging.numpy()          # shares the pinned memory
         order = tuple(e.request for e in entries)
         totals = []
-        if order == rec.order:
+        if kind == "d" and order == rec.order:
             # the same requests in the same places as last time: tokens, positions and slots change,
             # block tables only grow at their ends
             for b, e in enumerate(entries):
@@ -416,12 +478,12 @@ class ModelRunner:
                     st[off_slot + b] = table[done // ps] * ps + done % ps
         else:
             ctx = StepContext(self.device)
-            flat, layout, _ = self._describe(entries, ctx, table_width=width)
-            if len(flat) != rec.staging.numel():
+            flat, layout, _, tiles = self._tables_of(entries, ctx, width, rec.tiles or ())
+            if len(flat) != rec.staging.numel() or tiles != (rec.tiles or {}):
                 raise StepError("a recorded step was asked to run another shape")
             st[:] = flat
             rec.layout = layout
-            rec.order = order
+            rec.order = order if kind == "d" else ()
             rec.pages_written = [[len(g.tables[e.request]) for e in entries] for g in self.cache.groups]
             totals = ctx.context_len
         rec.meta.copy_(rec.staging, non_blocking=True)
@@ -429,9 +491,13 @@ class ModelRunner:
         rec.graph.replay()
         rec.replayed.record()
         self._last_context_len = totals
-        out = rec.logits.clone()          # the graph's own buffer is overwritten by its next replay
-        self._greedy_of = (out, rec)
-        return out
+        if rec.logits is None:
+            self._replayed_logits = None
+        else:
+            out = rec.logits.clone()      # the graph's own buffer is overwritten by its next replay
+            self._greedy_of = (out, rec)
+            self._replayed_logits = out
+        return True
 
     def step(self, entries: Sequence[StepEntry], end: Iterable[Hashable] = ()) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits ``[wanted, vocab]`` on the device, rows in the
@@ -444,10 +510,9 @@ class ModelRunner:
             self._check_and_reserve(entries)
             key = self._graph_shape(entries)
             totals = None
-            if key is not None:
-                logits = self._replay(key, entries)
-                if logits is not None:
-                    totals = self._last_context_len
+            if key is not None and self._replay(key, entries):
+                logits = self._replayed_logits
+                totals = self._last_context_len
             if totals is None:
                 ctx = StepContext(self.device, scratch_owner=self)
                 flat, layout, n_rows = self._describe(entries, ctx)

@@ -212,9 +212,12 @@ class Attention(Part):
             qkv = K.linear(x, self.w_qkv)
             K.rope_kv_write(qkv, ctx.positions, cos, sin, slots, cache.kpool, cache.vpool, self.H, self.KVH, self.hd)
         out = torch.empty(T, self.H * self.hd, dtype=x.dtype, device=x.device)
-        if (not ctx.recording and ctx.max_q_len >= self.MFMA_MIN_PORTION and K.mfma_attention_ok(x.dtype, self.hd)):
-            # prompt portions: tiles of tokens on the matrix cores
+        tiles = None
+        if ctx.max_q_len >= self.MFMA_MIN_PORTION and K.mfma_attention_ok(x.dtype, self.hd):
+            # prompt portions: tiles of tokens on the matrix cores (a recorded step has them only if
+            # it was recorded with them)
             tiles = ctx.q_tiles(K.mfma_tile_tokens(self.hd, self.H // self.KVH))
+        if tiles is not None:
             max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window + ctx.max_q_len)
             nsplit = K.mfma_splits(tiles.shape[0], self.KVH, self.H // self.KVH, max_keys)
             ws = ctx.workspace(T * self.H * nsplit * (self.hd + 2)) if nsplit > 1 else None

@@ -359,3 +359,62 @@ def test_recorded_steps_with_library_products_are_checked_before_use():
         assert float((a - b).abs().max()) <= 2e-3 * float(b.abs().max()), step
         toks = a.argmax(-1).tolist()
     assert len(recorded._recorded) + len(recorded._unrecordable) == 1
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_prompt_portions_equal_eager_ones(dtype):
+    """A prompt portion of 64 tokens or more that stands alone in its step is recorded per shape
+    and replayed at other positions and for other requests; every replay is checked against a
+    runner that records nothing, with decode steps and shorter portions between them, and the
+    whole against the plain implementation."""
+    from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
+    name = "B"
+    folder = model_folder(name)
+    vocab = ALL[name]["vocab_size"]
+    recorded = ModelRunner(folder, dtype=dtype, page_size=8, max_tokens=2048, max_requests=4)
+    eager = ModelRunner(folder, dtype=dtype, page_size=8, max_tokens=2048, max_requests=4, use_graphs=False)
+    reqs = {f"q{i}": random_tokens(vocab, n, 700 + i) for i, n in enumerate((300, 214, 129))}
+    done = {k: 0 for k in reqs}
+    got = {}
+
+    def both(entries, end=()):
+        a = recorded.step([StepEntry(*e) for e in entries], end=end)
+        b = eager.step([StepEntry(*e) for e in entries], end=end)
+        torch.cuda.synchronize()
+        assert (a is None) == (b is None)
+        if a is not None:
+            assert float((a - b).abs().max()) <= TOL[dtype] * float(b.abs().max()) * 0.1
+            row = 0
+            for rid, toks, want in entries:
+                for w in want:
+                    got[(rid, done[rid] + w)] = a[row].clone()
+                    row += 1
+        for rid, toks, _ in entries:
+            done[rid] += len(toks)
+
+    def portion(rid, n, want_last):
+        return (rid, list(reqs[rid][done[rid]:done[rid] + n]), [n - 1] if want_last else [])
+
+    both([portion("q0", 64, False)])                 # recorded now, no logits: judged by the keys and values it writes
+    both([portion("q0", 64, True)])                  # another recording: one row of logits
+    both([portion("q1", 64, False)])                 # replay for another request at position 0
+    both([portion("q0", 64, True)])                  # replay further on in q0 (same bucket of context)
+    both([portion("q1", 64, True), portion("q2", 64, False)])      # two portions in one step: not recorded, eager
+    both([portion("q0", 3, True)])                   # a short portion: eager
+    for _ in range(5):
+        both([("q0", [reqs["q0"][done["q0"]]], [0]), ("q1", [reqs["q1"][done["q1"]]], [0])])     # recorded decode steps between
+    both([portion("q0", 64, True)])                  # context now beyond 256: a new bucket, a new recording
+    both([portion("q1", 64, True)])
+    both([portion("q2", 64, True)])
+    both([portion("q0", 100 - 64, True)])
+    keys = list(recorded._recorded)
+    assert sum(1 for k in keys if k[0] == "p") >= 3 and sum(1 for k in keys if k[0] == "d") >= 1, keys
+    assert not eager._recorded
+    by_request = {}
+    for (rid, pos), row in got.items():
+        by_request.setdefault(rid, []).append((pos, row))
+    for rid, rows in by_request.items():
+        want = plain_logits(folder, tuple(reqs[rid]), dtype)
+        rows.sort(key=lambda x: x[0])
+        idx = [p for p, _ in rows]
+        assert_close(torch.stack([r for _, r in rows]), want[idx], dtype, f"recorded portions, request {rid}")
