@@ -301,39 +301,76 @@ def mfma_attention_ok(dtype: torch.dtype, hd: int) -> bool:
     return dtype == torch.bfloat16 and hd % 32 == 0 and 32 <= hd <= 256
 
 
-def mfma_tile_tokens(hd: int, group: int) -> int:
-    """Tokens of one tile of the matrix-core attention kernel for ``group`` query heads per kv head."""
-    return int(attention_mfma_lib(hd).ni_mfma_attention_tile_tokens(int(group)))
+COMPUTE_UNITS = 256      # of an MI355X
+
+
+def _heads_per_tile(group: int) -> int:
+    return 16 if group >= 16 else 8 if group > 4 else 4 if group > 2 else 2 if group > 1 else 1
+
+
+def mfma_tile_tokens(hd: int, group: int, n_tokens: Optional[int] = None, kv_heads: int = 1) -> int:
+    """Tokens of one tile of the matrix-core attention kernel for ``group`` query heads per kv head.
+    A wavefront owns one block of 16 rows, or two where the head size leaves registers for them.
+    More blocks share every staged key among more rows and give a wavefront more independent work,
+    but the kernel pairs long tiles with short ones, two to a workgroup, and wants two workgroups on
+    every compute unit: the largest number of blocks is taken that leaves a step of ``n_tokens``
+    tokens four tiles for every compute unit (measured at head size 64: 2,048 tokens 57 us with one
+    block, 63 with two; 4,096 tokens 197 and 134).  Without ``n_tokens``: the smallest tile."""
+    lib = attention_mfma_lib(hd)
+    hpt = _heads_per_tile(group)
+    blocks = 1
+    if n_tokens is not None:
+        chunks = (group + hpt - 1) // hpt
+        for b in (2,):
+            if b <= int(lib.ni_mfma_attention_max_blocks()) and \
+                    (n_tokens // (4 * b * 16 // hpt)) * kv_heads * chunks >= 4 * COMPUTE_UNITS:
+                blocks = b
+                break
+    return int(lib.ni_mfma_attention_tile_tokens(int(group), blocks))
 
 
 def build_q_tiles(q_start, q_len, context_len, tile_tokens: int):
     """Cut the portions of a step (host lists: first row, length, context after the step) into
-    tiles of at most ``tile_tokens`` tokens: flat list of (sequence, first row, tokens, first position)."""
-    flat = []
+    tiles of at most ``tile_tokens`` tokens: flat list of (sequence, first row, tokens, first position),
+    the tiles with the most keys before them first (the kernel deals them out in that order)."""
+    tiles = []
     for s, (row, n, total) in enumerate(zip(q_start, q_len, context_len)):
         first = total - n
         for t0 in range(0, n, tile_tokens):
-            flat.extend((s, row + t0, min(tile_tokens, n - t0), first + t0))
-    return flat
+            tiles.append((s, row + t0, min(tile_tokens, n - t0), first + t0))
+    tiles.sort(key=lambda t: -(t[3] + t[2]))
+    return [x for t in tiles for x in t]
 
 
 def mfma_splits(n_tiles: int, kv_heads: int, group: int, max_keys: int) -> int:
-    """Into how many runs the matrix-core kernel cuts the keys of every tile so that about a
-    thousand workgroups exist.  A run is never shorter than 2,048 keys: below that the second
-    kernel that merges the runs costs more than the cut gains (measured for portions of 512 tokens
-    at contexts of 512 to 8,192)."""
-    hpt = 16 if group >= 16 else 8 if group > 4 else 4 if group > 2 else 2 if group > 1 else 1
+    """Into how many runs the matrix-core kernel cuts the keys of every tile.  Cutting costs a
+    second kernel that merges the runs, and float32 partial results in between: a step with many
+    tiles is cut only into runs of 2,048 keys or more, up to about a thousand workgroups (measured
+    for portions of 512 tokens at contexts of 512 to 8,192); a step with fewer tiles than the chip
+    has compute units, into runs of 512 keys or more until every unit has one."""
+    hpt = _heads_per_tile(group)
     items = max(1, n_tiles * kv_heads * ((group + hpt - 1) // hpt))
-    return int(max(1, min(1024 // items, max_keys // 2048, 16)))
+    many = min(1024 // items, max_keys // 2048)
+    few = min(COMPUTE_UNITS // items, max_keys // 512)
+    return int(max(1, min(max(many, few), 16)))
 
 
 def mfma_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                    tiles: torch.Tensor, out: torch.Tensor, H: int, KVH: int, hd: int, scale: float,
-                   window: Optional[int], nsplit: int = 1, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   window: Optional[int], nsplit: int = 1, workspace: Optional[torch.Tensor] = None,
+                   tile_tokens: Optional[int] = None) -> torch.Tensor:
     """Attention of prompt portions on the matrix cores (bfloat16).  ``tiles`` is int32 [n, 4] from
-    :func:`build_q_tiles`; the pools already hold the keys and values of every position of the step.
-    ``workspace`` (float32, ``T*H*nsplit*(hd+2)`` elements) is needed when ``nsplit > 1``."""
+    :func:`build_q_tiles` with ``tile_tokens`` tokens a tile (a size that :func:`mfma_tile_tokens`
+    gives; default: its smallest); the pools already hold the keys and values of every position of
+    the step.  ``workspace`` (float32, ``T*H*nsplit*(hd+2)`` elements) is needed when ``nsplit > 1``."""
     T = qkv.shape[0]
+    smallest = mfma_tile_tokens(hd, H // max(KVH, 1))
+    tile_tokens = smallest if tile_tokens is None else int(tile_tokens)
+    blocks = tile_tokens // smallest
+    if not (blocks * smallest == tile_tokens and blocks >= 1
+            and blocks <= int(attention_mfma_lib(hd).ni_mfma_attention_max_blocks())):
+        raise KernelError(f"mfma_attention has no tiles of {tile_tokens} tokens at head size {hd} "
+                          f"(the smallest has {smallest})")
     _gpu(qkv, "qkv", torch.bfloat16)
     if not (mfma_attention_ok(qkv.dtype, hd)):
         raise KernelError(f"mfma_attention does not take {qkv.dtype} with head size {hd}")
@@ -365,7 +402,7 @@ def mfma_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
                                                     block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(out),
                                                     _ptr(part_o), _ptr(part_ml), H, KVH, kpool.shape[2],
                                                     int(window) if window else 0, ctypes.c_float(scale), nsplit,
-                                                    _stream()), "mfma_attention")
+                                                    blocks, _stream()), "mfma_attention")
     if nsplit > 1:
         _check(attention_lib(hd).ni_merge_splits(_ptr(part_o), _ptr(part_ml), _ptr(out), T, H, nsplit,
                                                  dtype_code(out.dtype), _stream()), "merge_splits")

@@ -158,7 +158,7 @@ def test_swiglu(K, dtype):
 
 # ------------------------------------------------------------------ attention over pages
 
-def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boost=None, kernel="token"):
+def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boost=None, kernel="token", blocks=1):
     """Sequences of ``lens`` keys each; the last ``q_lens`` of each are this step's queries.  The
     cache is filled through a shuffled block table; everything else in the pools is NaN so that a
     read outside a sequence's own keys poisons the result."""
@@ -205,10 +205,11 @@ def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boo
     ws = torch.empty(max(1, T * H * nsplit * (hd + 2)), device="cuda") if nsplit > 1 else None
     if kernel == "mfma":
         starts = [sum(q_lens[:b]) for b in range(B)]
-        flat = K.build_q_tiles(starts, q_lens, lens, K.mfma_tile_tokens(hd, H // KVH))
+        tile_tokens = K.mfma_tile_tokens(hd, H // KVH) * blocks      # a wavefront owns `blocks` blocks of 16 rows
+        flat = K.build_q_tiles(starts, q_lens, lens, tile_tokens)
         tiles = dev(torch.tensor(flat, dtype=torch.int32).view(-1, 4))
         K.mfma_attention(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table), tiles, out,
-                         H, KVH, hd, 1.0 / math.sqrt(hd), window, nsplit, ws)
+                         H, KVH, hd, 1.0 / math.sqrt(hd), window, nsplit, ws, tile_tokens)
     else:
         fn = {"token": K.token_attention, "token_wide": functools.partial(K.token_attention, wide=True),
               "mfma_token": K.mfma_token_attention}[kernel]
@@ -262,9 +263,10 @@ def test_attention_block_table_longer_than_one_segment(K, kernel):
     three slots a range of 2,500 keys needs several such segments; a boosted key is placed in the
     first, at the seam and in the last, so that a segment read through the wrong entries shows."""
     n = 2500
-    for ps, key_at in ((1, 5), (1, 1023), (1, 1024), (1, 2499), (3, 3071 % n), (3, 1)):
+    for i, (ps, key_at) in enumerate(((1, 5), (1, 1023), (1, 1024), (1, 2499), (3, 3071 % n), (3, 1))):
         out, want, (qs, ks, vs) = paged_case(K, "bfloat16", 4, 2, 64, ps, [n, 40], [3, 2], None, ps + key_at, 1,
-                                             boost=(0, key_at, n - 1, 6.0), kernel=kernel)
+                                             boost=(0, key_at, n - 1, 6.0), kernel=kernel,
+                                             blocks=(1, 2)[i % 2] if kernel == "mfma" else 1)
         assert not torch.isnan(out).any()
         assert rel(out, want) < KTOL["bfloat16"], (ps, key_at)
         got = out.double().cpu()[2].reshape(4, 64)
@@ -279,10 +281,36 @@ def test_attention_block_table_longer_than_one_segment(K, kernel):
 def test_mfma_attention_head_sizes_and_groups(K, H, KVH, hd, ps):
     # whole prompts, portions that start in the middle of a sequence, single tokens beside them, tile edges
     lens, q_lens = [1, 37, 130, 64, 200, 17], [1, 37, 2, 1, 77, 16]
-    for nsplit in (1, 3):
-        out, want, _ = paged_case(K, "bfloat16", H, KVH, hd, ps, lens, q_lens, None, hd + H, nsplit, kernel="mfma")
-        assert not torch.isnan(out).any(), "a key outside the sequence's own pages took part"
-        assert rel(out, want) < KTOL["bfloat16"], (H, KVH, hd, ps, nsplit)
+    for blocks in (1, 2, 4):
+        if blocks > mfma_max_blocks(K, hd):
+            with pytest.raises(K.KernelError, match="no tiles of"):
+                paged_case(K, "bfloat16", H, KVH, hd, ps, lens, q_lens, None, hd + H, 1, kernel="mfma", blocks=blocks)
+            continue
+        for nsplit in (1, 3):
+            out, want, _ = paged_case(K, "bfloat16", H, KVH, hd, ps, lens, q_lens, None, hd + H, nsplit, kernel="mfma",
+                                      blocks=blocks)
+            assert not torch.isnan(out).any(), "a key outside the sequence's own pages took part"
+            assert rel(out, want) < KTOL["bfloat16"], (H, KVH, hd, ps, nsplit, blocks)
+
+
+def mfma_max_blocks(K, hd):
+    return int(K.attention_mfma_lib(hd).ni_mfma_attention_max_blocks())
+
+
+def test_mfma_tile_size_and_splits_follow_the_step(K):
+    # 32 query heads on 8 kv heads, head size 64: tiles of 16 tokens, or of 32 where that leaves 1,024 tiles
+    assert K.mfma_tile_tokens(64, 4) == 16
+    assert K.mfma_tile_tokens(64, 4, 2048, 8) == 16
+    assert K.mfma_tile_tokens(64, 4, 4096, 8) == 32
+    assert K.mfma_tile_tokens(64, 4, 100, 8) == 16
+    assert K.mfma_tile_tokens(128, 4, 8192, 8) == 16        # head size 128 leaves registers for one block only
+    assert K.mfma_tile_tokens(256, 1, 8192, 8) == 64        # one head a tile: 4 wavefronts x 16 tokens, one block
+    # many tiles: runs of 2,048 keys or more; fewer tiles than compute units: runs of 512 or more
+    assert K.mfma_splits(128, 8, 4, 2048) == 1
+    assert K.mfma_splits(32, 8, 4, 8192) == 4
+    assert K.mfma_splits(8, 8, 4, 2048) == 4
+    assert K.mfma_splits(8, 8, 4, 300) == 1
+    assert K.mfma_splits(1, 1, 1, 10 ** 6) == 16
 
 
 @pytest.mark.parametrize("H,KVH,hd,ps", [(4, 2, 32, 8), (6, 1, 32, 8), (32, 8, 64, 16), (16, 2, 128, 16), (2, 2, 256, 16),
@@ -310,18 +338,22 @@ def test_mfma_token_attention_window_and_far_key(K):
         assert float((got - expect).abs().max()) < 0.05, key_at
 
 
-def test_mfma_attention_window_and_far_key(K):
+@pytest.mark.parametrize("blocks", [1, 2])
+def test_mfma_attention_window_and_far_key(K, blocks):
     for window in (1, 7, 16, 33, 100):
-        out, want, _ = paged_case(K, "bfloat16", 4, 2, 32, 8, [150, 9, 33], [150, 9, 2], window, window, 1, kernel="mfma")
+        out, want, _ = paged_case(K, "bfloat16", 4, 2, 32, 8, [150, 9, 33], [150, 9, 2], window, window, 1, kernel="mfma",
+                                  blocks=blocks)
         assert not torch.isnan(out).any()
         assert rel(out, want) < KTOL["bfloat16"], window
     for key_at in (37, 16, 15, 0, 31, 32, 698):
-        out, want, (qs, ks, vs) = paged_case(K, "bfloat16", 8, 2, 64, 16, [700], [5], None, 9, 1 + key_at % 4,
-                                             boost=(0, key_at, 699, 6.0), kernel="mfma")
-        assert rel(out, want) < KTOL["bfloat16"]
-        got = out.double().cpu()[-1].reshape(8, 64)
-        expect = vs[0][key_at].double().repeat_interleave(4, 0)
-        assert float((got - expect).abs().max()) < 0.05, key_at
+        # 5 queries, or 90 so that the large tiles are full and the last one is not
+        for n_q in (5, 90):
+            out, want, (qs, ks, vs) = paged_case(K, "bfloat16", 8, 2, 64, 16, [700], [n_q], None, 9, 1 + key_at % 4,
+                                                 boost=(0, key_at, 699, 6.0), kernel="mfma", blocks=blocks)
+            assert rel(out, want) < KTOL["bfloat16"]
+            got = out.double().cpu()[-1].reshape(8, 64)
+            expect = vs[0][key_at].double().repeat_interleave(4, 0)
+            assert float((got - expect).abs().max()) < 0.05, key_at
     with pytest.raises(Exception):
         K.attention_mfma_lib(48)
     assert not K.mfma_attention_ok(torch.float32, 64) and not K.mfma_attention_ok(torch.bfloat16, 48)
