@@ -41,6 +41,7 @@ PROMPT_LEN = 2048
 CONTEXT_LEN = 4096
 PREFILL_CHUNK = 512       # portions of the prefill measurement, as the benchmark configuration names them
 ENGINE_CHUNK = 2048       # the engine's own default: a portion as long as the step's token budget
+DECODE_RUN = 8            # the engine's own default of max_decode_run
 BLOCK_SIZE = 16
 HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
@@ -72,7 +73,7 @@ def prefill_flops(cfg: dict, tokens: int) -> float:
     return linear + attention + 2.0 * V * d
 
 
-def config_record(cfg: dict, layers: int, batch: int, mean_ctx: float, prefill_chunk: int) -> dict:
+def config_record(cfg: dict, layers: int, batch: int, mean_ctx: float, prefill_chunk: int, decode_run: int) -> dict:
     """Every size of the measured configuration, flat (nothing nested, at most 20 keys)."""
     return {
         "model": "llama-3.2-1b-shape", "layers": layers, "layers_full_model": FULL_LAYERS,
@@ -81,7 +82,7 @@ def config_record(cfg: dict, layers: int, batch: int, mean_ctx: float, prefill_c
         "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
         "tied_embeddings": True, "global_batch": batch, "prompt_len": PROMPT_LEN,
         "seq_len": CONTEXT_LEN, "decode_context_mean": round(mean_ctx, 1), "kv_block_size": BLOCK_SIZE,
-        "prefill_chunk": prefill_chunk, "parallelism": "single-gpu",
+        "prefill_chunk": prefill_chunk, "decode_run": decode_run, "parallelism": "single-gpu",
     }
 
 
@@ -94,6 +95,8 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (named in config)")
     ap.add_argument("--prefill-chunk", type=int, default=PREFILL_CHUNK, help="tokens of a prompt portion in the prefill measurement")
+    ap.add_argument("--decode-run", type=int, default=DECODE_RUN,
+                    help="decode steps on one scheduling decision (the engine's max_decode_run; 1: the host reads every token before the next step)")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
                     help="run one phase only (for profiling; prints no result line)")
@@ -155,17 +158,20 @@ def main() -> int:
             tokens.append(K.argmax(logits).tolist()[0])
         log(f"batch {batch}: prompts are in the cache")
 
-        def one_step(toks):
-            logits = runner.step([StepEntry(i, [t], [0]) for i, t in zip(ids, toks)])
-            return runner.greedy_tokens(logits)      # as the engine's sampler asks for the tokens of greedy requests
+        def decode(toks, n):
+            # as the engine decodes greedy requests: runs of steps on one scheduling decision, the
+            # tokens passing from step to step on the device
+            while n > 0:
+                k = min(args.decode_run, n)
+                toks = runner.decode_run([StepEntry(i, [t], [0]) for i, t in zip(ids, toks)], k)[-1]
+                n -= k
+            return toks
 
-        for _ in range(warmup):
-            tokens = one_step(tokens)
+        tokens = decode(tokens, warmup)
         torch.cuda.synchronize()
         first_ctx = runner.computed_tokens(ids[0])
         t = time.perf_counter()
-        for _ in range(steps):
-            tokens = one_step(tokens)
+        tokens = decode(tokens, steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         mean_ctx = first_ctx + (steps + 1) / 2.0
@@ -210,7 +216,7 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": args.dtype,
         "data": "synthetic: random weights (seed 0), uniform random token ids",
-        "config": config_record(cfg, args.layers, args.batch, mean_ctx, args.prefill_chunk),
+        "config": config_record(cfg, args.layers, args.batch, mean_ctx, args.prefill_chunk, args.decode_run),
         "prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(flops / prefill_s / FLOP_PEAK[args.dtype], 4)},
         "prefill_one_portion": {"value": round(PROMPT_LEN / whole_s, 1), "tokens": PROMPT_LEN, "ms": round(whole_s * 1e3, 3),

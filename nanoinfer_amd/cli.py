@@ -6,7 +6,7 @@ greedy), ``--top-k``, ``--top-p``, ``--rep-penalty``, ``--seed``, ``--max-tokens
 model folder here (the demos map a preset name to fixed paths), ``--dtype`` is fp32 or bf16 (the
 demos offer fp32 or int8).  What the demos fix at compile time (demo/batched_infer_multi_prompts.cpp:18-25)
 are options: ``--max-batch-size``, ``--max-sequences``, ``--prefill-chunk-size``, ``--block-size``,
-``--num-cache-blocks``.  Prompts are token ids (``--prompt-ids``) or random ids of given lengths
+``--num-cache-blocks``; ``--max-decode-run`` is this engine's own.  Prompts are token ids (``--prompt-ids``) or random ids of given lengths
 (``--prompt-len``): text goes through a tokenizer, which is outside this engine.
 """
 from __future__ import annotations
@@ -47,6 +47,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--num-cache-blocks", type=int, default=1024)
     ap.add_argument("--max-model-len", type=int, default=None)
+    ap.add_argument("--max-decode-run", type=int, default=8,
+                    help="decode steps run back to back on one scheduling decision (greedy requests only)")
     ap.add_argument("--json", action="store_true", help="print the generated ids as one JSON line per request")
     return ap
 
@@ -73,7 +75,7 @@ def main(argv: List[str] = None) -> int:
     cfg = EngineConfig(max_batch_size=args.max_batch_size, max_sequences=args.max_sequences,
                        prefill_chunk_size=args.prefill_chunk_size, block_size=args.block_size,
                        num_cache_blocks=args.num_cache_blocks, max_num_batched_tokens=args.max_num_batched_tokens,
-                       max_model_len=args.max_model_len, dtype=_DTYPES[args.dtype])
+                       max_model_len=args.max_model_len, max_decode_run=args.max_decode_run, dtype=_DTYPES[args.dtype])
     print(f"Model: {model_dir}  dtype: {args.dtype}", file=sys.stderr)
     t0 = time.perf_counter()
     engine = Engine(model_dir, cfg, ignore_eos=args.ignore_eos)

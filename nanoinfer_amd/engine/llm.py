@@ -15,7 +15,7 @@ from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence
 
 from ..sampling.params import SamplingParams
-from .scheduler import EngineConfig, Request, ScheduledBatch, Scheduler
+from .scheduler import EngineConfig, Request, ScheduledBatch, ScheduledItem, Scheduler
 
 
 @dataclass
@@ -95,6 +95,9 @@ class Engine:
             if item.samples:
                 sampling.append(item.request)
         self.last_prompt_tokens = sum(i.count for i in batch.items if i.count > 1 or not i.request.generated)
+        run = self.scheduler.decode_run_length(batch) if hasattr(self.runner, "decode_run") else 1
+        if run > 1:
+            return self._decode_run(batch, entries, run)
         logits = self.runner.step(entries)
         sampled: Dict[int, int] = {}
         if sampling:
@@ -104,6 +107,26 @@ class Engine:
             sampled = {r.request_id: int(t) for r, t in zip(sampling, ids)}
         self.num_steps += 1
         return self.scheduler.commit(batch, sampled)
+
+    def _decode_run(self, batch: ScheduledBatch, entries, run: int) -> List[Request]:
+        """``run`` greedy decode steps of the same batch on one scheduling decision: the runner
+        feeds every step's tokens to the next by itself; the scheduler then books the steps one by
+        one, and a request that stops on the way is finished there and its later tokens dropped."""
+        chosen = self.runner.decode_run(entries, run)
+        column = {item.request.request_id: b for b, item in enumerate(batch.items)}
+        finished: List[Request] = []
+        live = list(batch.items)
+        for k, tokens in enumerate(chosen):
+            if not live:
+                break
+            sub = batch if k == 0 else ScheduledBatch(
+                items=[ScheduledItem(i.request, i.request.num_computed, 1, True) for i in live])
+            sampled = {i.request.request_id: int(tokens[column[i.request.request_id]]) for i in sub.items}
+            finished.extend(self.scheduler.commit(sub, sampled))
+            live = [i for i in sub.items if i.request.finish_reason is None]
+            self.num_steps += 1
+        self.scheduler.last_scheduled_tokens = sum(len(t) for t in chosen)
+        return finished
 
     def run(self) -> List[Request]:
         """Step until nothing is left (src/engine/engine.cpp:191-198)."""

@@ -115,15 +115,19 @@ class _RecordedStep:
 
     graph: "torch.cuda.CUDAGraph"
     meta: torch.Tensor            # int32, device: every integer table of the step, fixed layout
-    staging: torch.Tensor         # the same, pinned host memory
+    stagings: list                # the same in pinned host memory: a few buffers used in turn, so that the host can
+                                  # write the tables of a step while the uploads of the steps before it are still queued
     logits: torch.Tensor
     ctx: StepContext
-    copied: "torch.cuda.Event" = None    # the last upload of the tables has left the staging buffer
+    copied: list = None                  # per staging buffer: its last upload has read it
+    turn: int = 0                        # the staging buffer that holds the tables of the last replay
     layout: list = None                  # per group (offset of slot mapping, offset of table, table width)
     order: tuple = ()                    # requests of the last replay, in batch order
     pages_written: list = None           # per group, per sequence: table entries already in the staging buffer
     tiles: dict = None                   # tile size -> (offset in the tables, number of tiles), for recorded prompt portions
     greedy: torch.Tensor = None          # int32, pinned host: argmax of every row of the logits, copied by the graph itself
+    amax: torch.Tensor = None            # the same on the device; a recorded decode step also leaves it in the place of
+                                         # its own token ids, where its next replay finds them without the host
     replayed: "torch.cuda.Event" = None  # the last replay has finished (and with it the copy into ``greedy``)
 
 
@@ -138,6 +142,8 @@ class ModelRunner:
     """
 
     GRAPH_MAX_BATCH = 64
+    STAGING_BUFFERS = 4           # pinned copies of a recorded step's tables, used in turn
+    HISTORY_ROWS = 16             # decode steps launched back to back before the host reads their tokens
     GRAPH_MIN_PORTION = 64        # a shorter prompt portion is not worth a recording
     GRAPH_MAX_PORTIONS = 24       # recordings of prompt portions kept (each holds its activations)
 
@@ -173,6 +179,8 @@ class ModelRunner:
         self._staging = [(None, None)] * 3     # pinned host buffers for the tables of eager steps, and their uploads' events
         self._staging_turn = 0
         self._greedy_of = None                 # (logits returned by the last recorded step, its recording)
+        self._history = None                   # pinned host: tokens chosen by decode steps launched back to back
+        self._history_done = None
 
     def _upload(self, flat: List[int]) -> torch.Tensor:
         """The integer tables of an eager step on the device.  They go through one of a few pinned
@@ -388,24 +396,34 @@ class ModelRunner:
         for ts, (off, count) in tiles.items():
             ctx._q_tiles[ts] = meta[off:off + 4 * count].view(-1, 4)
         greedy = torch.empty(max(n_rows, 1), dtype=torch.int32).pin_memory()
+        amax = None
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx, self._layer_cache(ctx))
             if logits is not None:
                 # greedy decoding needs only this: the recording picks the largest logit of every row
                 # and brings the ids to the host itself, so that no launch stands between step and token
-                greedy.copy_(K.argmax(logits), non_blocking=True)
+                amax = K.argmax(logits)
+                greedy.copy_(amax, non_blocking=True)
+                if kind == "d":
+                    # and leaves them where its own token ids stand: replayed again for the same requests
+                    # it decodes on, whether or not the host has looked at the tokens yet
+                    meta[0:size].copy_(amax)
         if ctx.tile_sizes_asked - set(tiles):
             self._unrecordable.add(key)       # the recorded run asked for tiles the eager run did not: not the same step
             return None
-        if K.library_calls() != calls_before and not self._replays_faithfully(graph, logits, warm, entries):
+        if K.library_calls() != calls_before and not self._replays_faithfully(graph, logits, warm, meta, staging):
             # a library routine ran inside and its recorded nodes do not reproduce the eager result
             # (some record memory-clearing nodes that misbehave on replay): this shape runs eagerly
             self._unrecordable.add(key)
             return None
-        rec = _RecordedStep(graph, meta, staging, logits, ctx, torch.cuda.Event())
-        rec.greedy, rec.replayed, rec.tiles = greedy, torch.cuda.Event(), tiles
-        rec.copied.record()
+        if kind == "d":
+            meta.copy_(staging)               # the recording's trial replays have put their own tokens there
+        stagings = [staging] + [torch.empty_like(staging).pin_memory() for _ in range(self.STAGING_BUFFERS - 1)]
+        rec = _RecordedStep(graph, meta, stagings, logits, ctx, [torch.cuda.Event() for _ in stagings])
+        rec.greedy, rec.amax, rec.replayed, rec.tiles = greedy, amax, torch.cuda.Event(), tiles
+        for done in rec.copied:
+            done.record()
         self._recorded[key] = rec
         return rec
 
@@ -422,12 +440,15 @@ class ModelRunner:
                 parts.append(g.vpools[cid][pages, :, offs].float().reshape(-1))
         return torch.cat(parts) if parts else torch.zeros(1, device=self.device)
 
-    def _replays_faithfully(self, graph, logits, warm: StepContext, entries: List[StepEntry], rounds: int = 3) -> bool:
+    def _replays_faithfully(self, graph, logits, warm: StepContext, meta: torch.Tensor, staging: torch.Tensor,
+                            rounds: int = 3) -> bool:
         """Replay a fresh recording several times, with the same step run eagerly and a
         synchronisation between the replays, and compare every replay with the eager run: the
         logits, or for a step that returns none the keys and values it wrote.  A step may be run any
-        number of times: it writes the same keys and values again."""
+        number of times: it writes the same keys and values again.  (Its tables are uploaded anew
+        each time: a recorded decode step overwrites its token ids with the ones it has chosen.)"""
         for _ in range(rounds):
+            meta.copy_(staging)
             graph.replay()
             torch.cuda.synchronize()
             got = logits.clone() if logits is not None else self._written_rows(warm)
@@ -440,25 +461,37 @@ class ModelRunner:
                 return False
         return True
 
-    def _replay(self, key, entries: List[StepEntry]) -> bool:
+    def _replay(self, key, entries: List[StepEntry], tokens_from: Optional[_RecordedStep] = None,
+                history_row: Optional[int] = None) -> bool:
         """Run the entries through the recording of their shape (made now if there is none).  False:
         this shape cannot be recorded and the step has not run.  The logits are left in
-        ``self._replayed_logits``."""
+        ``self._replayed_logits``.
+
+        ``tokens_from``: the token ids of the entries are not known to the host; they are what the
+        last replay of that recording (a decode step over the same requests in the same order)
+        chose, and are taken from where it left them on the device.  ``history_row``: the tokens
+        this replay chooses are also copied to that row of ``self._history`` (pinned host memory),
+        and its logits are not kept."""
         rec = self._recorded.get(key)
         if rec is None:
             rec = self._record(key, entries)
             if rec is None:
                 return False
             # the recording itself ran nothing: fall through to the first replay
-        rec.copied.synchronize()          # the previous upload must have read the staging buffer
         kind, B, width = key[0], key[1], key[2]
         ps = self.page_size
-        st = rec.staging.numpy()          # shares the pinned memory
+        # the tables are written into the next staging buffer in turn, starting from those of the last replay
+        last = rec.stagings[rec.turn]
+        rec.turn = (rec.turn + 1) % len(rec.stagings)
+        rec.copied[rec.turn].synchronize()          # the upload that last used this buffer has read it
+        staging = rec.stagings[rec.turn]
+        st = staging.numpy()                        # shares the pinned memory
         order = tuple(e.request for e in entries)
         totals = []
         if kind == "d" and order == rec.order:
             # the same requests in the same places as last time: tokens, positions and slots change,
             # block tables only grow at their ends
+            st[:] = last.numpy()
             for b, e in enumerate(entries):
                 done = self._done[e.request]
                 st[b] = int(e.tokens[0])
@@ -477,20 +510,33 @@ class ModelRunner:
                     done = totals[b] - 1
                     st[off_slot + b] = table[done // ps] * ps + done % ps
         else:
+            if tokens_from is not None:
+                raise StepError("tokens can stay on the device only between decode steps over the same requests")
             ctx = StepContext(self.device)
             flat, layout, _, tiles = self._tables_of(entries, ctx, width, rec.tiles or ())
-            if len(flat) != rec.staging.numel() or tiles != (rec.tiles or {}):
+            if len(flat) != staging.numel() or tiles != (rec.tiles or {}):
                 raise StepError("a recorded step was asked to run another shape")
             st[:] = flat
             rec.layout = layout
             rec.order = order if kind == "d" else ()
             rec.pages_written = [[len(g.tables[e.request]) for e in entries] for g in self.cache.groups]
             totals = ctx.context_len
-        rec.meta.copy_(rec.staging, non_blocking=True)
-        rec.copied.record()
+        if tokens_from is None:
+            rec.meta.copy_(staging, non_blocking=True)
+        else:
+            # everything but the token ids, which are on the device already: in this recording's own
+            # tables if it ran last, else in the other recording's choice
+            rec.meta[B:].copy_(staging[B:], non_blocking=True)
+            if tokens_from is not rec:
+                rec.meta[0:B].copy_(tokens_from.amax[0:B], non_blocking=True)
+        rec.copied[rec.turn].record()
         rec.graph.replay()
-        rec.replayed.record()
         self._last_context_len = totals
+        if history_row is not None:
+            self._history[history_row, 0:B].copy_(rec.amax[0:B], non_blocking=True)
+            self._replayed_logits = None
+            return True
+        rec.replayed.record()
         if rec.logits is None:
             self._replayed_logits = None
         else:
@@ -498,6 +544,11 @@ class ModelRunner:
             self._greedy_of = (out, rec)
             self._replayed_logits = out
         return True
+
+    def _book(self, entries: List[StepEntry], totals: Sequence[int]) -> None:
+        for e, total in zip(entries, totals):
+            self._done[e.request] = total
+            self.cache.release_passed(e.request, total)
 
     def step(self, entries: Sequence[StepEntry], end: Iterable[Hashable] = ()) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits ``[wanted, vocab]`` on the device, rows in the
@@ -519,9 +570,60 @@ class ModelRunner:
                 self._bind(ctx, self._upload(flat), layout, n_rows)
                 logits = self.model.forward(ctx, self._layer_cache(ctx))
                 totals = ctx.context_len
-            for e, total in zip(entries, totals):
-                self._done[e.request] = total
-                self.cache.release_passed(e.request, total)
+            self._book(entries, totals)
         for r in end:
             self.release(r)
         return logits
+
+    def decode_run(self, entries: Sequence[StepEntry], steps: int) -> List[List[int]]:
+        """Greedy decoding of ``steps`` tokens for every entry (one token each, wanting its logits):
+        the first step takes the entries' tokens, every later one the tokens that the step before
+        chose (the index of the largest logit, lowest index on ties).  Returns the chosen tokens,
+        ``[step][entry]``: what ``steps`` calls of :meth:`step` with :meth:`greedy_tokens` between
+        them return.  Where recordings of the steps' shapes exist, the steps are launched back to
+        back, the tokens passing from one to the next on the device, and the host waits once at
+        the end: the GPU is not idle while the host reads a token and launches the next step.
+        A shape without a recording runs the ordinary way (which records it)."""
+        entries = list(entries)
+        if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
+            raise StepError("decode_run takes entries of one token each that want its logits")
+        B = len(entries)
+        chosen: List[List[int]] = []
+        tokens: Optional[List[int]] = [int(e.tokens[0]) for e in entries]     # None: still on the device
+        launched = 0                # replays whose tokens the host has not read yet
+        last: Optional[_RecordedStep] = None
+        self._greedy_of = None
+        if self._history is None:
+            self._history = torch.zeros(self.HISTORY_ROWS, self.GRAPH_MAX_BATCH, dtype=torch.int32).pin_memory()
+            self._history_done = torch.cuda.Event()
+
+        def collect() -> None:
+            nonlocal launched, tokens
+            if launched:
+                self._history_done.record()
+                self._history_done.synchronize()
+                rows = self._history[0:launched, 0:B].tolist()
+                chosen.extend(rows)
+                tokens = rows[-1]
+                launched = 0
+
+        for _ in range(int(steps)):
+            cur = [StepEntry(e.request, [tokens[b] if tokens is not None else 0], [0]) for b, e in enumerate(entries)]
+            key = self._graph_shape(cur) if B else None
+            rec = self._recorded.get(key) if key is not None else None
+            if rec is None or rec.amax is None or launched == self.HISTORY_ROWS:
+                collect()
+                cur = [StepEntry(e.request, [tokens[b]], [0]) for b, e in enumerate(entries)]
+            if rec is None or rec.amax is None:
+                tokens = self.greedy_tokens(self.step(cur))
+                chosen.append(list(tokens))
+                last = None
+                continue
+            self._check_and_reserve(cur)
+            self._replay(key, cur, tokens_from=last if tokens is None else None, history_row=launched)
+            self._book(cur, self._last_context_len)
+            launched += 1
+            tokens = None
+            last = rec
+        collect()
+        return chosen

@@ -85,12 +85,13 @@ class EngineConfig:
     num_cache_blocks: int = 1024      # pages in the pool
     max_num_batched_tokens: int = 2048  # token budget of a step
     max_model_len: Optional[int] = None  # longest request (prompt + generated); None: what model and pool allow
+    max_decode_run: int = 8           # decode steps run back to back on one scheduling decision (1: never more than one)
     dtype: str = "bfloat16"
     seed: int = 0
 
     def validate(self) -> None:
         for name in ("max_batch_size", "max_sequences", "prefill_chunk_size", "block_size", "num_cache_blocks",
-                     "max_num_batched_tokens"):
+                     "max_num_batched_tokens", "max_decode_run"):
             if getattr(self, name) < 1:
                 raise ValueError(f"{name} must be at least 1, got {getattr(self, name)}")
 
@@ -221,6 +222,30 @@ class Scheduler:
             take(req, count)
         self.last_scheduled_tokens = batch.num_tokens
         return batch
+
+    def decode_run_length(self, batch: ScheduledBatch) -> int:
+        """For how many steps in a row ``batch`` can be run again on this one decision (at most
+        ``max_decode_run``; 1: only the step that was scheduled).  More than one only if a new
+        decision could change nothing but by a request's end: the batch is every running request,
+        one token each whose successor is wanted; nobody waits or was preempted; every request
+        decodes greedily without a repetition penalty (its next token is then the largest logit,
+        which the runner can feed back without the host); each has that many tokens left to
+        generate; and the pool has pages for all of them.  A request that meets its stop token
+        within the run has run a few tokens too far: they are dropped."""
+        steps = self.config.max_decode_run
+        if steps <= 1 or not batch.items or batch.preempted or self.waiting or len(batch.items) != len(self.running):
+            return 1
+        for item in batch.items:
+            req = item.request
+            if item.count != 1 or not item.samples:
+                return 1
+            if not req.params.use_greedy() or req.params.use_repetition_penalty():
+                return 1
+            steps = min(steps, req.max_new_tokens - len(req.generated))
+        while steps > 1 and not self.cache.can_reserve_all(
+                [(i.request.request_id, i.request.num_computed + steps) for i in batch.items]):
+            steps -= 1
+        return max(steps, 1)
 
     # ---------------------------------------------------------------- after the step
     def commit(self, batch: ScheduledBatch, sampled: Dict[int, int]) -> List[Request]:

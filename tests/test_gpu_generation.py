@@ -49,6 +49,26 @@ def test_greedy_generation_equals_plain(name):
     assert eng.runner.cache.free_pages() == 16
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_runs_do_not_change_the_tokens(dtype):
+    """Greedy requests decode in runs of steps on one scheduling decision (max_decode_run); the
+    tokens are those of an engine that decides before every step, also when requests end at
+    different times, join later and draw from a pool that runs short."""
+    from nanoinfer_amd.sampling.params import SamplingParams
+    folder = model_folder("B")
+    prompts = [list(random_tokens(1000, n, 80 + n)) for n in (9, 40, 23, 3)]
+    outs = []
+    for run in (1, 8):
+        eng = engine(folder, dtype=dtype, block_size=8, num_cache_blocks=24, max_sequences=3, max_decode_run=run)
+        ids = [eng.add_request(p, n, SamplingParams.greedy()) for p, n in zip(prompts, (30, 11, 50, 17))]
+        eng.run()
+        outs.append([eng.get_request(i).generated for i in ids])
+        assert eng.runner.cache.free_pages() == 24
+        assert all(eng.get_request(i).finish_reason == "length" for i in ids)
+    assert outs[0] == outs[1]
+    assert [len(t) for t in outs[1]] == [30, 11, 50, 17]
+
+
 def test_stop_token_from_the_configuration():
     from nanoinfer_amd.sampling.params import SamplingParams
     folder = model_folder("B")

@@ -418,3 +418,55 @@ def test_recorded_prompt_portions_equal_eager_ones(dtype):
         rows.sort(key=lambda x: x[0])
         idx = [p for p, _ in rows]
         assert_close(torch.stack([r for _, r in rows]), want[idx], dtype, f"recorded portions, request {rid}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_runs_equal_single_steps(dtype):
+    """Runs of decode steps launched back to back, the tokens passing from step to step on the
+    device, choose the tokens that single steps with the host between them choose.  The runs
+    cross page edges, the context bounds at which another recording takes over (256), the number
+    of steps whose tokens the host collects at once, and start before any recording exists; the
+    cache they leave gives the same logits afterwards.  Both runners replay the same recordings, so
+    their tokens are equal bit for bit.  A runner without recordings decodes in runs too, step by
+    step; its attention cuts the keys elsewhere, which may turn a tie of two logits the other way,
+    so its tokens are compared in float32 only, where ties are not met."""
+    from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
+    name = "B"
+    folder = model_folder(name)
+    vocab = ALL[name]["vocab_size"]
+    runs = ModelRunner(folder, dtype=dtype, page_size=8, max_tokens=2048, max_requests=4)
+    single = ModelRunner(folder, dtype=dtype, page_size=8, max_tokens=2048, max_requests=4)
+    eager = ModelRunner(folder, dtype=dtype, page_size=8, max_tokens=2048, max_requests=4, use_graphs=False)
+    prompts = {f"r{i}": list(random_tokens(vocab, n, 900 + i)) for i, n in enumerate((236, 150, 61))}
+    tokens = {}
+    with_eager = dtype == "float32"
+    for rid, p in prompts.items():
+        firsts = []
+        for runner in (runs, single, eager) if with_eager else (runs, single):
+            logits = runner.step([StepEntry(rid, p, [len(p) - 1])])
+            firsts.append(runner.greedy_tokens(logits)[0])
+        assert len(set(firsts)) == 1
+        tokens[rid] = firsts[0]
+    ids = list(prompts)
+    for k in (1, 3, 8, 20, 2, 33):
+        entries = [StepEntry(rid, [tokens[rid]], [0]) for rid in ids]
+        got = runs.decode_run(entries, k)
+        want = []
+        toks = [tokens[rid] for rid in ids]
+        for _ in range(k):
+            toks = single.greedy_tokens(single.step([StepEntry(rid, [t], [0]) for rid, t in zip(ids, toks)]))
+            want.append(list(toks))
+        assert got == want, k
+        if with_eager:
+            assert eager.decode_run([StepEntry(rid, [tokens[rid]], [0]) for rid in ids], k) == want, k
+        assert all(runs.computed_tokens(rid) == single.computed_tokens(rid) for rid in ids)
+        tokens = dict(zip(ids, want[-1]))
+    assert runs.computed_tokens("r0") == 236 + 67 > 256                  # the longest request has passed a bound
+    probe = [StepEntry(rid, [tokens[rid]], [0]) for rid in ids]
+    a, b = runs.step(probe), single.step(probe)
+    assert float((a - b).abs().max()) <= TOL[dtype] * float(b.abs().max()) * 0.1
+    # a batch of another make-up after a run: the tables are written anew
+    a, b = runs.step(probe[:2]), single.step(probe[:2])
+    assert float((a - b).abs().max()) <= TOL[dtype] * float(b.abs().max()) * 0.1
+    with pytest.raises(Exception):
+        runs.decode_run([StepEntry("r0", [1, 2], [1])], 2)

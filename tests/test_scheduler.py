@@ -219,3 +219,96 @@ def test_engine_never_plans_more_than_fits():
         assert eng.get_request(rid).generated == tokens
     assert runner.cache.free_pages() == 12 and eng.scheduler.stats()["num_finished"] == len(want)
     assert all(len(s) <= 4 and sum(n for _, n, _ in s) <= 16 for s in runner.steps)
+
+
+# ---- runs of decode steps on one scheduling decision
+
+class FakeRunnerWithRuns(FakeRunner):
+    """A runner that can also decode several steps in a row, feeding every step's largest logit to the next."""
+
+    def __init__(self, **kw):
+        super().__init__(**kw)
+        self.runs = []           # length of every run asked for
+
+    def decode_run(self, entries, steps):
+        from nanoinfer_amd.engine.runner import StepEntry
+        self.runs.append(steps)
+        chosen = []
+        tokens = [e.tokens[0] for e in entries]
+        for _ in range(steps):
+            logits = self.step([StepEntry(e.request, [t], [0]) for e, t in zip(entries, tokens)])
+            tokens = logits.argmax(dim=-1).tolist()
+            chosen.append(tokens)
+        return chosen
+
+
+def make_run_engine(**kw):
+    runner_kw = {k: kw.pop(k) for k in list(kw) if k in ("page_size", "num_pages", "max_requests", "max_positions", "eos")}
+    runner = FakeRunnerWithRuns(**runner_kw)
+    cfg = EngineConfig(block_size=runner.cache.page_size, num_cache_blocks=runner.cache.num_pages, **kw)
+    return Engine(config=cfg, runner=runner, sampler=ArgmaxSampler()), runner
+
+
+def test_decode_runs_give_the_tokens_of_single_steps():
+    outs = []
+    for run in (1, 8):
+        eng, runner = make_run_engine(max_decode_run=run, num_pages=32)
+        a = eng.add_request([7, 8, 9], max_new_tokens=12, params=SamplingParams.greedy())
+        b = eng.add_request([20], max_new_tokens=5, params=SamplingParams.greedy())
+        eng.run()
+        outs.append([(eng.get_request(r).generated, eng.get_request(r).finish_reason) for r in (a, b)])
+        assert not runner.cache.live_requests()
+        if run == 1:
+            assert runner.runs == []
+        else:
+            # both decode together for 4 steps (the shorter request has 4 tokens left), then the longer alone: 7 = 7
+            assert runner.runs == [4, 7]
+    assert outs[0] == outs[1]
+    assert outs[0][0] == (list(range(10, 22)), "length") and outs[0][1] == (list(range(21, 26)), "length")
+
+
+def test_a_stop_token_inside_a_run_ends_the_request_there():
+    eng, runner = make_run_engine(max_decode_run=8, eos=(13,), num_pages=32)
+    a = eng.add_request([8, 9], max_new_tokens=20, params=SamplingParams.greedy())      # 10, 11, 12, 13: stop
+    b = eng.add_request([19, 20], max_new_tokens=20, params=SamplingParams.greedy())
+    eng.step()                                     # the prompts (a prompt of one token would start a run itself)
+    finished = eng.step()                          # one run of 8 steps: a stops at its third
+    ra, rb = eng.get_request(a), eng.get_request(b)
+    assert [r.request_id for r in finished] == [a]
+    assert ra.generated == [10, 11, 12, 13] and ra.finish_reason == "stop"      # the stop token is kept, nothing after it
+    assert rb.generated == list(range(21, 30)) and rb.finish_reason is None
+    assert set(runner.cache.live_requests()) == {b}
+    eng.run()
+    assert rb.generated == list(range(21, 41)) and not runner.cache.live_requests()
+
+
+def test_what_keeps_a_decode_step_single():
+    greedy = SamplingParams.greedy()
+    # somebody waits (max_sequences 1 keeps the second request out)
+    eng, runner = make_run_engine(max_decode_run=8, max_sequences=1, num_pages=32)
+    eng.add_request([1, 2], max_new_tokens=4, params=greedy)
+    eng.add_request([3, 4], max_new_tokens=4, params=greedy)
+    eng.run()
+    assert runner.runs == [3]                       # only the second request, once the first has gone, decodes in a run
+    # a request that draws, or that has a repetition penalty
+    for params in (SamplingParams(temperature=0.7, seed=1), SamplingParams(temperature=0.0, repetition_penalty=1.3)):
+        eng, runner = make_run_engine(max_decode_run=8, num_pages=32)
+        eng.add_request([1, 2], max_new_tokens=6, params=params)
+        eng.run()
+        assert runner.runs == []
+    # a prompt portion in the batch
+    eng, runner = make_run_engine(max_decode_run=8, num_pages=32, max_num_batched_tokens=4)
+    eng.add_request([1, 2], max_new_tokens=6, params=greedy)
+    eng.step()
+    eng.add_request(list(range(10)), max_new_tokens=2, params=greedy)
+    eng.step()
+    assert runner.runs == []                        # the step mixed a decode token with a prompt portion
+    # pages: four tokens a page, five pages; one request of 3 + 14 tokens can run only as far as pages reach
+    eng, runner = make_run_engine(max_decode_run=8, num_pages=5, page_size=4)
+    r = eng.add_request([1, 2, 3], max_new_tokens=18, params=greedy)
+    eng.run()
+    assert eng.get_request(r).finish_reason == "length" and max(runner.runs) <= 8
+    sched = eng.scheduler
+    assert sched.config.max_decode_run == 8
+    with pytest.raises(ValueError):
+        EngineConfig(max_decode_run=0).validate()
