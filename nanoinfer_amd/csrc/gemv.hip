@@ -105,14 +105,22 @@ struct RopeArgs {
 
 // What follows the main loop of both kernels: the wavefronts' partial sums meet in LDS and the
 // epilogue stores them.
-template <typename T, typename TOUT, int MB, int NT, int EPI, int WV = GV_WAVES>
+template <typename T, typename TOUT, int MB, int NT, int EPI, int WV = GV_WAVES, bool EXT = false>
 __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TOUT* __restrict__ y, int M, int N, int I,
-                                              const RopeArgs& rope) {
+                                              const RopeArgs& rope, float* ext = nullptr) {
     const int tid = threadIdx.x;
     const int wave = tid / WAVE, lane = tid % WAVE;
     const int wg = blockIdx.x;
-    // partial sums of the wavefronts meet in LDS: red[wave][tile][lane * 4 + i]
-    __shared__ float red[WV][NT * MB][WAVE * 4];
+    // partial sums of the wavefronts meet in LDS: red[wave][tile][lane * 4 + i]; in memory of the
+    // function's own, or (EXT) in memory the kernel has no other use for any more
+    typedef float (*Red)[NT * MB][WAVE * 4];
+    Red red;
+    if constexpr (EXT) {
+        red = reinterpret_cast<Red>(ext);
+    } else {
+        __shared__ float red_own[WV][NT * MB][WAVE * 4];
+        red = red_own;
+    }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -506,6 +514,118 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
     skinny_finish<T, TOUT, 1, NT, EPI, WV>(acc, y, M, N, I, rope);
 }
 
+// 17 to 64 rows with re-tiled W.  The operand layout spreads a row of x over few lanes, so loaded
+// in that layout four blocks of rows cost the texture path twice the instructions of W itself (a
+// vector load takes it the same time whatever it fetches).  Here a wavefront brings the rows of x
+// that belong to its piece of K into LDS with full 16-byte loads of neighbouring lanes (eight
+// lanes a row), a slab of its own that needs no workgroup barrier, and picks the operands of all
+// its row blocks from there.  Two trips are in registers at a time, in two fixed sets, as in the
+// decode kernel.  The slabs' memory takes the partial sums at the end.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));    // 16 bytes that only pass through registers
+#define SLAB_ROW 144      // bytes: a 128-byte piece of a row and 16 of padding, so that the rows of a read fall on different banks
+
+template <typename T, typename TOUT, int MB, int NT, int EPI>
+__global__ __launch_bounds__(GV_THREADS) void skinny_rows_kernel(const T* __restrict__ x, const T* __restrict__ W,
+                                                                 TOUT* __restrict__ y, int M, int N, int K, int I,
+                                                                 RopeArgs rope) {
+    constexpr int EL = Piece<T>::ELEMS;
+    constexpr int CH = 4 * EL;
+    constexpr int WV = GV_WAVES;
+    constexpr int ROWS = MB * 16;
+    constexpr int XL = ROWS / 8;                       // 16-byte loads of a lane for one piece of all rows
+    constexpr int SLAB = ROWS * SLAB_ROW;
+    constexpr int RED = NT * MB * WAVE * 4 * static_cast<int>(sizeof(float));
+    __shared__ __attribute__((aligned(16))) unsigned char lds[WV * (SLAB > RED ? SLAB : RED)];
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;      // the same in every lane: say so
+    const int r = lane % 16, kg = lane / 16;
+    const int wg = blockIdx.x;
+    const int pieces = (K + CH - 1) / CH;
+    unsigned char* slab = lds + wave * SLAB;
+
+    const T* wrow[NT];      // first byte of this lane in piece 0 of each tile
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        int col0 = (EPI == EPI_SWIGLU) ? (wg * (NT / 2) + nt / 2) * 16 : (wg * NT + nt) * 16;
+        if (EPI == EPI_ROPE) {
+            const int per_head = rope.hd / 32;
+            col0 = (wg / per_head) * rope.hd + (wg % per_head) * 16 + nt * (rope.hd / 2);
+        }
+        const int shift = (EPI == EPI_SWIGLU && (nt % 2)) ? I : 0;
+        const int limit = (N + 15) / 16 - 1;         // a workgroup's last tiles may lie past the matrix: read the last one, store nothing
+        wrow[nt] = W + static_cast<size_t>(min((col0 + shift) / 16, limit)) * pieces * (WAVE * EL) + lane * EL;
+    }
+    floatx4_t acc[NT][MB];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    // pieces past the end of a row are read from its last piece and not multiplied: no load is under a branch
+    auto load_w = [&](int c, Piece<T> (&wa)[NT]) {
+        const int piece = min(c, pieces - 1);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) wa[nt].load(wrow[nt] + static_cast<size_t>(piece) * (WAVE * EL));
+    };
+    // x: lane l takes 16 bytes number l % 8 of the piece, of rows l / 8, l / 8 + 8, ...  (rows that do
+    // not exist read the last row; their columns are not stored).  K is a multiple of 32 bytes'
+    // worth of elements, so 16 bytes lie wholly inside a row or wholly past its end (then zeros:
+    // W is zero there, but zero times what lies behind x need not be)
+    constexpr int PER16 = 16 / static_cast<int>(sizeof(T));
+    auto load_x = [&](int c, u32x4_t (&xr)[XL]) {
+        const int k = min(c, pieces - 1) * CH + (lane % 8) * PER16;
+#pragma unroll
+        for (int i = 0; i < XL; ++i) {
+            const int row = min(i * 8 + lane / 8, M - 1);
+            const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(row) * K + min(k, K - PER16));
+            xr[i] = k < K ? v : u32x4_t{0u, 0u, 0u, 0u};
+        }
+    };
+    auto stage = [&](const u32x4_t (&xr)[XL]) {
+#pragma unroll
+        for (int i = 0; i < XL; ++i)
+            *reinterpret_cast<u32x4_t*>(slab + (i * 8 + lane / 8) * SLAB_ROW + (lane % 8) * 16) = xr[i];
+    };
+    // the lanes of one wavefront run together: ordering its own LDS writes and reads takes no barrier
+    auto wave_sync = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    auto multiply = [&](const Piece<T> (&wa)[NT]) {
+        Piece<T> xb[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) xb[mb].load(reinterpret_cast<const T*>(slab + (mb * 16 + r) * SLAB_ROW + kg * 32));
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = Piece<T>::mma(wa[nt], xb[mb], acc[nt][mb]);
+    };
+
+    Piece<T> wa_a[NT], wa_b[NT];
+    u32x4_t xr_a[XL], xr_b[XL];
+    load_w(wave, wa_a);
+    load_x(wave, xr_a);
+    for (int c = wave; c < pieces; c += 2 * WV) {
+        stage(xr_a);
+        wave_sync();
+        load_w(c + WV, wa_b);
+        load_x(c + WV, xr_b);
+        multiply(wa_a);
+        wave_sync();                       // the slab has been read: it may be written again
+        if (c + WV < pieces) {
+            stage(xr_b);
+            wave_sync();
+            load_w(c + 2 * WV, wa_a);
+            load_x(c + 2 * WV, xr_a);
+            multiply(wa_b);
+            wave_sync();
+        }
+    }
+    __syncthreads();                       // every wavefront is done with its slab: the partial sums take the memory
+    skinny_finish<T, TOUT, MB, NT, EPI, WV, true>(acc, y, M, N, I, rope, reinterpret_cast<float*>(lds));
+}
+
 template <typename T, typename TOUT, int MB, int EPI>
 static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, bool tiled,
                      hipStream_t stream, RopeArgs rope = RopeArgs{}) {
@@ -575,12 +695,41 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
     return NI_LAUNCH_RESULT();
 }
 
+// The kernel for 17 to 64 rows: MB blocks of 16 rows, NT as launch_nt chooses it, within the eight
+// fragments of partial sums a wavefront may hold.
+template <typename T, typename TOUT, int MB, int EPI>
+static int launch_rows(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream,
+                       RopeArgs rope = RopeArgs{}) {
+    const int out_width = (EPI == EPI_SWIGLU) ? I : N;
+    const int tiles = (out_width + 15) / 16;
+    auto run = [&](auto nt_tag) {
+        constexpr int NTc = decltype(nt_tag)::value;
+        constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
+        const int grid = (tiles + NOUT - 1) / NOUT;
+        skinny_rows_kernel<T, TOUT, MB, NTc, EPI><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope);
+    };
+    if constexpr (EPI == EPI_SWIGLU || EPI == EPI_ROPE) {
+        run(std::integral_constant<int, 2>{});
+    } else {
+        if constexpr (MB <= 2) {
+            if (NT >= 4) { run(std::integral_constant<int, 4>{}); return NI_LAUNCH_RESULT(); }
+        }
+        if (NT >= 2) run(std::integral_constant<int, 2>{});
+        else run(std::integral_constant<int, 1>{});
+    }
+    return NI_LAUNCH_RESULT();
+}
+
 template <typename T, typename TOUT, int EPI>
 static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, bool tiled,
                      hipStream_t stream, RopeArgs rope = RopeArgs{}) {
     if (M <= 16 && tiled) return launch_decode<T, TOUT, EPI, 0>(x, W, y, M, N, K, I, NT, stream, rope);
+    if (tiled) {
+        if (M <= 32) return launch_rows<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
+        return launch_rows<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
+    }
     if constexpr (EPI == EPI_RESIDUAL) {
-        return -7;      // the residual epilogue exists in the decode kernel only
+        return -7;      // the residual epilogue exists for re-tiled matrices only
     } else {
         if (M <= 16) return launch_nt<T, TOUT, 1, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
         if (M <= 32) return launch_nt<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
@@ -611,7 +760,7 @@ static int launch_normed(const NormArgs& norm, const void* W, void* y, int M, in
 }
 
 // epilogue: 0 store in the input type, 1 store float32, 2 SwiGLU (W is [2I, K], y is [M, I]),
-// 3 add into y, the float32 residual stream [M, N] (M <= 16, tiled W).
+// 3 add into y, the float32 residual stream [M, N] (tiled W).
 // K must be a multiple of 16 bytes' worth of elements x 2 (bf16: 16, f32: 8); M <= 64.
 // tiled: W is in the re-tiled order described at the top (swiglu then needs N/2 to be a multiple of 16).
 NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N, int K, int epilogue, int tiles_per_group,

@@ -444,7 +444,23 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
 # ------------------------------------------------------------------ matrix product (library)
 
 SKINNY_MAX_ROWS = 64        # what the kernel takes
-SKINNY_BEST_ROWS = 16       # up to here it beats the library product on this chip (measured at the 1B sizes)
+SKINNY_BEST_ROWS = 16       # up to here the skinny product beats the library's on this chip whatever the matrix
+
+
+def skinny_wins(M: int, K: int, dtype: torch.dtype, weight=None) -> bool:
+    """Whether the skinny product is the faster one for M rows of K elements (measured at the 1B
+    sizes, bfloat16).  Up to 16 rows always.  From 17 to 64 rows (re-tiled matrices only) every
+    workgroup reads the rows of x that belong to its columns' K range anew: that is worth it while
+    x is small beside the matrix, which ends at rows of more than 4,096 elements and over 32 rows
+    (the [2048, 8192] matrix: 20.8 us against the library's 19.5 at 64 rows, 14.0 : 13.7 at 32,
+    while [2048, 2048] takes 7.0 : 8.7 and the stacked [16384, 2048] with SwiGLU 21.8 : 25.5)."""
+    if not skinny_ok(M, K, dtype):
+        return False
+    if M <= SKINNY_BEST_ROWS:
+        return True
+    if not (isinstance(weight, Weight) and weight.tiles is not None):
+        return False
+    return M <= 32 or K <= 4096
 FUSE_NORMS = True           # residual sums and norms ride on the skinny products of a decode step where they can
 
 
@@ -540,8 +556,7 @@ def norm_prologue_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
 
 def residual_epilogue_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
     """Whether the skinny product can add its result straight into the float32 residual stream."""
-    return (isinstance(weight, Weight) and weight.tiles is not None and 0 < M <= SKINNY_BEST_ROWS
-            and skinny_ok(M, K, dtype))
+    return isinstance(weight, Weight) and weight.tiles is not None and skinny_wins(M, K, dtype, weight)
 
 
 def _check_normed(x: NormedInput, Kd: int) -> None:
@@ -577,8 +592,8 @@ def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bo
         _gpu(out, "out", dtype, (M, N // 2))
         epi = 2
     elif residual:
-        if not (tiles is not None and M <= 16):
-            raise KernelError("the residual epilogue needs a re-tiled matrix and at most 16 rows")
+        if not (tiles is not None):
+            raise KernelError("the residual epilogue needs a re-tiled matrix")
         _gpu(out, "out", torch.float32, (M, N))
         epi = 3
     else:
@@ -675,7 +690,7 @@ def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optiona
         skinny_gemm(x, weight, residual, residual=True)
         return None
     out_dtype = out_dtype or x.dtype
-    if x.shape[0] <= SKINNY_BEST_ROWS and skinny_ok(x.shape[0], x.shape[1], x.dtype):
+    if skinny_wins(x.shape[0], x.shape[1], x.dtype, weight):
         out = torch.empty(x.shape[0], rows.shape[0], dtype=out_dtype, device=x.device)
         return skinny_gemm(x, weight, out)
     rows_t = weight.rows_t if isinstance(weight, Weight) else rows.t()
@@ -691,7 +706,9 @@ def linear_swiglu(x, weight_gate_up) -> torch.Tensor:
     few rows, product then the SwiGLU kernel for many.  ``x`` may be a :class:`NormedInput`."""
     inter = weight_gate_up.shape[0] // 2
     out = torch.empty(x.shape[0], inter, dtype=x.dtype, device=x.device)
-    if isinstance(x, NormedInput) or (x.shape[0] <= SKINNY_BEST_ROWS and skinny_ok(x.shape[0], x.shape[1], x.dtype)):
+    # (past 16 rows only a matrix whose halves start on tile boundaries is streamed re-tiled)
+    if isinstance(x, NormedInput) or (skinny_wins(x.shape[0], x.shape[1], x.dtype, weight_gate_up)
+                                      and (x.shape[0] <= SKINNY_BEST_ROWS or inter % 16 == 0)):
         return skinny_gemm(x, weight_gate_up, out, swiglu=True)
     global _library_calls
     _library_calls += 1
