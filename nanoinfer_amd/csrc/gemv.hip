@@ -11,10 +11,12 @@
 // instructions per piece.  The MFMA's k index is only a label, so the same lane-to-k mapping on
 // both operands is all that is required.  Partial sums meet in LDS.
 //
-// W comes either as stored, [N, K] row-major, or re-tiled once at load into the order this kernel
-// reads it: [tile of 16 rows][128-byte piece][lane][32 bytes], zero-padded to whole tiles and
+// W comes either as stored, [N, K] row-major, or re-tiled once at load into the order the kernels
+// read it: [tile of 16 rows][128-byte piece][lane][32 bytes], zero-padded to whole tiles and
 // pieces.  A wavefront's load is then 2 KB of consecutive memory instead of sixteen 128-byte
-// runs 2*K bytes apart, which is worth about a third on the [2048, 8192] matrix.
+// runs 2*K bytes apart, which is worth about a third on the [2048, 8192] matrix.  Three kernels:
+// the first, described above, takes W as stored (any number of rows up to 64); the other two
+// take it re-tiled, one for the decode step proper (at most 16 rows), one for 17 to 64 rows.
 //
 // Epilogues: store (compute type or float32), or SwiGLU over paired tiles (tile 2j from the gate
 // rows, tile 2j+1 from the up rows of a stacked [2I, K] matrix): out[m, n] = silu(g) * u; or
@@ -24,13 +26,14 @@
 // or addition into the float32 residual stream (h[m, n] += the product, in place: a workgroup
 // reads and writes only its own columns).
 //
-// A second kernel serves the decode step proper: at most 16 rows and re-tiled weights.  It keeps two
+// The kernel of the decode step proper (at most 16 rows, re-tiled weights) keeps two
 // trips in registers (one multiplied while the other's loads are under way), and can take, instead
 // of x, the float32 residual stream h [M, K] with the weights and eps of an RMSNorm: every
 // workgroup then normalises the rows itself (sums of squares over the wavefronts' K slices, met in
 // LDS) while its first pieces of W are already on their way, and keeps the normalised operand in
 // registers (K up to XP * 8 pieces).  With that prologue and the residual epilogue a block of a
-// decoder needs no kernel of its own for the residual sum or the norm.
+// decoder needs no kernel of its own for the residual sum or the norm.  The kernel for 17 to 64
+// rows brings x through LDS (see there).
 // float32 inputs are multiplied in true float32 (no reduced-precision MFMA).
 #include <type_traits>
 
@@ -206,7 +209,7 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
     }
 }
 
-template <typename T, typename TOUT, int MB, int NT, int EPI, bool TILED>
+template <typename T, typename TOUT, int MB, int NT, int EPI>
 __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                                  TOUT* __restrict__ y, int M, int N, int K, int I,
                                                                  RopeArgs rope) {
@@ -229,10 +232,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
             col0 = (wg / per_head) * rope.hd + (wg % per_head) * 16 + nt * (rope.hd / 2);
         }
         const int shift = (EPI == EPI_SWIGLU && (nt % 2)) ? I : 0;      // odd tiles of a pair come from the up rows
-        if (TILED)      // first byte of this lane in piece 0 of the tile; a tile past the matrix reads the last one and stores nothing
-            wrow[nt] = W + static_cast<size_t>(min((col0 + shift) / 16, (N + 15) / 16 - 1)) * ((K + CH - 1) / CH) * (WAVE * EL) + lane * EL;
-        else
-            wrow[nt] = W + static_cast<size_t>(min(col0 + r, n_limit - 1) + shift) * K;
+        wrow[nt] = W + static_cast<size_t>(min(col0 + r, n_limit - 1) + shift) * K;
     }
     const T* xrow[MB];
     bool xok[MB];
@@ -262,11 +262,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
             const bool kok = k < K;                  // K is a multiple of EL: a lane's 32 bytes are all in or all out
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                if (TILED) {
-                    if (piece < pieces) wa[u][nt].load(wrow[nt] + static_cast<size_t>(piece) * (WAVE * EL)); else wa[u][nt].zero();
-                } else {
-                    if (kok) wa[u][nt].load(wrow[nt] + k); else wa[u][nt].zero();
-                }
+                if (kok) wa[u][nt].load(wrow[nt] + k); else wa[u][nt].zero();
             }
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
@@ -627,7 +623,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_rows_kernel(const T* __rest
 }
 
 template <typename T, typename TOUT, int MB, int EPI>
-static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, bool tiled,
+static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT,
                      hipStream_t stream, RopeArgs rope = RopeArgs{}) {
     const int out_width = (EPI == EPI_SWIGLU) ? I : N;
     const int tiles = (out_width + 15) / 16;
@@ -635,10 +631,7 @@ static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K,
         constexpr int NTc = decltype(nt_tag)::value;
         constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
         const int grid = (tiles + NOUT - 1) / NOUT;
-        if (tiled)
-            skinny_gemm_kernel<T, TOUT, MB, NTc, EPI, true><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope);
-        else
-            skinny_gemm_kernel<T, TOUT, MB, NTc, EPI, false><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope);
+        skinny_gemm_kernel<T, TOUT, MB, NTc, EPI><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope);
     };
     // NT * MB fragments of partial sums share 64 KB of LDS: at most 8
     if constexpr (MB <= 2 && EPI != EPI_ROPE) {
@@ -731,9 +724,9 @@ static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K,
     if constexpr (EPI == EPI_RESIDUAL) {
         return -7;      // the residual epilogue exists for re-tiled matrices only
     } else {
-        if (M <= 16) return launch_nt<T, TOUT, 1, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
-        if (M <= 32) return launch_nt<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
-        return launch_nt<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, tiled, stream, rope);
+        if (M <= 16) return launch_nt<T, TOUT, 1, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
+        if (M <= 32) return launch_nt<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
+        return launch_nt<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
     }
 }
 
