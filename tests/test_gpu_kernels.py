@@ -544,6 +544,35 @@ def test_skinny_product_with_norm_prologue_and_residual_epilogue(K, dtype, M, N,
         K.skinny_gemm(normed, dev(w), torch.empty(M, N, device="cuda", dtype=DT[dtype]))       # needs the re-tiled matrix
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("M,N,Kd", [(17, 96, 2048), (33, 778, 528), (64, 2064, 192), (40, 50, 4096), (24, 64, 8192)])
+def test_skinny_product_of_17_to_64_rows_adds_into_the_residual_stream(K, dtype, M, N, Kd):
+    """The kernel for 17 to 64 rows (re-tiled matrix, x through LDS): the residual epilogue, rows
+    that are no multiple of 16, a tile past the matrix, a row width that is no multiple of a piece."""
+    g = torch.Generator().manual_seed(M * 31 + N + Kd)
+    w = (torch.randn(N, Kd, generator=g) / math.sqrt(Kd)).to(DT[dtype])
+    W = K.Weight(dev(w))
+    x = torch.randn(M, Kd, generator=g).to(DT[dtype])
+    stream = torch.randn(M + 3, N, generator=g)
+    buf = dev(stream.clone())
+    assert K.skinny_wins(M, Kd, DT[dtype], W) and K.residual_epilogue_ok(M, Kd, DT[dtype], W)
+    assert not K.skinny_wins(M, Kd, DT[dtype], dev(w)), "past 16 rows only a re-tiled matrix is streamed"
+    assert K.linear(dev(x), W, residual=buf[:M]) is None
+    assert rel(buf[:M], stream[:M].double() + x.double() @ w.double().t()) < 3e-6
+    assert torch.equal(buf[M:].cpu(), stream[M:]), "rows past the batch were written"
+    assert rel(K.linear(dev(x), W), x.double() @ w.double().t()) < KTOL[dtype]
+
+
+def test_where_the_skinny_product_gives_way_to_the_library(K):
+    W = K.Weight(dev(torch.zeros(32, 8192, dtype=torch.bfloat16)))
+    assert K.skinny_wins(16, 8192, torch.bfloat16, W) and K.skinny_wins(32, 8192, torch.bfloat16, W)
+    assert not K.skinny_wins(33, 8192, torch.bfloat16, W) and K.skinny_wins(64, 4096, torch.bfloat16, W)
+    assert not K.skinny_wins(65, 2048, torch.bfloat16, W) and not K.skinny_wins(8, 2040, torch.bfloat16, W)
+    assert not K.residual_epilogue_ok(40, 8192, torch.bfloat16, W)
+    with pytest.raises(K.KernelError):
+        K.linear(dev(torch.zeros(40, 8192, dtype=torch.bfloat16)), W, residual=dev(torch.zeros(40, 32)))
+
+
 def test_skinny_product_reference_vector(K):
     # test/test_cuda_kernel/test_matmul_kernel.cpp:30-99: ones x 0.5 with K = 128 gives 64
     out = K.skinny_gemm(torch.ones(3, 128, device="cuda"), torch.full((7, 128), 0.5, device="cuda"),
