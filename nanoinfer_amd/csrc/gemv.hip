@@ -108,12 +108,15 @@ struct RopeArgs {
 
 // What follows the main loop of both kernels: the wavefronts' partial sums meet in LDS and the
 // epilogue stores them.
-template <typename T, typename TOUT, int MB, int NT, int EPI, int WV = GV_WAVES, bool EXT = false>
+// HALVES == 2: two workgroups share the tiles that one would own; the first stores the first eight
+// columns of every tile, the second the others (each has multiplied only its own rows of W).
+template <typename T, typename TOUT, int MB, int NT, int EPI, int WV = GV_WAVES, bool EXT = false, int HALVES = 1>
 __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TOUT* __restrict__ y, int M, int N, int I,
                                               const RopeArgs& rope, float* ext = nullptr) {
     const int tid = threadIdx.x;
     const int wave = tid / WAVE, lane = tid % WAVE;
-    const int wg = blockIdx.x;
+    const int wg = blockIdx.x / HALVES;
+    const int wg_half = blockIdx.x % HALVES;      // which eight columns of every tile are this workgroup's
     // partial sums of the wavefronts meet in LDS: red[wave][tile][lane * 4 + i]; in memory of the
     // function's own, or (EXT) in memory the kernel has no other use for any more
     typedef float (*Red)[NT * MB][WAVE * 4];
@@ -141,7 +144,7 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
         for (int item = tid; item < MB * 16 * 16; item += WV * WAVE) {
             const int n_local = item % 16;
             const int m = item / 16;
-            if (m >= M) continue;
+            if (m >= M || (HALVES == 2 && (n_local >> 3) != wg_half)) continue;
             const int mb = m / 16, m_local = m % 16;
             const int src = ((n_local / 4) * 16 + m_local) * 4 + (n_local % 4);
             float x0 = 0.f, x1 = 0.f;
@@ -187,7 +190,7 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
         const int ot = n_in / 16, n_local = n_in % 16;
         const int mb = m / 16, m_local = m % 16;
         const int n = out_n0 + n_in;
-        if (m >= M || n >= out_width) continue;
+        if (m >= M || n >= out_width || (HALVES == 2 && (n_local >> 3) != wg_half)) continue;
         const int src = ((n_local / 4) * 16 + m_local) * 4 + (n_local % 4);
         float v;
         if (EPI == EPI_SWIGLU) {
@@ -290,7 +293,12 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
 // few lanes: read in that layout, h and the norm's weights take twice the load instructions of W
 // itself.  Staged, the workgroup reads every element once with full loads, normalises, rounds, and
 // leaves the rows in LDS, from where the lanes pick their operands.
-template <typename T, typename TOUT, int NT, int EPI, int XP, int WV, int SR>
+// HALVES == 2: a matrix of few tiles is streamed by twice the workgroups, each taking eight of a
+// tile's sixteen rows (the lanes of the other eight load the same rows again, which costs no
+// memory traffic, and their columns of the product are not stored).  A compute unit alone draws
+// about 37 GB/s from memory, so a launch of fewer workgroups than compute units cannot stream at
+// the chip's rate.
+template <typename T, typename TOUT, int NT, int EPI, int XP, int WV, int SR, int HALVES = 1>
 __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                                    TOUT* __restrict__ y, int M, int N, int K, int I,
                                                                    RopeArgs rope, NormArgs norm) {
@@ -299,7 +307,10 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;      // the same in every lane: say so
     const int r = lane % 16, kg = lane / 16;
-    const int wg = blockIdx.x;
+    const int wg = blockIdx.x / HALVES;
+    // the lane of the re-tiled matrix that this lane reads: its own, or with HALVES == 2 the one of this
+    // workgroup's half that has the same row modulo eight
+    const int wlane = HALVES == 1 ? lane : kg * 16 + ((r & 7) | (static_cast<int>(blockIdx.x % HALVES) << 3));
     const int pieces = (K + CH - 1) / CH;
 
     const T* wrow[NT];      // first byte of this lane in piece 0 of each tile
@@ -312,7 +323,7 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
         }
         const int shift = (EPI == EPI_SWIGLU && (nt % 2)) ? I : 0;
         const int limit = (N + 15) / 16 - 1;         // a workgroup's last tiles may lie past the matrix: read the last one, store nothing
-        wrow[nt] = W + static_cast<size_t>(min((col0 + shift) / 16, limit)) * pieces * (WAVE * EL) + lane * EL;
+        wrow[nt] = W + static_cast<size_t>(min((col0 + shift) / 16, limit)) * pieces * (WAVE * EL) + wlane * EL;
     }
 
     floatx4_t acc[NT][1];
@@ -507,7 +518,7 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
             multiply(c + STRIDE, wa_b, xb_b);
         }
     }
-    skinny_finish<T, TOUT, 1, NT, EPI, WV>(acc, y, M, N, I, rope);
+    skinny_finish<T, TOUT, 1, NT, EPI, WV, false, HALVES>(acc, y, M, N, I, rope);
 }
 
 // 17 to 64 rows with re-tiled W.  The operand layout spreads a row of x over few lanes, so loaded
@@ -646,6 +657,8 @@ static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K,
     return NI_LAUNCH_RESULT();
 }
 
+#define HALVE_BELOW 160       // workgroups: a launch of no more than this many is doubled by halving the tiles
+
 // The decode kernel: NT as launch_nt chooses it.  XP: pieces per wavefront of the normalising prologue, 0 without.
 template <typename T, typename TOUT, int EPI, int XP>
 static int launch_decode(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream,
@@ -656,25 +669,41 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
         constexpr int NTc = decltype(nt_tag)::value;
         constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
         const int grid = (tiles + NOUT - 1) / NOUT;
+        // The stacked [q; k; v] matrix with rotation gives a workgroup two tiles (the partners of a
+        // rotation), which leaves a small model few workgroups (96 at the 1B shape): then two
+        // workgroups share every pair of tiles.  (For one tile a workgroup, 128 workgroups against
+        // 256, the same was measured and gained nothing: not compiled.)
+        constexpr bool CAN_HALVE = EPI == EPI_ROPE;
+        const bool halve = CAN_HALVE && grid <= HALVE_BELOW;
+        auto launch = [&](auto wv_tag, auto sr_tag, auto halves_tag) {
+            constexpr int WVc = decltype(wv_tag)::value, SRc = decltype(sr_tag)::value, Hc = decltype(halves_tag)::value;
+            skinny_decode_kernel<T, TOUT, NTc, EPI, XP, WVc, SRc, Hc><<<grid * Hc, WVc * WAVE, 0, stream>>>(
+                (const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm);
+        };
+        using One = std::integral_constant<int, 1>;
+        using Two = std::integral_constant<int, 2>;
+        using Waves8 = std::integral_constant<int, GV_WAVES>;
+        auto with_halves = [&](auto wv_tag, auto sr_tag) {
+            if constexpr (CAN_HALVE) {
+                if (halve) { launch(wv_tag, sr_tag, Two{}); return; }
+            }
+            launch(wv_tag, sr_tag, One{});
+        };
         if constexpr (XP == 0 && NTc == 1) {
-            // fewer workgroups than compute units and rows of 4,096 elements or more: sixteen wavefronts each
-            if (grid <= 160 && K >= 4096) {
-                skinny_decode_kernel<T, TOUT, NTc, EPI, XP, 16, 0><<<grid, 16 * WAVE, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm);
+            // rows of 4,096 elements or more in few workgroups: sixteen wavefronts each
+            if (grid <= HALVE_BELOW && K >= 4096) {
+                with_halves(std::integral_constant<int, 16>{}, std::integral_constant<int, 0>{});
                 return;
             }
         }
         if constexpr (XP == 4 && NTc <= 2) {
             // up to eight rows: the prologue staged through LDS (its rows and the partial sums both fit),
             // compiled for 1, 4 and 8 rows
-#define NI_STAGED(SR_)                                                                                                   \
-    skinny_decode_kernel<T, TOUT, NTc, EPI, XP, GV_WAVES, SR_><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, \
-                                                                                                 (TOUT*)y, M, N, K, I, rope, norm)
-            if (M == 1) { NI_STAGED(1); return; }
-            if (M <= 4) { NI_STAGED(4); return; }
-            if (M <= 8) { NI_STAGED(8); return; }
-#undef NI_STAGED
+            if (M == 1) { with_halves(Waves8{}, std::integral_constant<int, 1>{}); return; }
+            if (M <= 4) { with_halves(Waves8{}, std::integral_constant<int, 4>{}); return; }
+            if (M <= 8) { with_halves(Waves8{}, std::integral_constant<int, 8>{}); return; }
         }
-        skinny_decode_kernel<T, TOUT, NTc, EPI, XP, GV_WAVES, 0><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm);
+        with_halves(Waves8{}, std::integral_constant<int, 0>{});
     };
     if constexpr (EPI != EPI_ROPE) {
         if (NT >= 4) { run(std::integral_constant<int, 4>{}); return NI_LAUNCH_RESULT(); }
