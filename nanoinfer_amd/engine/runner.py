@@ -125,9 +125,9 @@ class _RecordedStep:
     order: tuple = ()                    # requests of the last replay, in batch order
     pages_written: list = None           # per group, per sequence: table entries already in the staging buffer
     tiles: dict = None                   # tile size -> (offset in the tables, number of tiles), for recorded prompt portions
-    greedy: torch.Tensor = None          # int32, pinned host: argmax of every row of the logits, copied by the graph itself
-    amax: torch.Tensor = None            # the same on the device; a recorded decode step also leaves it in the place of
-                                         # its own token ids, where its next replay finds them without the host
+    greedy: torch.Tensor = None          # int32, pinned host: argmax of every row of the logits, copied after a replay
+    amax: torch.Tensor = None            # the same on the device, picked by the recording itself; a recorded decode step
+                                         # writes it over its own token ids, where its next replay finds them without the host
     replayed: "torch.cuda.Event" = None  # the last replay has finished (and with it the copy into ``greedy``)
 
 
@@ -401,14 +401,11 @@ class ModelRunner:
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx, self._layer_cache(ctx))
             if logits is not None:
-                # greedy decoding needs only this: the recording picks the largest logit of every row
-                # and brings the ids to the host itself, so that no launch stands between step and token
-                amax = K.argmax(logits)
-                greedy.copy_(amax, non_blocking=True)
-                if kind == "d":
-                    # and leaves them where its own token ids stand: replayed again for the same requests
-                    # it decodes on, whether or not the host has looked at the tokens yet
-                    meta[0:size].copy_(amax)
+                # greedy decoding needs only this: the recording picks the largest logit of every row, so
+                # that one copy brings the ids to the host.  A decode step writes them where its own token
+                # ids stand: replayed again for the same requests it decodes on, whether or not the host
+                # has looked at the tokens yet.
+                amax = K.argmax(logits, out=meta[0:size]) if kind == "d" else K.argmax(logits)
         if ctx.tile_sizes_asked - set(tiles):
             self._unrecordable.add(key)       # the recorded run asked for tiles the eager run did not: not the same step
             return None
@@ -536,13 +533,14 @@ class ModelRunner:
             self._history[history_row, 0:B].copy_(rec.amax[0:B], non_blocking=True)
             self._replayed_logits = None
             return True
-        rec.replayed.record()
         if rec.logits is None:
             self._replayed_logits = None
         else:
+            rec.greedy.copy_(rec.amax, non_blocking=True)
             out = rec.logits.clone()      # the graph's own buffer is overwritten by its next replay
             self._greedy_of = (out, rec)
             self._replayed_logits = out
+        rec.replayed.record()
         return True
 
     def _book(self, entries: List[StepEntry], totals: Sequence[int]) -> None:
