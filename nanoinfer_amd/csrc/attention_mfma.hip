@@ -730,9 +730,9 @@ NI_EXPORT int ni_mfma_attention(const void* q, int q_stride, const void* kpool, 
             units[pow2] = cus;                                                                                      \
             slots[pow2] = cus * per_cu;                                                                             \
         }                                                                                                           \
-        /* an even number of rounds pairs long tiles with short ones; with few tiles every one gets a workgroup */  \
+        /* an even number of rounds pairs long tiles with short ones; with few tiles every one gets a workgroup  */  \
         int rounds = 1;                                                                                             \
-        if (n_tiles * per_tile >= 2 * units[pow2]) {                                                                \
+        if (n_tiles * per_tile >= 4 * units[pow2]) {                                                                \
             rounds = 2;                                                                                             \
             while ((n_tiles + rounds - 1) / rounds * per_tile > slots[pow2] && rounds < n_tiles) rounds += 2;       \
         }                                                                                                           \

@@ -216,11 +216,12 @@ class Attention(Part):
         if ctx.max_q_len >= self.MFMA_MIN_PORTION and K.mfma_attention_ok(x.dtype, self.hd):
             # prompt portions: tiles of tokens on the matrix cores (a recorded step has them only if
             # it was recorded with them)
-            tile_tokens = K.mfma_tile_tokens(self.hd, self.H // self.KVH, T, self.KVH)
+            max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window + ctx.max_q_len)
+            tile_tokens, nsplit = K.mfma_plan(self.hd, self.H // self.KVH, self.KVH, T, ctx.max_q_len, max_keys)
             tiles = ctx.q_tiles(tile_tokens)
         if tiles is not None:
-            max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window + ctx.max_q_len)
-            nsplit = K.mfma_splits(tiles.shape[0], self.KVH, self.H // self.KVH, max_keys)
+            if nsplit is None:
+                nsplit = K.mfma_splits(tiles.shape[0], self.KVH, self.H // self.KVH, max_keys)
             ws = ctx.workspace(T * self.H * nsplit * (self.hd + 2)) if nsplit > 1 else None
             K.mfma_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, out, self.H, self.KVH, self.hd,
                              self.scale, self.window, nsplit, ws, tile_tokens)

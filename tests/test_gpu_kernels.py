@@ -311,6 +311,14 @@ def test_mfma_tile_size_and_splits_follow_the_step(K):
     assert K.mfma_splits(8, 8, 4, 2048) == 4
     assert K.mfma_splits(8, 8, 4, 300) == 1
     assert K.mfma_splits(1, 1, 1, 10 ** 6) == 16
+    # one portion alone far into its sequence: two blocks and runs of 512 keys or more, if that fills the chip
+    assert K.mfma_plan(64, 4, 8, 512, 512, 2048) == (32, 4) == K.mfma_plan(64, 4, 8, 512, 512, 1100)
+    assert K.mfma_plan(64, 4, 8, 512, 512, 1024) == (16, None)        # the keys before it may be as few as its own
+    assert K.mfma_plan(64, 4, 8, 512, 512, 5000) == (32, 4)
+    assert K.mfma_plan(64, 4, 8, 2048, 2048, 2048) == (16, None)      # a whole prompt: short and long tiles, paired
+    assert K.mfma_plan(64, 4, 8, 4096, 4096, 4096) == (32, None)
+    assert K.mfma_plan(64, 4, 8, 512, 300, 2048) == (16, None)        # several portions in the step
+    assert K.mfma_plan(128, 4, 8, 512, 512, 2048) == (16, None)       # head size 128 has one block only
 
 
 @pytest.mark.parametrize("H,KVH,hd,ps", [(4, 2, 32, 8), (6, 1, 32, 8), (32, 8, 64, 16), (16, 2, 128, 16), (2, 2, 256, 16),
