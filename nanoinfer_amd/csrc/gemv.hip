@@ -805,13 +805,16 @@ NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N
     return launch_mb<bf16_t, bf16_t, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
 }
 
-// Whether the normalising prologue takes M rows of K elements of this type (1) or not (0).
+// Whether the normalising prologue takes M rows of K elements of this type (1) or not (0).  Every
+// workgroup reads all M rows of h: past eight rows that is more than the matrix it streams, and the
+// norm as a kernel of its own is faster (measured at the 1B shape: 6 % of a decode step at 9 to 16 rows).
+#define PROLOGUE_MAX_ROWS 8
 NI_EXPORT int ni_skinny_prologue_ok(int M, int K, int dtype) {
-    if (M < 1 || M > 16 || K % (dtype == 0 ? 8 : 16) != 0) return 0;
+    if (M < 1 || M > PROLOGUE_MAX_ROWS || K % (dtype == 0 ? 8 : 16) != 0) return 0;
     return (dtype == 0 ? prologue_pieces<float>(K) : prologue_pieces<bf16_t>(K)) != 0;
 }
 
-// The same product on RMSNorm(h) instead of a given x: h float32 [M <= 16, K], norm_weight float32 [K],
+// The same product on RMSNorm(h) instead of a given x: h float32 [M <= 8, K], norm_weight float32 [K],
 // W re-tiled.  epilogue 0 (store in the compute type) or 2 (SwiGLU).
 NI_EXPORT int ni_skinny_gemm_normed(const void* h, const void* norm_weight, float eps, const void* W, void* y, int M, int N,
                                     int K, int epilogue, int tiles_per_group, int dtype, hipStream_t stream) {
@@ -832,7 +835,7 @@ NI_EXPORT int ni_skinny_gemm_normed(const void* h, const void* norm_weight, floa
 // Product with the stacked [q; k; v] matrix ((H + 2 KVH) * hd rows), rotation of query and key
 // heads by the rows' positions, queries to q_out [M, H * hd], keys and values into the pools at
 // slot_mapping (null: not stored).  hd must be a multiple of 32 and fully rotated.
-// With x null the product is taken on RMSNorm(h): h float32 [M <= 16, K], norm_weight [K], W re-tiled.
+// With x null the product is taken on RMSNorm(h): h float32 [M <= 8, K], norm_weight [K], W re-tiled.
 NI_EXPORT int ni_skinny_qkv_rope(const void* x, const void* h, const void* norm_weight, float eps, const void* W,
                                  void* q_out, const void* positions, const void* cos_t, const void* sin_t,
                                  const void* slot_mapping, void* kpool, void* vpool, int M, int K, int H, int KVH, int hd,

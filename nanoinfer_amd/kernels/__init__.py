@@ -575,8 +575,9 @@ def _prologue_sizes_ok(M: int, K: int, code: int) -> bool:
 
 
 def norm_prologue_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
-    """Whether the skinny product can take RMSNorm(h) for its input: at most 16 rows, a re-tiled
-    matrix, rows short enough for the normalised operand to stay in registers."""
+    """Whether the skinny product can take RMSNorm(h) for its input: at most eight rows (every
+    workgroup normalises all of them: beyond that the norm as a kernel of its own is faster), a
+    re-tiled matrix, rows short enough for the normalised operand to stay in registers."""
     return (isinstance(weight, Weight) and weight.tiles is not None and dtype in _DTYPE_CODE
             and _prologue_sizes_ok(int(M), int(K), dtype_code(dtype)))
 
