@@ -264,11 +264,20 @@ def token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
 
 
 def mfma_token_splits(n_tokens: int, kv_heads: int, group: int, max_keys: int) -> int:
-    """Into how many runs the matrix-core kernel for single tokens cuts every key range: enough
-    for about one workgroup per compute unit, a run never shorter than 256 keys (measured at
-    batches 1 to 64 and contexts of 2,100 and 8,200 keys)."""
+    """Into how many runs the matrix-core kernel for single tokens cuts every key range.  Up to a
+    workgroup per compute unit: enough runs to give every unit one, none shorter than 256 keys
+    (measured at batches 1 to 64 and contexts of 2,100 and 8,200 keys).  Beyond that the units
+    that get one workgroup more than the others set the time, each drawing the same ~37 GB/s
+    whatever runs on it: 264 workgroups take 42 us where 256 take 26.  Two runs each even that out
+    a little where they leave the fullest unit three halves instead of two wholes (37 us there;
+    more runs lose to their own start-up and to the kernel that merges them)."""
+    units = COMPUTE_UNITS
     items = max(1, n_tokens * kv_heads * ((group + 15) // 16))
-    return int(max(1, min(256 // items, max_keys // 256, 64)))
+    if items <= units:
+        return int(max(1, min(units // items, max_keys // 256, 64)))
+    whole = -(-items // units)                       # workgroups on the fullest unit, uncut
+    halves = -(-2 * items // units)                  # and with two runs each
+    return 2 if max_keys >= 512 and halves / 2 + 0.2 < whole else 1
 
 
 def mfma_token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,

@@ -311,6 +311,9 @@ def test_mfma_tile_size_and_splits_follow_the_step(K):
     assert K.mfma_splits(8, 8, 4, 2048) == 4
     assert K.mfma_splits(8, 8, 4, 300) == 1
     assert K.mfma_splits(1, 1, 1, 10 ** 6) == 16
+    # single tokens: a workgroup for every compute unit, then two runs where that evens out the units' load
+    assert [K.mfma_token_splits(b, 8, 4, 2170) for b in (1, 8, 16, 32, 33, 48, 56, 64)] == [8, 4, 2, 1, 2, 2, 1, 1]
+    assert K.mfma_token_splits(40, 8, 4, 300) == 1 and K.mfma_token_splits(1, 8, 4, 100000) == 32
     # one portion alone far into its sequence: two blocks and runs of 512 keys or more, if that fills the chip
     assert K.mfma_plan(64, 4, 8, 512, 512, 2048) == (32, 4) == K.mfma_plan(64, 4, 8, 512, 512, 1100)
     assert K.mfma_plan(64, 4, 8, 512, 512, 1024) == (16, None)        # the keys before it may be as few as its own
