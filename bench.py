@@ -87,6 +87,7 @@ def config_record(cfg: dict, layers: int, batch: int, mean_ctx: float, prefill_c
 
 
 def main() -> int:
+    global PROMPT_LEN, CONTEXT_LEN
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
@@ -97,10 +98,17 @@ def main() -> int:
     ap.add_argument("--prefill-chunk", type=int, default=PREFILL_CHUNK, help="tokens of a prompt portion in the prefill measurement")
     ap.add_argument("--decode-run", type=int, default=DECODE_RUN,
                     help="decode steps on one scheduling decision (the engine's max_decode_run; 1: the host reads every token before the next step)")
+    ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
+                    help="tokens of every prompt (the measured prefill, and the context that decoding starts from); "
+                         "the pool holds 2,048 more for every request")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
                     help="run one phase only (for profiling; prints no result line)")
     args = ap.parse_args()
+    if args.prompt_len < 1 or args.prompt_len + 2048 > LLAMA_1B["max_position_embeddings"]:
+        print(f"--prompt-len must lie between 1 and {LLAMA_1B['max_position_embeddings'] - 2048}")
+        return 2
+    PROMPT_LEN, CONTEXT_LEN = args.prompt_len, args.prompt_len + 2048
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
         return 2
@@ -204,7 +212,7 @@ def main() -> int:
     achieved = decode_bytes(cfg, args.batch, mean_ctx, elem) / step_s
     flops = prefill_flops(cfg, PROMPT_LEN)
     result = {
-        "metric": "decode tok/s at batch 8 (Llama 3.2 1B shape, context 4096)",
+        "metric": f"decode tok/s at batch {args.batch} (Llama 3.2 1B shape, context {CONTEXT_LEN})",
         "value": round(args.batch / step_s, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
