@@ -93,7 +93,16 @@ struct NormArgs {
     const float* h;        // [M, K] residual stream
     const float* weight;   // [K]
     float eps;
+    // for the merging prologue instead: partial results of an attention whose keys were cut into runs
+    const float* part_o = nullptr;     // [M, heads, runs, hd]
+    const float* part_ml = nullptr;    // [M, heads, runs, 2]: maximum (base e) and sum of each run
+    int runs = 0, heads = 0, hd = 0;
 };
+#define PRO_NORM 0      // the prologue computes RMSNorm(h)
+#define PRO_MERGE 1     // the prologue merges the key runs of an attention
+#define MERGE_RUNS_MAX 16         // key runs the merging prologue takes for one row
+#define MERGE_RUNS_OF(SR) ((SR) == 1 ? MERGE_RUNS_MAX : 32 / (SR))      // and for up to SR rows: 8 for 4, 4 for 8
+#define MERGE_FACTORS_MAX 4096     // floats of LDS for the runs' weights: M * heads * (runs + 1) must fit
 
 // What the rotation epilogue needs beside the product.
 struct RopeArgs {
@@ -298,7 +307,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
 // memory traffic, and their columns of the product are not stored).  A compute unit alone draws
 // about 37 GB/s from memory, so a launch of fewer workgroups than compute units cannot stream at
 // the chip's rate.
-template <typename T, typename TOUT, int NT, int EPI, int XP, int WV, int SR, int HALVES = 1>
+template <typename T, typename TOUT, int NT, int EPI, int XP, int WV, int SR, int HALVES = 1, int PRO = PRO_NORM>
 __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                                    TOUT* __restrict__ y, int M, int N, int K, int I,
                                                                    RopeArgs rope, NormArgs norm) {
@@ -371,6 +380,78 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
             constexpr int QPT = (KMAX / 4 + THREADS - 1) / THREADS;      // groups of four columns per thread
             constexpr int XROW = KMAX + 16 / sizeof(T);        // 16 bytes of padding: rows start on different banks
             __shared__ __attribute__((aligned(16))) T xs[SR][XROW];
+            if constexpr (PRO == PRO_MERGE) {
+                // x is the output of an attention whose keys were cut into runs: row m, head h is
+                // sum_s o[m,h,s,:] * w_s / sum_s l[m,h,s] * w_s with w_s = exp(max[m,h,s] - max over s), as the
+                // merge kernel computes it.  The (maximum, sum) pairs are asked for first and the first trip
+                // of W right behind them; the weights of the runs meet in LDS, then every thread merges four
+                // columns of every row.
+                __shared__ float fs[MERGE_FACTORS_MAX];
+                constexpr bool FAST = sizeof(T) == 2;
+                constexpr int RC = MERGE_RUNS_OF(SR);      // runs whose pieces a thread can hold for all SR rows
+                static_assert(QPT == 1, "a thread merges one group of four columns");
+                const int runs = norm.runs, stride = runs + 1;
+                const int items = M * norm.heads;
+                constexpr int IPT = (SR * 128 + THREADS - 1) / THREADS;       // (row, head) items a thread may own
+                // everything the prologue reads is asked for before W, so that it is there while W is on its way
+                float2 ml[IPT][RC];
+#pragma unroll
+                for (int i = 0; i < IPT; ++i) {
+                    const int item = tid + i * THREADS;
+#pragma unroll
+                    for (int sp = 0; sp < RC; ++sp)
+                        ml[i][sp] = (item < items && sp < runs)
+                                        ? *reinterpret_cast<const float2*>(norm.part_ml + (static_cast<size_t>(item) * runs + sp) * 2)
+                                        : make_float2(-1.0e30f, 0.f);
+                }
+                const int k = 4 * tid;
+                const int head = min(k, K - 4) / norm.hd, dim = min(k, K - 4) % norm.hd;
+                float4 v[SR][RC];
+#pragma unroll
+                for (int m = 0; m < SR; ++m)
+#pragma unroll
+                    for (int sp = 0; sp < RC; ++sp) {
+                        const size_t at = (static_cast<size_t>(m * norm.heads + head) * runs + sp) * norm.hd + dim;
+                        v[m][sp] = (k < K && m < M && sp < runs) ? *reinterpret_cast<const float4*>(norm.part_o + at)
+                                                                 : make_float4(0.f, 0.f, 0.f, 0.f);
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+                load_w(wave, wa_a);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < IPT; ++i) {
+                    const int item = tid + i * THREADS;
+                    float run_max = -1.0e30f;
+#pragma unroll
+                    for (int sp = 0; sp < RC; ++sp) run_max = fmaxf(run_max, ml[i][sp].x);
+                    float total = 0.f;
+#pragma unroll
+                    for (int sp = 0; sp < RC; ++sp) {
+                        const float f = FAST ? __expf(ml[i][sp].x - run_max) : expf(ml[i][sp].x - run_max);
+                        total += ml[i][sp].y * f;             // runs that do not exist have sum 0
+                        if (item < items && sp < runs) fs[item * stride + sp] = f;
+                    }
+                    if (item < items) fs[item * stride + runs] = total;
+                }
+                __syncthreads();
+                if (k < K) {
+#pragma unroll
+                    for (int m = 0; m < SR; ++m) {
+                        if (m < M) {
+                            const float* w = fs + (m * norm.heads + head) * stride;
+                            float o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                            for (int sp = 0; sp < RC; ++sp) {
+                                const float f = sp < runs ? w[sp] : 0.f;
+                                o[0] += v[m][sp].x * f; o[1] += v[m][sp].y * f; o[2] += v[m][sp].z * f; o[3] += v[m][sp].w * f;
+                            }
+                            const float total = w[runs];
+                            const float f4[4] = {o[0] / total, o[1] / total, o[2] / total, o[3] / total};
+                            VecIO<T, 4>::store(&xs[m][k], f4);
+                        }
+                    }
+                }
+            } else {
             __shared__ float ssum[WV][SR];
             __shared__ float sinv[SR];
             float4 hv[SR][QPT], wv[QPT];
@@ -428,6 +509,7 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
                         VecIO<T, 4>::store(&xs[m][k], f);
                     }
                 }
+            }
             }
             __syncthreads();
 #pragma unroll
@@ -830,6 +912,45 @@ NI_EXPORT int ni_skinny_gemm_normed(const void* h, const void* norm_weight, floa
     }
     if (epilogue == 2) return launch_normed<bf16_t, EPI_SWIGLU>(norm, W, y, M, N, K, I, tiles_per_group, stream);
     return launch_normed<bf16_t, EPI_STORE>(norm, W, y, M, N, K, I, tiles_per_group, stream);
+}
+
+// The product on the output of an attention whose keys were cut into runs, merged in the prologue
+// instead of by a kernel of its own (same numbers): part_o float32 [M, heads, runs, hd], part_ml
+// float32 [M, heads, runs, 2] (maximum in base e, sum).  bfloat16, W re-tiled [N, heads * hd],
+// epilogue 0 (store in the compute type) or 3 (add into the float32 residual stream).
+NI_EXPORT int ni_skinny_merge_ok(int M, int heads, int hd, int runs, int dtype) {
+    if (dtype != 1 || M < 1 || M > PROLOGUE_MAX_ROWS || heads < 1 || heads > 128 || hd < 4 || hd % 4 != 0) return 0;
+    const int staged = M == 1 ? 1 : M <= 4 ? 4 : 8;       // the rows the prologue is compiled for
+    if (runs < 2 || runs > MERGE_RUNS_OF(staged) || M * heads * (runs + 1) > MERGE_FACTORS_MAX) return 0;
+    const long K = static_cast<long>(heads) * hd;
+    return K % 16 == 0 && K <= 65536 && prologue_pieces<bf16_t>(static_cast<int>(K)) == 4;
+}
+
+template <typename TOUT, int EPI>
+static int launch_merged(const NormArgs& merge, const void* W, void* y, int M, int N, int K, hipStream_t stream) {
+    const int tiles = (N + 15) / 16;
+    auto go = [&](auto sr_tag) {
+        constexpr int SRc = decltype(sr_tag)::value;
+        skinny_decode_kernel<bf16_t, TOUT, 1, EPI, 4, GV_WAVES, SRc, 1, PRO_MERGE><<<tiles, GV_THREADS, 0, stream>>>(
+            nullptr, (const bf16_t*)W, (TOUT*)y, M, N, K, 0, RopeArgs{}, merge);
+    };
+    if (M == 1) go(std::integral_constant<int, 1>{});
+    else if (M <= 4) go(std::integral_constant<int, 4>{});
+    else go(std::integral_constant<int, 8>{});
+    return NI_LAUNCH_RESULT();
+}
+
+NI_EXPORT int ni_skinny_gemm_merged(const void* part_o, const void* part_ml, int runs, int heads, int hd, const void* W,
+                                    void* y, int M, int N, int epilogue, int dtype, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (!part_o || !part_ml || !ni_skinny_merge_ok(M, heads, hd, runs, dtype)) return -5;
+    if (epilogue != 0 && epilogue != 3) return -6;
+    NormArgs merge{nullptr, nullptr, 0.f};
+    merge.part_o = (const float*)part_o;
+    merge.part_ml = (const float*)part_ml;
+    merge.runs = runs; merge.heads = heads; merge.hd = hd;
+    if (epilogue == 3) return launch_merged<float, EPI_RESIDUAL>(merge, W, y, M, N, heads * hd, stream);
+    return launch_merged<bf16_t, EPI_STORE>(merge, W, y, M, N, heads * hd, stream);
 }
 
 // Product with the stacked [q; k; v] matrix ((H + 2 KVH) * hd rows), rotation of query and key

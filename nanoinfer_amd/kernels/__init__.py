@@ -283,10 +283,11 @@ def mfma_token_splits(n_tokens: int, kv_heads: int, group: int, max_keys: int) -
 def mfma_token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                          seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, H: int, KVH: int,
                          hd: int, scale: float, window: Optional[int], nsplit: int,
-                         workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                         workspace: Optional[torch.Tensor] = None, merge: bool = True) -> torch.Tensor:
     """:func:`token_attention` on the matrix cores (bfloat16, head sizes that :func:`mfma_attention_ok`
     takes): the query heads of a kv head are the rows of the products, the wavefronts of a
-    workgroup share out the keys."""
+    workgroup share out the keys.  With ``nsplit > 1`` and ``merge=False`` the partial results of
+    the key runs are left in ``workspace`` for :func:`skinny_gemm_merged` and ``out`` is not written."""
     if not (mfma_attention_ok(qkv.dtype, hd)):
         raise KernelError(f"mfma_token_attention does not take {qkv.dtype} with head size {hd}")
     if not (qkv.shape[1] % 8 == 0):
@@ -299,7 +300,7 @@ def mfma_token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Te
         _ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table), block_table.shape[1],
         _ptr(seq_of_token), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), T, H, KVH, kpool.shape[2],
         int(window) if window else 0, ctypes.c_float(scale), nsplit, _stream()), "mfma_token_attention")
-    if nsplit > 1:
+    if nsplit > 1 and merge:
         _check(attention_lib(hd).ni_merge_splits(_ptr(part_o), _ptr(part_ml), _ptr(out), T, H, nsplit,
                                                  dtype_code(out.dtype), _stream()), "merge_splits")
     return out
@@ -498,6 +499,7 @@ def skinny_wins(M: int, K: int, dtype: torch.dtype, weight=None) -> bool:
         return False
     return M <= 32 or K <= 4096
 FUSE_NORMS = True           # residual sums and norms ride on the skinny products of a decode step where they can
+MERGE_IN_PRODUCT = True     # the key runs of a decode step's attention are merged by the output product where it can
 
 
 def tile_weight(w: torch.Tensor) -> torch.Tensor:
@@ -650,6 +652,52 @@ def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bo
     _gpu(x, "x")
     _check(skinny_lib().ni_skinny_gemm(_ptr(x), _ptr(rows if tiles is None else tiles), _ptr(out), M, N, Kd, epi,
                                        per_group, 0 if tiles is None else 1, dtype_code(dtype), _stream()), "skinny_gemm")
+    return out
+
+
+def skinny_merge_ok(M: int, H: int, hd: int, nsplit: int, dtype: torch.dtype, weight) -> bool:
+    """Whether the product of an attention's output with ``weight`` can merge the attention's
+    ``nsplit`` key runs in its prologue: bfloat16, a re-tiled matrix, few rows, and heads and runs
+    whose weights fit the workgroup's LDS."""
+    if not (isinstance(weight, Weight) and weight.tiles is not None and dtype == torch.bfloat16):
+        return False
+    return bool(skinny_lib().ni_skinny_merge_ok(int(M), int(H), int(hd), int(nsplit), dtype_code(dtype)))
+
+
+def skinny_merge_wins(M: int, H: int, hd: int, nsplit: int, dtype: torch.dtype, weight) -> bool:
+    """Whether merging in the product's prologue is also the faster way.  Every workgroup of the
+    product reads all partial results of all rows, 4 * nsplit times the bytes of the merged rows,
+    through its compute unit's one path of 64 bytes a cycle: that beats the merge kernel's launch
+    for one or two rows (measured at the 1B shape: a decode step at batch 1 0.819 -> 0.792 ms, at
+    batch 2 the same, at batch 4 0.894 -> 0.910, at batch 8 1.003 -> 1.051)."""
+    return M * nsplit <= 16 and skinny_merge_ok(M, H, hd, nsplit, dtype, weight)
+
+
+def skinny_gemm_merged(workspace: torch.Tensor, nsplit: int, M: int, H: int, hd: int, weight, out: torch.Tensor,
+                       residual: bool = False) -> torch.Tensor:
+    """``attn . weight^T`` where ``attn`` [M, H*hd] is still in the pieces that an attention kernel
+    left in ``workspace`` for ``nsplit`` key runs (float32: outputs [M, H, nsplit, hd], then
+    (maximum, sum) pairs [M, H, nsplit, 2]): the runs are merged in the product's prologue, with the
+    numbers the merge kernel gives.  ``out`` as for :func:`skinny_gemm`, with ``residual`` the
+    float32 residual stream."""
+    rows, tiles = _rows_and_tiles(weight)
+    N = rows.shape[0]
+    dtype = rows.dtype
+    if not skinny_merge_ok(M, H, hd, nsplit, dtype, weight):
+        raise KernelError(f"the merging prologue does not take M={M}, {H} heads of {hd}, {nsplit} runs in {dtype}")
+    _gpu(rows, "weight", dtype, (N, H * hd))
+    need = M * H * nsplit * (hd + 2)
+    _gpu(workspace, "workspace", torch.float32)
+    if not (workspace.numel() >= need):
+        raise KernelError(f"attention workspace of {need} floats needed for {nsplit} splits")
+    flat = workspace.view(-1)
+    part_o, part_ml = flat[: M * H * nsplit * hd], flat[M * H * nsplit * hd: need]
+    if residual:
+        _gpu(out, "out", torch.float32, (M, N))
+    else:
+        _gpu(out, "out", dtype, (M, N))
+    _check(skinny_lib().ni_skinny_gemm_merged(_ptr(part_o), _ptr(part_ml), nsplit, H, hd, _ptr(tiles), _ptr(out), M, N,
+                                              3 if residual else 0, dtype_code(dtype), _stream()), "skinny_gemm_merged")
     return out
 
 

@@ -232,6 +232,15 @@ class Attention(Part):
         choose = K.mfma_token_splits if on_matrix_cores else K.choose_splits
         nsplit = choose(T, self.KVH, self.H // self.KVH, max_keys)
         ws = ctx.workspace(T * self.H * nsplit * (self.hd + 2)) if nsplit > 1 else None
+        if on_matrix_cores and nsplit > 1 and K.MERGE_IN_PRODUCT and K.skinny_merge_wins(T, self.H, self.hd, nsplit, x.dtype, self.w_o):
+            # one or two rows: the output product merges the key runs in its prologue, no kernel of its own does
+            K.mfma_token_attention(qkv, cache.kpool, cache.vpool, cache.block_table, ctx.seq_of_token, ctx.positions,
+                                   out, self.H, self.KVH, self.hd, self.scale, self.window, nsplit, ws, merge=False)
+            if residual is not None:
+                K.skinny_gemm_merged(ws, nsplit, T, self.H, self.hd, self.w_o, residual, residual=True)
+                return None
+            y = torch.empty(T, self.w_o.rows.shape[0], dtype=x.dtype, device=x.device)
+            return K.skinny_gemm_merged(ws, nsplit, T, self.H, self.hd, self.w_o, y)
         attend = K.mfma_token_attention if on_matrix_cores else K.token_attention
         attend(qkv, cache.kpool, cache.vpool, cache.block_table, ctx.seq_of_token, ctx.positions, out,
                self.H, self.KVH, self.hd, self.scale, self.window, nsplit, ws)

@@ -574,6 +574,58 @@ def test_skinny_product_of_17_to_64_rows_adds_into_the_residual_stream(K, dtype,
     assert rel(K.linear(dev(x), W), x.double() @ w.double().t()) < KTOL[dtype]
 
 
+@pytest.mark.parametrize("M,H,hd,N,runs", [(1, 32, 64, 2048, 8), (8, 32, 64, 2048, 4), (3, 8, 128, 528, 8), (5, 24, 32, 96, 2),
+                                           (4, 6, 80, 272, 3), (8, 16, 128, 64, 4), (2, 1, 16, 48, 5), (1, 12, 96, 40, 16)])
+@pytest.mark.parametrize("residual", [False, True])
+def test_skinny_product_merges_the_key_runs_of_an_attention(K, M, H, hd, N, runs, residual):
+    # The attention's partial results go straight into the output product.  One run of one head
+    # dominates by e^12 and one is empty (maximum "minus infinity", sum 0), so that a wrong weight or
+    # a mixed-up index of (row, head, run) shows.
+    g = torch.Generator().manual_seed(M * 1000 + H * 10 + runs)
+    part_o = torch.randn(M, H, runs, hd, generator=g) * 5
+    part_m = torch.randn(M, H, runs, generator=g) * 3
+    part_l = torch.rand(M, H, runs, generator=g) * 50 + 1
+    part_m[M - 1, H // 2, runs - 1] += 12.0
+    part_m[0, 0, 0], part_l[0, 0, 0], part_o[0, 0, 0] = -1.0e30 * math.log(2.0), 0.0, 0.0
+    w = torch.randn(N, H * hd, generator=g) / math.sqrt(H * hd)
+    wt = K.Weight(dev(w, torch.bfloat16))
+    assert K.skinny_merge_ok(M, H, hd, runs, torch.bfloat16, wt)
+    ws = dev(torch.cat([part_o.reshape(-1), torch.stack([part_m, part_l], -1).reshape(-1)]))
+    f = torch.exp(part_m.double() - part_m.double().amax(-1, keepdim=True))
+    attn = ((part_o.double() * f[..., None]).sum(2) / (part_l.double() * f).sum(-1, keepdim=True)).reshape(M, H * hd)
+    want = attn.to(torch.bfloat16).double() @ w.to(torch.bfloat16).double().t()
+    if residual:
+        h0 = torch.randn(M, N, generator=g)
+        out = dev(h0.clone())
+        K.skinny_gemm_merged(ws, runs, M, H, hd, wt, out, residual=True)
+        got = out.cpu().double() - h0.double()
+    else:
+        out = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+        got = K.skinny_gemm_merged(ws, runs, M, H, hd, wt, out).cpu().double()
+    assert rel(got, want) < KTOL["bfloat16"], (M, H, hd, N, runs)
+
+
+def test_what_the_merging_prologue_refuses(K):
+    wt = K.Weight(dev(torch.zeros(64, 2048), torch.bfloat16))
+    assert K.skinny_merge_ok(8, 32, 64, 4, torch.bfloat16, wt)
+    assert not K.skinny_merge_ok(9, 32, 64, 4, torch.bfloat16, wt)          # more rows than the prologue stages
+    assert not K.skinny_merge_ok(8, 32, 64, 1, torch.bfloat16, wt)          # nothing to merge
+    assert not K.skinny_merge_ok(8, 32, 64, 17, torch.bfloat16, wt)         # more runs than it holds
+    assert K.skinny_merge_ok(1, 32, 64, 16, torch.bfloat16, wt) and K.skinny_merge_ok(4, 32, 64, 8, torch.bfloat16, wt)
+    assert not K.skinny_merge_ok(8, 32, 64, 5, torch.bfloat16, wt)          # eight rows: four runs fit a thread's registers
+    assert not K.skinny_merge_ok(3, 32, 64, 9, torch.bfloat16, wt)          # four rows: eight runs
+    assert not K.skinny_merge_ok(8, 48, 64, 4, torch.bfloat16, wt)          # rows of 3,072 elements: past the compiled size
+    assert not K.skinny_merge_ok(8, 32, 64, 4, torch.float32, wt)
+    # and where it is taken: one or two rows, beyond that the merge kernel is the faster way
+    assert K.skinny_merge_wins(1, 32, 64, 8, torch.bfloat16, wt) and K.skinny_merge_wins(2, 32, 64, 8, torch.bfloat16, wt)
+    assert not K.skinny_merge_wins(8, 32, 64, 4, torch.bfloat16, wt) and not K.skinny_merge_wins(3, 32, 64, 8, torch.bfloat16, wt)
+    assert not K.skinny_merge_ok(8, 32, 64, 4, torch.bfloat16, K.Weight(dev(torch.zeros(64, 2048), torch.bfloat16), tiled=False))
+    with pytest.raises(K.KernelError, match="merging prologue"):
+        K.skinny_gemm_merged(torch.zeros(1 << 20, device="cuda"), 17, 8, 32, 64, wt, torch.empty(8, 64, device="cuda", dtype=torch.bfloat16))
+    with pytest.raises(K.KernelError, match="workspace"):
+        K.skinny_gemm_merged(torch.zeros(100, device="cuda"), 4, 8, 32, 64, wt, torch.empty(8, 64, device="cuda", dtype=torch.bfloat16))
+
+
 def test_where_the_skinny_product_gives_way_to_the_library(K):
     W = K.Weight(dev(torch.zeros(32, 8192, dtype=torch.bfloat16)))
     assert K.skinny_wins(16, 8192, torch.bfloat16, W) and K.skinny_wins(32, 8192, torch.bfloat16, W)

@@ -204,7 +204,7 @@ def test_pages_whose_size_is_no_power_of_two(name, page, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_long_decoding(dtype):
+def test_long_decoding(dtype, monkeypatch):
     """A short prompt, then some four hundred tokens one at a time: positions far beyond the prompt,
     many page boundaries, the split key range of the decode path."""
     name = "B"
@@ -213,8 +213,13 @@ def test_long_decoding(dtype):
     steps = [([("long", list(toks[:3]), [0, 1, 2])], [])]
     steps += [([("long", [t], [0])], []) for t in toks[3:]]
     steps[-1] = (steps[-1][0], ["long"])
+    from nanoinfer_amd import kernels as K
+    merged, original = [], K.skinny_gemm_merged
+    monkeypatch.setattr(K, "skinny_gemm_merged", lambda *a, **kw: (merged.append(a[1]), original(*a, **kw))[1])
     got, _ = run_in_process(folder, dtype, PAGE[name], steps, 448)
     compare(got, {"long": toks}, folder, dtype, "long decoding")
+    # in bfloat16 the output product of a lone token merges the key runs itself once there are two of them
+    assert (dtype == "bfloat16") == bool(merged) and set(merged) <= {2}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
