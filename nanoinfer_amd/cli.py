@@ -48,7 +48,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--num-cache-blocks", type=int, default=1024)
     ap.add_argument("--max-model-len", type=int, default=None)
     ap.add_argument("--max-decode-run", type=int, default=8,
-                    help="decode steps run back to back on one scheduling decision (greedy requests only)")
+                    help="decode steps run back to back on one scheduling decision (requests without a repetition penalty)")
     ap.add_argument("--json", action="store_true", help="print the generated ids as one JSON line per request")
     return ap
 

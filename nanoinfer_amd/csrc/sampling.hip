@@ -2,7 +2,7 @@
 // repetition penalty -> temperature -> top-k -> softmax -> top-p -> renormalise -> inverse CDF
 // (order of src/sampler/configurable_sampler.cpp:93-120 of the reference).
 //
-// One workgroup of 1024 threads owns one row.  Thresholds are exact selections, not the
+// Thresholds are exact selections, not the
 // 16-step bisections of src/op/kernels/cuda/sampling_kernel.cu:202-296: a radix descent over
 // the order-preserving integer image of a float finds the k-th largest logit (counts) and the
 // smallest logit whose upper set still holds the mass top_p (sums).  Equal logits at a
@@ -11,8 +11,7 @@
 // u in (0, 1] comes from the host, which derives it from (seed, request, step).
 #include "common.h"
 
-#define SAMPLE_THREADS 1024
-#define SAMPLE_WAVES (SAMPLE_THREADS / WAVE)
+#include <type_traits>
 
 __device__ __forceinline__ uint32_t order_key(float f) {
     uint32_t u = __float_as_uint(f);
@@ -22,28 +21,6 @@ __device__ __forceinline__ uint32_t order_key(float f) {
 // argmax with the lowest index among equal values (src/op/kernels/cuda/argmax_kernel.cu:27).
 __device__ __forceinline__ void better(float& v, int& i, float v2, int i2) {
     if (v2 > v || (v2 == v && i2 < i)) { v = v2; i = i2; }
-}
-
-__device__ int block_argmax(const float* __restrict__ row, int V, float* out_max, float* s_val, int* s_idx) {
-    float best = -INFINITY;
-    int idx = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) better(best, idx, row[i], i);
-#pragma unroll
-    for (int off = WAVE / 2; off > 0; off >>= 1) {
-        float v2 = __shfl_xor(best, off, WAVE);
-        int i2 = __shfl_xor(idx, off, WAVE);
-        better(best, idx, v2, i2);
-    }
-    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-    __syncthreads();
-    if (lane == 0) { s_val[wave] = best; s_idx[wave] = idx; }
-    __syncthreads();
-    const int nw = (blockDim.x + WAVE - 1) / WAVE;
-    best = s_val[0]; idx = s_idx[0];
-    for (int w = 1; w < nw; ++w) better(best, idx, s_val[w], s_idx[w]);
-    if (idx == 0x7fffffff) idx = 0;  // a row of NaN or -inf: fall back to the first token
-    *out_max = best;
-    return idx;
 }
 
 // Stage one: ARGMAX_PARTS workgroups share a row, each finds the best of its slice (float4 loads
@@ -106,37 +83,104 @@ __global__ void argmax_final_kernel(const float* __restrict__ part_val, const in
     if (threadIdx.x == 0) out[r] = idx == 0x7fffffff ? 0 : idx;    // a row of NaN: the first token
 }
 
-__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
-    const float* __restrict__ logits, float* __restrict__ work, const float* __restrict__ temperature,
-    const int32_t* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ penalty,
-    const int32_t* __restrict__ pen_ids, const int32_t* __restrict__ pen_off, const float* __restrict__ uniform,
-    int32_t* __restrict__ out, int V) {
-    __shared__ float s_val[SAMPLE_WAVES];
-    __shared__ int s_idx[SAMPLE_WAVES];
-    __shared__ float s_red[SAMPLE_WAVES];
-    __shared__ float hist_f[256];
-    __shared__ uint32_t hist_u[256];
-    __shared__ uint32_t s_prefix;
-    __shared__ float s_remaining_f;
-    __shared__ uint32_t s_remaining_u;
-    __shared__ int s_pick;
-    __shared__ int s_last;
+// ---------------------------------------------------------------------------------------------
+// The sampling pipeline.  A row of a large vocabulary is far too long for one workgroup (one
+// compute unit draws a few per cent of the chip's bandwidth), so PARTS workgroups share a row, each
+// with a contiguous slice, and the pipeline is a chain of short launches; whatever one launch
+// decides for a row (a level of a radix descent, the mass of the kept tokens) every workgroup of
+// the next launch works out again from the per-part results, in the same fixed order, so that all
+// agree and no launch waits for another inside itself.  Per-part histograms and decisions of
+// successive levels alternate between two buffers: a workgroup may still be reading the last
+// level's while another writes the next one's.
+//
+// scratch, all sized by the host: work float [R, V]; part_max float / part_arg int32 [R, P];
+// part_z, part_mass float / part_last int32 [R, P]; hist uint32 [2, R, P, 256] (counts, or the
+// bits of float sums); state uint32 [R, 16]: words 2*l, 2*l + 1 = (prefix, remaining) after level
+// l of the top-k descent (l = 0..3), words 8 + 2*l likewise for top-p (remaining as float bits).
+struct SampleArgs {
+    const float* logits; float* work;
+    const float* temperature; const int32_t* top_k; const float* top_p; const float* penalty;
+    const int32_t* pen_ids; const int32_t* pen_off; const float* uniform; int32_t* out;
+    float* part_max; int32_t* part_arg; float* part_z; float* part_mass; int32_t* part_last;
+    uint32_t* hist; uint32_t* state;
+    int R, V, P;
+};
 
-    const int r = blockIdx.x;
-    const int tid = threadIdx.x;
-    const float* lrow = logits + static_cast<size_t>(r) * V;
-    float* w = work + static_cast<size_t>(r) * V;
-    const float T = temperature[r];
+#define SP_THREADS 256
+#define SP_WAVES (SP_THREADS / WAVE)
+
+struct Slice { int lo, hi; };
+__device__ __forceinline__ Slice slice_of(int part, int V, int P) {
+    const int per = ((V + P - 1) / P + 3) & ~3;
+    const int lo = min(V, part * per);
+    return Slice{lo, min(V, lo + per)};
+}
+__device__ __forceinline__ bool row_samples(const SampleArgs& a, int r) { return a.temperature[r] > 0.f; }
+__device__ __forceinline__ bool row_top_k(const SampleArgs& a, int r) { return row_samples(a, r) && a.top_k[r] > 0 && a.top_k[r] < a.V; }
+__device__ __forceinline__ bool row_top_p(const SampleArgs& a, int r) { return row_samples(a, r) && a.top_p[r] > 0.f && a.top_p[r] < 1.0f; }
+__device__ __forceinline__ uint32_t* hist_of(const SampleArgs& a, int which, int r, int part) {
+    return a.hist + ((static_cast<size_t>(which) * a.R + r) * a.P + part) * 256;
+}
+
+// One level of a radix descent, decided by every workgroup alike: the bins of all parts are summed in
+// the order of the parts, then the highest bin b is found whose bins from b upwards hold at least
+// `remaining`.  Returns b; `remaining` loses what the bins above b hold.  CT: uint32_t (counts) or float (sums).
+template <typename CT>
+__device__ int decide_level(const uint32_t* __restrict__ hist_row, int P, CT& remaining, CT* s_scan, int* s_bin) {
+    const int tid = threadIdx.x;                      // SP_THREADS == 256: thread t owns bin 255 - t
+    const int bin = 255 - tid;
+    CT mine = 0;
+    for (int p = 0; p < P; ++p) {
+        const uint32_t raw = hist_row[static_cast<size_t>(p) * 256 + bin];
+        if constexpr (std::is_same<CT, float>::value) mine += __uint_as_float(raw);
+        else mine += raw;
+    }
+    // inclusive scan over the threads = sum of the bins from `bin` upwards
+    CT incl = mine;
+#pragma unroll
+    for (int off = 1; off < WAVE; off <<= 1) {
+        const CT o = __shfl_up(incl, off, WAVE);
+        if ((tid % WAVE) >= off) incl += o;
+    }
+    const int wave = tid / WAVE, lane = tid % WAVE;
+    __syncthreads();
+    if (lane == WAVE - 1) s_scan[wave] = incl;
+    if (tid == 0) *s_bin = 0;
+    __syncthreads();
+    CT before = 0;
+    for (int w = 0; w < wave; ++w) before += s_scan[w];
+    incl += before;
+    if (incl >= remaining) atomicMax(s_bin, bin);
+    __syncthreads();
+    const int b = *s_bin;
+    // what the bins above b hold: the exclusive value of bin b's thread
+    __syncthreads();
+    if (bin == b) s_scan[SP_WAVES] = incl - mine;
+    __syncthreads();
+    remaining -= s_scan[SP_WAVES];
+    return b;
+}
+
+// Launch 1: penalty and temperature (src/op/kernels/cuda/sampling_kernel.cu:38-88), the slice's
+// largest value, and the counts of the first radix level for top-k.
+__global__ __launch_bounds__(SP_THREADS) void sample_prepare_kernel(SampleArgs a) {
+    __shared__ float s_val[SP_WAVES];
+    __shared__ int s_idx[SP_WAVES];
+    __shared__ uint32_t s_hist[256];
+    const int r = blockIdx.x, part = blockIdx.y, tid = threadIdx.x;
+    const Slice sl = slice_of(part, a.V, a.P);
+    const float* lrow = a.logits + static_cast<size_t>(r) * a.V;
+    float* w = a.work + static_cast<size_t>(r) * a.V;
+    const float T = a.temperature[r];
     const float inv_t = (T <= 0.f || T == 1.0f) ? 1.0f : 1.0f / T;
-    const float pen = penalty[r];
-
-    // penalty and temperature (src/op/kernels/cuda/sampling_kernel.cu:38-88)
-    for (int i = tid; i < V; i += SAMPLE_THREADS) w[i] = lrow[i] * inv_t;
+    const float pen = a.penalty[r];
+    for (int i = sl.lo + tid; i < sl.hi; i += SP_THREADS) w[i] = lrow[i] * inv_t;
+    s_hist[tid] = 0;
     __syncthreads();
     if (pen != 1.0f) {
-        for (int j = pen_off[r] + tid; j < pen_off[r + 1]; j += SAMPLE_THREADS) {
-            const int id = pen_ids[j];
-            if (id >= 0 && id < V) {
+        for (int j = a.pen_off[r] + tid; j < a.pen_off[r + 1]; j += SP_THREADS) {
+            const int id = a.pen_ids[j];
+            if (id >= sl.lo && id < sl.hi) {
                 float l = lrow[id];
                 l = l > 0.f ? l / pen : l * pen;
                 w[id] = l * inv_t;
@@ -144,121 +188,252 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         }
         __syncthreads();
     }
-
-    float M;
-    const int best = block_argmax(w, V, &M, s_val, s_idx);
-    if (T <= 0.f) {
-        if (tid == 0) out[r] = best;
-        return;
+    const bool counts = row_top_k(a, r);
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = sl.lo + tid; i < sl.hi; i += SP_THREADS) {
+        const float v = w[i];
+        better(best, idx, v, i);
+        if (counts) atomicAdd(&s_hist[order_key(v) >> 24], 1u);
     }
-
-    // top-k: the k-th largest key, by counts
-    uint32_t thr = 0;
-    const int k = top_k[r];
-    if (k > 0 && k < V) {
-        if (tid == 0) { s_prefix = 0; s_remaining_u = static_cast<uint32_t>(k); }
-        for (int shift = 24; shift >= 0; shift -= 8) {
-            if (tid < 256) hist_u[tid] = 0;
-            __syncthreads();
-            const uint32_t prefix = s_prefix;
-            const uint32_t mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
-            for (int i = tid; i < V; i += SAMPLE_THREADS) {
-                const uint32_t key = order_key(w[i]);
-                if ((key & mask) == prefix) atomicAdd(&hist_u[(key >> shift) & 255u], 1u);
-            }
-            __syncthreads();
-            if (tid == 0) {
-                uint32_t remaining = s_remaining_u, cum = 0;
-                int b = 255;
-                for (; b > 0; --b) {
-                    if (cum + hist_u[b] >= remaining) break;
-                    cum += hist_u[b];
-                }
-                s_remaining_u = remaining - cum;
-                s_prefix = prefix | (static_cast<uint32_t>(b) << shift);
-            }
-            __syncthreads();
-        }
-        thr = s_prefix;
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+        const float v2 = __shfl_xor(best, off, WAVE);
+        const int i2 = __shfl_xor(idx, off, WAVE);
+        better(best, idx, v2, i2);
     }
+    const int wave = tid / WAVE, lane = tid % WAVE;
+    if (lane == 0) { s_val[wave] = best; s_idx[wave] = idx; }
+    __syncthreads();
+    if (tid == 0) {
+        for (int wv = 1; wv < SP_WAVES; ++wv) better(best, idx, s_val[wv], s_idx[wv]);
+        a.part_max[r * a.P + part] = best;
+        a.part_arg[r * a.P + part] = idx;
+    }
+    if (counts) hist_of(a, 0, r, part)[tid] = s_hist[tid];
+}
 
-    // softmax mass of the kept tokens
+// Launches 2 to 4 (level = 1, 2, 3): decide level `level` - 1 of the top-k descent from the counts the
+// launch before left, then count the next eight bits of the keys that share the prefix so far.
+__global__ __launch_bounds__(SP_THREADS) void sample_top_k_kernel(SampleArgs a, int level) {
+    __shared__ uint32_t s_scan[SP_WAVES + 1];
+    __shared__ int s_bin;
+    __shared__ uint32_t s_hist[256];
+    const int r = blockIdx.x, part = blockIdx.y, tid = threadIdx.x;
+    if (!row_top_k(a, r)) return;
+    uint32_t* st = a.state + static_cast<size_t>(r) * 16;
+    uint32_t prefix = level == 1 ? 0u : st[2 * (level - 2)];
+    uint32_t remaining = level == 1 ? static_cast<uint32_t>(a.top_k[r]) : st[2 * (level - 2) + 1];
+    const int b = decide_level<uint32_t>(hist_of(a, (level - 1) & 1, r, 0), a.P, remaining, s_scan, &s_bin);
+    const int decided_shift = 24 - 8 * (level - 1);
+    prefix |= static_cast<uint32_t>(b) << decided_shift;
+    if (part == 0 && tid == 0) { st[2 * (level - 1)] = prefix; st[2 * (level - 1) + 1] = remaining; }
+    const int shift = decided_shift - 8;
+    const uint32_t mask = 0xffffffffu << decided_shift;
+    s_hist[tid] = 0;
+    __syncthreads();
+    const Slice sl = slice_of(part, a.V, a.P);
+    const float* w = a.work + static_cast<size_t>(r) * a.V;
+    for (int i = sl.lo + tid; i < sl.hi; i += SP_THREADS) {
+        const uint32_t key = order_key(w[i]);
+        if ((key & mask) == prefix) atomicAdd(&s_hist[(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    hist_of(a, level & 1, r, part)[tid] = s_hist[tid];
+}
+
+// The key of the k-th largest value once the counts of the last level are in (hist buffer 1), or 0.
+__device__ uint32_t top_k_threshold(const SampleArgs& a, int r, uint32_t* s_scan, int* s_bin) {
+    if (!row_top_k(a, r)) return 0u;
+    const uint32_t* st = a.state + static_cast<size_t>(r) * 16;
+    uint32_t remaining = st[5];
+    const int b = decide_level<uint32_t>(hist_of(a, 1, r, 0), a.P, remaining, s_scan, s_bin);
+    return st[4] | static_cast<uint32_t>(b);
+}
+
+__device__ float row_max(const SampleArgs& a, int r) {
+    float M = a.part_max[r * a.P];
+    for (int p = 1; p < a.P; ++p) M = fmaxf(M, a.part_max[r * a.P + p]);
+    return M;
+}
+
+// Launch 5: the softmax mass of the slice's kept tokens, and the sums of the first radix level for top-p.
+__global__ __launch_bounds__(SP_THREADS) void sample_mass_kernel(SampleArgs a) {
+    __shared__ uint32_t s_scan[SP_WAVES + 1];
+    __shared__ int s_bin;
+    __shared__ float s_red[16];
+    __shared__ float s_hist[256];
+    const int r = blockIdx.x, part = blockIdx.y, tid = threadIdx.x;
+    if (!row_samples(a, r)) return;
+    const uint32_t thr = top_k_threshold(a, r, s_scan, &s_bin);
+    if (part == 0 && tid == 0) a.state[static_cast<size_t>(r) * 16 + 6] = thr;
+    const float M = row_max(a, r);
+    const bool sums = row_top_p(a, r);
+    s_hist[tid] = 0.f;
+    __syncthreads();
+    const Slice sl = slice_of(part, a.V, a.P);
+    const float* w = a.work + static_cast<size_t>(r) * a.V;
     float z = 0.f;
-    for (int i = tid; i < V; i += SAMPLE_THREADS)
-        if (order_key(w[i]) >= thr) z += expf(w[i] - M);
-    z = block_sum(z, s_red);
-
-    // top-p: the largest key whose upper set holds at least top_p of the mass, by sums
-    const float p = top_p[r];
-    if (p > 0.f && p < 1.0f) {
-        __syncthreads();
-        if (tid == 0) { s_prefix = 0; s_remaining_f = p * z; }
-        for (int shift = 24; shift >= 0; shift -= 8) {
-            if (tid < 256) hist_f[tid] = 0.f;
-            __syncthreads();
-            const uint32_t prefix = s_prefix;
-            const uint32_t mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
-            for (int i = tid; i < V; i += SAMPLE_THREADS) {
-                const uint32_t key = order_key(w[i]);
-                if (key >= thr && (key & mask) == prefix) atomicAdd(&hist_f[(key >> shift) & 255u], expf(w[i] - M));
-            }
-            __syncthreads();
-            if (tid == 0) {
-                float remaining = s_remaining_f, cum = 0.f;
-                int b = 255;
-                for (; b > 0; --b) {
-                    if (cum + hist_f[b] >= remaining) break;
-                    cum += hist_f[b];
-                }
-                s_remaining_f = remaining - cum;
-                s_prefix = prefix | (static_cast<uint32_t>(b) << shift);
-            }
-            __syncthreads();
+    for (int i = sl.lo + tid; i < sl.hi; i += SP_THREADS) {
+        const uint32_t key = order_key(w[i]);
+        if (key >= thr) {
+            const float e = expf(w[i] - M);
+            z += e;
+            if (sums) atomicAdd(&s_hist[key >> 24], e);
         }
-        thr = max(thr, s_prefix);
     }
+    z = block_sum(z, s_red);
+    if (tid == 0) a.part_z[r * a.P + part] = z;
+    if (sums) hist_of(a, 0, r, part)[tid] = __float_as_uint(s_hist[tid]);
+}
 
-    // inverse CDF in vocabulary order over contiguous segments
-    const int seg = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-    const int i0 = min(V, tid * seg), i1 = min(V, i0 + seg);
+// Launches 6 to 8 (level = 1, 2, 3): the same descent for top-p, over sums of exp(w - max) of the kept tokens.
+__global__ __launch_bounds__(SP_THREADS) void sample_top_p_kernel(SampleArgs a, int level) {
+    __shared__ float s_scan[SP_WAVES + 1];
+    __shared__ int s_bin;
+    __shared__ float s_hist[256];
+    const int r = blockIdx.x, part = blockIdx.y, tid = threadIdx.x;
+    if (!row_top_p(a, r)) return;
+    uint32_t* st = a.state + static_cast<size_t>(r) * 16;
+    uint32_t prefix;
+    float remaining;
+    if (level == 1) {
+        float z = 0.f;
+        for (int p = 0; p < a.P; ++p) z += a.part_z[r * a.P + p];
+        prefix = 0u;
+        remaining = a.top_p[r] * z;
+    } else {
+        prefix = st[8 + 2 * (level - 2)];
+        remaining = __uint_as_float(st[8 + 2 * (level - 2) + 1]);
+    }
+    const int b = decide_level<float>(hist_of(a, (level - 1) & 1, r, 0), a.P, remaining, s_scan, &s_bin);
+    const int decided_shift = 24 - 8 * (level - 1);
+    prefix |= static_cast<uint32_t>(b) << decided_shift;
+    if (part == 0 && tid == 0) { st[8 + 2 * (level - 1)] = prefix; st[8 + 2 * (level - 1) + 1] = __float_as_uint(remaining); }
+    const int shift = decided_shift - 8;
+    const uint32_t mask = 0xffffffffu << decided_shift;
+    const uint32_t thr = st[6];
+    const float M = row_max(a, r);
+    s_hist[tid] = 0.f;
+    __syncthreads();
+    const Slice sl = slice_of(part, a.V, a.P);
+    const float* w = a.work + static_cast<size_t>(r) * a.V;
+    for (int i = sl.lo + tid; i < sl.hi; i += SP_THREADS) {
+        const uint32_t key = order_key(w[i]);
+        if (key >= thr && (key & mask) == prefix) atomicAdd(&s_hist[(key >> shift) & 255u], expf(w[i] - M));
+    }
+    __syncthreads();
+    hist_of(a, level & 1, r, part)[tid] = __float_as_uint(s_hist[tid]);
+}
+
+// Launch 9: the final threshold, and per slice the mass of the tokens it keeps and the last of them.
+__global__ __launch_bounds__(SP_THREADS) void sample_kept_kernel(SampleArgs a) {
+    __shared__ float s_scan[SP_WAVES + 1];
+    __shared__ int s_bin;
+    __shared__ float s_red[16];
+    __shared__ int s_last;
+    const int r = blockIdx.x, part = blockIdx.y, tid = threadIdx.x;
+    if (!row_samples(a, r)) return;
+    uint32_t* st = a.state + static_cast<size_t>(r) * 16;
+    uint32_t thr = st[6];
+    if (row_top_p(a, r)) {
+        float remaining = __uint_as_float(st[8 + 5]);
+        const int b = decide_level<float>(hist_of(a, 1, r, 0), a.P, remaining, s_scan, &s_bin);
+        thr = max(thr, st[8 + 4] | static_cast<uint32_t>(b));
+    }
+    if (part == 0 && tid == 0) st[7] = thr;
+    if (tid == 0) s_last = -1;
+    __syncthreads();
+    const float M = row_max(a, r);
+    const Slice sl = slice_of(part, a.V, a.P);
+    const float* w = a.work + static_cast<size_t>(r) * a.V;
+    // contiguous runs per thread, as the draw walks them
+    const int seg = (sl.hi - sl.lo + SP_THREADS - 1) / SP_THREADS;
+    const int i0 = min(sl.hi, sl.lo + tid * seg), i1 = min(sl.hi, i0 + seg);
     float mine = 0.f;
     int last_kept = -1;
     for (int i = i0; i < i1; ++i)
         if (order_key(w[i]) >= thr) { mine += expf(w[i] - M); last_kept = i; }
-    // inclusive scan over threads
-    float incl = mine;
-#pragma unroll
-    for (int off = 1; off < WAVE; off <<= 1) {
-        float o = __shfl_up(incl, off, WAVE);
-        if ((tid % WAVE) >= off) incl += o;
-    }
-    const int wave = tid / WAVE, lane = tid % WAVE;
-    __syncthreads();
-    if (tid == 0) { s_pick = 0x7fffffff; s_last = -1; }
-    if (lane == WAVE - 1) s_red[wave] = incl;
-    __syncthreads();
-    float before = 0.f, total = 0.f;
-    for (int wv = 0; wv < SAMPLE_WAVES; ++wv) {
-        if (wv < wave) before += s_red[wv];
-        total += s_red[wv];
-    }
-    incl += before;
-    const float excl = incl - mine;
-    const float target = uniform[r] * total;
     if (last_kept >= 0) atomicMax(&s_last, last_kept);
-    if (mine > 0.f && excl < target && target <= incl) {
-        float cum = excl;
-        int pick = last_kept;
-        for (int i = i0; i < i1; ++i) {
-            if (order_key(w[i]) >= thr) {
-                cum += expf(w[i] - M);
-                if (cum >= target) { pick = i; break; }
-            }
-        }
-        atomicMin(&s_pick, pick);
+    const float mass = block_sum(mine, s_red);
+    if (tid == 0) { a.part_mass[r * a.P + part] = mass; a.part_last[r * a.P + part] = s_last; }
+}
+
+// Launch 10, one workgroup per row: the slice in which the cumulative mass reaches u * total, and in
+// it the first token that does (src/op/kernels/cuda/sampling_kernel.cu:330-398); rows that do not
+// sample take the largest (penalised) logit.
+__global__ __launch_bounds__(SP_THREADS) void sample_draw_kernel(SampleArgs a) {
+    __shared__ float s_red[SP_WAVES];
+    __shared__ int s_pick;
+    const int r = blockIdx.x, tid = threadIdx.x;
+    float best_v = -INFINITY;
+    int best = 0x7fffffff;
+    for (int p = 0; p < a.P; ++p) better(best_v, best, a.part_max[r * a.P + p], a.part_arg[r * a.P + p]);
+    if (best == 0x7fffffff) best = 0;        // a row of NaN or -inf: the first token
+    if (!row_samples(a, r)) {
+        if (tid == 0) a.out[r] = best;
+        return;
     }
+    const float M = best_v;
+    const uint32_t thr = a.state[static_cast<size_t>(r) * 16 + 7];
+    float total = 0.f;
+    int last = -1;
+    for (int p = 0; p < a.P; ++p) { total += a.part_mass[r * a.P + p]; last = max(last, a.part_last[r * a.P + p]); }
+    const float target = a.uniform[r] * total;
+    // the first slice whose cumulative mass reaches the target
+    int part = -1;
+    float before_part = 0.f;
+    {
+        float cum = 0.f;
+        for (int p = 0; p < a.P; ++p) {
+            const float m = a.part_mass[r * a.P + p];
+            if (m > 0.f && cum < target && target <= cum + m) { part = p; before_part = cum; break; }
+            cum += m;
+        }
+    }
+    if (tid == 0) s_pick = 0x7fffffff;
     __syncthreads();
-    if (tid == 0) out[r] = s_pick != 0x7fffffff ? s_pick : (s_last >= 0 ? s_last : best);
+    if (part >= 0) {
+        const Slice sl = slice_of(part, a.V, a.P);
+        const float* w = a.work + static_cast<size_t>(r) * a.V;
+        const int seg = (sl.hi - sl.lo + SP_THREADS - 1) / SP_THREADS;
+        const int i0 = min(sl.hi, sl.lo + tid * seg), i1 = min(sl.hi, i0 + seg);
+        float mine = 0.f;
+        int last_kept = -1;
+        for (int i = i0; i < i1; ++i)
+            if (order_key(w[i]) >= thr) { mine += expf(w[i] - M); last_kept = i; }
+        float incl = mine;
+#pragma unroll
+        for (int off = 1; off < WAVE; off <<= 1) {
+            const float o = __shfl_up(incl, off, WAVE);
+            if ((tid % WAVE) >= off) incl += o;
+        }
+        const int wave = tid / WAVE, lane = tid % WAVE;
+        if (lane == WAVE - 1) s_red[wave] = incl;
+        __syncthreads();
+        float before = before_part;
+        for (int wv = 0; wv < wave; ++wv) before += s_red[wv];
+        incl += before;
+        const float excl = incl - mine;
+        if (mine > 0.f && excl < target && target <= incl) {
+            float cum = excl;
+            int pick = last_kept;
+            for (int i = i0; i < i1; ++i) {
+                if (order_key(w[i]) >= thr) {
+                    cum += expf(w[i] - M);
+                    if (cum >= target) { pick = i; break; }
+                }
+            }
+            atomicMin(&s_pick, pick);
+        }
+        __syncthreads();
+    }
+    // rounding may leave the target a hair past every running sum: then the last kept token of the slice, or of the row
+    if (tid == 0) {
+        int pick = s_pick;
+        if (pick == 0x7fffffff && part >= 0) pick = a.part_last[r * a.P + part] >= 0 ? a.part_last[r * a.P + part] : 0x7fffffff;
+        a.out[r] = pick != 0x7fffffff ? pick : (last >= 0 ? last : best);
+    }
 }
 
 // part_val: float [R, 32], part_idx: int32 [R, 32] scratch
@@ -272,13 +447,46 @@ NI_EXPORT int ni_argmax(const void* logits, void* out, void* part_val, void* par
     return NI_LAUNCH_RESULT();
 }
 
+// Workgroups that share a row, for R rows of V logits: enough to cover the chip, slices of at least 1,024 tokens.
+NI_EXPORT int ni_sample_parts(int R, int V) {
+    int P = 512 / (R > 0 ? R : 1);
+    P = P < 1 ? 1 : P > 32 ? 32 : P;
+    while (P > 1 && (V + P - 1) / P < 1024) --P;
+    return P;
+}
+
+// Scratch (see SampleArgs): work float [R, V]; parts float [R, P, 5] (maximum, its index, mass before top-p,
+// mass kept, last kept index: five arrays of R * P words one after another); hist uint32 [2, R, P, 256];
+// state uint32 [R, 16].  P must be ni_sample_parts(R, V).  uses_top_k / uses_top_p: 0 if no row asks for
+// it (their launches are skipped then).
 NI_EXPORT int ni_sample(const void* logits, void* work, const void* temperature, const void* top_k, const void* top_p,
                         const void* penalty, const void* pen_ids, const void* pen_off, const void* uniform, void* out,
-                        int R, int V, hipStream_t stream) {
+                        void* parts, void* hist, void* state, int R, int V, int P, int uses_top_k, int uses_top_p,
+                        hipStream_t stream) {
     if (R <= 0) return 0;
-    sample_kernel<<<R, SAMPLE_THREADS, 0, stream>>>((const float*)logits, (float*)work, (const float*)temperature,
-                                                    (const int32_t*)top_k, (const float*)top_p, (const float*)penalty,
-                                                    (const int32_t*)pen_ids, (const int32_t*)pen_off,
-                                                    (const float*)uniform, (int32_t*)out, V);
-    return NI_LAUNCH_RESULT();
+    if (V < 1 || P != ni_sample_parts(R, V) || !parts || !hist || !state) return -1;
+    SampleArgs a;
+    a.logits = (const float*)logits; a.work = (float*)work;
+    a.temperature = (const float*)temperature; a.top_k = (const int32_t*)top_k; a.top_p = (const float*)top_p;
+    a.penalty = (const float*)penalty; a.pen_ids = (const int32_t*)pen_ids; a.pen_off = (const int32_t*)pen_off;
+    a.uniform = (const float*)uniform; a.out = (int32_t*)out;
+    float* pf = (float*)parts;
+    const size_t n = static_cast<size_t>(R) * P;
+    a.part_max = pf; a.part_arg = (int32_t*)(pf + n); a.part_z = pf + 2 * n; a.part_mass = pf + 3 * n;
+    a.part_last = (int32_t*)(pf + 4 * n);
+    a.hist = (uint32_t*)hist; a.state = (uint32_t*)state;
+    a.R = R; a.V = V; a.P = P;
+    const dim3 grid(R, P);
+    int err;
+#define SP_STEP(call) call; if ((err = NI_LAUNCH_RESULT()) != 0) return err;
+    SP_STEP((sample_prepare_kernel<<<grid, SP_THREADS, 0, stream>>>(a)))
+    if (uses_top_k)
+        for (int level = 1; level <= 3; ++level) { SP_STEP((sample_top_k_kernel<<<grid, SP_THREADS, 0, stream>>>(a, level))) }
+    SP_STEP((sample_mass_kernel<<<grid, SP_THREADS, 0, stream>>>(a)))
+    if (uses_top_p)
+        for (int level = 1; level <= 3; ++level) { SP_STEP((sample_top_p_kernel<<<grid, SP_THREADS, 0, stream>>>(a, level))) }
+    SP_STEP((sample_kept_kernel<<<grid, SP_THREADS, 0, stream>>>(a)))
+    SP_STEP((sample_draw_kernel<<<R, SP_THREADS, 0, stream>>>(a)))
+#undef SP_STEP
+    return 0;
 }

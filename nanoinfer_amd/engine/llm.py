@@ -95,7 +95,9 @@ class Engine:
             if item.samples:
                 sampling.append(item.request)
         self.last_prompt_tokens = sum(i.count for i in batch.items if i.count > 1 or not i.request.generated)
-        run = self.scheduler.decode_run_length(batch) if hasattr(self.runner, "decode_run") else 1
+        run = 1
+        if hasattr(self.runner, "decode_run"):
+            run = self.scheduler.decode_run_length(batch, draws=hasattr(self.sampler, "plan"))
         if run > 1:
             return self._decode_run(batch, entries, run)
         logits = self.runner.step(entries)
@@ -109,10 +111,16 @@ class Engine:
         return self.scheduler.commit(batch, sampled)
 
     def _decode_run(self, batch: ScheduledBatch, entries, run: int) -> List[Request]:
-        """``run`` greedy decode steps of the same batch on one scheduling decision: the runner
-        feeds every step's tokens to the next by itself; the scheduler then books the steps one by
-        one, and a request that stops on the way is finished there and its later tokens dropped."""
-        chosen = self.runner.decode_run(entries, run)
+        """``run`` decode steps of the same batch on one scheduling decision: the runner
+        feeds every step's tokens to the next by itself (the largest logits, or what the sampler's
+        plan draws); the scheduler then books the steps one by one, and a request that stops on the
+        way is finished there and its later tokens dropped."""
+        requests = [item.request for item in batch.items]
+        if all(r.params.use_greedy() for r in requests):
+            chosen = self.runner.decode_run(entries, run)
+        else:
+            plan = self.sampler.plan([r.params for r in requests], [len(r.generated) for r in requests], run)
+            chosen = self.runner.decode_run(entries, run, pick=plan.launch)
         column = {item.request.request_id: b for b, item in enumerate(batch.items)}
         finished: List[Request] = []
         live = list(batch.items)

@@ -459,7 +459,7 @@ class ModelRunner:
         return True
 
     def _replay(self, key, entries: List[StepEntry], tokens_from: Optional[_RecordedStep] = None,
-                history_row: Optional[int] = None) -> bool:
+                history_row: Optional[int] = None, pick=None) -> bool:
         """Run the entries through the recording of their shape (made now if there is none).  False:
         this shape cannot be recorded and the step has not run.  The logits are left in
         ``self._replayed_logits``.
@@ -468,7 +468,8 @@ class ModelRunner:
         last replay of that recording (a decode step over the same requests in the same order)
         chose, and are taken from where it left them on the device.  ``history_row``: the tokens
         this replay chooses are also copied to that row of ``self._history`` (pinned host memory),
-        and its logits are not kept."""
+        and its logits are not kept.  ``pick(logits, out)``: launched behind the replay, it puts other
+        tokens than the largest logits where the step leaves its choice."""
         rec = self._recorded.get(key)
         if rec is None:
             rec = self._record(key, entries)
@@ -528,6 +529,8 @@ class ModelRunner:
                 rec.meta[0:B].copy_(tokens_from.amax[0:B], non_blocking=True)
         rec.copied[rec.turn].record()
         rec.graph.replay()
+        if pick is not None:
+            pick(rec.logits, rec.amax[0:B])
         self._last_context_len = totals
         if history_row is not None:
             self._history[history_row, 0:B].copy_(rec.amax[0:B], non_blocking=True)
@@ -573,10 +576,12 @@ class ModelRunner:
             self.release(r)
         return logits
 
-    def decode_run(self, entries: Sequence[StepEntry], steps: int) -> List[List[int]]:
-        """Greedy decoding of ``steps`` tokens for every entry (one token each, wanting its logits):
+    def decode_run(self, entries: Sequence[StepEntry], steps: int, pick=None) -> List[List[int]]:
+        """Decoding of ``steps`` tokens for every entry (one token each, wanting its logits):
         the first step takes the entries' tokens, every later one the tokens that the step before
-        chose (the index of the largest logit, lowest index on ties).  Returns the chosen tokens,
+        chose: the index of the largest logit, lowest index on ties, or with ``pick`` what
+        ``pick(i, logits, out)`` launches into ``out`` (int32 [entries], on the device) for step
+        ``i`` without waiting for anything.  Returns the chosen tokens,
         ``[step][entry]``: what ``steps`` calls of :meth:`step` with :meth:`greedy_tokens` between
         them return.  Where recordings of the steps' shapes exist, the steps are launched back to
         back, the tokens passing from one to the next on the device, and the host waits once at
@@ -613,12 +618,20 @@ class ModelRunner:
                 collect()
                 cur = [StepEntry(e.request, [tokens[b]], [0]) for b, e in enumerate(entries)]
             if rec is None or rec.amax is None:
-                tokens = self.greedy_tokens(self.step(cur))
+                logits = self.step(cur)
+                if pick is None:
+                    tokens = self.greedy_tokens(logits)
+                else:
+                    out = torch.empty(B, dtype=torch.int32, device=self.device)
+                    pick(len(chosen), logits, out)
+                    tokens = out.tolist()
                 chosen.append(list(tokens))
                 last = None
                 continue
             self._check_and_reserve(cur)
-            self._replay(key, cur, tokens_from=last if tokens is None else None, history_row=launched)
+            at = len(chosen) + launched
+            self._replay(key, cur, tokens_from=last if tokens is None else None, history_row=launched,
+                         pick=None if pick is None else (lambda logits, out, at=at: pick(at, logits, out)))
             self._book(cur, self._last_context_len)
             launched += 1
             tokens = None

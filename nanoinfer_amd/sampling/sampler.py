@@ -1,9 +1,10 @@
 """The sampler above the kernels: from logits and per-request options to one token per row.
 
 Pipeline and fast path follow src/sampler/configurable_sampler.cpp:65-174 of the reference: when
-every row is greedy one argmax kernel runs; otherwise one kernel per row does penalty ->
-temperature -> top-k -> softmax -> top-p -> renormalise -> draw, and takes the argmax for rows
-whose temperature is <= 0 (the reference fixes those up through the host afterwards).
+every row is greedy one argmax kernel runs; otherwise a chain of short kernels, in which several
+workgroups share a row, does penalty -> temperature -> top-k -> softmax -> top-p -> renormalise ->
+draw, and takes the argmax for rows whose temperature is <= 0 (the reference fixes those up through
+the host afterwards).
 
 Two things differ on purpose.  The uniform number of a draw comes from a counter-based generator
 keyed by (seed, tokens generated so far), so a seeded request gives the same tokens whatever
@@ -15,6 +16,7 @@ from __future__ import annotations
 
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from .. import kernels as K
@@ -56,17 +58,60 @@ class Sampler:
             if p.use_repetition_penalty():
                 pen_ids.extend(sorted(set(int(t) for t in g)))
             pen_off.append(len(pen_ids))
-        dev = self.device
-        f32, i32 = torch.float32, torch.int32
-        temperature = torch.tensor([p.temperature for p in params], dtype=f32).to(dev)
-        top_k = torch.tensor([p.top_k if p.use_top_k() else 0 for p in params], dtype=i32).to(dev)
-        top_p = torch.tensor([p.top_p if p.use_top_p() else 1.0 for p in params], dtype=f32).to(dev)
-        penalty = torch.tensor([p.repetition_penalty for p in params], dtype=f32).to(dev)
-        uniform = torch.tensor([uniform_from_counter(max(p.seed, 0), c) for p, c in zip(params, counters)],
-                               dtype=f32).to(dev)
-        ids = torch.tensor(pen_ids if pen_ids else [0], dtype=i32).to(dev)
-        off = torch.tensor(pen_off, dtype=i32).to(dev)
+        # every per-row option in one upload: four float arrays and three int arrays, as int32 words
+        floats = np.array([[p.temperature for p in params],
+                           [p.top_p if p.use_top_p() else 1.0 for p in params],
+                           [p.repetition_penalty for p in params],
+                           [uniform_from_counter(max(p.seed, 0), c) for p, c in zip(params, counters)]], dtype=np.float32)
+        ints = np.array([p.top_k if p.use_top_k() else 0 for p in params] + pen_off + (pen_ids or [0]), dtype=np.int32)
+        packed = torch.from_numpy(np.concatenate([floats.reshape(-1).view(np.int32), ints])).to(self.device)
+        as_float = packed[: 4 * R].view(torch.float32)
+        temperature, top_p, penalty, uniform = (as_float[i * R:(i + 1) * R] for i in range(4))
+        top_k = packed[4 * R: 5 * R]
+        off = packed[5 * R: 6 * R + 1]
+        ids = packed[6 * R + 1:]
         work = torch.empty_like(logits)
-        out = torch.empty(R, dtype=i32, device=dev)
-        K.sample(logits, work, temperature, top_k, top_p, penalty, ids, off, uniform, out)
+        out = torch.empty(R, dtype=torch.int32, device=self.device)
+        K.sample(logits, work, temperature, top_k, top_p, penalty, ids, off, uniform, out,
+                 uses_top_k=any(p.use_top_k() and p.temperature > 0 for p in params),
+                 uses_top_p=any(p.use_top_p() and p.temperature > 0 for p in params))
         return out.tolist()
+
+    def plan(self, params: Sequence[SamplingParams], counters: Sequence[int], steps: int) -> "SamplingPlan":
+        """The draws of ``steps`` successive tokens for the same rows, prepared in one upload: the
+        uniform numbers of a seeded request do not depend on the tokens drawn before (they are keyed
+        by the seed and the count of generated tokens), so a caller can launch step after step
+        without reading a token in between.  No row may have a repetition penalty (that needs the
+        tokens)."""
+        if any(p.use_repetition_penalty() for p in params):
+            raise ValueError("a repetition penalty needs the generated tokens: it cannot be planned ahead")
+        return SamplingPlan(self.device, params, counters, steps)
+
+
+class SamplingPlan:
+    """Options of R rows and their uniform numbers for ``steps`` draws, on the device."""
+
+    def __init__(self, device, params: Sequence[SamplingParams], counters: Sequence[int], steps: int):
+        R = len(params)
+        floats = np.array([[p.temperature for p in params],
+                           [p.top_p if p.use_top_p() else 1.0 for p in params],
+                           [1.0] * R], dtype=np.float32)
+        uniform = np.array([[uniform_from_counter(max(p.seed, 0), c + i) for p, c in zip(params, counters)]
+                            for i in range(steps)], dtype=np.float32)
+        ints = np.array([p.top_k if p.use_top_k() else 0 for p in params] + [0] * (R + 2), dtype=np.int32)
+        packed = torch.from_numpy(np.concatenate([floats.reshape(-1).view(np.int32), ints,
+                                                  uniform.reshape(-1).view(np.int32)])).to(device)
+        as_float = packed[: 3 * R].view(torch.float32)
+        self.temperature, self.top_p, self.penalty = (as_float[i * R:(i + 1) * R] for i in range(3))
+        self.top_k = packed[3 * R: 4 * R]
+        self.pen_off = packed[4 * R: 5 * R + 1]
+        self.pen_ids = packed[5 * R + 1: 5 * R + 2]
+        self.uniform = packed[5 * R + 2:].view(torch.float32).view(steps, R)
+        self.uses_top_k = any(p.use_top_k() and p.temperature > 0 for p in params)
+        self.uses_top_p = any(p.use_top_p() and p.temperature > 0 for p in params)
+        self.steps = steps
+
+    def launch(self, i: int, logits: torch.Tensor, out: torch.Tensor) -> None:
+        """Launch draw ``i`` over ``logits`` [R, vocab] into ``out`` (int32 [R], device); nothing waits."""
+        K.sample(logits, torch.empty_like(logits), self.temperature, self.top_k, self.top_p, self.penalty,
+                 self.pen_ids, self.pen_off, self.uniform[i], out, uses_top_k=self.uses_top_k, uses_top_p=self.uses_top_p)

@@ -69,6 +69,37 @@ def test_decode_runs_do_not_change_the_tokens(dtype):
     assert [len(t) for t in outs[1]] == [30, 11, 50, 17]
 
 
+def test_decode_runs_with_planned_draws_give_the_tokens_of_single_steps():
+    """Requests that draw (temperature, top-k, top-p; no repetition penalty) decode in runs too: the
+    uniform numbers of their draws are known ahead, and every step's draw is launched behind the
+    step.  Float32, so that the two ways see the same logits to the last bit but for the attention's
+    key runs; a request with a repetition penalty keeps every step single."""
+    from nanoinfer_amd.sampling.params import SamplingParams
+    folder = model_folder("B")
+    prompts = [list(random_tokens(1000, n, 60 + n)) for n in (9, 40, 23, 3)]
+    options = [SamplingParams(temperature=0.8, seed=5), SamplingParams(temperature=1.3, top_k=40, top_p=0.9, seed=6),
+               SamplingParams.greedy(), SamplingParams(temperature=0.6, top_p=0.5, seed=7)]
+    outs, runs = [], []
+    for run in (1, 8):
+        eng = engine(folder, dtype="float32", block_size=8, num_cache_blocks=24, max_sequences=3, max_decode_run=run)
+        asked, original = [], eng.runner.decode_run
+        eng.runner.decode_run = lambda entries, steps, pick=None: (asked.append((steps, pick is not None)), original(entries, steps, pick))[1]
+        ids = [eng.add_request(p, n, o) for p, n, o in zip(prompts, (30, 11, 50, 17), options)]
+        eng.run()
+        outs.append([eng.get_request(i).generated for i in ids])
+        runs.append(asked)
+        assert eng.runner.cache.free_pages() == 24
+    assert outs[0] == outs[1]
+    assert [len(t) for t in outs[1]] == [30, 11, 50, 17]
+    assert not runs[0] and any(steps == 8 and draws for steps, draws in runs[1])
+    assert len({tuple(t) for t in outs[1]}) == 4 and outs[1][2] != outs[1][0]
+    # with a repetition penalty every decision is taken step by step
+    eng = engine(folder, dtype="float32", block_size=8, num_cache_blocks=24, max_decode_run=8)
+    eng.runner.decode_run = None
+    eng.add_request(prompts[0], 6, SamplingParams(temperature=0.8, repetition_penalty=1.2, seed=5))
+    eng.run()
+
+
 def test_stop_token_from_the_configuration():
     from nanoinfer_amd.sampling.params import SamplingParams
     folder = model_folder("B")

@@ -425,7 +425,7 @@ def plain_pick(logits, temperature, top_k, top_p, penalty, generated, u):
     return P.inverse_cdf(P.filtered_distribution(l, top_k, top_p), u)
 
 
-@pytest.mark.parametrize("V", [50, 1000, 5003])
+@pytest.mark.parametrize("V", [50, 1000, 5003, 40000])
 def test_sampling_matches_plain(K, V):
     g = torch.Generator().manual_seed(V)
     rng = random.Random(V)

@@ -3,6 +3,8 @@
 The fake runner keeps real cache books (a KVCacheManager without pools) and returns logits whose
 argmax is a known function of the request, as the reference's mock model does with a fixed
 argmax of 3 (test/test_engine/test_engine.cpp:11-80)."""
+import types
+
 import pytest
 import torch
 
@@ -230,14 +232,19 @@ class FakeRunnerWithRuns(FakeRunner):
         super().__init__(**kw)
         self.runs = []           # length of every run asked for
 
-    def decode_run(self, entries, steps):
+    def decode_run(self, entries, steps, pick=None):
         from nanoinfer_amd.engine.runner import StepEntry
         self.runs.append(steps)
         chosen = []
         tokens = [e.tokens[0] for e in entries]
-        for _ in range(steps):
+        for k in range(steps):
             logits = self.step([StepEntry(e.request, [t], [0]) for e, t in zip(entries, tokens)])
-            tokens = logits.argmax(dim=-1).tolist()
+            if pick is None:
+                tokens = logits.argmax(dim=-1).tolist()
+            else:
+                out = torch.empty(len(entries), dtype=torch.int32)
+                pick(k, logits, out)
+                tokens = out.tolist()
             chosen.append(tokens)
         return chosen
 
@@ -296,6 +303,22 @@ def test_what_keeps_a_decode_step_single():
         eng.add_request([1, 2], max_new_tokens=6, params=params)
         eng.run()
         assert runner.runs == []
+    # unless the sampler can plan the draws ahead (never with a repetition penalty: that needs the tokens)
+    class PlanningSampler(ArgmaxSampler):
+        def __init__(self):
+            self.plans = []
+
+        def plan(self, params, counters, steps):
+            self.plans.append((list(counters), steps))
+            assert not any(p.use_repetition_penalty() for p in params)
+            return types.SimpleNamespace(launch=lambda i, logits, out: out.copy_(logits.argmax(dim=-1)))
+    for params, runs in ((SamplingParams(temperature=0.7, seed=1), [5]), (SamplingParams(temperature=0.7, repetition_penalty=1.3, seed=1), [])):
+        eng, runner = make_run_engine(max_decode_run=8, num_pages=32)
+        eng.sampler = PlanningSampler()
+        r = eng.add_request([1, 2], max_new_tokens=6, params=params)
+        eng.run()
+        assert runner.runs == runs and eng.get_request(r).generated == [3, 4, 5, 6, 7, 8]
+        assert eng.sampler.plans == ([([1], 5)] if runs else [])
     # a prompt portion in the batch
     eng, runner = make_run_engine(max_decode_run=8, num_pages=32, max_num_batched_tokens=4)
     eng.add_request([1, 2], max_new_tokens=6, params=greedy)
