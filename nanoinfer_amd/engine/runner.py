@@ -148,7 +148,8 @@ class ModelRunner:
     GRAPH_MAX_PORTIONS = 24       # recordings of prompt portions kept (each holds its activations)
 
     def __init__(self, model_dir: str, dtype: str = "bfloat16", page_size: int = 16, max_tokens: int = 4096,
-                 max_requests: int = 64, device: Optional[torch.device] = None, use_graphs: bool = True):
+                 max_requests: int = 64, device: Optional[torch.device] = None, use_graphs: bool = True,
+                 warm_up: bool = True):
         self.device = device or K.require_gpu()
         torch_dtype = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
                        "float32": torch.float32, "fp32": torch.float32}.get(dtype)
@@ -170,6 +171,26 @@ class ModelRunner:
         self._done: Dict[Hashable, int] = {}   # tokens of each live request already in the cache
         self._scratch: Optional[torch.Tensor] = None
         self._init_graphs(use_graphs)
+        if warm_up:
+            self._warm_up()
+
+    def _warm_up(self) -> None:
+        """One short prompt and one decode step of a request of the runner's own, run eagerly and given
+        back: the code objects of the kernels and the matrix library's set-up are loaded while the model
+        is, not during the first request (on the 1B shape that is 0.2 s of its first step)."""
+        n = min(128, self.max_positions - 1, (self.cache.min_free_pages() - 1) * self.page_size)
+        if n < 2:
+            return
+        me = ("warm-up", id(self))
+        graphs, self.use_graphs = self.use_graphs, False
+        try:
+            self.step([StepEntry(me, [0] * n, [n - 1])])
+            logits = self.step([StepEntry(me, [0], [0])])
+            K.argmax(logits)
+            torch.cuda.synchronize()
+        finally:
+            self.use_graphs = graphs
+            self.release(me)
 
     def _init_graphs(self, use_graphs: bool) -> None:
         import os
