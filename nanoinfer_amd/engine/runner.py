@@ -146,6 +146,8 @@ class ModelRunner:
     HISTORY_ROWS = 16             # decode steps launched back to back before the host reads their tokens
     GRAPH_MIN_PORTION = 64        # a shorter prompt portion is not worth a recording
     GRAPH_MAX_PORTIONS = 24       # recordings of prompt portions kept (each holds its activations)
+    GRAPH_PORTION_SIGHTS = 2      # a portion's shape is recorded when it comes this many times: recording costs
+                                  # seven runs of the step and gains a few per cent of a run (a lone length never pays)
 
     def __init__(self, model_dir: str, dtype: str = "bfloat16", page_size: int = 16, max_tokens: int = 4096,
                  max_requests: int = 64, device: Optional[torch.device] = None, use_graphs: bool = True,
@@ -197,6 +199,7 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and self.model.graph_safe() and not os.environ.get("NANOINFER_NO_GRAPHS")
         self._recorded: Dict[tuple, _RecordedStep] = {}
         self._unrecordable = set()
+        self._portion_sights: Dict[tuple, int] = {}      # how often a prompt portion's shape has come without a recording
         self._staging = [(None, None)] * 3     # pinned host buffers for the tables of eager steps, and their uploads' events
         self._staging_turn = 0
         self._greedy_of = None                 # (logits returned by the last recorded step, its recording)
@@ -379,9 +382,12 @@ class ModelRunner:
         key = (kind, size, pages, bound, rows)
         if key in self._unrecordable:
             return None
-        if kind == "p" and key not in self._recorded and \
-                sum(1 for k in self._recorded if k[0] == "p") >= self.GRAPH_MAX_PORTIONS:
-            return None
+        if kind == "p" and key not in self._recorded:
+            if sum(1 for k in self._recorded if k[0] == "p") >= self.GRAPH_MAX_PORTIONS:
+                return None
+            seen = self._portion_sights[key] = self._portion_sights.get(key, 0) + 1
+            if seen < self.GRAPH_PORTION_SIGHTS:
+                return None
         return key
 
     def _tables_of(self, entries: List[StepEntry], ctx: StepContext, width: int, tile_sizes):

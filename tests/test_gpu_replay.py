@@ -377,6 +377,8 @@ def test_recorded_prompt_portions_equal_eager_ones(dtype):
     folder = model_folder(name)
     vocab = ALL[name]["vocab_size"]
     recorded = ModelRunner(folder, dtype=dtype, page_size=8, max_tokens=2048, max_requests=4)
+    assert recorded.GRAPH_PORTION_SIGHTS == 2        # by default a shape is recorded when it comes the second time
+    recorded.GRAPH_PORTION_SIGHTS = 1                # here: at once
     eager = ModelRunner(folder, dtype=dtype, page_size=8, max_tokens=2048, max_requests=4, use_graphs=False)
     reqs = {f"q{i}": random_tokens(vocab, n, 700 + i) for i, n in enumerate((300, 214, 129))}
     done = {k: 0 for k in reqs}
@@ -423,6 +425,23 @@ def test_recorded_prompt_portions_equal_eager_ones(dtype):
         rows.sort(key=lambda x: x[0])
         idx = [p for p, _ in rows]
         assert_close(torch.stack([r for _, r in rows]), want[idx], dtype, f"recorded portions, request {rid}")
+
+
+def test_a_portion_shape_is_recorded_when_it_comes_again():
+    """A recording costs several runs of its step: a prompt portion's shape that has come once runs
+    the ordinary way, the second time it is recorded, from then on replayed."""
+    from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
+    folder = model_folder("B")
+    vocab = ALL["B"]["vocab_size"]
+    runner = ModelRunner(folder, dtype="float32", page_size=8, max_tokens=1024, max_requests=4)
+    eager = ModelRunner(folder, dtype="float32", page_size=8, max_tokens=1024, max_requests=4, use_graphs=False)
+    portions = lambda: sum(1 for k in runner._recorded if k[0] == "p")
+    for i, (n, recorded_after) in enumerate(((80, 0), (96, 0), (80, 1), (80, 1), (96, 2), (70, 2))):
+        toks = random_tokens(vocab, n, 900 + i)
+        a = runner.step([StepEntry(i, toks, [n - 1])], end=[i])
+        b = eager.step([StepEntry(i, toks, [n - 1])], end=[i])
+        assert float((a - b).abs().max()) <= 1e-4 * float(b.abs().max()), (i, n)
+        assert portions() == recorded_after, (i, n)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
