@@ -37,6 +37,19 @@ LLAMA_1B = {
     "bos_token_id": 128000, "eos_token_id": 128001,
 }
 FULL_LAYERS = 16
+
+
+def _family(hidden, layers, heads, kv_heads, head_dim, inter, factor, tied):
+    cfg = dict(LLAMA_1B, hidden_size=hidden, num_hidden_layers=layers, num_attention_heads=heads,
+               num_key_value_heads=kv_heads, head_dim=head_dim, intermediate_size=inter, tie_word_embeddings=tied)
+    cfg["rope_scaling"] = dict(LLAMA_1B["rope_scaling"], factor=factor)
+    return cfg
+
+
+# other sizes of the family, for --shape (the default and the result line's contract is the 1B shape)
+SHAPES = {"1b": ("llama-3.2-1b-shape", "Llama 3.2 1B", LLAMA_1B),
+          "3b": ("llama-3.2-3b-shape", "Llama 3.2 3B", _family(3072, 28, 24, 8, 128, 8192, 32.0, True)),
+          "8b": ("llama-3.1-8b-shape", "Llama 3.1 8B", _family(4096, 32, 32, 8, 128, 14336, 8.0, False))}
 PROMPT_LEN = 2048
 CONTEXT_LEN = 4096
 PREFILL_CHUNK = 512       # portions of the prefill measurement, as the benchmark configuration names them
@@ -73,14 +86,15 @@ def prefill_flops(cfg: dict, tokens: int) -> float:
     return linear + attention + 2.0 * V * d
 
 
-def config_record(cfg: dict, layers: int, batch: int, mean_ctx: float, prefill_chunk: int, decode_run: int) -> dict:
+def config_record(cfg: dict, layers: int, batch: int, mean_ctx: float, prefill_chunk: int, decode_run: int,
+                  model: str = "llama-3.2-1b-shape", full_layers: int = FULL_LAYERS) -> dict:
     """Every size of the measured configuration, flat (nothing nested, at most 20 keys)."""
     return {
-        "model": "llama-3.2-1b-shape", "layers": layers, "layers_full_model": FULL_LAYERS,
+        "model": model, "layers": layers, "layers_full_model": full_layers,
         "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
         "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
         "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
-        "tied_embeddings": True, "global_batch": batch, "prompt_len": PROMPT_LEN,
+        "tied_embeddings": bool(cfg["tie_word_embeddings"]), "global_batch": batch, "prompt_len": PROMPT_LEN,
         "seq_len": CONTEXT_LEN, "decode_context_mean": round(mean_ctx, 1), "kv_block_size": BLOCK_SIZE,
         "prefill_chunk": prefill_chunk, "decode_run": decode_run, "parallelism": "single-gpu",
     }
@@ -94,7 +108,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes of the family member to measure (default: 1b)")
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--prefill-chunk", type=int, default=PREFILL_CHUNK, help="tokens of a prompt portion in the prefill measurement")
     ap.add_argument("--decode-run", type=int, default=DECODE_RUN,
                     help="decode steps on one scheduling decision (the engine's max_decode_run; 1: the host reads every token before the next step)")
@@ -121,7 +136,10 @@ def main() -> int:
     from nanoinfer_amd.weights.loader import make_random_model
 
     torch.cuda.set_device(0)
-    cfg = dict(LLAMA_1B)
+    model_name, shown_name, full = SHAPES[args.shape]
+    cfg = dict(full)
+    if args.layers is None:
+        args.layers = full["num_hidden_layers"]
     cfg["num_hidden_layers"] = args.layers
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[args.dtype]
     elem = 2 if args.dtype == "bf16" else 4
@@ -212,7 +230,7 @@ def main() -> int:
     achieved = decode_bytes(cfg, args.batch, mean_ctx, elem) / step_s
     flops = prefill_flops(cfg, PROMPT_LEN)
     result = {
-        "metric": f"decode tok/s at batch {args.batch} (Llama 3.2 1B shape, context {CONTEXT_LEN})",
+        "metric": f"decode tok/s at batch {args.batch} ({shown_name} shape, context {CONTEXT_LEN})",
         "value": round(args.batch / step_s, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -224,7 +242,8 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": args.dtype,
         "data": "synthetic: random weights (seed 0), uniform random token ids",
-        "config": config_record(cfg, args.layers, args.batch, mean_ctx, args.prefill_chunk, args.decode_run),
+        "config": config_record(cfg, args.layers, args.batch, mean_ctx, args.prefill_chunk, args.decode_run,
+                                model_name, full["num_hidden_layers"]),
         "prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(flops / prefill_s / FLOP_PEAK[args.dtype], 4)},
         "prefill_one_portion": {"value": round(PROMPT_LEN / whole_s, 1), "tokens": PROMPT_LEN, "ms": round(whole_s * 1e3, 3),
