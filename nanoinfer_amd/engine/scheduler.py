@@ -227,14 +227,16 @@ class Scheduler:
         """For how many steps in a row ``batch`` can be run again on this one decision (at most
         ``max_decode_run``; 1: only the step that was scheduled).  More than one only if a new
         decision could change nothing but by a request's end: the batch is every running request,
-        one token each whose successor is wanted; nobody waits or was preempted; no request has
-        a repetition penalty, and every one decodes greedily (its next token is then the largest
-        logit, which the runner can feed back without the host) unless ``draws`` says that the
-        sampler can plan a request's draws ahead too; each has that many tokens left to
-        generate; and the pool has pages for all of them.  A request that meets its stop token
-        within the run has run a few tokens too far: they are dropped."""
+        one token each whose successor is wanted; nobody was preempted; no request has a repetition
+        penalty, and every one decodes greedily (its next token is then the largest logit, which
+        the runner can feed back without the host) unless ``draws`` says that the sampler can plan
+        a request's draws ahead too; each has that many tokens left to generate; and the pool has
+        pages for all of them.  Requests may wait meanwhile: this decision has just refused the
+        first of them for want of a place or of pages, and neither comes back before a request
+        ends.  A request that meets its stop token within the run has run a few tokens too far:
+        they are dropped, and whoever waits for its place gets it that many steps later."""
         steps = self.config.max_decode_run
-        if steps <= 1 or not batch.items or batch.preempted or self.waiting or len(batch.items) != len(self.running):
+        if steps <= 1 or not batch.items or batch.preempted or len(batch.items) != len(self.running):
             return 1
         for item in batch.items:
             req = item.request

@@ -291,12 +291,14 @@ def test_a_stop_token_inside_a_run_ends_the_request_there():
 
 def test_what_keeps_a_decode_step_single():
     greedy = SamplingParams.greedy()
-    # somebody waits (max_sequences 1 keeps the second request out)
+    # somebody who waits for a place keeps nothing single: the decision has just refused it, and nothing changes
+    # before a request ends (max_sequences 1 keeps the second request out until the first has gone)
     eng, runner = make_run_engine(max_decode_run=8, max_sequences=1, num_pages=32)
-    eng.add_request([1, 2], max_new_tokens=4, params=greedy)
-    eng.add_request([3, 4], max_new_tokens=4, params=greedy)
+    a = eng.add_request([1, 2], max_new_tokens=4, params=greedy)
+    b = eng.add_request([3, 4], max_new_tokens=4, params=greedy)
     eng.run()
-    assert runner.runs == [3]                       # only the second request, once the first has gone, decodes in a run
+    assert runner.runs == [3, 3]
+    assert eng.get_request(a).generated == [3, 4, 5, 6] and eng.get_request(b).generated == [5, 6, 7, 8]
     # a request that draws, or that has a repetition penalty
     for params in (SamplingParams(temperature=0.7, seed=1), SamplingParams(temperature=0.0, repetition_penalty=1.3)):
         eng, runner = make_run_engine(max_decode_run=8, num_pages=32)
