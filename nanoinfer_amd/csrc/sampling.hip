@@ -100,7 +100,7 @@ __global__ void argmax_final_kernel(const float* __restrict__ part_val, const in
 struct SampleArgs {
     const float* logits; float* work;
     const float* temperature; const int32_t* top_k; const float* top_p; const float* penalty;
-    const int32_t* pen_ids; const int32_t* pen_off; const float* uniform; int32_t* out;
+    int32_t* pen_ids; const int32_t* pen_off; int32_t* pen_count; const float* uniform; int32_t* out;
     float* part_max; int32_t* part_arg; float* part_z; float* part_mass; int32_t* part_last;
     uint32_t* hist; uint32_t* state;
     int R, V, P;
@@ -178,8 +178,10 @@ __global__ __launch_bounds__(SP_THREADS) void sample_prepare_kernel(SampleArgs a
     s_hist[tid] = 0;
     __syncthreads();
     if (pen != 1.0f) {
-        for (int j = a.pen_off[r] + tid; j < a.pen_off[r + 1]; j += SP_THREADS) {
-            const int id = a.pen_ids[j];
+        const int first = a.pen_off[r];
+        const int n_pen = a.pen_count ? a.pen_count[r] : a.pen_off[r + 1] - first;
+        for (int j = tid; j < n_pen; j += SP_THREADS) {
+            const int id = a.pen_ids[first + j];
             if (id >= sl.lo && id < sl.hi) {
                 float l = lrow[id];
                 l = l > 0.f ? l / pen : l * pen;
@@ -370,8 +372,17 @@ __global__ __launch_bounds__(SP_THREADS) void sample_draw_kernel(SampleArgs a) {
     int best = 0x7fffffff;
     for (int p = 0; p < a.P; ++p) better(best_v, best, a.part_max[r * a.P + p], a.part_arg[r * a.P + p]);
     if (best == 0x7fffffff) best = 0;        // a row of NaN or -inf: the first token
+    // with pen_count the chosen token joins the row's penalised tokens: the next draw of a run sees it
+    auto choose = [&](int token) {
+        a.out[r] = token;
+        if (a.pen_count) {
+            const int n = a.pen_count[r];
+            a.pen_ids[a.pen_off[r] + n] = token;
+            a.pen_count[r] = n + 1;
+        }
+    };
     if (!row_samples(a, r)) {
-        if (tid == 0) a.out[r] = best;
+        if (tid == 0) choose(best);
         return;
     }
     const float M = best_v;
@@ -432,7 +443,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_draw_kernel(SampleArgs a) {
     if (tid == 0) {
         int pick = s_pick;
         if (pick == 0x7fffffff && part >= 0) pick = a.part_last[r * a.P + part] >= 0 ? a.part_last[r * a.P + part] : 0x7fffffff;
-        a.out[r] = pick != 0x7fffffff ? pick : (last >= 0 ? last : best);
+        choose(pick != 0x7fffffff ? pick : (last >= 0 ? last : best));
     }
 }
 
@@ -458,17 +469,20 @@ NI_EXPORT int ni_sample_parts(int R, int V) {
 // Scratch (see SampleArgs): work float [R, V]; parts float [R, P, 5] (maximum, its index, mass before top-p,
 // mass kept, last kept index: five arrays of R * P words one after another); hist uint32 [2, R, P, 256];
 // state uint32 [R, 16].  P must be ni_sample_parts(R, V).  uses_top_k / uses_top_p: 0 if no row asks for
-// it (their launches are skipped then).
+// it (their launches are skipped then).  Row r's penalised tokens are pen_ids[pen_off[r] .. pen_off[r + 1]),
+// or with pen_count (int32 [R]) the first pen_count[r] of them; then the chosen token is appended and the
+// count raised, for the next draw of the same rows (the caller leaves room).
 NI_EXPORT int ni_sample(const void* logits, void* work, const void* temperature, const void* top_k, const void* top_p,
-                        const void* penalty, const void* pen_ids, const void* pen_off, const void* uniform, void* out,
-                        void* parts, void* hist, void* state, int R, int V, int P, int uses_top_k, int uses_top_p,
-                        hipStream_t stream) {
+                        const void* penalty, void* pen_ids, const void* pen_off, void* pen_count, const void* uniform,
+                        void* out, void* parts, void* hist, void* state, int R, int V, int P, int uses_top_k,
+                        int uses_top_p, hipStream_t stream) {
     if (R <= 0) return 0;
     if (V < 1 || P != ni_sample_parts(R, V) || !parts || !hist || !state) return -1;
     SampleArgs a;
     a.logits = (const float*)logits; a.work = (float*)work;
     a.temperature = (const float*)temperature; a.top_k = (const int32_t*)top_k; a.top_p = (const float*)top_p;
-    a.penalty = (const float*)penalty; a.pen_ids = (const int32_t*)pen_ids; a.pen_off = (const int32_t*)pen_off;
+    a.penalty = (const float*)penalty; a.pen_ids = (int32_t*)pen_ids; a.pen_off = (const int32_t*)pen_off;
+    a.pen_count = (int32_t*)pen_count;
     a.uniform = (const float*)uniform; a.out = (int32_t*)out;
     float* pf = (float*)parts;
     const size_t n = static_cast<size_t>(R) * P;

@@ -116,10 +116,10 @@ class Engine:
         plan draws); the scheduler then books the steps one by one, and a request that stops on the
         way is finished there and its later tokens dropped."""
         requests = [item.request for item in batch.items]
-        if all(r.params.use_greedy() for r in requests):
+        if all(r.params.use_greedy() and not r.params.use_repetition_penalty() for r in requests):
             chosen = self.runner.decode_run(entries, run)
         else:
-            plan = self.sampler.plan([r.params for r in requests], [len(r.generated) for r in requests], run)
+            plan = self.sampler.plan([r.params for r in requests], [r.generated for r in requests], run)
             chosen = self.runner.decode_run(entries, run, pick=plan.launch)
         column = {item.request.request_id: b for b, item in enumerate(batch.items)}
         finished: List[Request] = []

@@ -227,10 +227,10 @@ class Scheduler:
         """For how many steps in a row ``batch`` can be run again on this one decision (at most
         ``max_decode_run``; 1: only the step that was scheduled).  More than one only if a new
         decision could change nothing but by a request's end: the batch is every running request,
-        one token each whose successor is wanted; nobody was preempted; no request has a repetition
-        penalty, and every one decodes greedily (its next token is then the largest logit, which
+        one token each whose successor is wanted; nobody was preempted; every request decodes
+        greedily without a repetition penalty (its next token is then the largest logit, which
         the runner can feed back without the host) unless ``draws`` says that the sampler can plan
-        a request's draws ahead too; each has that many tokens left to generate; and the pool has
+        a request's choices ahead; each has that many tokens left to generate; and the pool has
         pages for all of them.  Requests may wait meanwhile: this decision has just refused the
         first of them for want of a place or of pages, and neither comes back before a request
         ends.  A request that meets its stop token within the run has run a few tokens too far:
@@ -242,7 +242,7 @@ class Scheduler:
             req = item.request
             if item.count != 1 or not item.samples:
                 return 1
-            if req.params.use_repetition_penalty() or not (draws or req.params.use_greedy()):
+            if not draws and (req.params.use_repetition_penalty() or not req.params.use_greedy()):
                 return 1
             steps = min(steps, req.max_new_tokens - len(req.generated))
         while steps > 1 and not self.cache.can_reserve_all(

@@ -462,12 +462,16 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
 
 def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
            top_p: torch.Tensor, penalty: torch.Tensor, pen_ids: torch.Tensor, pen_off: torch.Tensor,
-           uniform: torch.Tensor, out: torch.Tensor, uses_top_k: bool = True, uses_top_p: bool = True) -> torch.Tensor:
+           uniform: torch.Tensor, out: torch.Tensor, uses_top_k: bool = True, uses_top_p: bool = True,
+           pen_count: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One token per row of ``logits`` [R, V]: repetition penalty on the tokens ``pen_ids[pen_off[r]:
     pen_off[r+1]]``, temperature, top-k, softmax, top-p, and the token at which the cumulative mass
     in vocabulary order reaches ``uniform[r]`` times the kept mass; rows with temperature <= 0 take
     the largest (penalised) logit.  ``work`` [R, V] is scratch.  ``uses_top_k`` / ``uses_top_p``
-    may be False when no row asks for it: their launches are then left out."""
+    may be False when no row asks for it: their launches are then left out.  With ``pen_count``
+    (int32 [R]) row r's penalised tokens are the first ``pen_count[r]`` from ``pen_off[r]`` on, and
+    the chosen token is appended to them and counted, for the next draw of the same rows: the
+    caller leaves room behind every row's tokens."""
     R, V = logits.shape
     _gpu(logits, "logits", torch.float32)
     _gpu(work, "work", torch.float32, (R, V))
@@ -477,13 +481,15 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
         _gpu(t, name, dt, (R,))
     _gpu(pen_off, "pen_off", torch.int32, (R + 1,))
     _gpu(pen_ids, "pen_ids", torch.int32)
+    if pen_count is not None:
+        _gpu(pen_count, "pen_count", torch.int32, (R,))
     lib = sampling_lib()
     P = int(lib.ni_sample_parts(R, V))
     # per-part results, two sets of per-part histograms, the decisions of the levels
     scratch = torch.empty(R * P * 5 + 2 * R * P * 256 + R * 16, dtype=torch.int32, device=logits.device)
     parts, hist, state = scratch[: R * P * 5], scratch[R * P * 5: R * P * 5 + 2 * R * P * 256], scratch[-R * 16:]
     _check(lib.ni_sample(_ptr(logits), _ptr(work), _ptr(temperature), _ptr(top_k), _ptr(top_p),
-                         _ptr(penalty), _ptr(pen_ids), _ptr(pen_off), _ptr(uniform), _ptr(out),
+                         _ptr(penalty), _ptr(pen_ids), _ptr(pen_off), _ptr(pen_count), _ptr(uniform), _ptr(out),
                          _ptr(parts), _ptr(hist), _ptr(state), R, V, P, int(bool(uses_top_k)), int(bool(uses_top_p)),
                          _stream()), "sample")
     return out

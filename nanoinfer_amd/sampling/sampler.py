@@ -77,36 +77,43 @@ class Sampler:
                  uses_top_p=any(p.use_top_p() and p.temperature > 0 for p in params))
         return out.tolist()
 
-    def plan(self, params: Sequence[SamplingParams], counters: Sequence[int], steps: int) -> "SamplingPlan":
+    def plan(self, params: Sequence[SamplingParams], generated: Sequence[Sequence[int]], steps: int) -> "SamplingPlan":
         """The draws of ``steps`` successive tokens for the same rows, prepared in one upload: the
         uniform numbers of a seeded request do not depend on the tokens drawn before (they are keyed
         by the seed and the count of generated tokens), so a caller can launch step after step
-        without reading a token in between.  No row may have a repetition penalty (that needs the
-        tokens)."""
-        if any(p.use_repetition_penalty() for p in params):
-            raise ValueError("a repetition penalty needs the generated tokens: it cannot be planned ahead")
-        return SamplingPlan(self.device, params, counters, steps)
+        without reading a token in between.  The tokens of a row with a repetition penalty are kept
+        on the device, where every draw adds the token it chose."""
+        return SamplingPlan(self.device, params, generated, steps)
 
 
 class SamplingPlan:
     """Options of R rows and their uniform numbers for ``steps`` draws, on the device."""
 
-    def __init__(self, device, params: Sequence[SamplingParams], counters: Sequence[int], steps: int):
+    def __init__(self, device, params: Sequence[SamplingParams], generated: Sequence[Sequence[int]], steps: int):
         R = len(params)
         floats = np.array([[p.temperature for p in params],
                            [p.top_p if p.use_top_p() else 1.0 for p in params],
-                           [1.0] * R], dtype=np.float32)
-        uniform = np.array([[uniform_from_counter(max(p.seed, 0), c + i) for p, c in zip(params, counters)]
+                           [p.repetition_penalty for p in params]], dtype=np.float32)
+        uniform = np.array([[uniform_from_counter(max(p.seed, 0), len(g) + i) for p, g in zip(params, generated)]
                             for i in range(steps)], dtype=np.float32)
-        ints = np.array([p.top_k if p.use_top_k() else 0 for p in params] + [0] * (R + 2), dtype=np.int32)
-        packed = torch.from_numpy(np.concatenate([floats.reshape(-1).view(np.int32), ints,
-                                                  uniform.reshape(-1).view(np.int32)])).to(device)
-        as_float = packed[: 3 * R].view(torch.float32)
+        # penalised tokens: what a row has generated, and room for the tokens of the run
+        pen_ids, pen_off, pen_count = [], [0], []
+        for p, g in zip(params, generated):
+            mine = sorted(set(int(t) for t in g)) if p.use_repetition_penalty() else []
+            pen_count.append(len(mine))
+            pen_ids.extend(mine + [0] * steps)
+            pen_off.append(len(pen_ids))
+        ints = np.array([p.top_k if p.use_top_k() else 0 for p in params] + pen_off + pen_count + pen_ids, dtype=np.int32)
+        packed = torch.from_numpy(np.concatenate([floats.reshape(-1).view(np.int32), uniform.reshape(-1).view(np.int32),
+                                                  ints])).to(device)
+        as_float = packed[: (3 + steps) * R].view(torch.float32)
         self.temperature, self.top_p, self.penalty = (as_float[i * R:(i + 1) * R] for i in range(3))
-        self.top_k = packed[3 * R: 4 * R]
-        self.pen_off = packed[4 * R: 5 * R + 1]
-        self.pen_ids = packed[5 * R + 1: 5 * R + 2]
-        self.uniform = packed[5 * R + 2:].view(torch.float32).view(steps, R)
+        self.uniform = as_float[3 * R:].view(steps, R)
+        ints_dev = packed[(3 + steps) * R:]
+        self.top_k = ints_dev[:R]
+        self.pen_off = ints_dev[R: 2 * R + 1]
+        self.pen_count = ints_dev[2 * R + 1: 3 * R + 1]
+        self.pen_ids = ints_dev[3 * R + 1:]
         self.uses_top_k = any(p.use_top_k() and p.temperature > 0 for p in params)
         self.uses_top_p = any(p.use_top_p() and p.temperature > 0 for p in params)
         self.steps = steps
@@ -114,4 +121,5 @@ class SamplingPlan:
     def launch(self, i: int, logits: torch.Tensor, out: torch.Tensor) -> None:
         """Launch draw ``i`` over ``logits`` [R, vocab] into ``out`` (int32 [R], device); nothing waits."""
         K.sample(logits, torch.empty_like(logits), self.temperature, self.top_k, self.top_p, self.penalty,
-                 self.pen_ids, self.pen_off, self.uniform[i], out, uses_top_k=self.uses_top_k, uses_top_p=self.uses_top_p)
+                 self.pen_ids, self.pen_off, self.uniform[i], out, uses_top_k=self.uses_top_k, uses_top_p=self.uses_top_p,
+                 pen_count=self.pen_count)

@@ -70,15 +70,15 @@ def test_decode_runs_do_not_change_the_tokens(dtype):
 
 
 def test_decode_runs_with_planned_draws_give_the_tokens_of_single_steps():
-    """Requests that draw (temperature, top-k, top-p; no repetition penalty) decode in runs too: the
-    uniform numbers of their draws are known ahead, and every step's draw is launched behind the
-    step.  Float32, so that the two ways see the same logits to the last bit but for the attention's
-    key runs; a request with a repetition penalty keeps every step single."""
+    """Requests that draw (temperature, top-k, top-p, repetition penalty) decode in runs too: the
+    uniform numbers of their draws are known ahead, every step's draw is launched behind the step,
+    and the tokens that a penalty looks at grow on the device.  Float32, so that the two ways see
+    the same logits to the last bit but for the attention's key runs."""
     from nanoinfer_amd.sampling.params import SamplingParams
     folder = model_folder("B")
     prompts = [list(random_tokens(1000, n, 60 + n)) for n in (9, 40, 23, 3)]
     options = [SamplingParams(temperature=0.8, seed=5), SamplingParams(temperature=1.3, top_k=40, top_p=0.9, seed=6),
-               SamplingParams.greedy(), SamplingParams(temperature=0.6, top_p=0.5, seed=7)]
+               SamplingParams.greedy(), SamplingParams(temperature=0.9, top_p=0.8, repetition_penalty=1.6, seed=7)]
     outs, runs = [], []
     for run in (1, 8):
         eng = engine(folder, dtype="float32", block_size=8, num_cache_blocks=24, max_sequences=3, max_decode_run=run)
@@ -93,11 +93,15 @@ def test_decode_runs_with_planned_draws_give_the_tokens_of_single_steps():
     assert [len(t) for t in outs[1]] == [30, 11, 50, 17]
     assert not runs[0] and any(steps == 8 and draws for steps, draws in runs[1])
     assert len({tuple(t) for t in outs[1]}) == 4 and outs[1][2] != outs[1][0]
-    # with a repetition penalty every decision is taken step by step
-    eng = engine(folder, dtype="float32", block_size=8, num_cache_blocks=24, max_decode_run=8)
-    eng.runner.decode_run = None
-    eng.add_request(prompts[0], 6, SamplingParams(temperature=0.8, repetition_penalty=1.2, seed=5))
-    eng.run()
+    # the penalty changed what was drawn, and a greedy request with a penalty runs through the same plan
+    other = engine(folder, dtype="float32", block_size=8, num_cache_blocks=24, max_decode_run=8)
+    plain = other.generate([prompts[3]], 17, SamplingParams(temperature=0.9, top_p=0.8, seed=7))[0].tokens
+    assert plain != outs[1][3]
+    greedy = []
+    for run in (1, 8):
+        eng = engine(folder, dtype="float32", block_size=8, num_cache_blocks=24, max_decode_run=run)
+        greedy.append(eng.generate([prompts[0]], 24, SamplingParams(temperature=0.0, repetition_penalty=1.5))[0].tokens)
+    assert greedy[0] == greedy[1] and greedy[0] != outs[1][2][:24]
 
 
 def test_stop_token_from_the_configuration():

@@ -472,6 +472,45 @@ def test_sampling_closed_forms(K):
     assert again == got
 
 
+def test_sampling_keeps_the_penalised_tokens_of_a_run(K):
+    """With a count of its own on the device, a row's list of penalised tokens takes every token the
+    row is given, and the next call over the same rows penalises it: three calls in a row equal three
+    calls whose lists the host has extended."""
+    V, R = 3000, 3
+    g = torch.Generator().manual_seed(11)
+    logits = [torch.randn(R, V, generator=g) * 2 for _ in range(3)]
+    for lg in logits:
+        lg[0] *= 0.05
+        lg[0, 7] = 30.0            # row 0 (greedy, penalty 5): 7 wins once, then its penalised logit 6 still does,
+        lg[0, 9] = 6.5             # unless 9 has not been chosen yet
+    temperature, top_k, top_p, penalty = [0.0, 0.9, 1.0], [0, 20, 0], [1.0, 1.0, 0.7], [5.0, 1.4, 1.0]
+    us = [[0.5, 0.3, 0.9], [0.5, 0.6, 0.2], [0.5, 0.1, 0.4]]
+    start = [[], [5, 6], [1]]
+    want, lists = [], [list(x) for x in start]
+    for i in range(3):
+        got = sample_rows(K, logits[i], temperature, top_k, top_p, penalty, lists, us[i])
+        want.append(got)
+        for r in range(R):
+            lists[r].append(got[r])
+    assert [w[0] for w in want] == [7, 9, 7]
+    f32, i32 = torch.float32, torch.int32
+    pen_ids, pen_off = [], [0]
+    for x in start:
+        pen_ids += sorted(set(x)) + [0] * 3
+        pen_off.append(len(pen_ids))
+    ids, off = dev(torch.tensor(pen_ids, dtype=i32)), dev(torch.tensor(pen_off, dtype=i32))
+    count = dev(torch.tensor([len(set(x)) for x in start], dtype=i32))
+    opts = [dev(torch.tensor(temperature, dtype=f32)), dev(torch.tensor(top_k, dtype=i32)), dev(torch.tensor(top_p, dtype=f32)),
+            dev(torch.tensor(penalty, dtype=f32))]
+    for i in range(3):
+        out = torch.empty(R, dtype=i32, device="cuda")
+        K.sample(dev(logits[i]), torch.empty(R, V, device="cuda"), *opts, ids, off, dev(torch.tensor(us[i], dtype=f32)), out,
+                 pen_count=count)
+        assert out.tolist() == want[i], i
+    assert count.tolist() == [len(set(x)) + 3 for x in start]
+    assert ids.tolist()[0:3] == [w[0] for w in want]
+
+
 # ------------------------------------------------------------------ skinny matrix product
 
 def _skinny_case(Kmod, dtype, M, N, Kd):

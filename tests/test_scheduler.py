@@ -305,22 +305,21 @@ def test_what_keeps_a_decode_step_single():
         eng.add_request([1, 2], max_new_tokens=6, params=params)
         eng.run()
         assert runner.runs == []
-    # unless the sampler can plan the draws ahead (never with a repetition penalty: that needs the tokens)
+    # unless the sampler can plan a request's choices ahead (it then keeps the tokens of a penalty itself)
     class PlanningSampler(ArgmaxSampler):
         def __init__(self):
             self.plans = []
 
-        def plan(self, params, counters, steps):
-            self.plans.append((list(counters), steps))
-            assert not any(p.use_repetition_penalty() for p in params)
+        def plan(self, params, generated, steps):
+            self.plans.append(([list(g) for g in generated], steps))
             return types.SimpleNamespace(launch=lambda i, logits, out: out.copy_(logits.argmax(dim=-1)))
-    for params, runs in ((SamplingParams(temperature=0.7, seed=1), [5]), (SamplingParams(temperature=0.7, repetition_penalty=1.3, seed=1), [])):
+    for params in (SamplingParams(temperature=0.7, seed=1), SamplingParams(temperature=0.0, repetition_penalty=1.3)):
         eng, runner = make_run_engine(max_decode_run=8, num_pages=32)
         eng.sampler = PlanningSampler()
         r = eng.add_request([1, 2], max_new_tokens=6, params=params)
         eng.run()
-        assert runner.runs == runs and eng.get_request(r).generated == [3, 4, 5, 6, 7, 8]
-        assert eng.sampler.plans == ([([1], 5)] if runs else [])
+        assert runner.runs == [5] and eng.get_request(r).generated == [3, 4, 5, 6, 7, 8]
+        assert eng.sampler.plans == [([[3]], 5)]
     # a prompt portion in the batch
     eng, runner = make_run_engine(max_decode_run=8, num_pages=32, max_num_batched_tokens=4)
     eng.add_request([1, 2], max_new_tokens=6, params=greedy)
