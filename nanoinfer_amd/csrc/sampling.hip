@@ -2,10 +2,10 @@
 // repetition penalty -> temperature -> top-k -> softmax -> top-p -> renormalise -> inverse CDF
 // (order of src/sampler/configurable_sampler.cpp:93-120 of the reference).
 //
-// Thresholds are exact selections, not the
-// 16-step bisections of src/op/kernels/cuda/sampling_kernel.cu:202-296: a radix descent over
-// the order-preserving integer image of a float finds the k-th largest logit (counts) and the
-// smallest logit whose upper set still holds the mass top_p (sums).  Equal logits at a
+// Thresholds are exact selections, not the 16-step bisections of
+// src/op/kernels/cuda/sampling_kernel.cu:202-296: a radix descent over the order-preserving
+// integer image of a float finds the k-th largest logit (counts) and the smallest logit whose
+// upper set still holds the mass top_p (sums).  Equal logits at a
 // threshold are kept together.  The draw walks the kept tokens in vocabulary order and takes
 // the first whose cumulative mass reaches u * total (src/op/kernels/cuda/sampling_kernel.cu:330-398);
 // u in (0, 1] comes from the host, which derives it from (seed, request, step).
