@@ -453,6 +453,29 @@ def test_sampling_matches_plain(K, V):
             assert probs[got[r]] > 0 and abs(float(cum[lo]) - c["u"]) < 1e-5, (r, c, got[r], want)
 
 
+def test_sampling_at_the_family_vocabulary(K):
+    # eight rows of 128,256 logits: 32 workgroups share a row
+    V = 128256
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(8, V, generator=g) * 3
+    opts = [(0.8, 0, 1.0, 1.0), (1.0, 50, 1.0, 1.0), (0.7, 0, 0.9, 1.0), (1.2, 200, 0.5, 1.3), (0.0, 0, 1.0, 1.0),
+            (0.0, 0, 1.0, 2.0), (1.5, 1, 1.0, 1.0), (0.9, 1000, 0.99, 1.0)]
+    generated = [[], [], [5], [int(logits[3].argmax()), 7, 7], [], [int(logits[5].argmax())], [], []]
+    us = [0.37, 0.81, 0.05, 0.66, 0.5, 0.5, 0.93, 0.999]
+    got = sample_rows(K, logits, [o[0] for o in opts], [o[1] for o in opts], [o[2] for o in opts], [o[3] for o in opts], generated, us)
+    for r, (t, k, p, pen) in enumerate(opts):
+        want = plain_pick(logits[r], t, k, p, pen, generated[r], us[r])
+        if got[r] != want:
+            l = logits[r].double()
+            if pen != 1.0:
+                l = P.repetition_penalty(l, generated[r], pen)
+            probs = P.filtered_distribution(P.temperature_scale(l, t), k, p)
+            cum = torch.cumsum(probs, 0)
+            lo = min(got[r], want)
+            assert t > 0 and probs[got[r]] > 0 and abs(float(cum[lo]) - us[r]) < 1e-5, (r, got[r], want)
+    assert got[5] != int(logits[5].argmax())         # the penalised maximum lost
+
+
 def test_sampling_closed_forms(K):
     V = 10
     logits = torch.tensor([[2.0, -1.0, 3.0, 0.0, -2.0, 1.0, 0.5, -0.5, 1.5, -1.5]]).repeat(5, 1)
