@@ -125,8 +125,8 @@ def main(argv: List[str] = None) -> int:
         print(f"Prefill:  {prefill_tokens} tokens, {prefill_s * 1e3:.2f} ms ({prefill_tokens / prefill_s:.1f} tok/s)")
     if decode_s > 0:
         print(f"Decode:   {decode_tokens} tokens, {decode_s * 1e3:.2f} ms ({decode_tokens / decode_s:.1f} tok/s)")
-    print(f"Total:    {prefill_tokens + decode_tokens} tokens run, {generated} generated, {steps} steps, "
-          f"{elapsed * 1e3:.2f} ms")
+    print(f"Total:    {prefill_tokens + decode_tokens} tokens run, {generated} generated, {engine.num_steps} steps "
+          f"on {steps} scheduling decisions, {elapsed * 1e3:.2f} ms")
     st = engine.scheduler.stats()
     print(f"Scheduler - Finished: {st['num_finished']}  Running: {st['num_running']}  Waiting: {st['num_waiting']}  "
           f"Preemptions: {st['num_preemptions']}")
