@@ -616,7 +616,7 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));    // 16 bytes tha
 template <typename T, typename TOUT, int MB, int NT, int EPI>
 __global__ __launch_bounds__(GV_THREADS) void skinny_rows_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                                  TOUT* __restrict__ y, int M, int N, int K, int I,
-                                                                 RopeArgs rope) {
+                                                                 RopeArgs rope, int splits) {
     constexpr int EL = Piece<T>::ELEMS;
     constexpr int CH = 4 * EL;
     constexpr int WV = GV_WAVES;
@@ -630,6 +630,10 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_rows_kernel(const T* __rest
     const int r = lane % 16, kg = lane / 16;
     const int wg = blockIdx.x;
     const int pieces = (K + CH - 1) / CH;
+    // with splits > 1 workgroup (x, y) multiplies the y-th share of the pieces and stores its sums in the y-th [M, N] of y
+    const int share = (pieces + splits - 1) / splits;
+    const int p_begin = min(pieces, static_cast<int>(blockIdx.y) * share), p_end = min(pieces, p_begin + share);
+    y += static_cast<size_t>(blockIdx.y) * M * N;
     unsigned char* slab = lds + wave * SLAB;
 
     const T* wrow[NT];      // first byte of this lane in piece 0 of each tile
@@ -652,7 +656,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_rows_kernel(const T* __rest
 
     // pieces past the end of a row are read from its last piece and not multiplied: no load is under a branch
     auto load_w = [&](int c, Piece<T> (&wa)[NT]) {
-        const int piece = min(c, pieces - 1);
+        const int piece = min(c, p_end - 1);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) wa[nt].load(wrow[nt] + static_cast<size_t>(piece) * (WAVE * EL));
     };
@@ -662,7 +666,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_rows_kernel(const T* __rest
     // W is zero there, but zero times what lies behind x need not be)
     constexpr int PER16 = 16 / static_cast<int>(sizeof(T));
     auto load_x = [&](int c, u32x4_t (&xr)[XL]) {
-        const int k = min(c, pieces - 1) * CH + (lane % 8) * PER16;
+        const int k = min(c, p_end - 1) * CH + (lane % 8) * PER16;
 #pragma unroll
         for (int i = 0; i < XL; ++i) {
             const int row = min(i * 8 + lane / 8, M - 1);
@@ -693,16 +697,16 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_rows_kernel(const T* __rest
 
     Piece<T> wa_a[NT], wa_b[NT];
     u32x4_t xr_a[XL], xr_b[XL];
-    load_w(wave, wa_a);
-    load_x(wave, xr_a);
-    for (int c = wave; c < pieces; c += 2 * WV) {
+    load_w(p_begin + wave, wa_a);
+    load_x(p_begin + wave, xr_a);
+    for (int c = p_begin + wave; c < p_end; c += 2 * WV) {
         stage(xr_a);
         wave_sync();
         load_w(c + WV, wa_b);
         load_x(c + WV, xr_b);
         multiply(wa_a);
         wave_sync();                       // the slab has been read: it may be written again
-        if (c + WV < pieces) {
+        if (c + WV < p_end) {
             stage(xr_b);
             wave_sync();
             load_w(c + 2 * WV, wa_a);
@@ -803,14 +807,14 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
 // fragments of partial sums a wavefront may hold.
 template <typename T, typename TOUT, int MB, int EPI>
 static int launch_rows(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream,
-                       RopeArgs rope = RopeArgs{}) {
+                       RopeArgs rope = RopeArgs{}, int splits = 1) {
     const int out_width = (EPI == EPI_SWIGLU) ? I : N;
     const int tiles = (out_width + 15) / 16;
     auto run = [&](auto nt_tag) {
         constexpr int NTc = decltype(nt_tag)::value;
         constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
         const int grid = (tiles + NOUT - 1) / NOUT;
-        skinny_rows_kernel<T, TOUT, MB, NTc, EPI><<<grid, GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope);
+        skinny_rows_kernel<T, TOUT, MB, NTc, EPI><<<dim3(grid, splits), GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, splits);
     };
     if constexpr (EPI == EPI_SWIGLU || EPI == EPI_ROPE) {
         run(std::integral_constant<int, 2>{});
@@ -885,6 +889,16 @@ NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N
     if (epilogue == 2) return launch_mb<bf16_t, bf16_t, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
     if (epilogue == 1) return launch_mb<bf16_t, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
     return launch_mb<bf16_t, bf16_t, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
+}
+
+// 17 to 64 rows of bfloat16, re-tiled W: the K range cut into `splits` shares of whole 128-byte pieces, the sums of
+// share s stored as float32 in y[s] ([splits, M, N]); whoever reads y adds the shares in their order.  A matrix of
+// few tiles then fills the chip: 128 tiles in two or four shares are 256 workgroups.
+NI_EXPORT int ni_skinny_gemm_ksplit(const void* x, const void* W, void* y, int M, int N, int K, int tiles_per_group, int splits,
+                                    hipStream_t stream) {
+    if (M <= 16 || M > 64 || N <= 0 || K % 16 != 0 || splits < 1 || splits > 16) return -1;
+    if (M <= 32) return launch_rows<bf16_t, float, 2, EPI_STORE>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, splits);
+    return launch_rows<bf16_t, float, 4, EPI_STORE>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, splits);
 }
 
 // Whether the normalising prologue takes M rows of K elements of this type (1) or not (0).  Every

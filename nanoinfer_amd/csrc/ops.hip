@@ -31,7 +31,7 @@ __global__ void embedding_kernel(const int32_t* __restrict__ ids, const T* __res
 // Rows of up to NV * blockDim elements are held in registers: every load of the row is issued
 // before anything waits, and the row is read from memory once.
 template <typename TP, typename TO, int NV>
-__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TP* __restrict__ pending,
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TP* __restrict__ pending, int addends, size_t addend_stride,
                                    const float* __restrict__ w, TO* __restrict__ out,
                                    const int32_t* __restrict__ rows, int d, float eps) {
     __shared__ float scratch[16];
@@ -47,10 +47,21 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TP* __restrict__
         wv[j] = i < d ? w[i] : 0.f;
     }
     if (prow) {
+        // several addends (the shares of a product whose K range was cut) are added in their order;
+        // four at a time are asked for before any is added, so that their loads overlap
+        for (int a0 = 0; a0 < addends; a0 += 4) {
+            float t[4][NV];
 #pragma unroll
-        for (int j = 0; j < NV; ++j) {
-            const int i = threadIdx.x + j * blockDim.x;
-            if (i < d) v[j] += ld(prow + i);
+            for (int b = 0; b < 4; ++b)
+#pragma unroll
+                for (int j = 0; j < NV; ++j) {
+                    const int i = threadIdx.x + j * blockDim.x;
+                    t[b][j] = (a0 + b < addends && i < d) ? ld(prow + (a0 + b) * addend_stride + i) : 0.f;
+                }
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+#pragma unroll
+                for (int j = 0; j < NV; ++j) v[j] += t[b][j];
         }
     }
     float ss = 0.f;
@@ -75,7 +86,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TP* __restrict__
 
 // Rows of any width: two passes over memory.
 template <typename TP, typename TO>
-__global__ void add_rmsnorm_wide_kernel(float* __restrict__ h, const TP* __restrict__ pending,
+__global__ void add_rmsnorm_wide_kernel(float* __restrict__ h, const TP* __restrict__ pending, int addends, size_t addend_stride,
                                         const float* __restrict__ w, TO* __restrict__ out,
                                         const int32_t* __restrict__ rows, int d, float eps) {
     __shared__ float scratch[16];
@@ -84,9 +95,14 @@ __global__ void add_rmsnorm_wide_kernel(float* __restrict__ h, const TP* __restr
     float* hrow = h + src * d;
     const TP* prow = pending ? pending + src * d : nullptr;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    auto sum_at = [&](int i) {
         float v = hrow[i];
-        if (prow) v += ld(prow + i);
+        if (prow)
+            for (int a = 0; a < addends; ++a) v += ld(prow + a * addend_stride + i);
+        return v;
+    };
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        const float v = sum_at(i);
         if (!rows && prow) hrow[i] = v;
         ss += v * v;
     }
@@ -94,8 +110,7 @@ __global__ void add_rmsnorm_wide_kernel(float* __restrict__ h, const TP* __restr
     const float inv = 1.0f / sqrtf(ss / static_cast<float>(d) + eps);
     TO* orow = out + static_cast<size_t>(r) * d;
     for (int i = threadIdx.x; i < d; i += blockDim.x) {
-        float v = hrow[i];
-        if (rows && prow) v += ld(prow + i);
+        const float v = (rows && prow) ? sum_at(i) : hrow[i];
         st(orow + i, (v * inv) * w[i]);
     }
 }
@@ -237,26 +252,33 @@ NI_EXPORT int ni_embedding(const void* ids, const void* table, void* out, int T,
 }
 
 template <typename TP, typename TO>
-static void launch_add_rmsnorm(float* h, const TP* pending, const float* w, TO* out, const int32_t* rows, int n_rows,
-                               int d, float eps, hipStream_t stream) {
+static void launch_add_rmsnorm(float* h, const TP* pending, int addends, size_t addend_stride, const float* w, TO* out,
+                               const int32_t* rows, int n_rows, int d, float eps, hipStream_t stream) {
     constexpr int NV = 8;
     if (d <= NV * 1024) {
         const int threads = d <= NV * 64 ? 64 : d <= NV * 128 ? 128 : d <= NV * 256 ? 256 : d <= NV * 512 ? 512 : 1024;
-        add_rmsnorm_kernel<TP, TO, NV><<<n_rows, threads, 0, stream>>>(h, pending, w, out, rows, d, eps);
+        add_rmsnorm_kernel<TP, TO, NV><<<n_rows, threads, 0, stream>>>(h, pending, addends, addend_stride, w, out, rows, d, eps);
     } else {
-        add_rmsnorm_wide_kernel<TP, TO><<<n_rows, 1024, 0, stream>>>(h, pending, w, out, rows, d, eps);
+        add_rmsnorm_wide_kernel<TP, TO><<<n_rows, 1024, 0, stream>>>(h, pending, addends, addend_stride, w, out, rows, d, eps);
     }
 }
 
-NI_EXPORT int ni_add_rmsnorm(void* h, const void* pending, const void* w, void* out, const void* rows,
-                             int n_rows, int d, float eps, int dtype, hipStream_t stream) {
+// pending: null, or [T, d] of the output type, or (addends >= 1 with float_addends) float32 [addends, T, d], whose
+// slices are added in their order.
+NI_EXPORT int ni_add_rmsnorm(void* h, const void* pending, int addends, int float_addends, size_t addend_stride,
+                             const void* w, void* out, const void* rows, int n_rows, int d, float eps, int dtype,
+                             hipStream_t stream) {
     if (n_rows <= 0) return 0;
+    if (pending && (addends < 1 || (addends > 1 && !float_addends))) return -1;
     if (dtype == 0)
-        launch_add_rmsnorm<float, float>((float*)h, (const float*)pending, (const float*)w, (float*)out,
-                                         (const int32_t*)rows, n_rows, d, eps, stream);
+        launch_add_rmsnorm<float, float>((float*)h, (const float*)pending, addends, addend_stride, (const float*)w,
+                                         (float*)out, (const int32_t*)rows, n_rows, d, eps, stream);
+    else if (float_addends)
+        launch_add_rmsnorm<float, bf16_t>((float*)h, (const float*)pending, addends, addend_stride, (const float*)w,
+                                          (bf16_t*)out, (const int32_t*)rows, n_rows, d, eps, stream);
     else
-        launch_add_rmsnorm<bf16_t, bf16_t>((float*)h, (const bf16_t*)pending, (const float*)w, (bf16_t*)out,
-                                           (const int32_t*)rows, n_rows, d, eps, stream);
+        launch_add_rmsnorm<bf16_t, bf16_t>((float*)h, (const bf16_t*)pending, addends, addend_stride, (const float*)w,
+                                           (bf16_t*)out, (const int32_t*)rows, n_rows, d, eps, stream);
     return NI_LAUNCH_RESULT();
 }
 

@@ -12,7 +12,7 @@ from typing import Dict, Optional
 import torch
 
 from ..config.spec import ModelSpec
-from ..parts.base import CacheNeed, LayerCache, Runtime
+from ..parts.base import CacheNeed, LayerCache, Runtime, pending_for
 from ..parts.standard import build_part
 from ..registry import get_part
 
@@ -63,5 +63,5 @@ class Model:
             h, pending = self.blocks[run.block].forward(h, pending, ctx, cache)
         if ctx.logit_rows is None or ctx.logit_rows.shape[0] == 0:
             return None
-        x = self.final_norm.forward(h, pending, rows=ctx.logit_rows)
+        x = self.final_norm.forward(h, pending_for(self.final_norm, pending, self.rt.dtype), rows=ctx.logit_rows)
         return self.head.forward(x)

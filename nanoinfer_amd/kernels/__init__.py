@@ -119,18 +119,25 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torc
 def add_rmsnorm(h: torch.Tensor, pending: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
                 out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``h += pending`` (when no ``rows``) and ``out = rmsnorm(h) * weight``; with ``rows`` only those
-    rows are read and ``h`` stays as it is."""
+    rows are read and ``h`` stays as it is.  ``pending`` is [T, d] of the output's type, or float32
+    [S, T, d]: S addends (the shares of a product whose K range was cut), added in their order."""
     T, d = h.shape
     _gpu(h, "h", torch.float32)
     _gpu(weight, "weight", torch.float32, (d,))
     n = T if rows is None else rows.shape[0]
     _gpu(out, "out", None, (n, d))
+    addends, float_addends = 1, 0
     if pending is not None:
-        _gpu(pending, "pending", out.dtype, (T, d))
+        if pending.dim() == 3:
+            _gpu(pending, "pending", torch.float32, (pending.shape[0], T, d))
+            addends, float_addends = pending.shape[0], 1
+        else:
+            _gpu(pending, "pending", out.dtype, (T, d))
     if rows is not None:
         _gpu(rows, "rows", torch.int32, (n,))
-    _check(core().ni_add_rmsnorm(_ptr(h), _ptr(pending), _ptr(weight), _ptr(out), _ptr(rows), n, d,
-                                 ctypes.c_float(eps), dtype_code(out.dtype), _stream()), "add_rmsnorm")
+    _check(core().ni_add_rmsnorm(_ptr(h), _ptr(pending), addends, float_addends, ctypes.c_size_t(T * d), _ptr(weight),
+                                 _ptr(out), _ptr(rows), n, d, ctypes.c_float(eps), dtype_code(out.dtype), _stream()),
+           "add_rmsnorm")
     return out
 
 
@@ -517,6 +524,7 @@ def skinny_wins(M: int, K: int, dtype: torch.dtype, weight=None) -> bool:
     return M <= 32 or K <= 4096
 FUSE_NORMS = True           # residual sums and norms ride on the skinny products of a decode step where they can
 MERGE_IN_PRODUCT = True     # the key runs of a decode step's attention are merged by the output product where it can
+SPLIT_K = True              # products of 17 to 64 rows on matrices of few tiles are cut along K, the next norm adds the shares
 
 
 def tile_weight(w: torch.Tensor) -> torch.Tensor:
@@ -610,9 +618,44 @@ def norm_prologue_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
             and _prologue_sizes_ok(int(M), int(K), dtype_code(dtype)))
 
 
+def skinny_ksplit(M: int, K: int, dtype: torch.dtype, weight):
+    """(shares, tiles per workgroup) for a product of 17 to 64 bfloat16 rows whose K range is worth
+    cutting: a matrix of few 16-row tiles (the [2048, K] matrices of the 1B shape have 128) leaves
+    half the chip idle with one workgroup a tile, and every compute unit that does work loads all of
+    x.  Cut into shares the product runs on about 256 workgroups, each loading its share of x only;
+    the shares' float32 sums are added by the kernel that adds the product to the residual stream.
+    Measured at the 1B shape (us): [2048, 8192] at 64 rows 20.9 -> 12.0 (the library 20.4), at 32 rows
+    14.2 -> 9.1; [2048, 2048] at 64 rows 7.3 -> 5.5, at 32 rows 5.0 -> 4.0.  (1, .): not cut."""
+    if not (SPLIT_K and isinstance(weight, Weight) and weight.tiles is not None and dtype == torch.bfloat16
+            and SKINNY_BEST_ROWS < M <= SKINNY_MAX_ROWS and skinny_ok(M, K, dtype)):
+        return 1, 1
+    per = 2 if (M > 32 and K >= 4096) else 1
+    groups = -(-((weight.rows.shape[0] + 15) // 16) // per)
+    pieces = (K + 63) // 64
+    return max(1, min(-(-COMPUTE_UNITS // groups), pieces // 16, 16)), per
+
+
+def skinny_gemm_ksplit(x: torch.Tensor, weight, shares: int, per_group: int) -> torch.Tensor:
+    """``x . weight^T`` as ``shares`` float32 addends [shares, M, N] (see :func:`skinny_ksplit`)."""
+    M, Kd = x.shape
+    rows, tiles = _rows_and_tiles(weight)
+    N = rows.shape[0]
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(rows, "weight", torch.bfloat16, (N, Kd))
+    if not (tiles is not None and SKINNY_BEST_ROWS < M <= SKINNY_MAX_ROWS and skinny_ok(M, Kd, x.dtype) and 1 <= shares <= 16):
+        raise KernelError(f"the product in shares does not take M={M}, K={Kd}, {shares} shares with this matrix")
+    out = torch.empty(shares, M, N, dtype=torch.float32, device=x.device)
+    _check(skinny_lib().ni_skinny_gemm_ksplit(_ptr(x), _ptr(tiles), _ptr(out), M, N, Kd, int(per_group), int(shares),
+                                              _stream()), "skinny_gemm_ksplit")
+    return out
+
+
 def residual_epilogue_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
-    """Whether the skinny product can add its result straight into the float32 residual stream."""
-    return isinstance(weight, Weight) and weight.tiles is not None and skinny_wins(M, K, dtype, weight)
+    """Whether a product can go to the float32 residual stream without a kernel of its own for the
+    sum: added by the skinny product's epilogue, or left as float32 shares for the next norm."""
+    if not (isinstance(weight, Weight) and weight.tiles is not None):
+        return False
+    return skinny_wins(M, K, dtype, weight) or skinny_ksplit(M, K, dtype, weight)[0] > 1
 
 
 def _check_normed(x: NormedInput, Kd: int) -> None:
@@ -773,7 +816,8 @@ def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optiona
     ``out_dtype`` float32 keeps the float32 accumulators of a bfloat16 product.  ``x`` may be a
     :class:`NormedInput` where :func:`norm_prologue_ok` holds.  With ``residual`` (the float32
     residual stream, where :func:`residual_epilogue_ok` holds) the product is added into it and
-    nothing is returned."""
+    nothing is returned, or (17 to 64 rows on a matrix of few tiles, :func:`skinny_ksplit`) it is
+    returned as float32 addends [S, M, N] that the next norm adds to the stream."""
     rows, _ = _rows_and_tiles(weight)
     if isinstance(x, NormedInput):
         if not (residual is None):
@@ -789,6 +833,9 @@ def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optiona
     if residual is not None:
         if not (residual_epilogue_ok(x.shape[0], x.shape[1], x.dtype, weight)):
             raise KernelError("the residual epilogue does not take this product")
+        shares, per = skinny_ksplit(x.shape[0], x.shape[1], x.dtype, weight)
+        if shares > 1:
+            return skinny_gemm_ksplit(x, weight, shares, per)      # addends for the next norm
         skinny_gemm(x, weight, residual, residual=True)
         return None
     out_dtype = out_dtype or x.dtype

@@ -15,7 +15,7 @@ import torch
 from .. import kernels as K
 from ..config.spec import BlockSpec, PartSpec
 from ..registry import get_part, register_part
-from .base import CacheNeed, KVNeed, LayerCache, Part, Runtime, WeightRequest
+from .base import CacheNeed, KVNeed, LayerCache, Part, Runtime, WeightRequest, pending_for
 
 
 def build_part(family: str, spec: PartSpec, tensors: Dict[str, torch.Tensor], rt: Runtime) -> Part:
@@ -60,6 +60,7 @@ class RMSNorm(Part):
     params: size, eps.  weights: weight [size]."""
 
     graph_safe = True
+    takes_addends = True      # ``pending`` may be float32 [S, T, size]: S addends, summed in their order
 
     @classmethod
     def weight_requests(cls, spec):
@@ -196,7 +197,8 @@ class Attention(Part):
                 and K.norm_prologue_ok(T, d, self.rt.dtype, self.w_qkv))
 
     def adds_residual(self, T: int) -> bool:
-        """Whether ``forward`` can add its output straight into the residual stream for T tokens."""
+        """Whether ``forward`` can take ``residual=h`` for T tokens: its output then goes into the residual
+        stream without a kernel for the sum (added by the product itself, or left as float32 addends)."""
         return K.FUSE_NORMS and K.residual_epilogue_ok(T, self.H * self.hd, self.rt.dtype, self.w_o)
 
     def forward(self, x, ctx, cache: LayerCache, residual: Optional[torch.Tensor] = None):
@@ -291,7 +293,8 @@ class PreNormBlock:
     The residual stream ``h`` is float32.  The last addend is handed on as ``pending`` and is
     summed into ``h`` by the next norm, in float32, in the same pass that normalises.  Two optional
     abilities of a mixer or feed-forward shorten this for steps of few tokens: ``adds_residual(T)``
-    (its last product adds into ``h`` itself: nothing is pending) and ``takes_normed(T)`` (its first
+    (given ``residual=h`` its last product adds into ``h`` itself and nothing is pending, or it
+    returns float32 addends [S, T, d] for the next norm to sum) and ``takes_normed(T)`` (its first
     product normalises ``h`` itself, given the norm's ``as_prologue(h)``).  A part without them is
     run the plain way.
     """
@@ -306,6 +309,7 @@ class PreNormBlock:
 
     def __init__(self, spec: BlockSpec, tensors: Dict[str, torch.Tensor], rt: Runtime):
         self.spec = spec
+        self.rt = rt
         self.mixer_norm = build_part("norm", spec.mixer_norm, tensors, rt)
         self.mixer = build_part("mixer", spec.mixer, tensors, rt)
         self.ffn_norm = build_part("norm", spec.ffn_norm, tensors, rt)
@@ -317,15 +321,14 @@ class PreNormBlock:
     def graph_safe(self) -> bool:
         return all(p.graph_safe is True for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn))
 
-    @staticmethod
-    def _normed_input(norm, part, h, pending):
+    def _normed_input(self, norm, part, h, pending):
         """What ``part`` is given for ``norm(h + pending)``: the norm as a prologue where both sides can, else its output."""
         T = h.shape[0]
         takes = getattr(part, "takes_normed", None)
         prologue = getattr(norm, "as_prologue", None)
         if pending is None and takes is not None and prologue is not None and takes(T):
             return prologue(h)
-        return norm.forward(h, pending)
+        return norm.forward(h, pending_for(norm, pending, self.rt.dtype))
 
     def forward(self, h, pending, ctx, cache: LayerCache):
         T = h.shape[0]

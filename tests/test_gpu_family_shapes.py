@@ -3,7 +3,8 @@ step function against the plain implementation: a prompt in one portion and in t
 tokens one by one (recorded steps), in float32 and bfloat16.  These are the hidden widths, head
 sizes and groups at which the kernels' other code paths run: head size 128, rows of 3,072 and
 4,096 elements (too long for the norm prologue in bfloat16, so the separate norm kernel runs),
-three query heads per kv head, an intermediate size of 14,336, the family's vocabulary."""
+three query heads per kv head, an intermediate size of 14,336, the family's vocabulary; and
+portions of 17 to 64 tokens, whose output and down products are cut along K in bfloat16."""
 import pytest
 import torch
 
@@ -41,9 +42,19 @@ def test_family_layer_sizes(name, dtype):
     for i in range(69, 75):
         out = runner.step([StepEntry("a", [a[i]], [0])])
         got_a[i] = out[0].clone()
-    runner.release("a"), runner.release("b")
+    # c: portions of 40 and 24 tokens, steps of 17 to 64 rows (in bfloat16 the products onto the residual
+    # stream are cut along K there and the norms add their shares)
+    c = random_tokens(vocab, 64, 13)
+    got_c = {}
+    out = runner.step([StepEntry("c", c[:40], list(range(40)))])
+    for i in range(40):
+        got_c[i] = out[i].clone()
+    out = runner.step([StepEntry("c", c[40:], list(range(24)))])
+    for i in range(24):
+        got_c[40 + i] = out[i].clone()
+    runner.release("a"), runner.release("b"), runner.release("c")
     runner.cache.check()
-    for tokens, got, rid in ((a, got_a, "a"), (b[:41], got_b, "b")):
+    for tokens, got, rid in ((a, got_a, "a"), (b[:41], got_b, "b"), (c, got_c, "c")):
         want = plain_logits(folder, tuple(tokens), dtype)
         idx = sorted(got)
         assert_close(torch.stack([got[i] for i in idx]), want[idx], dtype, f"{name} {dtype} request {rid}")

@@ -618,7 +618,8 @@ def test_skinny_product_with_norm_prologue_and_residual_epilogue(K, dtype, M, N,
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("M,N,Kd", [(17, 96, 2048), (33, 778, 528), (64, 2064, 192), (40, 50, 4096), (24, 64, 8192)])
+@pytest.mark.parametrize("M,N,Kd", [(17, 96, 2048), (33, 778, 528), (64, 2064, 192), (40, 50, 4096), (24, 64, 8192), (64, 2048, 8192),
+                                    (20, 3000, 2048), (48, 272, 4112)])
 def test_skinny_product_of_17_to_64_rows_adds_into_the_residual_stream(K, dtype, M, N, Kd):
     """The kernel for 17 to 64 rows (re-tiled matrix, x through LDS): the residual epilogue, rows
     that are no multiple of 16, a tile past the matrix, a row width that is no multiple of a piece."""
@@ -628,10 +629,36 @@ def test_skinny_product_of_17_to_64_rows_adds_into_the_residual_stream(K, dtype,
     x = torch.randn(M, Kd, generator=g).to(DT[dtype])
     stream = torch.randn(M + 3, N, generator=g)
     buf = dev(stream.clone())
-    assert K.skinny_wins(M, Kd, DT[dtype], W) and K.residual_epilogue_ok(M, Kd, DT[dtype], W)
     assert not K.skinny_wins(M, Kd, DT[dtype], dev(w)), "past 16 rows only a re-tiled matrix is streamed"
-    assert K.linear(dev(x), W, residual=buf[:M]) is None
-    assert rel(buf[:M], stream[:M].double() + x.double() @ w.double().t()) < 3e-6
+    ok = K.residual_epilogue_ok(M, Kd, DT[dtype], W)
+    assert ok == (K.skinny_wins(M, Kd, DT[dtype], W) or (dtype == "bfloat16" and Kd >= 2048))
+    if not ok:      # float32 rows of more than 4,096 elements past 32 rows: the library's product, and a kernel for the sum
+        with pytest.raises(K.KernelError):
+            K.linear(dev(x), W, residual=buf[:M])
+        return
+    got = K.linear(dev(x), W, residual=buf[:M])
+    shares = K.skinny_ksplit(M, Kd, DT[dtype], W)[0]
+    groups = -(-((N + 15) // 16) // (2 if M > 32 and Kd >= 4096 else 1))
+    assert shares == (min(-(-256 // groups), Kd // 64 // 16, 16) if dtype == "bfloat16" and Kd >= 2048 else 1), \
+        "bfloat16 rows of 32 pieces or more are cut, towards 256 workgroups"
+    if shares > 1:
+        # the K range was cut: float32 addends for the next norm, the stream itself untouched
+        assert got.dtype == torch.float32 and tuple(got.shape) == (shares, M, N)
+        assert torch.equal(buf.cpu(), stream)
+        total = buf[:M].double() + got.double().sum(0)
+        # ... which adds them in its pass: h += sum of the addends, out = rmsnorm(h)
+        nw = 1 + 0.1 * torch.randn(N, generator=g)
+        out = K.add_rmsnorm(buf[:M], got, dev(nw), 1e-5, torch.empty(M, N, device="cuda", dtype=DT[dtype]))
+        assert rel(buf[:M], total.cpu()) < 1e-6
+        assert rel(out, P.rmsnorm(total.cpu(), nw, 1e-5)) < KTOL[dtype]
+        picked = dev(torch.tensor([M - 1, 0, 3], dtype=torch.int32))
+        buf2 = dev(stream.clone())
+        out = K.add_rmsnorm(buf2[:M], got, dev(nw), 1e-5, torch.empty(3, N, device="cuda", dtype=DT[dtype]), picked)
+        assert rel(out, P.rmsnorm(total.cpu(), nw, 1e-5)[[M - 1, 0, 3]]) < KTOL[dtype] and torch.equal(buf2.cpu(), stream)
+    else:
+        assert got is None
+        total = buf[:M].double()
+    assert rel(total, stream[:M].double() + x.double() @ w.double().t()) < 3e-6
     assert torch.equal(buf[M:].cpu(), stream[M:]), "rows past the batch were written"
     assert rel(K.linear(dev(x), W), x.double() @ w.double().t()) < KTOL[dtype]
 
@@ -693,9 +720,13 @@ def test_where_the_skinny_product_gives_way_to_the_library(K):
     assert K.skinny_wins(16, 8192, torch.bfloat16, W) and K.skinny_wins(32, 8192, torch.bfloat16, W)
     assert not K.skinny_wins(33, 8192, torch.bfloat16, W) and K.skinny_wins(64, 4096, torch.bfloat16, W)
     assert not K.skinny_wins(65, 2048, torch.bfloat16, W) and not K.skinny_wins(8, 2040, torch.bfloat16, W)
-    assert not K.residual_epilogue_ok(40, 8192, torch.bfloat16, W)
+    # with the next norm to add them, 40 rows of 8,192 go in eight shares of K instead
+    assert K.residual_epilogue_ok(40, 8192, torch.bfloat16, W) and K.skinny_ksplit(40, 8192, torch.bfloat16, W) == (8, 2)
+    assert K.skinny_ksplit(16, 8192, torch.bfloat16, W) == (1, 1) == K.skinny_ksplit(65, 8192, torch.bfloat16, W)
+    Wf = K.Weight(dev(torch.zeros(32, 8192)))
+    assert not K.residual_epilogue_ok(40, 8192, torch.float32, Wf)
     with pytest.raises(K.KernelError):
-        K.linear(dev(torch.zeros(40, 8192, dtype=torch.bfloat16)), W, residual=dev(torch.zeros(40, 32)))
+        K.linear(dev(torch.zeros(40, 8192)), Wf, residual=dev(torch.zeros(40, 32)))
 
 
 def test_skinny_product_reference_vector(K):
