@@ -310,7 +310,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
 template <typename T, typename TOUT, int NT, int EPI, int XP, int WV, int SR, int HALVES = 1, int PRO = PRO_NORM>
 __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                                    TOUT* __restrict__ y, int M, int N, int K, int I,
-                                                                   RopeArgs rope, NormArgs norm) {
+                                                                   RopeArgs rope, NormArgs norm, int splits) {
     constexpr int EL = Piece<T>::ELEMS;
     constexpr int CH = 4 * EL;
     const int tid = threadIdx.x;
@@ -321,6 +321,10 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
     // workgroup's half that has the same row modulo eight
     const int wlane = HALVES == 1 ? lane : kg * 16 + ((r & 7) | (static_cast<int>(blockIdx.x % HALVES) << 3));
     const int pieces = (K + CH - 1) / CH;
+    // with splits > 1 (no prologue) workgroup (x, y) multiplies the y-th share of the pieces and stores its sums in the y-th [M, N] of y
+    const int share = (pieces + splits - 1) / splits;
+    const int p_begin = min(pieces, static_cast<int>(blockIdx.y) * share), p_end = min(pieces, p_begin + share);
+    y += static_cast<size_t>(blockIdx.y) * M * N;
 
     const T* wrow[NT];      // first byte of this lane in piece 0 of each tile
 #pragma unroll
@@ -347,7 +351,7 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
     auto load_w = [&](int c, Piece<T> (&wa)[PT][NT]) {
 #pragma unroll
         for (int u = 0; u < PT; ++u) {
-            const int piece = min(c + u * WV, pieces - 1);
+            const int piece = min(c + u * WV, p_end - 1);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) wa[u][nt].load(wrow[nt] + static_cast<size_t>(piece) * (WAVE * EL));
         }
@@ -355,7 +359,7 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
     auto multiply = [&](int c, const Piece<T> (&wa)[PT][NT], const Piece<T> (&xb)[PT][1]) {
 #pragma unroll
         for (int u = 0; u < PT; ++u) {
-            if (c + u * WV < pieces) {
+            if (c + u * WV < p_end) {
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) acc[nt][0] = Piece<T>::mma(wa[u][nt], xb[u][0], acc[nt][0]);
             }
@@ -585,18 +589,18 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
             if (t + 1 < TRIPS) multiply(c + STRIDE, wa_b, xn[t + 1 < TRIPS ? t + 1 : t]);
         }
     } else {
-        load_w(wave, wa_a);
+        load_w(p_begin + wave, wa_a);
         const T* xrow = x + static_cast<size_t>(row) * K;
         auto load_x = [&](int c, Piece<T> (&xb)[PT][1]) {
 #pragma unroll
             for (int u = 0; u < PT; ++u) xb[u][0].load(xrow + min((c + u * WV) * CH + kg * EL, K - EL));
         };
         Piece<T> xb_a[PT][1], xb_b[PT][1];
-        load_x(wave, xb_a);
-        for (int c = wave; c < pieces; c += 2 * STRIDE) {
-            if (c + STRIDE < pieces) { load_w(c + STRIDE, wa_b); load_x(c + STRIDE, xb_b); }
+        load_x(p_begin + wave, xb_a);
+        for (int c = p_begin + wave; c < p_end; c += 2 * STRIDE) {
+            if (c + STRIDE < p_end) { load_w(c + STRIDE, wa_b); load_x(c + STRIDE, xb_b); }
             multiply(c, wa_a, xb_a);
-            if (c + 2 * STRIDE < pieces) { load_w(c + 2 * STRIDE, wa_a); load_x(c + 2 * STRIDE, xb_a); }
+            if (c + 2 * STRIDE < p_end) { load_w(c + 2 * STRIDE, wa_a); load_x(c + 2 * STRIDE, xb_a); }
             multiply(c + STRIDE, wa_b, xb_b);
         }
     }
@@ -748,7 +752,8 @@ static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K,
 // The decode kernel: NT as launch_nt chooses it.  XP: pieces per wavefront of the normalising prologue, 0 without.
 template <typename T, typename TOUT, int EPI, int XP>
 static int launch_decode(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream,
-                         RopeArgs rope = RopeArgs{}, NormArgs norm = NormArgs{}) {
+                         RopeArgs rope = RopeArgs{}, NormArgs norm = NormArgs{}, int splits = 1) {
+    if (splits != 1 && (XP != 0 || EPI != EPI_STORE)) return -8;      // shares are stored, not finished
     const int out_width = (EPI == EPI_SWIGLU) ? I : N;
     const int tiles = (out_width + 15) / 16;
     auto run = [&](auto nt_tag) {
@@ -763,8 +768,8 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
         const bool halve = CAN_HALVE && grid <= HALVE_BELOW;
         auto launch = [&](auto wv_tag, auto sr_tag, auto halves_tag) {
             constexpr int WVc = decltype(wv_tag)::value, SRc = decltype(sr_tag)::value, Hc = decltype(halves_tag)::value;
-            skinny_decode_kernel<T, TOUT, NTc, EPI, XP, WVc, SRc, Hc><<<grid * Hc, WVc * WAVE, 0, stream>>>(
-                (const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm);
+            skinny_decode_kernel<T, TOUT, NTc, EPI, XP, WVc, SRc, Hc><<<dim3(grid * Hc, splits), WVc * WAVE, 0, stream>>>(
+                (const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm, splits);
         };
         using One = std::integral_constant<int, 1>;
         using Two = std::integral_constant<int, 2>;
@@ -891,12 +896,13 @@ NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N
     return launch_mb<bf16_t, bf16_t, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
 }
 
-// 17 to 64 rows of bfloat16, re-tiled W: the K range cut into `splits` shares of whole 128-byte pieces, the sums of
+// Up to 64 rows of bfloat16, re-tiled W: the K range cut into `splits` shares of whole 128-byte pieces, the sums of
 // share s stored as float32 in y[s] ([splits, M, N]); whoever reads y adds the shares in their order.  A matrix of
 // few tiles then fills the chip: 128 tiles in two or four shares are 256 workgroups.
 NI_EXPORT int ni_skinny_gemm_ksplit(const void* x, const void* W, void* y, int M, int N, int K, int tiles_per_group, int splits,
                                     hipStream_t stream) {
-    if (M <= 16 || M > 64 || N <= 0 || K % 16 != 0 || splits < 1 || splits > 16) return -1;
+    if (M <= 0 || M > 64 || N <= 0 || K % 16 != 0 || splits < 1 || splits > 16) return -1;
+    if (M <= 16) return launch_decode<bf16_t, float, EPI_STORE, 0>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, NormArgs{}, splits);
     if (M <= 32) return launch_rows<bf16_t, float, 2, EPI_STORE>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, splits);
     return launch_rows<bf16_t, float, 4, EPI_STORE>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, splits);
 }
@@ -946,7 +952,7 @@ static int launch_merged(const NormArgs& merge, const void* W, void* y, int M, i
     auto go = [&](auto sr_tag) {
         constexpr int SRc = decltype(sr_tag)::value;
         skinny_decode_kernel<bf16_t, TOUT, 1, EPI, 4, GV_WAVES, SRc, 1, PRO_MERGE><<<tiles, GV_THREADS, 0, stream>>>(
-            nullptr, (const bf16_t*)W, (TOUT*)y, M, N, K, 0, RopeArgs{}, merge);
+            nullptr, (const bf16_t*)W, (TOUT*)y, M, N, K, 0, RopeArgs{}, merge, 1);
     };
     if (M == 1) go(std::integral_constant<int, 1>{});
     else if (M <= 4) go(std::integral_constant<int, 4>{});

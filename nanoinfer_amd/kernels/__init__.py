@@ -619,20 +619,28 @@ def norm_prologue_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
 
 
 def skinny_ksplit(M: int, K: int, dtype: torch.dtype, weight):
-    """(shares, tiles per workgroup) for a product of 17 to 64 bfloat16 rows whose K range is worth
-    cutting: a matrix of few 16-row tiles (the [2048, K] matrices of the 1B shape have 128) leaves
-    half the chip idle with one workgroup a tile, and every compute unit that does work loads all of
-    x.  Cut into shares the product runs on about 256 workgroups, each loading its share of x only;
-    the shares' float32 sums are added by the kernel that adds the product to the residual stream.
-    Measured at the 1B shape (us): [2048, 8192] at 64 rows 20.9 -> 12.0 (the library 20.4), at 32 rows
-    14.2 -> 9.1; [2048, 2048] at 64 rows 7.3 -> 5.5, at 32 rows 5.0 -> 4.0.  (1, .): not cut."""
+    """(shares, tiles per workgroup) for a product of bfloat16 rows onto the residual stream whose K
+    range is worth cutting: a matrix of few 16-row tiles (the [2048, K] matrices of the 1B shape have
+    128) leaves half the chip idle with one workgroup a tile, and every compute unit that does work
+    loads all of x.  Cut into shares the product runs on about 256 workgroups, each loading its share
+    of x only; the shares' float32 sums are added by the kernel that adds the product to the residual
+    stream.  Measured at the 1B shape (us): [2048, 8192] at 64 rows 20.9 -> 12.0 (the library 20.4), at
+    32 rows 14.2 -> 9.1, at 16 rows 12.7 -> 8.1, at 9 rows 9.8 -> 7.5; [2048, 2048] at 64 rows 7.3 -> 5.5,
+    at 32 rows 5.0 -> 4.0, at 16 rows 4.65 -> 4.4.  Up to 16 rows only rows of 4,096 elements or more are
+    cut, and only where the norm that follows is a kernel of its own anyway (where the next product can
+    normalise in its prologue that is worth more than the cut).  (1, .): not cut."""
     if not (SPLIT_K and isinstance(weight, Weight) and weight.tiles is not None and dtype == torch.bfloat16
-            and SKINNY_BEST_ROWS < M <= SKINNY_MAX_ROWS and skinny_ok(M, K, dtype)):
+            and 1 <= M <= SKINNY_MAX_ROWS and skinny_ok(M, K, dtype)):
+        return 1, 1
+    N = weight.rows.shape[0]
+    if M <= SKINNY_BEST_ROWS and (K < 4096 or _prologue_sizes_ok(int(M), int(N), dtype_code(dtype))):
         return 1, 1
     per = 2 if (M > 32 and K >= 4096) else 1
-    groups = -(-((weight.rows.shape[0] + 15) // 16) // per)
+    groups = -(-((N + 15) // 16) // per)
     pieces = (K + 63) // 64
-    return max(1, min(-(-COMPUTE_UNITS // groups), pieces // 16, 16)), per
+    # as many shares as keep the workgroups within one to a compute unit (192 groups in two shares are one and a
+    # half rounds: measured slower), each share at least sixteen pieces
+    return max(1, min(COMPUTE_UNITS // groups, pieces // 16, 16)), per
 
 
 def skinny_gemm_ksplit(x: torch.Tensor, weight, shares: int, per_group: int) -> torch.Tensor:
@@ -642,7 +650,7 @@ def skinny_gemm_ksplit(x: torch.Tensor, weight, shares: int, per_group: int) -> 
     N = rows.shape[0]
     _gpu(x, "x", torch.bfloat16)
     _gpu(rows, "weight", torch.bfloat16, (N, Kd))
-    if not (tiles is not None and SKINNY_BEST_ROWS < M <= SKINNY_MAX_ROWS and skinny_ok(M, Kd, x.dtype) and 1 <= shares <= 16):
+    if not (tiles is not None and 1 <= M <= SKINNY_MAX_ROWS and skinny_ok(M, Kd, x.dtype) and 1 <= shares <= 16):
         raise KernelError(f"the product in shares does not take M={M}, K={Kd}, {shares} shares with this matrix")
     out = torch.empty(shares, M, N, dtype=torch.float32, device=x.device)
     _check(skinny_lib().ni_skinny_gemm_ksplit(_ptr(x), _ptr(tiles), _ptr(out), M, N, Kd, int(per_group), int(shares),

@@ -631,7 +631,7 @@ def test_skinny_product_of_17_to_64_rows_adds_into_the_residual_stream(K, dtype,
     buf = dev(stream.clone())
     assert not K.skinny_wins(M, Kd, DT[dtype], dev(w)), "past 16 rows only a re-tiled matrix is streamed"
     ok = K.residual_epilogue_ok(M, Kd, DT[dtype], W)
-    assert ok == (K.skinny_wins(M, Kd, DT[dtype], W) or (dtype == "bfloat16" and Kd >= 2048))
+    assert ok == (K.skinny_wins(M, Kd, DT[dtype], W) or K.skinny_ksplit(M, Kd, DT[dtype], W)[0] > 1)
     if not ok:      # float32 rows of more than 4,096 elements past 32 rows: the library's product, and a kernel for the sum
         with pytest.raises(K.KernelError):
             K.linear(dev(x), W, residual=buf[:M])
@@ -639,7 +639,7 @@ def test_skinny_product_of_17_to_64_rows_adds_into_the_residual_stream(K, dtype,
     got = K.linear(dev(x), W, residual=buf[:M])
     shares = K.skinny_ksplit(M, Kd, DT[dtype], W)[0]
     groups = -(-((N + 15) // 16) // (2 if M > 32 and Kd >= 4096 else 1))
-    assert shares == (min(-(-256 // groups), Kd // 64 // 16, 16) if dtype == "bfloat16" and Kd >= 2048 else 1), \
+    assert shares == (max(1, min(256 // groups, Kd // 64 // 16, 16)) if dtype == "bfloat16" and Kd >= 2048 else 1), \
         "bfloat16 rows of 32 pieces or more are cut, towards 256 workgroups"
     if shares > 1:
         # the K range was cut: float32 addends for the next norm, the stream itself untouched
@@ -661,6 +661,31 @@ def test_skinny_product_of_17_to_64_rows_adds_into_the_residual_stream(K, dtype,
     assert rel(total, stream[:M].double() + x.double() @ w.double().t()) < 3e-6
     assert torch.equal(buf[M:].cpu(), stream[M:]), "rows past the batch were written"
     assert rel(K.linear(dev(x), W), x.double() @ w.double().t()) < KTOL[dtype]
+
+
+@pytest.mark.parametrize("M,N,Kd,shares", [(9, 2048, 8192, 2), (16, 96, 4096, 4), (12, 272, 4112, 4), (8, 2048, 8192, 1),
+                                           (8, 3072, 8192, 1), (1, 4096, 14336, 1), (12, 3072, 8192, 1), (16, 2048, 2048, 1)])
+def test_long_products_of_up_to_16_rows_are_cut_where_a_norm_kernel_follows(K, M, N, Kd, shares):
+    """Up to 16 bfloat16 rows of 4,096 elements or more onto the residual stream go in shares of K
+    where the norm that follows is a kernel of its own (past eight rows; up to eight the next product
+    normalises in its prologue, which is worth more) and the shares still make no more workgroups
+    than the chip has compute units (not the 192 tiles of the 3B shape in two shares)."""
+    g = torch.Generator().manual_seed(M + N + Kd)
+    w = (torch.randn(N, Kd, generator=g) / math.sqrt(Kd)).to(torch.bfloat16)
+    W = K.Weight(dev(w))
+    x = torch.randn(M, Kd, generator=g).to(torch.bfloat16)
+    stream = torch.randn(M + 1, N, generator=g)
+    buf = dev(stream.clone())
+    assert K.skinny_ksplit(M, Kd, torch.bfloat16, W)[0] == shares
+    got = K.linear(dev(x), W, residual=buf[:M])
+    if shares == 1:
+        assert got is None
+        total = buf[:M].double().cpu()
+    else:
+        assert tuple(got.shape) == (shares, M, N) and got.dtype == torch.float32 and torch.equal(buf.cpu(), stream)
+        total = stream[:M].double() + got.double().sum(0).cpu()
+    assert rel(total, stream[:M].double() + x.double() @ w.double().t()) < 3e-6
+    assert torch.equal(buf[M:].cpu(), stream[M:])
 
 
 @pytest.mark.parametrize("M,H,hd,N,runs", [(1, 32, 64, 2048, 8), (8, 32, 64, 2048, 4), (3, 8, 128, 528, 8), (5, 24, 32, 96, 2),
@@ -722,7 +747,7 @@ def test_where_the_skinny_product_gives_way_to_the_library(K):
     assert not K.skinny_wins(65, 2048, torch.bfloat16, W) and not K.skinny_wins(8, 2040, torch.bfloat16, W)
     # with the next norm to add them, 40 rows of 8,192 go in eight shares of K instead
     assert K.residual_epilogue_ok(40, 8192, torch.bfloat16, W) and K.skinny_ksplit(40, 8192, torch.bfloat16, W) == (8, 2)
-    assert K.skinny_ksplit(16, 8192, torch.bfloat16, W) == (1, 1) == K.skinny_ksplit(65, 8192, torch.bfloat16, W)
+    assert K.skinny_ksplit(65, 8192, torch.bfloat16, W) == (1, 1) == K.skinny_ksplit(8, 8192, torch.bfloat16, W)
     Wf = K.Weight(dev(torch.zeros(32, 8192)))
     assert not K.residual_epilogue_ok(40, 8192, torch.float32, Wf)
     with pytest.raises(K.KernelError):
