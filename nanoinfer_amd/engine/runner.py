@@ -505,13 +505,16 @@ class ModelRunner:
             # the recording itself ran nothing: fall through to the first replay
         kind, B, width = key[0], key[1], key[2]
         ps = self.page_size
+        order = tuple(e.request for e in entries)
+        if tokens_from is not None and not (kind == "d" and order == rec.order):
+            # refused before anything is changed: the caller's books and this recording's stay as they were
+            raise StepError("tokens can stay on the device only between decode steps over the same requests")
         # the tables are written into the next staging buffer in turn, starting from those of the last replay
         last = rec.stagings[rec.turn]
         rec.turn = (rec.turn + 1) % len(rec.stagings)
         rec.copied[rec.turn].synchronize()          # the upload that last used this buffer has read it
         staging = rec.stagings[rec.turn]
         st = staging.numpy()                        # shares the pinned memory
-        order = tuple(e.request for e in entries)
         totals = []
         if kind == "d" and order == rec.order:
             # the same requests in the same places as last time: tokens, positions and slots change,
@@ -535,8 +538,6 @@ class ModelRunner:
                     done = totals[b] - 1
                     st[off_slot + b] = table[done // ps] * ps + done % ps
         else:
-            if tokens_from is not None:
-                raise StepError("tokens can stay on the device only between decode steps over the same requests")
             ctx = StepContext(self.device)
             flat, layout, _, tiles = self._tables_of(entries, ctx, width, rec.tiles or ())
             if len(flat) != staging.numel() or tiles != (rec.tiles or {}):
@@ -637,11 +638,15 @@ class ModelRunner:
                 tokens = rows[-1]
                 launched = 0
 
+        order = tuple(e.request for e in entries)
         for _ in range(int(steps)):
             cur = [StepEntry(e.request, [tokens[b] if tokens is not None else 0], [0]) for b, e in enumerate(entries)]
             key = self._graph_shape(cur) if B else None
             rec = self._recorded.get(key) if key is not None else None
-            if rec is None or rec.amax is None or launched == self.HISTORY_ROWS:
+            if rec is None or rec.amax is None or launched == self.HISTORY_ROWS or \
+                    (tokens is None and rec.order != order):
+                # also when the run passes into a recording of another shape (a longer context, a wider
+                # table) that last ran other requests: its tables are written anew, from tokens the host knows
                 collect()
                 cur = [StepEntry(e.request, [tokens[b]], [0]) for b, e in enumerate(entries)]
             if rec is None or rec.amax is None:

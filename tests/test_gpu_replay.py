@@ -494,3 +494,39 @@ def test_decode_runs_equal_single_steps(dtype):
     assert float((a - b).abs().max()) <= TOL[dtype] * float(b.abs().max()) * 0.1
     with pytest.raises(Exception):
         runs.decode_run([StepEntry("r0", [1, 2], [1])], 2)
+
+
+@pytest.mark.parametrize("page, prompt_len", [(16, 250), (8, 121)])
+def test_a_later_wave_of_requests_decodes_in_runs_across_a_recording_s_bounds(page, prompt_len):
+    """Waves of fresh requests of one batch size, each decoding in runs of eight: the runs pass,
+    in their middle, from one recording into the next (the context bound of 256, or with pages of
+    8 tokens the table width of 16 pages at 128 tokens).  From the second wave on both recordings
+    exist and hold the tables of requests that are gone.  Tokens equal those of single steps."""
+    from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
+    name = "B"
+    folder = model_folder(name)
+    vocab = ALL[name]["vocab_size"]
+    runs = ModelRunner(folder, dtype="float32", page_size=page, max_tokens=1024, max_requests=4)
+    single = ModelRunner(folder, dtype="float32", page_size=page, max_tokens=1024, max_requests=4)
+    for wave in range(3):
+        ids = [f"w{wave}r{i}" for i in range(2)]
+        toks = []
+        for i, rid in enumerate(ids):
+            p = list(random_tokens(vocab, prompt_len + i, 70 + 10 * wave + i))
+            a = runs.greedy_tokens(runs.step([StepEntry(rid, p, [len(p) - 1])]))[0]
+            b = single.greedy_tokens(single.step([StepEntry(rid, p, [len(p) - 1])]))[0]
+            assert a == b
+            toks.append(a)
+        for _ in range(3):
+            got = runs.decode_run([StepEntry(rid, [t], [0]) for rid, t in zip(ids, toks)], 8)
+            want = []
+            for _ in range(8):
+                toks = single.greedy_tokens(single.step([StepEntry(rid, [t], [0]) for rid, t in zip(ids, toks)]))
+                want.append(list(toks))
+            assert got == want, wave
+        assert runs.computed_tokens(ids[0]) == prompt_len + 24
+        for rid in ids:
+            runs.release(rid)
+            single.release(rid)
+        runs.cache.check()
+    assert runs.cache.free_pages() == runs.cache.num_pages

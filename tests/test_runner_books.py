@@ -1,0 +1,174 @@
+"""The runner's host side without a GPU: the real ``decode_run``, ``_replay``, ``_graph_shape`` and cache
+books, over a recording whose graph is a stand-in that "chooses" the next token by a formula.  Every
+replay checks the tables it was given against the cache manager's books."""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from nanoinfer_amd.cache.manager import KVCacheManager
+from nanoinfer_amd.engine.runner import ModelRunner, StepContext, StepEntry, StepError, _RecordedStep
+from nanoinfer_amd.parts.base import CacheNeed, KVNeed
+
+VOCAB = 97
+
+
+def next_token(token: int, position: int) -> int:
+    return (token * 31 + position * 7 + 1) % VOCAB
+
+
+class _Event:
+    def record(self):
+        pass
+
+    def synchronize(self):
+        pass
+
+
+class _Graph:
+    """Stands for a recorded decode step: reads its tables, checks them, leaves its choice where the
+    token ids stood."""
+
+    def __init__(self, runner, rec_of):
+        self.runner, self.rec_of, self.replays = runner, rec_of, 0
+
+    def replay(self):
+        rec = self.rec_of()
+        r, B = self.runner, len(rec.order)
+        meta = rec.meta
+        (off_slot, off_table, width) = rec.layout[0]
+        g = r.cache.groups[0]
+        ps = r.page_size
+        for b, request in enumerate(rec.order):
+            pos = int(meta[B + b])
+            assert pos == r._done[request], "position of the replay is the request's next one"
+            table = g.tables[request]
+            assert int(meta[off_slot + b]) == table[pos // ps] * ps + pos % ps
+            row = meta[off_table + b * width: off_table + (b + 1) * width].tolist()
+            assert row[:len(table)] == table and all(x == -1 for x in row[len(table):])
+            meta[b] = next_token(int(meta[b]), pos)
+        rec.logits.zero_()
+        for b in range(B):
+            rec.logits[b, int(meta[b])] = 1.0
+        self.replays += 1
+
+
+def make_runner(page_size=8, num_pages=200, max_requests=8):
+    r = object.__new__(ModelRunner)
+    r.device = torch.device("cpu")
+    r.page_size = page_size
+    r.cache = KVCacheManager({0: CacheNeed(kv=KVNeed(1, 16))}, page_size, num_pages, max_requests, device=None)
+    r.vocab_size = VOCAB
+    r.model = SimpleNamespace(max_positions=8192, graph_safe=lambda: True)
+    r.max_positions = 8192
+    r._done = {}
+    r._scratch = None
+    r._init_graphs(True)
+    r._history = torch.zeros(r.HISTORY_ROWS, r.GRAPH_MAX_BATCH, dtype=torch.int32)
+    r._history_done = _Event()
+    r.recordings_made = []
+
+    def record(key, entries):
+        kind, size, pages, bound, _ = key
+        assert kind == "d"
+        ctx = StepContext(r.device, recording=True)
+        flat, layout, n_rows, tiles = r._tables_of(entries, ctx, pages, ())
+        staging = torch.tensor(flat, dtype=torch.int32)
+        meta = staging.clone()
+        holder = {}
+        rec = _RecordedStep(_Graph(r, lambda: holder["rec"]), meta,
+                            [staging] + [torch.empty_like(staging) for _ in range(r.STAGING_BUFFERS - 1)],
+                            torch.zeros(size, VOCAB), ctx, [_Event() for _ in range(r.STAGING_BUFFERS)])
+        rec.greedy = torch.zeros(size, dtype=torch.int32)
+        rec.amax, rec.replayed, rec.tiles = meta[0:size], _Event(), tiles
+        holder["rec"] = rec
+        r._recorded[key] = rec
+        r.recordings_made.append(key)
+        return rec
+
+    r._record = record
+    r.greedy_tokens = lambda logits: logits.argmax(dim=1).tolist()
+    return r
+
+
+def start(r, request, context):
+    """A request whose first ``context`` tokens are in the cache already."""
+    assert r.cache.reserve(request, context)
+    r._done[request] = context
+
+
+def expected(first_tokens, contexts, steps):
+    toks, out = list(first_tokens), []
+    for k in range(steps):
+        toks = [next_token(t, c + k) for t, c in zip(toks, contexts)]
+        out.append(list(toks))
+    return out
+
+
+def run_wave(r, names, context, first_tokens, steps, run):
+    got = []
+    toks = list(first_tokens)
+    left = steps
+    while left:
+        k = min(run, left)
+        rows = r.decode_run([StepEntry(n, [t], [0]) for n, t in zip(names, toks)], k)
+        assert len(rows) == k
+        got.extend(rows)
+        toks = rows[-1]
+        left -= k
+    assert got == expected(first_tokens, [context] * len(names), steps)
+    for n in names:
+        assert r._done[n] == context + steps == r.cache.num_tokens(n)
+
+
+def test_a_second_wave_of_requests_crosses_a_context_bucket_inside_a_run():
+    """Two requests decode in runs of eight from context 252: the run passes from the recording
+    for contexts up to 256 into the one for up to 512.  A second pair of fresh requests does the
+    same afterwards, when both recordings exist and hold the first pair's tables."""
+    r = make_runner(page_size=16)
+    for wave, names in enumerate((("a", "b"), ("c", "d"), ("e", "f"))):
+        for n in names:
+            start(r, n, 252)
+        run_wave(r, names, 252, [3 + wave, 50 + wave], steps=24, run=8)
+        for n in names:
+            r.release(n)
+        r.cache.check()
+    assert len(r.recordings_made) == 2       # one per bucket, made by the first wave only
+    assert r.cache.free_pages() == r.cache.num_pages
+
+
+def test_a_second_wave_crosses_a_page_bucket_inside_a_run():
+    """Pages of 8 tokens: the table's width passes from 16 to 32 pages at 128 tokens while the
+    context bound stays."""
+    r = make_runner(page_size=8)
+    for wave, names in enumerate((("a", "b", "c"), ("d", "e", "f"))):
+        for n in names:
+            start(r, n, 123)
+        run_wave(r, names, 123, [1, 2, 3 + wave], steps=16, run=8)
+        for n in names:
+            r.release(n)
+    assert {k[2] for k in r.recordings_made} == {16, 32}
+
+
+def test_the_same_requests_in_another_order_get_their_tables_written_anew():
+    r = make_runner(page_size=16)
+    for n in ("a", "b"):
+        start(r, n, 40)
+    run_wave(r, ("a", "b"), 40, [5, 6], steps=8, run=4)
+    got = r.decode_run([StepEntry("b", [9], [0]), StepEntry("a", [11], [0])], 4)
+    assert got == expected([9, 11], [48, 48], 4)
+
+
+def test_tokens_on_the_device_are_refused_before_anything_changes():
+    """``_replay`` with ``tokens_from`` for other requests than the recording's last: an error, and
+    neither the recording's turn nor the books have moved."""
+    r = make_runner(page_size=16)
+    for n in ("a", "b", "c", "d"):
+        start(r, n, 40)
+    run_wave(r, ("a", "b"), 40, [5, 6], steps=2, run=2)
+    key = r.recordings_made[0]
+    rec = r._recorded[key]
+    turn, books = rec.turn, dict(r._done)
+    with pytest.raises(StepError):
+        r._replay(key, [StepEntry("c", [0], [0]), StepEntry("d", [0], [0])], tokens_from=rec, history_row=0)
+    assert rec.turn == turn and r._done == books
