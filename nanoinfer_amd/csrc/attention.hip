@@ -22,6 +22,8 @@
 // plain sum.  A prompt portion is handled as its tokens one by one: each reads the cache, which
 // the step has already filled up to and including that token.
 #include "common.h"
+#include "attention_api.h"
+#include <mutex>
 
 #ifndef HEAD_DIM
 #error "HEAD_DIM must be defined"
@@ -342,4 +344,54 @@ NI_EXPORT int ni_merge_splits(const void* part_o, const void* part_ml, void* out
         merge_splits_kernel<bf16_t><<<dim3(T_tokens, H), 64, 0, stream>>>((const float*)part_o, (const float*)part_ml,
                                                                          (bf16_t*)out, H, nsplit);
     return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- the entry point that allocates nothing
+// The partial results of the key runs, held by the library itself.  In host code the array's
+// name is only a handle for hipGetSymbolAddress: the address that kernels are given is asked for
+// once per device and kept.
+#define STATIC_SCRATCH_FLOATS (1L << 20)
+#define STATIC_MAX_DEVICES 64
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
+static float* scratch_of_device[STATIC_MAX_DEVICES];
+static std::mutex scratch_lock;
+
+// Address of the current device's copy of the array (each GPU has its own), or null with *err set.
+static float* static_scratch(int* err) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { *err = static_cast<int>(e); return nullptr; }
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES) { *err = -4; return nullptr; }
+    std::lock_guard<std::mutex> hold(scratch_lock);
+    if (!scratch_of_device[dev]) {
+        float* ptr = nullptr;
+        e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) { *err = e != hipSuccess ? static_cast<int>(e) : -5; return nullptr; }
+        scratch_of_device[dev] = ptr;
+    }
+    return scratch_of_device[dev];
+}
+
+NI_EXPORT long ni_token_attention_static_floats(void) { return STATIC_SCRATCH_FLOATS; }
+
+NI_EXPORT int ni_token_attention_static(const void* q, int q_stride, const void* kpool, const void* vpool,
+                                        const void* block_table, int table_stride, const void* seq_of_token,
+                                        const void* positions, void* out, int T_tokens, int H, int KVH,
+                                        int page_size, int window, float scale, int nsplit, int wide, int dtype,
+                                        hipStream_t stream) {
+    if (T_tokens <= 0) return 0;
+    if (H < 1 || KVH < 1 || H % KVH != 0 || nsplit < 1 || nsplit > 65535 || page_size < 1) return -1;
+    float* part_o = nullptr;
+    float* part_ml = nullptr;
+    if (nsplit > 1) {
+        const long long rows = static_cast<long long>(T_tokens) * H * nsplit;
+        if (rows * (HEAD_DIM + 2) > STATIC_SCRATCH_FLOATS) return -3;      // more than the array holds
+        int err = 0;
+        float* base = static_scratch(&err);
+        if (!base) return err;
+        part_o = base;
+        part_ml = base + rows * HEAD_DIM;
+    }
+    return ni_token_attention(q, q_stride, kpool, vpool, block_table, table_stride, seq_of_token, positions, out,
+                              part_o, part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, wide, dtype, stream);
 }

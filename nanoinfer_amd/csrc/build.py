@@ -23,7 +23,7 @@ FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          # packed float32 arithmetic is kept out of the generated code
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-value", "-Wno-unknown-warning-option"]
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "attention_api.h"]
 
 
 class BuildError(RuntimeError):
