@@ -100,6 +100,137 @@ def config_record(cfg: dict, layers: int, batch: int, mean_ctx: float, prefill_c
     }
 
 
+def percentile(values, q: float) -> float:
+    values = sorted(values)
+    if not values:
+        return 0.0
+    return values[min(len(values) - 1, int(q * len(values)))]
+
+
+def serving(args) -> int:
+    """``--workload serving``: requests through the engine's own scheduler, as a user's program
+    drives it (``Engine.add_request`` / ``Engine.step``): 64 requests arrive at once, prompts of
+    uniform random length in [128, 2048] (seeded), 256 new tokens each, greedy, continuous
+    batching with prompt portions beside decode tokens.  The report follows the reference's demo
+    (demo/batched_infer_multi_prompts.cpp:356-362: prefill and decode tokens a second) and adds
+    the step times, the share of the HBM roofline of the decode steps, and the host's share of
+    the wall time (wall minus the spans between the GPU events around every step's launches)."""
+    import torch
+
+    import nanoinfer_amd  # noqa: F401
+    from nanoinfer_amd.engine.llm import Engine
+    from nanoinfer_amd.engine.scheduler import EngineConfig
+    from nanoinfer_amd.sampling.params import SamplingParams
+    from nanoinfer_amd.weights.loader import make_random_model
+
+    torch.cuda.set_device(0)
+    model_name, shown_name, full = SHAPES[args.shape]
+    cfg = dict(full)
+    layers = args.layers or full["num_hidden_layers"]
+    cfg["num_hidden_layers"] = layers
+    dtype = {"bf16": "bfloat16", "fp32": "float32"}[args.dtype]
+    elem = 2 if args.dtype == "bf16" else 4
+    rng = random.Random(0)
+    n_req, new_tokens = args.requests, args.new_tokens
+    lengths = [rng.randint(args.min_prompt, args.max_prompt) for _ in range(n_req)]
+    prompts = [[rng.randrange(cfg["vocab_size"]) for _ in range(n)] for n in lengths]
+    pages = sum(-(-(n + new_tokens) // BLOCK_SIZE) for n in lengths) + n_req
+    if args.pool_share < 1.0:
+        pages = max(int(pages * args.pool_share), -(-(max(lengths) + new_tokens) // BLOCK_SIZE) + 1)
+    with tempfile.TemporaryDirectory(prefix="nanoinfer-bench-") as folder:
+        t0 = time.perf_counter()
+        make_random_model(folder, cfg, seed=0, dtype=dtype)
+        log(f"random model written in {time.perf_counter() - t0:.1f} s")
+        t0 = time.perf_counter()
+        engine = Engine(folder, EngineConfig(max_batch_size=n_req, max_sequences=n_req, block_size=BLOCK_SIZE,
+                                             num_cache_blocks=pages, prefill_chunk_size=args.prefill_chunk or ENGINE_CHUNK,
+                                             max_num_batched_tokens=args.token_budget, max_decode_run=args.decode_run,
+                                             dtype=dtype), ignore_eos=True)
+        log(f"model loaded in {time.perf_counter() - t0:.1f} s")
+    runner = engine.runner
+
+    def one_pass(measure: bool):
+        for p in prompts:
+            engine.add_request(p, new_tokens, SamplingParams.greedy())
+        runner.timeline = [] if measure else None
+        rows = []           # per scheduling decision: wall s, gpu s, model steps, prompt tokens, decode tokens, bytes
+        torch.cuda.synchronize()
+        t_begin = time.perf_counter()
+        while engine.has_work():
+            live = [(r.num_computed, r) for r in engine.scheduler.running]
+            steps_before = engine.num_steps
+            t1 = time.perf_counter()
+            engine.step()
+            wall = time.perf_counter() - t1
+            n = engine.scheduler.last_scheduled_tokens
+            prompt_tokens = engine.last_prompt_tokens
+            model_steps = engine.num_steps - steps_before
+            gpu = 0.0
+            if measure:
+                torch.cuda.synchronize()
+                gpu = sum(a.elapsed_time(b) for a, b in runner.timeline) * 1e-3
+                runner.timeline.clear()
+            # keys a decode-only decision reads: a request with c tokens in the cache reads c + 1 + k in step k
+            kv_tokens = 0 if prompt_tokens else sum(model_steps * (c + 1) + model_steps * (model_steps - 1) // 2
+                                                    for c, _ in live)
+            rows.append((wall, gpu, model_steps, prompt_tokens, n - prompt_tokens, kv_tokens))
+        torch.cuda.synchronize()
+        total = time.perf_counter() - t_begin
+        engine.scheduler.clear_finished()
+        return rows, total
+
+    log("first pass (records the decode shapes) ...")
+    one_pass(False)
+    log("measured pass ...")
+    rows, total = one_pass(True)
+    plain_rows, plain_total = one_pass(False)      # without events and their synchronisation: the figure that counts
+
+    generated = n_req * new_tokens
+    prefill_s = sum(w * (p / (p + d)) for w, _, _, p, d, _ in plain_rows if p + d)
+    decode_s = sum(w * (d / (p + d)) for w, _, _, p, d, _ in plain_rows if p + d)
+    prompt_total = sum(lengths)
+    decode_rows = [r for r in rows if r[3] == 0 and r[4] > 0]
+    per_step = [r[0] / r[2] for r in decode_rows for _ in range(r[2])]
+    weights = decode_bytes(cfg, 0, 0, elem)
+    kv_per_token = cfg["num_hidden_layers"] * 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * elem
+    decode_time = sum(r[0] for r in decode_rows)
+    decode_read = sum(weights * r[2] + kv_per_token * r[5] for r in decode_rows)
+    wall_sum = sum(r[0] for r in rows)
+    gpu_sum = sum(r[1] for r in rows)
+    host_share_decode = 1.0 - sum(r[1] for r in decode_rows) / decode_time if decode_time else 0.0
+    result = {
+        "metric": f"serving: generated tok/s, {n_req} concurrent requests ({shown_name} shape, continuous batching)",
+        "value": round(generated / plain_total, 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": sum(r[2] for r in plain_rows), "warmup": 1,
+        "ms_per_step": round(1e3 * (sum(per_step) / len(per_step) if per_step else 0.0), 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic: random weights (seed 0), uniform random token ids, prompt lengths uniform (seed 0)",
+        "config": {"model": model_name, "layers": layers, "layers_full_model": full["num_hidden_layers"],
+                   "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
+                   "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+                   "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
+                   "requests": n_req, "prompt_len_min": args.min_prompt, "prompt_len_max": args.max_prompt,
+                   "new_tokens": new_tokens, "kv_block_size": BLOCK_SIZE, "cache_pages": pages,
+                   "token_budget": args.token_budget, "decode_run": args.decode_run, "parallelism": "single-gpu"},
+        "total_ms": round(plain_total * 1e3, 1),
+        "prefill": {"value": round(prompt_total / prefill_s, 1) if prefill_s else None, "tokens": prompt_total,
+                    "ms": round(prefill_s * 1e3, 2)},
+        "decode": {"value": round((generated - n_req) / decode_s, 1) if decode_s else None, "tokens": generated - n_req,
+                   "ms": round(decode_s * 1e3, 2)},
+        "decode_step_ms": {"mean": round(1e3 * sum(per_step) / max(len(per_step), 1), 4),
+                           "p50": round(1e3 * percentile(per_step, 0.5), 4), "p99": round(1e3 * percentile(per_step, 0.99), 4)},
+        "roofline": {"bound": "hbm", "achieved": round(decode_read / decode_time / 1e9, 1) if decode_time else None,
+                     "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(decode_read / decode_time / HBM_PEAK, 4) if decode_time else None},
+        "host_share": {"all_steps": round(1.0 - gpu_sum / wall_sum, 4) if wall_sum else None,
+                       "decode_steps": round(host_share_decode, 4),
+                       "measured_pass_ms": round(total * 1e3, 1)},
+        "preemptions": engine.scheduler.num_preemptions,
+    }
+    print(json.dumps(result))
+    return 0
+
+
 def main() -> int:
     global PROMPT_LEN, CONTEXT_LEN
     ap = argparse.ArgumentParser()
@@ -110,13 +241,26 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes of the family member to measure (default: 1b)")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
-    ap.add_argument("--prefill-chunk", type=int, default=PREFILL_CHUNK, help="tokens of a prompt portion in the prefill measurement")
+    ap.add_argument("--prefill-chunk", type=int, default=None,
+                    help="tokens of a prompt portion in the prefill measurement (default 512); serving: the engine's "
+                         "prefill_chunk_size (default: the token budget)")
     ap.add_argument("--decode-run", type=int, default=DECODE_RUN,
                     help="decode steps on one scheduling decision (the engine's max_decode_run; 1: the host reads every token before the next step)")
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
                     help="tokens of every prompt (the measured prefill, and the context that decoding starts from); "
                          "the pool holds 2,048 more for every request")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--workload", default="steps", choices=["steps", "serving"],
+                    help="steps: the decode step and prefill of the result line's contract (default); "
+                         "serving: concurrent requests through the engine's scheduler, a line of its own")
+    ap.add_argument("--requests", type=int, default=64, help="serving: concurrent requests")
+    ap.add_argument("--new-tokens", type=int, default=256, help="serving: tokens generated per request")
+    ap.add_argument("--min-prompt", type=int, default=128, help="serving: shortest prompt")
+    ap.add_argument("--max-prompt", type=int, default=2048, help="serving: longest prompt")
+    ap.add_argument("--token-budget", type=int, default=2048, help="serving: tokens of one step (max_num_batched_tokens)")
+    ap.add_argument("--pool-share", type=float, default=1.0,
+                    help="serving: pages of the pool as a share of what all requests need at their ends "
+                         "(below 1 requests wait or are preempted)")
     ap.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
                     help="run one phase only (for profiling; prints no result line)")
     args = ap.parse_args()
@@ -127,6 +271,9 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
         return 2
+    if args.workload == "serving":
+        return serving(args)
+    args.prefill_chunk = args.prefill_chunk or PREFILL_CHUNK
 
     import torch
 

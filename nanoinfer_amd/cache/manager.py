@@ -85,6 +85,37 @@ class KVGroup:
         return first_key // self.page_size
 
 
+class ReservationPlan:
+    """Reservations that are to be made together, collected one by one: ``fits`` says whether one
+    more ``(request, total_tokens)`` can be reserved beside those already added, in time that does
+    not grow with their number (a scheduler asks once per request and step).  Pages that are
+    freed while the plan is filled only make more fit; the plan reserves nothing itself."""
+
+    def __init__(self, cache: "KVCacheManager"):
+        self.cache = cache
+        self.new_pages = [0] * len(cache.groups)
+        self.new_requests = 0
+        self.wanted: List[Tuple[Hashable, int]] = []
+
+    def _needs(self, request: Hashable, total_tokens: int):
+        c = self.cache
+        return [c._new_pages_needed(g, request, total_tokens) for g in c.groups]
+
+    def fits(self, request: Hashable, total_tokens: int) -> bool:
+        c = self.cache
+        if request not in c._tokens and self.new_requests + 1 > c.slots.num_free:
+            return False
+        return all(g.pages.can_allocate(have + n)
+                   for g, have, n in zip(c.groups, self.new_pages, self._needs(request, total_tokens)))
+
+    def add(self, request: Hashable, total_tokens: int) -> None:
+        if request not in self.cache._tokens:
+            self.new_requests += 1
+        for i, n in enumerate(self._needs(request, total_tokens)):
+            self.new_pages[i] += n
+        self.wanted.append((request, total_tokens))
+
+
 class KVCacheManager:
     """Pages and state slots for the caches of one model.
 
@@ -174,6 +205,10 @@ class KVCacheManager:
         if new_requests > self.slots.num_free:
             return False
         return all(g.pages.can_allocate(sum(self._new_pages_needed(g, r, t) for r, t in wanted)) for g in self.groups)
+
+    def plan(self) -> "ReservationPlan":
+        """An empty plan of reservations to be made together (what a scheduler fills for one step)."""
+        return ReservationPlan(self)
 
     def max_tokens_per_request(self) -> int:
         """The longest request the pools can ever hold (it then holds every page of a group)."""

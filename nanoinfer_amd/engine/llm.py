@@ -90,7 +90,7 @@ class Engine:
         entries = []
         sampling = []
         for item in batch.items:
-            toks = item.request.tokens[item.start:item.start + item.count]
+            toks = item.request.tokens_from(item.start, item.count)
             entries.append(StepEntry(item.request.request_id, toks, [item.count - 1] if item.samples else []))
             if item.samples:
                 sampling.append(item.request)

@@ -14,6 +14,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, Iterable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from .. import kernels as K
@@ -205,8 +206,10 @@ class ModelRunner:
         self._greedy_of = None                 # (logits returned by the last recorded step, its recording)
         self._history = None                   # pinned host: tokens chosen by decode steps launched back to back
         self._history_done = None
+        self.timeline = None                   # a list: every step appends (event before its first launch, event
+                                               # behind its last), for whoever measures the GPU's share of a step
 
-    def _upload(self, flat: List[int]) -> torch.Tensor:
+    def _upload(self, flat) -> torch.Tensor:
         """The integer tables of an eager step on the device.  They go through one of a few pinned
         host buffers used in turn, so that the copy is asynchronous and the host can prepare and
         launch a step while the one before it still runs."""
@@ -217,7 +220,7 @@ class ModelRunner:
             done.synchronize()            # the upload that last used this buffer has read it
         if buf is None or buf.numel() < n:
             buf = torch.empty(max(n, 4096, 2 * (buf.numel() if buf is not None else 0)), dtype=torch.int32).pin_memory()
-        buf[:n] = torch.tensor(flat, dtype=torch.int32)
+        buf.numpy()[:n] = flat
         dev = torch.empty(n, dtype=torch.int32, device=self.device)
         dev.copy_(buf[:n], non_blocking=True)
         done = done or torch.cuda.Event()
@@ -253,38 +256,40 @@ class ModelRunner:
     # ---------------------------------------------------------------- the step
     def _check_and_reserve(self, entries: List[StepEntry]) -> None:
         seen = set()
+        vocab = self.vocab_size
+        limit = self.model.max_positions
+        totals = []
         for e in entries:
             if e.request in seen:
                 raise StepError(f"request {e.request!r} appears twice in one step")
             seen.add(e.request)
-            n = len(e.tokens)
+            toks = e.tokens
+            n = len(toks)
             if n == 0:
                 raise StepError(f"request {e.request!r} brings no tokens")
-            for t in e.tokens:
-                if not 0 <= int(t) < self.vocab_size:
-                    raise StepError(f"token id {t} of request {e.request!r} is outside the vocabulary "
-                                    f"of {self.vocab_size}")
+            if not (0 <= min(toks) and max(toks) < vocab):
+                bad = next(t for t in toks if not 0 <= int(t) < vocab)
+                raise StepError(f"token id {bad} of request {e.request!r} is outside the vocabulary of {vocab}")
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"request {e.request!r} wants the logits of place {w} among {n} tokens")
-            done = self._done.get(e.request, 0)
-            if done + n > self.model.max_positions:
-                raise StepError(f"request {e.request!r} would reach {done + n} tokens, the model's positions "
-                                f"end at {self.model.max_positions}")
+            total = self._done.get(e.request, 0) + n
+            if total > limit:
+                raise StepError(f"request {e.request!r} would reach {total} tokens, the model's positions "
+                                f"end at {limit}")
+            totals.append((e.request, total))
         # reserve for all entries, or for none
-        totals = [(e.request, self._done.get(e.request, 0) + len(e.tokens)) for e in entries]
         if not self.cache.reserve_all(totals):
             raise OutOfPages(f"the step needs more pages or state slots than are free "
                              f"({self.cache.min_free_pages()} pages, {self.cache.slots.num_free} slots free)")
 
     def _describe(self, entries: List[StepEntry], ctx: StepContext, table_width: Optional[int] = None):
         """Fill the host side of ``ctx`` and return every integer table of the step as one flat
-        list, with the places of its parts: [token ids | positions | sequence of token | logit rows |
-        per group: slot mapping, block table]."""
+        int32 array, with the places of its parts: [token ids | positions | sequence of token |
+        logit rows | per group: slot mapping, block table]."""
         ps = self.page_size
-        token_ids: List[int] = []
-        positions: List[int] = []
-        seq_of_token: List[int] = []
+        i32 = np.int32
+        token_ids, positions, seq_of_token = [], [], []
         logit_rows: List[int] = []
         row = 0
         for si, e in enumerate(entries):
@@ -295,36 +300,37 @@ class ModelRunner:
             ctx.q_len.append(n)
             ctx.context_len.append(done + n)
             ctx.state_slot.append(self.cache.state_slot(e.request))
-            token_ids.extend(int(t) for t in e.tokens)
-            positions.extend(range(done, done + n))
-            seq_of_token.extend([si] * n)
-            logit_rows.extend(row + int(w) for w in e.want)
+            token_ids.append(np.asarray(e.tokens, dtype=i32))
+            positions.append(np.arange(done, done + n, dtype=i32))
+            seq_of_token.append(np.full(n, si, dtype=i32))
+            for w in e.want:
+                logit_rows.append(row + int(w))
             row += n
         ctx.n_tokens = row
         ctx.n_seqs = len(entries)
         ctx.max_context = max(ctx.context_len)
         ctx.max_q_len = max(ctx.q_len)
-        flat: List[int] = token_ids + positions + seq_of_token + logit_rows
+        pieces = token_ids + positions + seq_of_token + [np.asarray(logit_rows, dtype=i32)]
+        at = 3 * row + len(logit_rows)
         layout = []
+        B = len(entries)
         for g in self.cache.groups:
             tables = [g.tables[e.request] for e in entries]
             width = table_width or max(len(t) for t in tables)
-            slot_mapping: List[int] = []
-            for e, table in zip(entries, tables):
-                done = self._done.get(e.request, 0)
-                for p in range(done, done + len(e.tokens)):
-                    page = table[p // ps]
-                    if page < 0:
-                        raise StepError(f"request {e.request!r}: position {p} lies in a page already given back")
-                    slot_mapping.append(page * ps + p % ps)
-            off_slot = len(flat)
-            flat.extend(slot_mapping)
-            off_table = len(flat)
-            for t in tables:
-                flat.extend(t)
-                flat.extend([-1] * (width - len(t)))
-            layout.append((off_slot, off_table, width))
-        return flat, layout, len(logit_rows)
+            block_table = np.full((B, width), -1, dtype=i32)
+            off_slot = at
+            for b, (table, pos) in enumerate(zip(tables, positions)):
+                block_table[b, :len(table)] = table
+                pages = block_table[b, pos // ps]
+                if (pages < 0).any():
+                    p = int(pos[int(np.argmax(pages < 0))])
+                    raise StepError(f"request {entries[b].request!r}: position {p} lies in a page already given back")
+                pieces.append(pages * ps + pos % ps)
+            at += row
+            pieces.append(block_table.reshape(-1))
+            layout.append((off_slot, at, width))
+            at += B * width
+        return np.concatenate(pieces), layout, len(logit_rows)
 
     def _bind(self, ctx: StepContext, dev: torch.Tensor, layout, n_rows: int) -> None:
         T, B = ctx.n_tokens, ctx.n_seqs
@@ -395,11 +401,13 @@ class ModelRunner:
         the attention tiles of each tile size the model asked for."""
         flat, layout, n_rows = self._describe(entries, ctx, table_width=width)
         tiles = {}
+        pieces, at = [flat], len(flat)
         for ts in sorted(tile_sizes):
             rows = K.build_q_tiles(ctx.q_start, ctx.q_len, ctx.context_len, ts)
-            tiles[ts] = (len(flat), len(rows) // 4)        # where they start, how many
-            flat.extend(rows)
-        return flat, layout, n_rows, tiles
+            tiles[ts] = (at, len(rows) // 4)        # where they start, how many
+            pieces.append(np.asarray(rows, dtype=np.int32))
+            at += len(rows)
+        return (np.concatenate(pieces) if len(pieces) > 1 else flat), layout, n_rows, tiles
 
     def _record(self, key, entries: List[StepEntry]) -> Optional[_RecordedStep]:
         kind, size, pages, bound, _ = key
@@ -409,7 +417,7 @@ class ModelRunner:
         # harmless: it writes the same keys, values and logits again.
         warm = StepContext(self.device, scratch_owner=self)
         flat_w, layout_w, rows_w = self._describe(entries, warm)
-        self._bind(warm, torch.tensor(flat_w, dtype=torch.int32).to(self.device), layout_w, rows_w)
+        self._bind(warm, torch.from_numpy(flat_w).to(self.device), layout_w, rows_w)
         warm_logits = self.model.forward(warm, self._layer_cache(warm))
         if warm_logits is not None:
             K.argmax(warm_logits)
@@ -417,7 +425,7 @@ class ModelRunner:
         ctx = StepContext(self.device, recording=True)
         flat, layout, n_rows, tiles = self._tables_of(entries, ctx, pages, warm.tile_sizes_asked)
         ctx.max_context = bound
-        staging = torch.tensor(flat, dtype=torch.int32).pin_memory()
+        staging = torch.from_numpy(flat).pin_memory()
         meta = staging.to(self.device)
         self._bind(ctx, meta, layout, n_rows)
         for ts, (off, count) in tiles.items():
@@ -574,6 +582,20 @@ class ModelRunner:
         rec.replayed.record()
         return True
 
+    def _span(self):
+        """An event recorded now, and a function that records its partner and notes the pair in
+        ``self.timeline``; (None, no-op) when nobody measures."""
+        if self.timeline is None:
+            return None, lambda: None
+        first = torch.cuda.Event(enable_timing=True)
+        first.record()
+
+        def close():
+            last = torch.cuda.Event(enable_timing=True)
+            last.record()
+            self.timeline.append((first, last))
+        return first, close
+
     def _book(self, entries: List[StepEntry], totals: Sequence[int]) -> None:
         for e, total in zip(entries, totals):
             self._done[e.request] = total
@@ -590,6 +612,7 @@ class ModelRunner:
             self._check_and_reserve(entries)
             key = self._graph_shape(entries)
             totals = None
+            _, close = self._span()
             if key is not None and self._replay(key, entries):
                 logits = self._replayed_logits
                 totals = self._last_context_len
@@ -599,6 +622,7 @@ class ModelRunner:
                 self._bind(ctx, self._upload(flat), layout, n_rows)
                 logits = self.model.forward(ctx, self._layer_cache(ctx))
                 totals = ctx.context_len
+            close()
             self._book(entries, totals)
         for r in end:
             self.release(r)
@@ -662,8 +686,10 @@ class ModelRunner:
                 continue
             self._check_and_reserve(cur)
             at = len(chosen) + launched
+            _, close = self._span()
             self._replay(key, cur, tokens_from=last if tokens is None else None, history_row=launched,
                          pick=None if pick is None else (lambda logits, out, at=at: pick(at, logits, out)))
+            close()
             self._book(cur, self._last_context_len)
             launched += 1
             tokens = None

@@ -33,9 +33,11 @@ class RequestState(enum.Enum):
     FINISHED = "finished"
 
 
-@dataclass
+@dataclass(eq=False)
 class Request:
-    """Token-level state of one request (include/nanoinfer/engine/inference_request.h:32-169)."""
+    """Token-level state of one request (include/nanoinfer/engine/inference_request.h:32-169).
+    Two requests are the same only if they are the same object (the queues look requests up by
+    identity, never by comparing token lists)."""
 
     request_id: int
     prompt: List[int]
@@ -53,6 +55,16 @@ class Request:
     @property
     def tokens(self) -> List[int]:
         return self.prompt + self.generated
+
+    def tokens_from(self, start: int, count: int) -> List[int]:
+        """``tokens[start:start + count]`` without putting prompt and generated tokens together first."""
+        n = len(self.prompt)
+        stop = start + count
+        if stop <= n:
+            return self.prompt[start:stop]
+        if start >= n:
+            return self.generated[start - n:stop - n]
+        return self.prompt[start:] + self.generated[:stop - n]
 
     @property
     def num_tokens(self) -> int:
@@ -161,9 +173,6 @@ class Scheduler:
         return rid
 
     # ---------------------------------------------------------------- one step's decision
-    def _fits(self, chosen: List[Tuple[Hashable, int]], request: Request, count: int) -> bool:
-        return self.cache.can_reserve_all(chosen + [(request.request_id, request.num_computed + count)])
-
     def _preempt(self, victim: Request, batch: ScheduledBatch) -> None:
         if self.cache.has(victim.request_id):
             self.release(victim)
@@ -183,12 +192,15 @@ class Scheduler:
         cfg = self.config
         batch = ScheduledBatch()
         budget = cfg.max_num_batched_tokens
-        chosen: List[Tuple[Hashable, int]] = []
+        plan = self.cache.plan()         # what this step will reserve, filled request by request
+
+        def fits(req: Request, count: int) -> bool:
+            return plan.fits(req.request_id, req.num_computed + count)
 
         def take(req: Request, count: int) -> None:
             nonlocal budget
             batch.items.append(ScheduledItem(req, req.num_computed, count, req.num_computed + count == req.num_tokens))
-            chosen.append((req.request_id, req.num_computed + count))
+            plan.add(req.request_id, req.num_computed + count)
             budget -= count
 
         # 1. running requests, decode tokens before prompt portions, each group in admission order
@@ -199,7 +211,7 @@ class Scheduler:
             if len(batch.items) >= cfg.max_batch_size or budget <= 0:
                 break
             count = min(req.remaining, cfg.prefill_chunk_size, budget)
-            while not self._fits(chosen, req, count):
+            while not fits(req, count):
                 # the youngest running request that this step has not already planned for gives way;
                 # that may be the request that does not fit itself
                 in_batch = {id(i.request) for i in batch.items}
@@ -214,7 +226,7 @@ class Scheduler:
                 and budget > 0:
             req = self.waiting[0]
             count = min(req.remaining, cfg.prefill_chunk_size, budget)
-            if not self._fits(chosen, req, count):
+            if not fits(req, count):
                 break                          # strict FCFS: nobody overtakes the head of the queue
             self.waiting.popleft()
             req.state = RequestState.RUNNING
