@@ -140,8 +140,16 @@ def attention_mfma_target(head_dim: int):
     return (f"ni_attention_mfma_hd{head_dim}", ["attention_mfma.hip"], {"HEAD_DIM": head_dim})
 
 
+def attention_mfma_f32_target(head_dim: int):
+    if head_dim % 16 or not 16 <= head_dim <= 256:
+        raise BuildError(f"head size {head_dim} is not supported by the float32 matrix-core attention kernel: "
+                         "it must be a multiple of 16 between 16 and 256")
+    return (f"ni_attention_mfma_f32_hd{head_dim}", ["attention_mfma_f32.hip"], {"HEAD_DIM": head_dim})
+
+
 def build_all(head_dims: Iterable[int] = COMMON_HEAD_DIMS, force: bool = True, verbose: bool = True) -> List[str]:
     """Compile every library (attention for the given head sizes)."""
     targets = [CORE, SAMPLING, SKINNY] + [attention_target(h) for h in head_dims] + \
-        [attention_mfma_target(h) for h in head_dims if h % 32 == 0]
+        [attention_mfma_target(h) for h in head_dims if h % 32 == 0] + \
+        [attention_mfma_f32_target(h) for h in head_dims]
     return [library_path(n, s, d, force=force, verbose=verbose) for n, s, d in targets]

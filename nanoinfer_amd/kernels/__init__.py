@@ -58,6 +58,10 @@ def attention_mfma_lib(head_dim: int) -> ctypes.CDLL:
     return _load(_build.attention_mfma_target(head_dim))
 
 
+def attention_mfma_f32_lib(head_dim: int) -> ctypes.CDLL:
+    return _load(_build.attention_mfma_f32_target(head_dim))
+
+
 def dtype_code(dtype: torch.dtype) -> int:
     try:
         return _DTYPE_CODE[dtype]
@@ -291,11 +295,11 @@ def mfma_token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Te
                          seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, H: int, KVH: int,
                          hd: int, scale: float, window: Optional[int], nsplit: int,
                          workspace: Optional[torch.Tensor] = None, merge: bool = True) -> torch.Tensor:
-    """:func:`token_attention` on the matrix cores (bfloat16, head sizes that :func:`mfma_attention_ok`
+    """:func:`token_attention` on the matrix cores (bfloat16, head sizes that :func:`mfma_token_ok`
     takes): the query heads of a kv head are the rows of the products, the wavefronts of a
     workgroup share out the keys.  With ``nsplit > 1`` and ``merge=False`` the partial results of
     the key runs are left in ``workspace`` for :func:`skinny_gemm_merged` and ``out`` is not written."""
-    if not (mfma_attention_ok(qkv.dtype, hd)):
+    if not (mfma_token_ok(qkv.dtype, hd)):
         raise KernelError(f"mfma_token_attention does not take {qkv.dtype} with head size {hd}")
     if not (qkv.shape[1] % 8 == 0):
         raise KernelError("rows of qkv are not aligned to 16 bytes")
@@ -314,7 +318,15 @@ def mfma_token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Te
 
 
 def mfma_attention_ok(dtype: torch.dtype, hd: int) -> bool:
-    """Whether the matrix-core attention kernel takes this type and head size."""
+    """Whether a matrix-core attention kernel for prompt portions takes this type and head size:
+    bfloat16 with head sizes in steps of 32, float32 in steps of 16."""
+    if dtype == torch.bfloat16:
+        return hd % 32 == 0 and 32 <= hd <= 256
+    return dtype == torch.float32 and hd % 16 == 0 and 16 <= hd <= 256
+
+
+def mfma_token_ok(dtype: torch.dtype, hd: int) -> bool:
+    """Whether the matrix-core kernel for single tokens takes this type and head size (bfloat16 only)."""
     return dtype == torch.bfloat16 and hd % 32 == 0 and 32 <= hd <= 256
 
 
@@ -325,14 +337,18 @@ def _heads_per_tile(group: int) -> int:
     return 16 if group >= 16 else 8 if group > 4 else 4 if group > 2 else 2 if group > 1 else 1
 
 
-def mfma_tile_tokens(hd: int, group: int, n_tokens: Optional[int] = None, kv_heads: int = 1) -> int:
+def mfma_tile_tokens(hd: int, group: int, n_tokens: Optional[int] = None, kv_heads: int = 1,
+                     dtype: torch.dtype = torch.bfloat16) -> int:
     """Tokens of one tile of the matrix-core attention kernel for ``group`` query heads per kv head.
     A wavefront owns one block of 16 rows, or two where the head size leaves registers for them.
     More blocks share every staged key among more rows and give a wavefront more independent work,
     but the kernel pairs long tiles with short ones, two to a workgroup, and wants two workgroups on
     every compute unit: the largest number of blocks is taken that leaves a step of ``n_tokens``
     tokens four tiles for every compute unit (measured at head size 64: 2,048 tokens 57 us with one
-    block, 63 with two; 4,096 tokens 197 and 134).  Without ``n_tokens``: the smallest tile."""
+    block, 63 with two; 4,096 tokens 197 and 134).  Without ``n_tokens``: the smallest tile.  The
+    float32 kernel has one tile size."""
+    if dtype == torch.float32:
+        return int(attention_mfma_f32_lib(hd).ni_mfma_attention_f32_tile_tokens(int(group)))
     lib = attention_mfma_lib(hd)
     hpt = _heads_per_tile(group)
     blocks = 1
@@ -346,7 +362,8 @@ def mfma_tile_tokens(hd: int, group: int, n_tokens: Optional[int] = None, kv_hea
     return int(lib.ni_mfma_attention_tile_tokens(int(group), blocks))
 
 
-def mfma_plan(hd: int, group: int, kv_heads: int, n_tokens: int, max_q_len: int, max_keys: int):
+def mfma_plan(hd: int, group: int, kv_heads: int, n_tokens: int, max_q_len: int, max_keys: int,
+              dtype: torch.dtype = torch.bfloat16):
     """Tile size and number of key runs for the matrix-core attention of a step of ``n_tokens``
     tokens whose longest portion has ``max_q_len`` and whose rows read at most ``max_keys`` keys:
     ``(tile_tokens, nsplit)``, ``nsplit`` None where :func:`mfma_splits` is to decide from the
@@ -357,6 +374,8 @@ def mfma_plan(hd: int, group: int, kv_heads: int, n_tokens: int, max_q_len: int,
     and need no pairing, and cutting their keys into runs of 512 or more fills the chip (measured at
     head size 64: 512 tokens at context 2,048 take 36.8 us with one block and no cut, 30.8 with two
     blocks and four runs; at context 4,096 68.4 and 45.7)."""
+    if dtype == torch.float32:
+        return mfma_tile_tokens(hd, group, dtype=dtype), None
     small = mfma_tile_tokens(hd, group)
     tile = mfma_tile_tokens(hd, group, n_tokens, kv_heads)
     if tile != small:
@@ -403,27 +422,29 @@ def mfma_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
                    tiles: torch.Tensor, out: torch.Tensor, H: int, KVH: int, hd: int, scale: float,
                    window: Optional[int], nsplit: int = 1, workspace: Optional[torch.Tensor] = None,
                    tile_tokens: Optional[int] = None) -> torch.Tensor:
-    """Attention of prompt portions on the matrix cores (bfloat16).  ``tiles`` is int32 [n, 4] from
-    :func:`build_q_tiles` with ``tile_tokens`` tokens a tile (a size that :func:`mfma_tile_tokens`
-    gives; default: its smallest); the pools already hold the keys and values of every position of
-    the step.  ``workspace`` (float32, ``T*H*nsplit*(hd+2)`` elements) is needed when ``nsplit > 1``."""
+    """Attention of prompt portions on the matrix cores, in bfloat16 or in true float32 (a kernel
+    each).  ``tiles`` is int32 [n, 4] from :func:`build_q_tiles` with ``tile_tokens`` tokens a tile (a
+    size that :func:`mfma_tile_tokens` gives for the type; default: its smallest); the pools already
+    hold the keys and values of every position of the step.  ``workspace`` (float32,
+    ``T*H*nsplit*(hd+2)`` elements) is needed when ``nsplit > 1``."""
     T = qkv.shape[0]
-    smallest = mfma_tile_tokens(hd, H // max(KVH, 1))
+    dtype = qkv.dtype
+    _gpu(qkv, "qkv")
+    if not (mfma_attention_ok(dtype, hd)):
+        raise KernelError(f"mfma_attention does not take {dtype} with head size {hd}")
+    if not (H >= 1 and KVH >= 1 and H % KVH == 0):
+        raise KernelError(f"{H} query heads do not divide into {KVH} kv heads")
+    smallest = mfma_tile_tokens(hd, H // KVH, dtype=dtype)
     tile_tokens = smallest if tile_tokens is None else int(tile_tokens)
     blocks = tile_tokens // smallest
-    if not (blocks * smallest == tile_tokens and blocks >= 1
-            and blocks <= int(attention_mfma_lib(hd).ni_mfma_attention_max_blocks())):
-        raise KernelError(f"mfma_attention has no tiles of {tile_tokens} tokens at head size {hd} "
+    most = 1 if dtype == torch.float32 else int(attention_mfma_lib(hd).ni_mfma_attention_max_blocks())
+    if not (blocks * smallest == tile_tokens and 1 <= blocks <= most):
+        raise KernelError(f"mfma_attention has no tiles of {tile_tokens} tokens at head size {hd} in {dtype} "
                           f"(the smallest has {smallest})")
-    _gpu(qkv, "qkv", torch.bfloat16)
-    if not (mfma_attention_ok(qkv.dtype, hd)):
-        raise KernelError(f"mfma_attention does not take {qkv.dtype} with head size {hd}")
     if not (qkv.shape[1] >= H * hd and qkv.shape[1] % 8 == 0):
         raise KernelError("qkv is narrower than the query heads or its rows are unaligned")
-    if not (H % KVH == 0):
-        raise KernelError(f"{H} query heads do not divide into {KVH} kv heads")
-    _gpu(kpool, "kpool", torch.bfloat16)
-    _gpu(vpool, "vpool", torch.bfloat16, kpool.shape)
+    _gpu(kpool, "kpool", dtype)
+    _gpu(vpool, "vpool", dtype, kpool.shape)
     if not (kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd):
         raise KernelError(f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
     if not (kpool.numel() // hd < 2 ** 32):
@@ -432,7 +453,9 @@ def mfma_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
     _gpu(tiles, "tiles", torch.int32)
     if not (tiles.dim() == 2 and tiles.shape[1] == 4):
         raise KernelError("tiles must be [n, 4]")
-    _gpu(out, "out", torch.bfloat16, (T, H * hd))
+    _gpu(out, "out", dtype, (T, H * hd))
+    if not (1 <= nsplit <= 64):
+        raise KernelError(f"mfma_attention cuts the keys into 1 to 64 runs, not {nsplit}")
     part_o = part_ml = None
     if nsplit > 1:
         need = T * H * nsplit * (hd + 2)
@@ -442,11 +465,16 @@ def mfma_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
         flat = workspace.view(-1)
         part_o = flat[: T * H * nsplit * hd]
         part_ml = flat[T * H * nsplit * hd: need]
-    _check(attention_mfma_lib(hd).ni_mfma_attention(_ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table),
-                                                    block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(out),
-                                                    _ptr(part_o), _ptr(part_ml), H, KVH, kpool.shape[2],
-                                                    int(window) if window else 0, ctypes.c_float(scale), nsplit,
-                                                    blocks, _stream()), "mfma_attention")
+    if dtype == torch.float32:
+        _check(attention_mfma_f32_lib(hd).ni_mfma_attention_f32(
+            _ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table), block_table.shape[1], _ptr(tiles),
+            tiles.shape[0], _ptr(out), _ptr(part_o), _ptr(part_ml), H, KVH, kpool.shape[2],
+            int(window) if window else 0, ctypes.c_float(scale), nsplit, _stream()), "mfma_attention (float32)")
+    else:
+        _check(attention_mfma_lib(hd).ni_mfma_attention(
+            _ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table), block_table.shape[1], _ptr(tiles),
+            tiles.shape[0], _ptr(out), _ptr(part_o), _ptr(part_ml), H, KVH, kpool.shape[2],
+            int(window) if window else 0, ctypes.c_float(scale), nsplit, blocks, _stream()), "mfma_attention")
     if nsplit > 1:
         _check(attention_lib(hd).ni_merge_splits(_ptr(part_o), _ptr(part_ml), _ptr(out), T, H, nsplit,
                                                  dtype_code(out.dtype), _stream()), "merge_splits")

@@ -219,7 +219,7 @@ class Attention(Part):
             # prompt portions: tiles of tokens on the matrix cores (a recorded step has them only if
             # it was recorded with them)
             max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window + ctx.max_q_len)
-            tile_tokens, nsplit = K.mfma_plan(self.hd, self.H // self.KVH, self.KVH, T, ctx.max_q_len, max_keys)
+            tile_tokens, nsplit = K.mfma_plan(self.hd, self.H // self.KVH, self.KVH, T, ctx.max_q_len, max_keys, x.dtype)
             tiles = ctx.q_tiles(tile_tokens)
         if tiles is not None:
             if nsplit is None:
@@ -230,7 +230,7 @@ class Attention(Part):
             return K.linear(out, self.w_o, residual=residual)
         # single tokens and short portions, token by token
         max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window)
-        on_matrix_cores = K.mfma_attention_ok(x.dtype, self.hd)
+        on_matrix_cores = K.mfma_token_ok(x.dtype, self.hd)
         choose = K.mfma_token_splits if on_matrix_cores else K.choose_splits
         nsplit = choose(T, self.KVH, self.H // self.KVH, max_keys)
         ws = ctx.workspace(T * self.H * nsplit * (self.hd + 2)) if nsplit > 1 else None

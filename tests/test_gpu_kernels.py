@@ -205,7 +205,7 @@ def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boo
     ws = torch.empty(max(1, T * H * nsplit * (hd + 2)), device="cuda") if nsplit > 1 else None
     if kernel == "mfma":
         starts = [sum(q_lens[:b]) for b in range(B)]
-        tile_tokens = K.mfma_tile_tokens(hd, H // KVH) * blocks      # a wavefront owns `blocks` blocks of 16 rows
+        tile_tokens = K.mfma_tile_tokens(hd, H // KVH, dtype=DT[dtype]) * blocks      # a wavefront owns `blocks` blocks of 16 rows
         flat = K.build_q_tiles(starts, q_lens, lens, tile_tokens)
         tiles = dev(torch.tensor(flat, dtype=torch.int32).view(-1, 4))
         K.mfma_attention(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table), tiles, out,
@@ -367,7 +367,53 @@ def test_mfma_attention_window_and_far_key(K, blocks):
             assert float((got - expect).abs().max()) < 0.05, key_at
     with pytest.raises(Exception):
         K.attention_mfma_lib(48)
-    assert not K.mfma_attention_ok(torch.float32, 64) and not K.mfma_attention_ok(torch.bfloat16, 48)
+    assert not K.mfma_token_ok(torch.float32, 64) and not K.mfma_attention_ok(torch.bfloat16, 48)
+    assert K.mfma_attention_ok(torch.float32, 48) and not K.mfma_attention_ok(torch.float32, 40)
+
+
+# ---- the matrix-core kernel for prompt portions in float32
+
+@pytest.mark.parametrize("H,KVH,hd,ps", [(4, 2, 16, 16), (6, 1, 32, 8), (5, 5, 48, 5), (32, 8, 64, 16), (3, 3, 80, 16),
+                                         (8, 2, 96, 4), (2, 1, 112, 16), (16, 2, 128, 16), (2, 2, 256, 16), (32, 1, 64, 16),
+                                         (12, 4, 64, 3)])
+def test_mfma_attention_float32_head_sizes_and_groups(K, H, KVH, hd, ps):
+    # whole prompts, portions that start in the middle of a sequence, single tokens beside them, tile edges
+    lens, q_lens = [1, 37, 130, 64, 200, 17], [1, 37, 2, 1, 77, 16]
+    for nsplit in (1, 3):
+        out, want, _ = paged_case(K, "float32", H, KVH, hd, ps, lens, q_lens, None, hd + H, nsplit, kernel="mfma")
+        assert not torch.isnan(out).any(), "a key outside the sequence's own pages took part"
+        assert rel(out, want) < KTOL["float32"], (H, KVH, hd, ps, nsplit)
+    with pytest.raises(K.KernelError, match="no tiles of"):
+        paged_case(K, "float32", H, KVH, hd, ps, lens, q_lens, None, 1, 1, kernel="mfma", blocks=2)
+
+
+def test_mfma_attention_float32_window_and_far_key(K):
+    for window in (1, 7, 16, 33, 100):
+        for nsplit in (1, 2):
+            out, want, _ = paged_case(K, "float32", 4, 2, 32, 8, [150, 9, 33], [150, 9, 2], window, window, nsplit,
+                                      kernel="mfma")
+            assert not torch.isnan(out).any()
+            assert rel(out, want) < KTOL["float32"], (window, nsplit)
+    for key_at in (37, 16, 15, 0, 31, 32, 698):
+        for n_q in (5, 90):
+            out, want, (qs, ks, vs) = paged_case(K, "float32", 8, 2, 64, 16, [700], [n_q], None, 9, 1 + key_at % 4,
+                                                 boost=(0, key_at, 699, 6.0), kernel="mfma")
+            assert rel(out, want) < KTOL["float32"]
+            got = out.double().cpu()[-1].reshape(8, 64)
+            expect = vs[0][key_at].double().repeat_interleave(4, 0)
+            assert float((got - expect).abs().max()) < 0.05, key_at
+
+
+def test_mfma_attention_float32_block_table_longer_than_one_segment(K):
+    n = 2500
+    for ps, key_at in ((1, 5), (1, 1023), (1, 1024), (1, 2499), (3, 3071 % n), (3, 1)):
+        out, want, (qs, ks, vs) = paged_case(K, "float32", 4, 2, 64, ps, [n, 40], [3, 2], None, ps + key_at, 1,
+                                             boost=(0, key_at, n - 1, 6.0), kernel="mfma")
+        assert not torch.isnan(out).any()
+        assert rel(out, want) < KTOL["float32"], (ps, key_at)
+        got = out.double().cpu()[2].reshape(4, 64)
+        expect = vs[0][key_at].double().repeat_interleave(2, 0)
+        assert float((got - expect).abs().max()) < 0.05, (ps, key_at)
 
 
 def test_attention_uniform_keys_reference_vector(K):
