@@ -1,16 +1,22 @@
 """Decode and prefill throughput of the engine on one MI355X, Llama 3.2 1B shape, random weights.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--shape 1b|3b|8b] [--layers L]
+    python bench.py --workload serving [--shape 3b] [--dtype fp32]
 
 A step is one decode step of a batch of 8 requests whose prompts of 2,048 random tokens are in
 the cache (context limit 4,096): the step function runs the 8 new tokens as one batch, the
 argmax kernels pick the next ones, and they come back to the host, as in greedy generation.  ``value``
 is decoded tokens per second.  The same line carries the prefill of one 2,048-token prompt in
-portions of 512 (``prefill``; ``--prefill-chunk`` changes the cut) and in one portion, the engine's
-default (``prefill_one_portion``), the decode step's fraction of the HBM roofline, and
-decode at batch 1 and 64.  Peaks are MI355X's published ones: HBM 8 TB/s, dense bf16 MFMA
-2.5 PFLOP/s, fp32 157.3 TFLOP/s.  The reference publishes no numbers for this model, so
-``vs_baseline`` is null.
+portions of 512 (``prefill``; ``--prefill-chunk`` changes the cut), in one portion, the engine's
+default (``prefill_one_portion``, and ``prefill_one_portion_eager`` with every kernel launched from
+the host instead of a recorded step), the decode step's fraction of the HBM roofline, and in
+``points`` decode at batch 1 and 64.  The default line (1B shape, bfloat16) adds further points, each
+timed over 96 steps: decode at batch 8 from contexts of 8,192 and 32,768 tokens, the same model in
+true float32 (``decode_b8_fp32``, ``prefill_fp32``: the reference's own precision), and the 3B shape
+(``decode_b8_3b``), with the roofline fraction of each.  Peaks are MI355X's published ones: HBM
+8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s.  The reference publishes no numbers for
+this model, so ``vs_baseline`` is null.  ``--workload serving`` measures requests through the
+scheduler instead and prints a line of its own.
 """
 from __future__ import annotations
 
@@ -98,6 +104,109 @@ def config_record(cfg: dict, layers: int, batch: int, mean_ctx: float, prefill_c
         "seq_len": CONTEXT_LEN, "decode_context_mean": round(mean_ctx, 1), "kv_block_size": BLOCK_SIZE,
         "prefill_chunk": prefill_chunk, "decode_run": decode_run, "parallelism": "single-gpu",
     }
+
+
+LONG_CONTEXTS = (8192, 32768)   # further decode points at batch 8
+POINT_STEPS = 96               # timed steps of every point beside the headline (whatever --steps says):
+POINT_WARMUP = 16              # enough for batch 64 to repeat within a few per cent
+
+
+class Rig:
+    """A random model of the given sizes in a runner, and the two measurements over it."""
+
+    def __init__(self, cfg: dict, dtype: str, pool_tokens: int, max_requests: int, decode_run: int):
+        import torch
+
+        import nanoinfer_amd  # noqa: F401
+        from nanoinfer_amd.engine.runner import ModelRunner
+        from nanoinfer_amd.weights.loader import make_random_model
+
+        self.cfg, self.decode_run = cfg, decode_run
+        self.rng = random.Random(0)
+        name = {"bf16": "bfloat16", "fp32": "float32"}[dtype]
+        with tempfile.TemporaryDirectory(prefix="nanoinfer-bench-") as folder:
+            t0 = time.perf_counter()
+            make_random_model(folder, cfg, seed=0, dtype=name)
+            log(f"random model ({cfg['num_hidden_layers']} layers of {cfg['hidden_size']}, {dtype}) written in "
+                f"{time.perf_counter() - t0:.1f} s")
+            t0 = time.perf_counter()
+            self.runner = ModelRunner(folder, dtype=name, page_size=BLOCK_SIZE, max_tokens=pool_tokens,
+                                      max_requests=max_requests)
+            log(f"model loaded in {time.perf_counter() - t0:.1f} s")
+        self.torch = torch
+
+    def close(self) -> None:
+        self.runner = None
+        import gc
+        gc.collect()
+        self.torch.cuda.empty_cache()
+
+    def prompt(self, n: int):
+        V = self.cfg["vocab_size"]
+        return [self.rng.randrange(V) for _ in range(n)]
+
+    def prefill(self, length: int, chunk: int, recorded: bool = True) -> float:
+        """Seconds for one prompt of ``length`` tokens in portions of ``chunk``, up to its first
+        token on the host; the best of the second and third of three prompts.  ``recorded`` False:
+        every kernel launched from the host, as a portion's shape runs when it comes the first time."""
+        from nanoinfer_amd import kernels as K
+        from nanoinfer_amd.engine.runner import StepEntry
+
+        runner, torch = self.runner, self.torch
+        graphs, runner.use_graphs = runner.use_graphs, runner.use_graphs and recorded
+        times = []
+        try:
+            for rep in range(3):
+                toks = self.prompt(length)
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                for s in range(0, length, chunk):
+                    part = toks[s:s + chunk]
+                    last = s + chunk >= length
+                    logits = runner.step([StepEntry("p", part, [len(part) - 1] if last else [])])
+                K.argmax(logits).tolist()
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t)
+                runner.release("p")
+        finally:
+            runner.use_graphs = graphs
+        return min(times[1:])
+
+    def decode(self, batch: int, context: int, steps: int, warmup: int):
+        """(seconds a step, mean context) of ``steps`` decode steps of ``batch`` requests whose
+        prompts of ``context`` tokens are in the cache, as the engine decodes greedy requests: runs
+        of steps on one scheduling decision, the tokens passing from step to step on the device."""
+        from nanoinfer_amd import kernels as K
+        from nanoinfer_amd.engine.runner import StepEntry
+
+        runner, torch = self.runner, self.torch
+        ids = [f"d{i}" for i in range(batch)]
+        tokens = []
+        for i in ids:   # fill the cache: one request at a time, in portions of the engine's token budget
+            toks = self.prompt(context)
+            for s in range(0, context, ENGINE_CHUNK):
+                part = toks[s:s + ENGINE_CHUNK]
+                logits = runner.step([StepEntry(i, part, [len(part) - 1] if s + ENGINE_CHUNK >= context else [])])
+            tokens.append(K.argmax(logits).tolist()[0])
+        log(f"batch {batch}: prompts of {context} tokens are in the cache")
+
+        def run(toks, n):
+            while n > 0:
+                k = min(self.decode_run, n)
+                toks = runner.decode_run([StepEntry(i, [t], [0]) for i, t in zip(ids, toks)], k)[-1]
+                n -= k
+            return toks
+
+        tokens = run(tokens, warmup)
+        torch.cuda.synchronize()
+        first_ctx = runner.computed_tokens(ids[0])
+        t = time.perf_counter()
+        tokens = run(tokens, steps)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        for i in ids:
+            runner.release(i)
+        return dt / steps, first_ctx + (steps + 1) / 2.0
 
 
 def percentile(values, q: float) -> float:
@@ -249,7 +358,9 @@ def main() -> int:
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
                     help="tokens of every prompt (the measured prefill, and the context that decoding starts from); "
                          "the pool holds 2,048 more for every request")
-    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the further points")
+    ap.add_argument("--no-further", action="store_true",
+                    help="skip the points beyond the contract's: contexts of 8k and 32k, float32, the 3B shape")
     ap.add_argument("--workload", default="steps", choices=["steps", "serving"],
                     help="steps: the decode step and prefill of the result line's contract (default); "
                          "serving: concurrent requests through the engine's scheduler, a line of its own")
@@ -277,105 +388,84 @@ def main() -> int:
 
     import torch
 
-    import nanoinfer_amd  # noqa: F401
-    from nanoinfer_amd import kernels as K
-    from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
-    from nanoinfer_amd.weights.loader import make_random_model
-
     torch.cuda.set_device(0)
     model_name, shown_name, full = SHAPES[args.shape]
     cfg = dict(full)
     if args.layers is None:
         args.layers = full["num_hidden_layers"]
     cfg["num_hidden_layers"] = args.layers
-    dtype = {"bf16": "bfloat16", "fp32": "float32"}[args.dtype]
     elem = 2 if args.dtype == "bf16" else 4
-    rng = random.Random(0)
-    V = cfg["vocab_size"]
+    extras = not args.no_points and args.phase == "all"
+    # the further points (longer contexts, float32, the 3B shape) belong to the default line only
+    further = extras and args.shape == "1b" and args.dtype == "bf16" and args.layers == full["num_hidden_layers"] \
+        and args.prompt_len == 2048 and not args.no_further
 
-    with tempfile.TemporaryDirectory(prefix="nanoinfer-bench-") as folder:
-        t0 = time.perf_counter()
-        make_random_model(folder, cfg, seed=0, dtype=dtype)
-        log(f"random model written in {time.perf_counter() - t0:.1f} s")
-        max_batch = args.batch if args.no_points else max(args.batch, 64)
-        t0 = time.perf_counter()
-        runner = ModelRunner(folder, dtype=dtype, page_size=BLOCK_SIZE, max_tokens=max_batch * CONTEXT_LEN,
-                             max_requests=max_batch)
-        log(f"model loaded in {time.perf_counter() - t0:.1f} s")
-
-    def prompt():
-        return [rng.randrange(V) for _ in range(PROMPT_LEN)]
-
-    def measure_prefill(chunk):
-        """One prompt of 2,048 tokens in portions of ``chunk``; the last portion yields the first token."""
-        times = []
-        for rep in range(3):
-            toks = prompt()
-            torch.cuda.synchronize()
-            t = time.perf_counter()
-            for s in range(0, PROMPT_LEN, chunk):
-                part = toks[s:s + chunk]
-                last = s + chunk >= PROMPT_LEN
-                logits = runner.step([StepEntry("p", part, [len(part) - 1] if last else [])])
-            K.argmax(logits).tolist()
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t)
-            runner.release("p")
-        return min(times[1:])
-
-    def measure_decode(batch: int, steps: int, warmup: int):
-        ids = [f"d{i}" for i in range(batch)]
-        tokens = []
-        for i in ids:   # fill the cache: whole prompts, one request a step
-            logits = runner.step([StepEntry(i, prompt(), [PROMPT_LEN - 1])])
-            tokens.append(K.argmax(logits).tolist()[0])
-        log(f"batch {batch}: prompts are in the cache")
-
-        def decode(toks, n):
-            # as the engine decodes greedy requests: runs of steps on one scheduling decision, the
-            # tokens passing from step to step on the device
-            while n > 0:
-                k = min(args.decode_run, n)
-                toks = runner.decode_run([StepEntry(i, [t], [0]) for i, t in zip(ids, toks)], k)[-1]
-                n -= k
-            return toks
-
-        tokens = decode(tokens, warmup)
-        torch.cuda.synchronize()
-        first_ctx = runner.computed_tokens(ids[0])
-        t = time.perf_counter()
-        tokens = decode(tokens, steps)
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t
-        mean_ctx = first_ctx + (steps + 1) / 2.0
-        for i in ids:
-            runner.release(i)
-        return dt / steps, mean_ctx
+    max_batch = max(args.batch, 64) if extras else args.batch
+    pool = max_batch * CONTEXT_LEN
+    if further:
+        pool = max(pool, 8 * (LONG_CONTEXTS[-1] + 512))
+    rig = Rig(cfg, args.dtype, pool, max_batch, args.decode_run)
 
     if args.phase == "prefill":
-        log(f"prefill of {PROMPT_LEN} in portions of {args.prefill_chunk}: {measure_prefill(args.prefill_chunk) * 1e3:.2f} ms")
+        log(f"prefill of {PROMPT_LEN} in portions of {args.prefill_chunk}: "
+            f"{rig.prefill(PROMPT_LEN, args.prefill_chunk) * 1e3:.2f} ms")
         return 0
     if args.phase == "decode":
-        step_s, _ = measure_decode(args.batch, args.steps, args.warmup)
+        step_s, _ = rig.decode(args.batch, PROMPT_LEN, args.steps, args.warmup)
         log(f"decode batch {args.batch}: {step_s * 1e3:.3f} ms a step")
         return 0
+    flops = prefill_flops(cfg, PROMPT_LEN)
+
+    def prefill_record(seconds: float, dtype: str = args.dtype, fl: float = flops) -> dict:
+        return {"value": round(PROMPT_LEN / seconds, 1), "tokens": PROMPT_LEN, "ms": round(seconds * 1e3, 3),
+                "frac": round(fl / seconds / FLOP_PEAK[dtype], 4)}
+
     log("prefill ...")
-    prefill_s = measure_prefill(args.prefill_chunk)
+    prefill_s = rig.prefill(PROMPT_LEN, args.prefill_chunk)
     log(f"prefill of {PROMPT_LEN} in portions of {args.prefill_chunk}: {prefill_s * 1e3:.2f} ms")
-    whole_s = measure_prefill(ENGINE_CHUNK)
+    whole_s = rig.prefill(PROMPT_LEN, ENGINE_CHUNK)
     log(f"prefill of {PROMPT_LEN} in one portion: {whole_s * 1e3:.2f} ms")
-    step_s, mean_ctx = measure_decode(args.batch, args.steps, args.warmup)
+    eager_s = rig.prefill(PROMPT_LEN, ENGINE_CHUNK, recorded=False)
+    log(f"prefill of {PROMPT_LEN} in one portion, launched kernel by kernel: {eager_s * 1e3:.2f} ms")
+    step_s, mean_ctx = rig.decode(args.batch, PROMPT_LEN, args.steps, args.warmup)
     log(f"decode batch {args.batch}: {step_s * 1e3:.3f} ms a step")
     points = {}
-    if not args.no_points:
+    more = {}
+    if extras:
         for b in (1, 64):
-            n = max(20, min(args.steps, 100))
-            s, _ = measure_decode(b, n, max(5, args.warmup // 2))
-            points[f"decode_b{b}"] = round(b / s, 1)
-            log(f"decode batch {b}: {s * 1e3:.3f} ms a step")
+            sec, _ = rig.decode(b, PROMPT_LEN, POINT_STEPS, POINT_WARMUP)
+            points[f"decode_b{b}"] = round(b / sec, 1)
+            log(f"decode batch {b}: {sec * 1e3:.3f} ms a step")
+    if further:
+        for n in LONG_CONTEXTS:
+            sec, ctx = rig.decode(8, n, POINT_STEPS, POINT_WARMUP)
+            points[f"decode_b8_ctx{n // 1024}k"] = round(8 / sec, 1)
+            more[f"roofline_ctx{n // 1024}k"] = round(decode_bytes(cfg, 8, ctx, elem) / sec / HBM_PEAK, 4)
+            log(f"decode batch 8 at context {n}: {sec * 1e3:.3f} ms a step")
+        rig.close()
+        # the reference's own precision: the same model in true float32
+        rig32 = Rig(cfg, "fp32", 8 * CONTEXT_LEN, 8, args.decode_run)
+        sec = rig32.prefill(PROMPT_LEN, args.prefill_chunk)
+        more["prefill_fp32"] = prefill_record(sec, "fp32")
+        more["prefill_fp32_one_portion"] = prefill_record(rig32.prefill(PROMPT_LEN, ENGINE_CHUNK), "fp32")
+        log(f"float32: prefill of {PROMPT_LEN} in portions of {args.prefill_chunk}: {sec * 1e3:.2f} ms")
+        sec, ctx = rig32.decode(8, PROMPT_LEN, POINT_STEPS, POINT_WARMUP)
+        points["decode_b8_fp32"] = round(8 / sec, 1)
+        more["roofline_fp32"] = round(decode_bytes(cfg, 8, ctx, 4) / sec / HBM_PEAK, 4)
+        log(f"float32: decode batch 8: {sec * 1e3:.3f} ms a step")
+        rig32.close()
+        # the next size of the family
+        cfg3 = dict(SHAPES["3b"][2])
+        rig3 = Rig(cfg3, "bf16", 8 * CONTEXT_LEN, 8, args.decode_run)
+        sec = rig3.prefill(PROMPT_LEN, ENGINE_CHUNK)
+        more["prefill_3b_one_portion"] = prefill_record(sec, "bf16", prefill_flops(cfg3, PROMPT_LEN))
+        sec, ctx = rig3.decode(8, PROMPT_LEN, POINT_STEPS, POINT_WARMUP)
+        points["decode_b8_3b"] = round(8 / sec, 1)
+        more["roofline_3b"] = round(decode_bytes(cfg3, 8, ctx, 2) / sec / HBM_PEAK, 4)
+        log(f"3B shape: decode batch 8: {sec * 1e3:.3f} ms a step")
+        rig3.close()
 
     achieved = decode_bytes(cfg, args.batch, mean_ctx, elem) / step_s
-    flops = prefill_flops(cfg, PROMPT_LEN)
     result = {
         "metric": f"decode tok/s at batch {args.batch} ({shown_name} shape, context {CONTEXT_LEN})",
         "value": round(args.batch / step_s, 1),
@@ -391,14 +481,14 @@ def main() -> int:
         "data": "synthetic: random weights (seed 0), uniform random token ids",
         "config": config_record(cfg, args.layers, args.batch, mean_ctx, args.prefill_chunk, args.decode_run,
                                 model_name, full["num_hidden_layers"]),
-        "prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN, "ms": round(prefill_s * 1e3, 3),
-                    "frac": round(flops / prefill_s / FLOP_PEAK[args.dtype], 4)},
-        "prefill_one_portion": {"value": round(PROMPT_LEN / whole_s, 1), "tokens": PROMPT_LEN, "ms": round(whole_s * 1e3, 3),
-                                "frac": round(flops / whole_s / FLOP_PEAK[args.dtype], 4)},
+        "prefill": prefill_record(prefill_s),
+        "prefill_one_portion": prefill_record(whole_s),
+        "prefill_one_portion_eager": prefill_record(eager_s),
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
         "points": points,
     }
+    result.update(more)
     print(json.dumps(result))
     return 0
 

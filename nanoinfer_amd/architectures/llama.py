@@ -8,14 +8,10 @@ output head, which is the embedding matrix when ``tie_word_embeddings`` holds
 """
 from __future__ import annotations
 
-import hashlib
-from typing import Dict
-
-import torch
-
 from ..config.model_config import LlamaConfig
 from ..config.spec import BlockSpec, LayerRun, ModelSpec, PartSpec
 from ..registry import Architecture, register_architecture
+from ..weights.random_init import InitRule
 
 
 def build_spec(cfg: LlamaConfig) -> ModelSpec:
@@ -61,45 +57,13 @@ def build_spec(cfg: LlamaConfig) -> ModelSpec:
         bos_token_id=cfg.bos_token_id,
         eos_token_ids=cfg.eos_token_ids,
         duplicates={"lm_head.weight": embed_name} if cfg.tie_word_embeddings else {},
+        ignorable_suffixes=("rotary_emb.inv_freq",),
     )
-
-
-def _generator(seed: int, name: str) -> torch.Generator:
-    digest = hashlib.sha256(f"{seed}:{name}".encode()).digest()
-    g = torch.Generator(device="cpu")
-    g.manual_seed(int.from_bytes(digest[:8], "little") & 0x7FFFFFFFFFFFFFFF)
-    return g
-
-
-def random_weights(cfg: LlamaConfig, seed: int, dtype: torch.dtype = torch.bfloat16, std: float = 0.02,
-                   norm_std: float = 0.05) -> Dict[str, torch.Tensor]:
-    """Every tensor of the checkpoint from a seed: matrices N(0, std), norm weights 1 + N(0, norm_std).
-    Each tensor has a generator of its own, keyed by (seed, name), so the values do not depend on
-    the order of creation.  Matrices are stored in ``dtype``; norm weights stay float32 when the
-    matrices are float32 and are stored in ``dtype`` otherwise."""
-    from ..parts.standard import PreNormBlock, requests_of
-
-    spec = build_spec(cfg)
-    requests = requests_of("embedding", spec.embedding)
-    for b in spec.blocks:
-        requests += PreNormBlock.weight_requests(b)
-    requests += requests_of("norm", spec.final_norm) + requests_of("head", spec.head)
-    out: Dict[str, torch.Tensor] = {}
-    for req in requests:
-        if req.name in out:
-            continue
-        g = _generator(seed, req.name)
-        if len(req.shape) == 1:
-            t = 1.0 + norm_std * torch.randn(req.shape, generator=g, dtype=torch.float32)
-        else:
-            t = std * torch.randn(req.shape, generator=g, dtype=torch.float32)
-        out[req.name] = t.to(dtype)
-    return out
 
 
 LLAMA = register_architecture(Architecture(
     name="LlamaForCausalLM",
     config_from_dict=LlamaConfig.from_dict,
     build_spec=build_spec,
-    random_weights=random_weights,
+    init=InitRule(matrix_std=0.02, vector_mean=1.0, vector_std=0.05),
 ))

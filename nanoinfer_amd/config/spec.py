@@ -65,6 +65,9 @@ class ModelSpec:
     # tensor name -> name of the tensor it may merely repeat (a tied head stored a second time);
     # such a tensor is accepted in a checkpoint when it equals the original and is not loaded
     duplicates: Dict[str, str] = field(default_factory=dict)
+    # endings of tensor names that a checkpoint may hold without the model asking for them (buffers that
+    # exporters write along, such as a rotation's stored frequencies); they are not loaded
+    ignorable_suffixes: tuple = ()
 
     def num_caches(self) -> int:
         return 1 + max((r.cache for r in self.order), default=-1)

@@ -30,8 +30,7 @@
 #endif
 static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256, "head size: multiple of 16, at most 256");
 
-#define ATT_THREADS 256        // threads of a workgroup, narrow form
-#define ATT_THREADS_WIDE 512   // wide form
+#define ATT_THREADS 256        // threads of a workgroup
 #define GT 4  // query heads handled together by one workgroup
 
 template <typename T> struct Lanes {
@@ -286,7 +285,7 @@ template <typename T>
 static int launch(const void* q, int q_stride, const void* kpool, const void* vpool, const void* block_table,
                   int table_stride, const void* seq_of_token, const void* positions, void* out, void* part_o,
                   void* part_ml, int T_tokens, int H, int KVH, int page_size, int window, float scale,
-                  int nsplit, bool wide, hipStream_t stream) {
+                  int nsplit, hipStream_t stream) {
     const int G = H / KVH;
     const int chunks = (G + GT - 1) / GT;
     dim3 grid(T_tokens, KVH * chunks, nsplit);
@@ -298,13 +297,8 @@ static int launch(const void* q, int q_stride, const void* kpool, const void* vp
     (const T*)q, q_stride, (const T*)kpool, (const T*)vpool, (const int32_t*)block_table, table_stride,            \
         (const int32_t*)seq_of_token, (const int32_t*)positions, (T*)out, (float*)part_o, (float*)part_ml, H, KVH, \
         page_size, page_shift, window, scale, nsplit
-    if (wide) {
-        auto kernel = pow2 ? token_attention_kernel<T, true, ATT_THREADS_WIDE> : token_attention_kernel<T, false, ATT_THREADS_WIDE>;
-        kernel<<<grid, ATT_THREADS_WIDE, 0, stream>>>(TA_ARGS);
-    } else {
-        auto kernel = pow2 ? token_attention_kernel<T, true, ATT_THREADS> : token_attention_kernel<T, false, ATT_THREADS>;
-        kernel<<<grid, ATT_THREADS, 0, stream>>>(TA_ARGS);
-    }
+    auto kernel = pow2 ? token_attention_kernel<T, true, ATT_THREADS> : token_attention_kernel<T, false, ATT_THREADS>;
+    kernel<<<grid, ATT_THREADS, 0, stream>>>(TA_ARGS);
 #undef TA_ARGS
     int err = NI_LAUNCH_RESULT();
     if (err || nsplit == 1) return err;
@@ -317,20 +311,19 @@ NI_EXPORT int ni_attention_head_dim() { return HEAD_DIM; }
 NI_EXPORT int ni_attention_heads_per_group() { return GT; }
 
 // part_o: float [T, H, nsplit, HEAD_DIM], part_ml: float [T, H, nsplit, 2]; unused when nsplit == 1.
-// wide != 0 asks for workgroups of 512 threads instead of 256.
 NI_EXPORT int ni_token_attention(const void* q, int q_stride, const void* kpool, const void* vpool,
                                  const void* block_table, int table_stride, const void* seq_of_token,
                                  const void* positions, void* out, void* part_o, void* part_ml,
                                  int T_tokens, int H, int KVH, int page_size, int window, float scale, int nsplit,
-                                 int wide, int dtype, hipStream_t stream) {
+                                 int dtype, hipStream_t stream) {
     if (T_tokens <= 0) return 0;
     if (H % KVH != 0 || nsplit < 1 || nsplit > 65535 || page_size < 1) return -1;
     if (nsplit > 1 && (!part_o || !part_ml)) return -2;
     if (dtype == 0)
         return launch<float>(q, q_stride, kpool, vpool, block_table, table_stride, seq_of_token, positions, out,
-                             part_o, part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, wide != 0, stream);
+                             part_o, part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, stream);
     return launch<bf16_t>(q, q_stride, kpool, vpool, block_table, table_stride, seq_of_token, positions, out, part_o,
-                          part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, wide != 0, stream);
+                          part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, stream);
 }
 
 // Merge of partial results in the layout above, for kernels of other libraries that split the keys.
@@ -377,7 +370,7 @@ NI_EXPORT long ni_token_attention_static_floats(void) { return STATIC_SCRATCH_FL
 NI_EXPORT int ni_token_attention_static(const void* q, int q_stride, const void* kpool, const void* vpool,
                                         const void* block_table, int table_stride, const void* seq_of_token,
                                         const void* positions, void* out, int T_tokens, int H, int KVH,
-                                        int page_size, int window, float scale, int nsplit, int wide, int dtype,
+                                        int page_size, int window, float scale, int nsplit, int dtype,
                                         hipStream_t stream) {
     if (T_tokens <= 0) return 0;
     if (H < 1 || KVH < 1 || H % KVH != 0 || nsplit < 1 || nsplit > 65535 || page_size < 1) return -1;
@@ -393,5 +386,5 @@ NI_EXPORT int ni_token_attention_static(const void* q, int q_stride, const void*
         part_ml = base + rows * HEAD_DIM;
     }
     return ni_token_attention(q, q_stride, kpool, vpool, block_table, table_stride, seq_of_token, positions, out,
-                              part_o, part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, wide, dtype, stream);
+                              part_o, part_ml, T_tokens, H, KVH, page_size, window, scale, nsplit, dtype, stream);
 }

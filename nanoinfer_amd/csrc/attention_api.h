@@ -15,7 +15,7 @@ extern "C" {
 int ni_token_attention(const void* q, int q_stride, const void* kpool, const void* vpool, const void* block_table,
                        int table_stride, const void* seq_of_token, const void* positions, void* out, void* part_o,
                        void* part_ml, int T_tokens, int H, int KVH, int page_size, int window, float scale, int nsplit,
-                       int wide, int dtype, hipStream_t stream);
+                       int dtype, hipStream_t stream);
 
 // The same attention for callers that cannot allocate device memory and so cannot bring a
 // workspace: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
@@ -31,7 +31,7 @@ int ni_token_attention(const void* q, int q_stride, const void* kpool, const voi
 int ni_token_attention_static(const void* q, int q_stride, const void* kpool, const void* vpool,
                               const void* block_table, int table_stride, const void* seq_of_token,
                               const void* positions, void* out, int T_tokens, int H, int KVH, int page_size,
-                              int window, float scale, int nsplit, int wide, int dtype, hipStream_t stream);
+                              int window, float scale, int nsplit, int dtype, hipStream_t stream);
 
 // Capacity of the library's own array, in floats.
 long ni_token_attention_static_floats(void);

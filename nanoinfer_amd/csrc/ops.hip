@@ -9,6 +9,8 @@
 //     returns 0 or the hipError_t of its launch.  Shapes are checked by the host wrapper.
 #include "common.h"
 
+#include <algorithm>
+
 // ---------------------------------------------------------------- embedding
 // out[t, :] = table[ids[t], :]   (src/op/kernels/cuda/embedding_kernel.cu:30-48 of the reference;
 // ids are range-checked on the host before upload, an id outside the table never reaches here.)
@@ -113,13 +115,6 @@ __global__ void add_rmsnorm_wide_kernel(float* __restrict__ h, const TP* __restr
         const float v = (rows && prow) ? sum_at(i) : hrow[i];
         st(orow + i, (v * inv) * w[i]);
     }
-}
-
-// h[row] += pending[row] without a norm (the last residual sum when no norm follows).
-template <typename TP>
-__global__ void residual_add_kernel(float* __restrict__ h, const TP* __restrict__ pending, size_t n) {
-    size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i < n) h[i] += ld(pending + i);
 }
 
 // ---------------------------------------------------------------- rotation table
@@ -229,11 +224,65 @@ __global__ void swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out,
     VecIO<T, V>::store(out + t * I + i, y);
 }
 
-// ---------------------------------------------------------------- float32 <- any
+// ---------------------------------------------------------------- random weights
+// Element `start + i` of the normal stream of `key`: a counter-based generator (splitmix64 over
+// key + (index + 1) * gamma, Box-Muller over two 24-bit fractions).  Every operation is an IEEE
+// float32 operation rounded on its own (contraction into fused multiply-adds is switched off in
+// these routines; division and square root are the correctly rounded ones), and logarithm and
+// cosine are fixed polynomials, so that the host's numpy twin of this routine
+// (nanoinfer_amd/weights/random_init.py) gives the same bits.
+__device__ __forceinline__ float rn_poly6(float x2, float c0, float c1, float c2, float c3, float c4, float c5) {
+#pragma clang fp contract(off)
+    float acc = c5;
+    acc = acc * x2; acc = acc + c4;
+    acc = acc * x2; acc = acc + c3;
+    acc = acc * x2; acc = acc + c2;
+    acc = acc * x2; acc = acc + c1;
+    acc = acc * x2; acc = acc + c0;
+    return acc;
+}
+
+__device__ __forceinline__ float counter_normal(uint64_t key, uint64_t index, float mean, float std) {
+#pragma clang fp contract(off)
+    uint64_t z = key + (index + 1) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z = z ^ (z >> 31);
+    const int k1 = static_cast<int>(z >> 40) + 1;          // 1 .. 2^24
+    const int k2 = static_cast<int>(z & 0xFFFFFFull);      // 0 .. 2^24 - 1
+    // -2 ln(k1 / 2^24): k1 = m * 2^e, m brought into [sqrt(1/2), sqrt(2)); ln m = 2 atanh((m-1)/(m+1))
+    int e;
+    float m = frexpf(static_cast<float>(k1), &e);          // m in [0.5, 1), exact
+    if (m < 0.7071067811865476f) { m = m * 2.0f; e -= 1; }
+    const float ef = static_cast<float>(e - 24);
+    const float num = m - 1.0f, den = m + 1.0f;
+    const float s = num / den;                             // correctly rounded (the compiler's default for HIP)
+    const float s2 = s * s;
+    const float ln_m = s * rn_poly6(s2, 2.0f / 1, 2.0f / 3, 2.0f / 5, 2.0f / 7, 2.0f / 9, 2.0f / 11);
+    const float e_ln2 = ef * 0.6931471805599453f;
+    const float ln_u = e_ln2 + ln_m;
+    const float radius = sqrtf(-2.0f * ln_u);              // correctly rounded as well
+    // cos(2 pi k2 / 2^24): quarter turns q, the rest f in [0, 1) folded to [0, 1/2], x = pi/2 f
+    const int q = k2 >> 22;
+    const float f = static_cast<float>(k2 & 0x3FFFFF) * (1.0f / 4194304.0f);
+    const bool fold = f > 0.5f;
+    const float x = (fold ? 1.0f - f : f) * 1.5707963267948966f;
+    const float x2 = x * x;
+    const float sin_x = x * rn_poly6(x2, 1.0f, -1.0f / 6, 1.0f / 120, -1.0f / 5040, 1.0f / 362880, -1.0f / 39916800);
+    const float cos_x = rn_poly6(x2, 1.0f, -0.5f, 1.0f / 24, -1.0f / 720, 1.0f / 40320, -1.0f / 3628800);
+    const float sin_f = fold ? cos_x : sin_x;
+    const float cos_f = fold ? sin_x : cos_x;
+    const float c = q == 0 ? cos_f : q == 1 ? -sin_f : q == 2 ? -cos_f : sin_f;
+    const float n = radius * c;
+    const float scaled = std * n;
+    return scaled + mean;
+}
+
 template <typename T>
-__global__ void to_float_kernel(const T* __restrict__ in, float* __restrict__ out, size_t n) {
-    size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = ld(in + i);
+__global__ void random_normal_kernel(T* __restrict__ out, size_t count, uint64_t key, uint64_t start, float mean, float std) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += stride)
+        st(out + i, counter_normal(key, start + i, mean, std));
 }
 
 // ================================================================ entry points
@@ -282,15 +331,6 @@ NI_EXPORT int ni_add_rmsnorm(void* h, const void* pending, int addends, int floa
     return NI_LAUNCH_RESULT();
 }
 
-NI_EXPORT int ni_residual_add(void* h, const void* pending, size_t n, int dtype, hipStream_t stream) {
-    if (n == 0) return 0;
-    if (dtype == 0)
-        residual_add_kernel<float><<<blocks_for(n, 256), 256, 0, stream>>>((float*)h, (const float*)pending, n);
-    else
-        residual_add_kernel<bf16_t><<<blocks_for(n, 256), 256, 0, stream>>>((float*)h, (const bf16_t*)pending, n);
-    return NI_LAUNCH_RESULT();
-}
-
 NI_EXPORT int ni_rope_table(const void* inv_freq, void* cos_t, void* sin_t, int max_pos, int half,
                             hipStream_t stream) {
     size_t n = static_cast<size_t>(max_pos) * half;
@@ -333,11 +373,14 @@ NI_EXPORT int ni_swiglu(const void* gu, void* out, int T, int I, int dtype, hipS
     return NI_LAUNCH_RESULT();
 }
 
-NI_EXPORT int ni_to_float(const void* in, void* out, size_t n, int dtype, hipStream_t stream) {
-    if (n == 0) return 0;
+// out[i] = mean + std * normal(key, start + i), i < count, in the output's type (see counter_normal).
+NI_EXPORT int ni_random_normal(void* out, size_t count, uint64_t key, uint64_t start, float mean, float std, int dtype,
+                               hipStream_t stream) {
+    if (count == 0) return 0;
+    const unsigned blocks = static_cast<unsigned>(std::min<size_t>((count + 255) / 256, 65536));
     if (dtype == 0)
-        to_float_kernel<float><<<blocks_for(n, 256), 256, 0, stream>>>((const float*)in, (float*)out, n);
+        random_normal_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, count, key, start, mean, std);
     else
-        to_float_kernel<bf16_t><<<blocks_for(n, 256), 256, 0, stream>>>((const bf16_t*)in, (float*)out, n);
+        random_normal_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, count, key, start, mean, std);
     return NI_LAUNCH_RESULT();
 }

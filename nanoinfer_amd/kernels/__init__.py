@@ -145,14 +145,6 @@ def add_rmsnorm(h: torch.Tensor, pending: Optional[torch.Tensor], weight: torch.
     return out
 
 
-def residual_add(h: torch.Tensor, pending: torch.Tensor) -> torch.Tensor:
-    _gpu(h, "h", torch.float32)
-    _gpu(pending, "pending", None, h.shape)
-    _check(core().ni_residual_add(_ptr(h), _ptr(pending), ctypes.c_size_t(h.numel()), dtype_code(pending.dtype),
-                                  _stream()), "residual_add")
-    return h
-
-
 def rope_table(inv_freq: torch.Tensor, max_pos: int):
     """cos and sin of ``pos * inv_freq[p]`` in float32, each ``[max_pos, len(inv_freq)]``."""
     _gpu(inv_freq, "inv_freq", torch.float32)
@@ -204,11 +196,16 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def to_float(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    _gpu(x, "x")
-    _gpu(out, "out", torch.float32, x.shape)
-    _check(core().ni_to_float(_ptr(x), _ptr(out), ctypes.c_size_t(x.numel()), dtype_code(x.dtype), _stream()),
-           "to_float")
+def random_normal(out: torch.Tensor, key: int, start: int, mean: float, std: float) -> torch.Tensor:
+    """``out[i] = mean + std * n(key, start + i)`` for the flat tensor ``out`` (float32 or bfloat16):
+    the counter-based normal stream of :mod:`nanoinfer_amd.weights.random_init`, same bits as its
+    numpy routine."""
+    _gpu(out, "out")
+    if not (out.dim() == 1 and 0 <= int(key) < 2 ** 64 and int(start) >= 0):
+        raise KernelError("random_normal fills a flat tensor from a 64-bit key and a non-negative start")
+    _check(core().ni_random_normal(_ptr(out), ctypes.c_size_t(out.numel()), ctypes.c_uint64(int(key)),
+                                   ctypes.c_uint64(int(start)), ctypes.c_float(mean), ctypes.c_float(std),
+                                   dtype_code(out.dtype), _stream()), "random_normal")
     return out
 
 
@@ -255,13 +252,12 @@ def _token_attention_checks(qkv, kpool, vpool, block_table, seq_of_token, positi
 def token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                     seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, H: int, KVH: int,
                     hd: int, scale: float, window: Optional[int], nsplit: int,
-                    workspace: Optional[torch.Tensor] = None, wide: bool = False) -> torch.Tensor:
+                    workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of every token of ``qkv`` over the paged cache of its sequence.
 
     ``qkv`` is [T, >= H*hd] with the (rotated) query heads first; the pools already hold the keys
     and values of all positions up to each token's own.  ``workspace`` (float32, at least
-    ``T*H*nsplit*(hd+2)`` elements) is needed when ``nsplit > 1``.  ``wide`` asks for workgroups
-    of 512 threads instead of 256.
+    ``T*H*nsplit*(hd+2)`` elements) is needed when ``nsplit > 1``.
     """
     T, part_o, part_ml = _token_attention_checks(qkv, kpool, vpool, block_table, seq_of_token, positions, out,
                                                  H, KVH, hd, nsplit, workspace)
@@ -269,7 +265,7 @@ def token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
     _check(lib.ni_token_attention(_ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table),
                                   block_table.shape[1], _ptr(seq_of_token), _ptr(positions), _ptr(out),
                                   _ptr(part_o), _ptr(part_ml), T, H, KVH, kpool.shape[2],
-                                  int(window) if window else 0, ctypes.c_float(scale), nsplit, int(bool(wide)),
+                                  int(window) if window else 0, ctypes.c_float(scale), nsplit,
                                   dtype_code(qkv.dtype), _stream()), "token_attention")
     return out
 

@@ -7,18 +7,23 @@ The reference chooses a C++ class and an enum by a preset name in each demo
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Any, Callable, Dict, List
 
 from .config.spec import ModelSpec
+from .weights.random_init import InitRule
 
 
 @dataclass
 class Architecture:
+    """All an architecture has to say: how its ``config.json`` is read, how its model is described
+    as parts, and (as data) how its random weights are drawn.  The typed configuration needs a
+    ``to_dict()`` that gives back ``config.json`` keys, for the random-weights mode's folder."""
+
     name: str
     config_from_dict: Callable[[Dict[str, Any]], Any]   # config.json -> typed configuration
     build_spec: Callable[[Any], ModelSpec]               # typed configuration -> model as data
-    random_weights: Callable[..., Dict[str, Any]]        # typed configuration, seed -> tensors by name
+    init: InitRule = field(default_factory=InitRule)     # distribution of each tensor of the random-weights mode
 
 
 ARCHITECTURES: Dict[str, Architecture] = {}

@@ -20,7 +20,7 @@ import torch
 from ..config.model_config import read_config_json
 from ..config.spec import ModelSpec
 from ..registry import architecture_of, get_part
-from .safetensors_io import SafetensorsFile, WeightFileError, write_safetensors
+from .safetensors_io import SafetensorsFile, WeightFileError, write_safetensors, write_safetensors_streamed
 
 
 class WeightMismatchError(WeightFileError):
@@ -130,6 +130,8 @@ def load_tensors(folder: str, spec: ModelSpec) -> Dict[str, torch.Tensor]:
         orig = spec.duplicates.get(n)
         if orig in have and tuple(f.shape(n)) == tuple(f.shape(orig)) and torch.equal(f.tensor(n), f.tensor(orig)):
             continue  # a second copy of a tensor the model shares
+        if any(n.endswith(suffix) for suffix in spec.ignorable_suffixes):
+            continue  # a buffer that exporters write along and the model does not use
         unexpected.append(n)
     wrong = sorted((n, want[n], f.shape(n)) for n in want if n in have and tuple(f.shape(n)) != want[n])
     if missing or unexpected or wrong:
@@ -167,17 +169,59 @@ _TORCH_DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": to
 
 
 def make_random_model(folder: str, config_json: Dict[str, Any], seed: int, dtype: str = "bfloat16",
-                      shards: int = 1, **init) -> str:
-    """Random-weights mode: write ``config.json`` and ``model.safetensors`` for the architecture
-    that ``config_json`` names, from a seed.  ``dtype`` is the type the matrices are stored in."""
+                      shards: int = 1, device=None, **init) -> str:
+    """Random-weights mode: write ``config.json`` and ``model.safetensors`` (or ``shards`` files and
+    their index) for the architecture that ``config_json`` names, from a seed.  ``dtype`` is the type
+    every tensor is stored in.  What is drawn is the architecture's :class:`InitRule`, of which
+    ``init`` may replace fields (``matrix_std=...``); which tensors exist, and their shapes, is what
+    the parts of the model ask for.  Every element is a function of (seed, tensor name, element
+    index), so the file does not depend on where it is made: with a GPU (``device``; default: the
+    current one when there is one) large tensors are generated there and streamed to the file piece
+    by piece, which a model of tens of gigabytes needs; without, numpy gives the same bits."""
     if dtype not in _TORCH_DTYPES:
         raise WeightFileError(f"dtype {dtype!r} is not one of {sorted(_TORCH_DTYPES)}")
+    import dataclasses
+
+    from . import random_init
+
     arch = architecture_of(config_json)
     cfg = arch.config_from_dict(config_json)
-    tensors = arch.random_weights(cfg, seed, dtype=_TORCH_DTYPES[dtype], **init)
+    spec = arch.build_spec(cfg)
+    rule = dataclasses.replace(arch.init, **init) if init else arch.init
+    store = _TORCH_DTYPES[dtype]
+    if device is None and torch.cuda.is_available():
+        device = torch.device("cuda", torch.cuda.current_device())
+    entries = []
+    for name, shape in expected_tensors(spec).items():
+        mean, std = rule.mean_std(name, shape)
+        entries.append((name, store, shape,
+                        lambda name=name, shape=shape, mean=mean, std=std:
+                        random_init.pieces(seed, name, shape, mean, std, store, device)))
     out = dict(cfg.to_dict())
-    out["torch_dtype"] = "bfloat16" if _TORCH_DTYPES[dtype] == torch.bfloat16 else "float32"
-    return write_model_folder(folder, out, tensors, shards=shards)
+    out["torch_dtype"] = "bfloat16" if store == torch.bfloat16 else "float32"
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as fh:
+        json.dump(out, fh, indent=2)
+    if shards <= 1:
+        write_safetensors_streamed(os.path.join(folder, "model.safetensors"), entries, {"format": "pt"})
+        return folder
+    per = -(-len(entries) // shards)
+    weight_map, total = {}, 0
+    for i in range(shards):
+        part = entries[i * per:(i + 1) * per]
+        if not part:
+            continue
+        fname = f"model-{i + 1:05d}-of-{shards:05d}.safetensors"
+        write_safetensors_streamed(os.path.join(folder, fname), part, {"format": "pt"})
+        for name, dt, shape, _ in part:
+            weight_map[name] = fname
+            n = 1
+            for d in shape:
+                n *= int(d)
+            total += n * (2 if dt == torch.bfloat16 else 4)
+    with open(os.path.join(folder, INDEX_NAME), "w") as fh:
+        json.dump({"metadata": {"total_size": total}, "weight_map": weight_map}, fh, indent=2)
+    return folder
 
 
 def read_model_folder(folder: str):

@@ -117,27 +117,60 @@ class SafetensorsFile:
         self._fh.close()
 
 
-def write_safetensors(path: str, tensors: Dict[str, torch.Tensor], metadata: Dict[str, str] = None) -> None:
-    """Write CPU tensors under their names, in the given order, 8-byte aligned header."""
+def _raw(t: torch.Tensor) -> memoryview:
+    """The bytes of a contiguous CPU tensor, without a copy."""
+    t = t.detach().contiguous()
+    arr = t.view(torch.uint16).numpy() if t.dtype == torch.bfloat16 else t.numpy()
+    return memoryview(arr.reshape(-1)).cast("B")
+
+
+def write_safetensors_streamed(path: str, entries, metadata: Dict[str, str] = None) -> None:
+    """Write tensors that are produced piece by piece.  ``entries`` is a list of ``(name, dtype,
+    shape, pieces)``; ``pieces()`` returns an iterator of flat CPU tensors of that type which
+    together hold the tensor's elements in order.  The header is written first, from the shapes
+    alone, and every piece goes to the file as it comes: no tensor is ever held whole, so a model
+    larger than the host's memory can be written (the reference's loader, for contrast, maps views
+    of a file that an exporter held whole: src/model/llama.cpp:568-706)."""
     header = {}
     if metadata:
         header["__metadata__"] = {str(k): str(v) for k, v in metadata.items()}
     offset = 0
-    blobs = []
-    for name, t in tensors.items():
-        t = t.detach().cpu().contiguous()
-        if t.dtype not in _TAG_OF:
-            raise WeightFileError(f"tensor {name!r}: type {t.dtype} cannot be stored")
-        raw = t.view(torch.uint16).numpy().tobytes() if t.dtype == torch.bfloat16 else t.numpy().tobytes()
-        header[name] = {"dtype": _TAG_OF[t.dtype], "shape": list(t.shape), "data_offsets": [offset, offset + len(raw)]}
-        offset += len(raw)
-        blobs.append(raw)
+    sizes = []
+    for name, dtype, shape, _ in entries:
+        if dtype not in _TAG_OF:
+            raise WeightFileError(f"tensor {name!r}: type {dtype} cannot be stored")
+        n = 1
+        for d in shape:
+            n *= int(d)
+        nbytes = n * _DTYPES[_TAG_OF[dtype]][1]
+        if name in header:
+            raise WeightFileError(f"tensor {name!r} is listed twice")
+        header[name] = {"dtype": _TAG_OF[dtype], "shape": [int(d) for d in shape], "data_offsets": [offset, offset + nbytes]}
+        offset += nbytes
+        sizes.append(nbytes)
     hjson = json.dumps(header, separators=(",", ":")).encode("utf-8")
     hjson += b" " * ((8 - len(hjson) % 8) % 8)
     tmp = path + ".tmp"
     with open(tmp, "wb") as fh:
         fh.write(struct.pack("<Q", len(hjson)))
         fh.write(hjson)
-        for raw in blobs:
-            fh.write(raw)
+        for (name, dtype, shape, pieces), nbytes in zip(entries, sizes):
+            written = 0
+            for piece in pieces():
+                if piece.dtype != dtype:
+                    raise WeightFileError(f"tensor {name!r}: a piece of type {piece.dtype} for a tensor of type {dtype}")
+                raw = _raw(piece)
+                fh.write(raw)
+                written += len(raw)
+            if written != nbytes:
+                raise WeightFileError(f"tensor {name!r} of shape {tuple(shape)} takes {nbytes} bytes, its pieces gave {written}")
     os.replace(tmp, path)
+
+
+def write_safetensors(path: str, tensors: Dict[str, torch.Tensor], metadata: Dict[str, str] = None) -> None:
+    """Write CPU tensors under their names, in the given order, 8-byte aligned header."""
+    entries = []
+    for name, t in tensors.items():
+        t = t.detach().cpu()
+        entries.append((name, t.dtype, tuple(t.shape), lambda t=t: iter([t.reshape(-1)])))
+    write_safetensors_streamed(path, entries, metadata)

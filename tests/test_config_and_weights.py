@@ -267,3 +267,75 @@ def test_sharded_checkpoint_is_read_through_its_index(tmp_path):
     with pytest.raises(Exception) as e:
         load_tensors(three, spec)
     assert "weight_map" in str(e.value)
+
+
+# ------------------------------------------------------------------ random weights: the generator and the streamed file
+
+def test_random_elements_depend_on_seed_name_and_index_only():
+    from nanoinfer_amd.weights import random_init as R
+    key = R.tensor_key(3, "model.embed_tokens.weight")
+    whole = R.standard_normal(key, 0, 70000)                     # more than one block of the routine
+    assert whole.dtype.name == "float32"
+    cut = [R.standard_normal(key, s, n) for s, n in ((0, 1), (1, 4999), (5000, 32768), (37768, 32232))]
+    assert (torch.from_numpy(whole) == torch.cat([torch.from_numpy(c) for c in cut])).all()
+    far = R.standard_normal(key, (1 << 33) + 5, 100)             # indices beyond 32 bits
+    assert (far != whole[:100]).any() and abs(float(far.mean())) < 0.5
+    other = R.standard_normal(R.tensor_key(3, "model.norm.weight"), 0, 1000)
+    again = R.standard_normal(R.tensor_key(4, "model.embed_tokens.weight"), 0, 1000)
+    assert (other != whole[:1000]).any() and (again != whole[:1000]).any()
+    # a standard normal: moments, tails, no trace of the neighbour
+    x = torch.from_numpy(R.standard_normal(key, 0, 400000)).double()
+    assert abs(float(x.mean())) < 0.01 and abs(float(x.std()) - 1.0) < 0.01
+    assert abs(float((x ** 4).mean() / x.var() ** 2) - 3.0) < 0.05
+    assert abs(float((x.abs() > 1.959964).double().mean()) - 0.05) < 0.003
+    assert abs(float((x[:-1] * x[1:]).mean())) < 0.01
+    assert float(x.abs().max()) < 6.0
+
+
+def test_random_model_follows_the_architecture_s_rule_and_its_parts(tmp_path):
+    from nanoinfer_amd.weights import random_init as R
+    d = make_random_model(str(tmp_path / "m"), TINY_B, seed=9, dtype="float32", matrix_std=0.5, vector_mean=-2.0)
+    f = SafetensorsFile(os.path.join(d, "model.safetensors"))
+    _, _, spec = read_model_folder(d)
+    assert set(f.names()) == set(expected_tensors(spec))
+    w = f.tensor("model.layers.2.mlp.up_proj.weight")
+    assert abs(float(w.std()) - 0.5) < 0.01
+    assert abs(float(f.tensor("model.layers.1.input_layernorm.weight").mean()) + 2.0) < 0.05
+    # an element is what the generator says for (seed, name, index), whatever the piece it was written in
+    want = R.random_tensor(9, "model.layers.2.mlp.up_proj.weight", tuple(w.shape), 0.0, 0.5)
+    assert torch.equal(w, want)
+    with pytest.raises(TypeError):
+        make_random_model(str(tmp_path / "n"), TINY_B, seed=9, dtype="float32", no_such_field=1.0)
+
+
+def test_streamed_file_equals_the_file_written_whole(tmp_path, monkeypatch):
+    from nanoinfer_amd.weights import random_init as R
+    from nanoinfer_amd.weights.safetensors_io import write_safetensors_streamed
+    whole = make_random_model(str(tmp_path / "whole"), TINY_A, seed=2, dtype="bfloat16")
+    monkeypatch.setattr(R, "PIECE", 1000)                       # every matrix now comes in many pieces
+    pieces = make_random_model(str(tmp_path / "pieces"), TINY_A, seed=2, dtype="bfloat16")
+    a, b = (open(os.path.join(x, "model.safetensors"), "rb").read() for x in (whole, pieces))
+    assert a == b
+    # pieces that do not add up to the tensor, or are of another type, are an error, not a damaged file
+    with pytest.raises(WeightFileError, match="pieces gave"):
+        write_safetensors_streamed(str(tmp_path / "short.safetensors"),
+                                   [("t", torch.float32, (4, 4), lambda: iter([torch.zeros(10)]))])
+    with pytest.raises(WeightFileError, match="piece of type"):
+        write_safetensors_streamed(str(tmp_path / "typed.safetensors"),
+                                   [("t", torch.float32, (4,), lambda: iter([torch.zeros(4, dtype=torch.bfloat16)]))])
+    assert not os.path.exists(str(tmp_path / "short.safetensors"))
+
+
+def test_buffers_that_exporters_write_along_are_ignored_other_extras_are_not(tmp_path):
+    d = make_random_model(str(tmp_path / "m"), TINY_A, seed=1, dtype="float32")
+    cfg_json = json.load(open(os.path.join(d, "config.json")))
+    tensors = dict(SafetensorsFile(os.path.join(d, "model.safetensors")).items())
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.ones(8)
+    ok = write_model_folder(str(tmp_path / "ok"), cfg_json, tensors)
+    _, _, spec = read_model_folder(ok)
+    assert set(load_tensors(ok, spec)) == set(expected_tensors(spec))
+    tensors["model.layers.0.self_attn.q_proj.bias"] = torch.ones(64)
+    bad = write_model_folder(str(tmp_path / "bad"), cfg_json, tensors)
+    with pytest.raises(WeightMismatchError) as e:
+        load_tensors(bad, spec)
+    assert e.value.unexpected == ["model.layers.0.self_attn.q_proj.bias"]

@@ -42,6 +42,39 @@ def test_missing_gpu_tensor_is_refused(K):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_random_weights_kernel_gives_the_bits_of_the_host_routine(K, dtype):
+    """Every element is a function of (key, index): the kernel and numpy agree bit for bit, at
+    any start (also beyond 32 bits) and for mean and deviation of both kinds of tensor."""
+    from nanoinfer_amd.weights import random_init as R
+    for name, start, count, mean, std in (("model.embed_tokens.weight", 0, 300001, 0.0, 0.02),
+                                          ("model.norm.weight", 12345, 70000, 1.0, 0.05),
+                                          ("x", (1 << 35) + 7, 4099, -3.0, 2.5), ("y", 0, 1, 0.0, 1.0)):
+        key = R.tensor_key(5, name)
+        want = R.normal_cpu(key, start, count, mean, std, DT[dtype])
+        got = K.random_normal(torch.empty(count, dtype=DT[dtype], device="cuda"), key, start, mean, std).cpu()
+        assert torch.equal(got.view(torch.int16 if dtype == "bfloat16" else torch.int32),
+                           want.view(torch.int16 if dtype == "bfloat16" else torch.int32)), (name, start)
+    with pytest.raises(K.KernelError):
+        K.random_normal(torch.empty(2, 2, device="cuda"), 1, 0, 0.0, 1.0)
+
+
+def test_large_tensors_of_a_random_model_are_made_on_the_gpu_with_the_same_bits(tmp_path, monkeypatch):
+    from nanoinfer_amd.weights import random_init as R
+    from nanoinfer_amd.weights.loader import make_random_model
+    from tiny_configs import TINY_B
+    cpu = make_random_model(str(tmp_path / "cpu"), TINY_B, seed=8, dtype="bfloat16", device=None)
+    monkeypatch.setattr(R, "GPU_WORTH_IT", 1000)         # now every matrix goes through the kernel
+    monkeypatch.setattr(R, "PIECE", 50000)
+    made = []
+    original = R.normal_gpu
+    monkeypatch.setattr(R, "normal_gpu", lambda *a: (made.append(a[2]), original(*a))[1])
+    gpu = make_random_model(str(tmp_path / "gpu"), TINY_B, seed=8, dtype="bfloat16")
+    assert made and max(made) == 50000
+    assert open(str(tmp_path / "cpu" / "model.safetensors"), "rb").read() == \
+        open(str(tmp_path / "gpu" / "model.safetensors"), "rb").read()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_embedding(K, dtype):
     g = torch.Generator().manual_seed(0)
     table = torch.randn(1003, 70, generator=g).to(DT[dtype])
@@ -211,8 +244,7 @@ def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boo
         K.mfma_attention(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table), tiles, out,
                          H, KVH, hd, 1.0 / math.sqrt(hd), window, nsplit, ws, tile_tokens)
     else:
-        fn = {"token": K.token_attention, "token_wide": functools.partial(K.token_attention, wide=True),
-              "mfma_token": K.mfma_token_attention}[kernel]
+        fn = {"token": K.token_attention, "mfma_token": K.mfma_token_attention}[kernel]
         fn(dev(qkv, DT[dtype]), dev(kpool, DT[dtype]), dev(vpool, DT[dtype]), dev(table),
            dev(torch.tensor(seq_of, dtype=torch.int32)), dev(torch.tensor(positions, dtype=torch.int32)),
            out, H, KVH, hd, 1.0 / math.sqrt(hd), window, nsplit, ws)
@@ -226,7 +258,7 @@ def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boo
                                          (8, 2, 96, 4), (2, 1, 112, 16), (16, 2, 128, 16), (2, 2, 256, 16)])
 def test_attention_head_sizes_and_groups(K, dtype, H, KVH, hd, ps):
     lens, q_lens = [1, 37, 130, 64], [1, 37, 2, 1]
-    for nsplit, kernel in ((1, "token"), (3, "token"), (1, "token_wide"), (2, "token_wide")):
+    for nsplit, kernel in ((1, "token"), (3, "token")):
         out, want, _ = paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, None, hd + nsplit, nsplit, kernel=kernel)
         assert not torch.isnan(out).any(), "a key outside the sequence's own pages was read"
         assert rel(out, want) < KTOL[dtype], (H, KVH, hd, ps, nsplit, kernel)

@@ -54,12 +54,12 @@ def _both(lib, n_tokens, context, nsplit, dtype, seed):
     part_o, part_ml = work[: rows * HD], work[rows * HD:]
     err = lib.ni_token_attention(_ptr(q), H * HD, _ptr(kpool), _ptr(vpool), _ptr(table), table.shape[1], _ptr(seq),
                                  _ptr(pos), _ptr(want), _ptr(part_o), _ptr(part_ml), n_tokens, H, KVH, PAGE, 0, scale,
-                                 nsplit, 0, code, stream)
+                                 nsplit, code, stream)
     assert err == 0
     torch.cuda.synchronize()
     held = torch.cuda.memory_allocated()
     err = lib.ni_token_attention_static(_ptr(q), H * HD, _ptr(kpool), _ptr(vpool), _ptr(table), table.shape[1],
-                                        _ptr(seq), _ptr(pos), _ptr(got), n_tokens, H, KVH, PAGE, 0, scale, nsplit, 0,
+                                        _ptr(seq), _ptr(pos), _ptr(got), n_tokens, H, KVH, PAGE, 0, scale, nsplit,
                                         code, stream)
     assert err == 0
     torch.cuda.synchronize()
@@ -87,7 +87,7 @@ def test_more_than_the_array_holds_is_refused():
     out = torch.zeros(n_tokens, H * HD, device=q.device)
     err = lib.ni_token_attention_static(_ptr(q), H * HD, _ptr(kpool), _ptr(vpool), _ptr(table), table.shape[1],
                                         _ptr(seq), _ptr(pos), _ptr(out), n_tokens, H, KVH, PAGE, 0,
-                                        ctypes.c_float(0.125), nsplit, 0, 0,
+                                        ctypes.c_float(0.125), nsplit, 0,
                                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
     assert err == -3
