@@ -17,6 +17,7 @@ from ..weights.random_init import InitRule
 def build_spec(cfg: LlamaConfig) -> ModelSpec:
     d = cfg.hidden_size
     scaling = None if cfg.rope_scaling is None else {
+        "kind": cfg.rope_scaling.rope_type,
         "factor": cfg.rope_scaling.factor,
         "low_freq_factor": cfg.rope_scaling.low_freq_factor,
         "high_freq_factor": cfg.rope_scaling.high_freq_factor,

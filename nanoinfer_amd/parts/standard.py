@@ -84,32 +84,63 @@ class RMSNorm(Part):
 
 # ------------------------------------------------------------------ position
 
+ROPE_SCALINGS = {}     # kind -> rule(frequencies float32 [pairs], params dict) -> frequencies float32 [pairs]
+
+
+def register_rope_scaling(kind: str):
+    """``@register_rope_scaling("<kind>")`` over a function ``(freqs, params) -> freqs`` (numpy float32):
+    another way to stretch the rotation to longer contexts is another entry here, named by the
+    ``kind`` of the ``scaling`` parameter of a ``rope`` position part."""
+    def deco(fn):
+        ROPE_SCALINGS[kind] = fn
+        return fn
+    return deco
+
+
+@register_rope_scaling("llama3")
+def llama3_scaling(freqs: np.ndarray, params: dict) -> np.ndarray:
+    """Long waves divided by ``factor``, short ones kept, a linear blend between, in float32
+    arithmetic (src/op/kernels/cuda/rope_kernel.cu:108-127, src/op/kernels/cpu/rope_kernel.cpp:121-139)."""
+    f32 = np.float32
+    factor, low, high = f32(params["factor"]), f32(params["low_freq_factor"]), f32(params["high_freq_factor"])
+    orig = f32(params["original_max_position_embeddings"])
+    out = freqs.astype(f32).copy()
+    for p in range(out.shape[0]):
+        freq = out[p]
+        wavelen = f32(f32(2.0) * f32(math.pi) / freq)
+        if wavelen >= f32(orig / low):
+            freq = f32(freq / factor)
+        elif wavelen > f32(orig / high):
+            smooth = f32(f32(orig / wavelen - low) / f32(high - low))
+            freq = f32(f32(f32(1.0) - smooth) * freq / factor + smooth * freq)
+        out[p] = freq
+    return out
+
+
 def rope_inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[dict]) -> np.ndarray:
-    """Frequency of each rotated pair in float32 arithmetic, with llama3 scaling when given:
-    long waves divided by ``factor``, short ones kept, a linear blend between
-    (src/op/kernels/cuda/rope_kernel.cu:108-127, src/op/kernels/cpu/rope_kernel.cpp:121-139)."""
+    """Frequency of each rotated pair, ``theta^(-2p/rotary_dim)`` in float32 arithmetic
+    (src/op/kernels/cuda/rope_kernel.cu:103-106), then the scaling rule that ``scaling["kind"]``
+    names, if any, applied with the other entries of ``scaling`` as its parameters."""
     f32 = np.float32
     half = rotary_dim // 2
     out = np.empty(half, dtype=f32)
     for p in range(half):
-        freq = f32(1.0) / f32(np.power(f32(theta), f32(f32(2 * p) / f32(rotary_dim)), dtype=f32))
-        if scaling is not None:
-            factor, low, high = f32(scaling["factor"]), f32(scaling["low_freq_factor"]), f32(scaling["high_freq_factor"])
-            orig = f32(scaling["original_max_position_embeddings"])
-            wavelen = f32(f32(2.0) * f32(math.pi) / freq)
-            if wavelen >= f32(orig / low):
-                freq = f32(freq / factor)
-            elif wavelen > f32(orig / high):
-                smooth = f32(f32(orig / wavelen - low) / f32(high - low))
-                freq = f32(f32(f32(1.0) - smooth) * freq / factor + smooth * freq)
-        out[p] = freq
+        out[p] = f32(1.0) / f32(np.power(f32(theta), f32(f32(2 * p) / f32(rotary_dim)), dtype=f32))
+    if scaling is not None:
+        kind = scaling.get("kind")
+        if kind not in ROPE_SCALINGS:
+            raise ValueError(f"rotation scaling of kind {kind!r} is not registered; known: {sorted(ROPE_SCALINGS)}")
+        out = np.asarray(ROPE_SCALINGS[kind](out, scaling), dtype=f32)
+        if out.shape != (half,):
+            raise ValueError(f"rotation scaling {kind!r} returned {out.shape} frequencies for {half} pairs")
     return out
 
 
 @register_part("position", "rope")
 class RotaryPosition(Part):
-    """Rotation of pairs by ``pos * f_p``.  params: rotary_dim, theta, scaling (dict or None),
-    max_positions.  One table per distinct set of constants is shared by all layers."""
+    """Rotation of pairs by ``pos * f_p``.  params: rotary_dim, theta, max_positions, scaling (None,
+    or a dict with the ``kind`` of a registered rule and that rule's parameters).  One table per
+    distinct set of constants is shared by all layers."""
 
     graph_safe = True
 

@@ -4,6 +4,7 @@ import functools
 import math
 import random
 
+import numpy as np
 import pytest
 import torch
 
@@ -109,15 +110,20 @@ def test_add_rmsnorm(K, dtype, d):
     assert rel(out2, P.rmsnorm(total[rows.long()], w, eps)) < KTOL[dtype]
 
 
-def test_rope_table_matches_plain(K):
-    from nanoinfer_amd.parts.standard import rope_inverse_frequencies
-    scaling = {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": 128}
-    for hd, theta, sc in [(48, 10000.0, None), (64, 500000.0, scaling), (16, 1234.5, scaling)]:
-        inv = rope_inverse_frequencies(hd, theta, sc)
-        assert (inv == P.rope_frequencies(hd, theta, sc)).all()          # bit for bit: same float32 steps
-        cos, sin = K.rope_table(dev(torch.from_numpy(inv)), 3000)
-        s, c = P.rope_tables(range(3000), inv)
-        assert float((sin.double().cpu() - s).abs().max()) < 2e-6 and float((cos.double().cpu() - c).abs().max()) < 2e-6
+def test_rope_table_holds_the_sines_of_position_times_frequency(K):
+    """The table against numbers: cos and sin of pos * f in float64, for frequencies that come from
+    nowhere but this test (a geometric run, and the worked llama3 numbers of tests/rope_literals.py)."""
+    from rope_literals import CASES
+    runs = [np.array([1.0 / 3.7 ** p for p in range(24)], dtype=np.float32)]
+    runs += [np.array([value for _, value in pairs.values()], dtype=np.float32) for _, _, _, pairs in CASES]
+    for inv in runs:
+        n = 3000
+        cos, sin = K.rope_table(dev(torch.from_numpy(inv)), n)
+        assert cos.shape == sin.shape == (n, len(inv))
+        angle = (np.arange(n, dtype=np.float32)[:, None] * inv[None, :]).astype(np.float64)     # the product is float32
+        assert float((sin.double().cpu() - torch.from_numpy(np.sin(angle))).abs().max()) < 2e-6
+        assert float((cos.double().cpu() - torch.from_numpy(np.cos(angle))).abs().max()) < 2e-6
+    assert bool((sin[0] == 0).all()) and bool((cos[0] == 1).all())
 
 
 def plain_rotate_half(x, sin, cos, rot):

@@ -72,7 +72,7 @@ def test_position_part_shares_one_table():
     from nanoinfer_amd.parts.standard import build_part
     rt = runtime("float32")
     sc = dict(TINY_B["rope_scaling"])
-    sc.pop("rope_type")
+    sc["kind"] = sc.pop("rope_type")
     spec = PartSpec("rope", {"rotary_dim": 32, "theta": 500000.0, "scaling": sc, "max_positions": 300})
     a = build_part("position", spec, {}, rt)
     b = build_part("position", spec, {}, rt)

@@ -102,6 +102,37 @@ def test_rope_llama3_scaling_branches():
     assert abs(math.sin(float(f[-1]))) < 0.1 and f[-1] == pytest.approx(1 / 500000 ** (62 / 64) / 32, rel=1e-5)
 
 
+def test_rope_llama3_frequencies_as_numbers():
+    """The three bands, and above all the blend of the middle one, against numbers worked out from
+    the rule independently (tests/rope_literals.py): a blend the other way round, a band edge
+    moved to the other constant or a factor applied twice all miss them by far more than 1e-5."""
+    from rope_literals import CASES
+    for hd, theta, scaling, pairs in CASES:
+        f = P.rope_frequencies(hd, theta, scaling)
+        assert f.dtype == np.float32 and f.shape == (hd // 2,)
+        for p, (band, value) in pairs.items():
+            assert float(f[p]) == pytest.approx(value, rel=1e-5), (hd, p, band)
+    assert {band for _, _, _, pairs in CASES for band, _ in pairs.values()} == {"short", "middle", "long"}
+
+
+def test_rope_llama3_blend_meets_both_neighbours_at_the_band_edges():
+    """With a factor other than 1: a pair whose wavelength lies a hair inside the middle band has
+    nearly the frequency of a pair a hair outside it, at the long edge (f / factor) and at the short
+    edge (f).  The wavelength of pair 3 is held fixed and the band is moved across it."""
+    hd, theta, p = 32, 10000.0, 3
+    base = float(P.rope_frequencies(hd, theta, None)[p])
+    wl = 2 * math.pi / base
+    for edge, expect in (("long", base / 8.0), ("short", base)):
+        got = []
+        for nudge in (1 - 2e-4, 1 + 2e-4):
+            # long edge: wl = orig / low; short edge: wl = orig / high
+            orig = wl * (1.0 if edge == "long" else 4.0) * nudge
+            s = {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": orig}
+            got.append(float(P.rope_frequencies(hd, theta, s)[p]))
+        assert got[0] == pytest.approx(expect, rel=2e-3) and got[1] == pytest.approx(expect, rel=2e-3), (edge, got)
+        assert got[0] != got[1]                      # one of them really is in the middle band
+
+
 def test_rope_invariants():
     g = torch.Generator().manual_seed(2)
     hd = 16
