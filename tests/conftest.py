@@ -22,3 +22,15 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter):
+    """The worst row-wise error the comparisons with the plain implementation have met, for the record."""
+    try:
+        import gpu_common
+    except Exception:
+        return
+    seen = {k: v for k, v in gpu_common.worst_row_seen.items() if v}
+    if seen:
+        terminalreporter.write_line("worst row of any comparison with the plain implementation, relative to the row's "
+                                    "largest logit: " + ", ".join(f"{k} {v:.2e}" for k, v in seen.items()))

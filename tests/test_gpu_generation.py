@@ -181,12 +181,15 @@ def test_bfloat16_generation_runs_and_agrees_on_clear_choices():
     got = eng.generate([prompt], max_new_tokens=8, params=SamplingParams.greedy())[0].tokens
     config, tensors = P.read_model_folder(folder)
     toks = list(prompt)
+    compared = 0
     for t in got:
         l = P.forward(config, tensors, toks)[-1]
         top = torch.topk(l, 2).values
         if float(top[0] - top[1]) > 0.05 * float(l.abs().max()):
             assert t == int(l.argmax())
+            compared += 1
         toks.append(t)
+    assert compared >= 6, f"only {compared} of {len(got)} choices were clear enough to compare"
 
 
 def test_command_line(tmp_path):

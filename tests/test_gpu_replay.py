@@ -530,3 +530,33 @@ def test_a_later_wave_of_requests_decodes_in_runs_across_a_recording_s_bounds(pa
             single.release(rid)
         runs.cache.check()
     assert runs.cache.free_pages() == runs.cache.num_pages
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_long_sequences_reach_the_larger_tiles_and_the_key_runs_of_prompt_attention(dtype, monkeypatch):
+    """Configuration D (32 query heads on 8): a prompt of 4,200 tokens in one step takes the tiles
+    of two blocks a wavefront; a lone portion of 512 tokens that starts 1,100 tokens into its
+    sequence takes two-block tiles with its keys cut into runs.  What the attention was asked for is
+    noted, so that the test fails if these paths are no longer the ones taken (bfloat16; the float32
+    kernel has one tile size and cuts keys for few tiles only)."""
+    from nanoinfer_amd import kernels as K
+    name = "D"
+    folder = model_folder(name)
+    vocab = ALL[name]["vocab_size"]
+    asked, original = [], K.mfma_attention
+    monkeypatch.setattr(K, "mfma_attention", lambda *a, **kw: (asked.append((a[0].shape[0], a[11], a[13])), original(*a, **kw))[1])
+    small = K.mfma_tile_tokens(32, 4, dtype=torch.bfloat16 if dtype == "bfloat16" else torch.float32)
+    long_prompt = random_tokens(vocab, 4200, 41)
+    deep = random_tokens(vocab, 1100 + 512 + 30, 42)
+    steps = [([("long", list(long_prompt), [0, 1, 2047, 2048, 4095, 4199])], ["long"]),
+             ([("deep", list(deep[:1100]), [1099])], []),
+             ([("deep", list(deep[1100:1612]), [0, 255, 511])], []),
+             ([("deep", list(deep[1612:]), list(range(30)))], ["deep"])]
+    got, _ = run_in_process(folder, dtype, 16, steps, 4200 + 64)
+    compare(got, {"long": long_prompt, "deep": deep}, folder, dtype, "configuration D")
+    by_tokens = {t: (nsplit, tile) for t, nsplit, tile in asked}
+    if dtype == "bfloat16":
+        assert by_tokens[4200] == (1, 2 * small)
+        assert by_tokens[512] == (4, 2 * small)
+    else:
+        assert by_tokens[4200][1] == small

@@ -32,6 +32,18 @@ TINY_C = {
 }
 
 
+# many heads on few kv heads and positions for long sequences: with 32 query heads a lone portion of
+# 512 tokens far into its sequence, or a prompt of 4,096, reaches the attention's larger tiles and key runs
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 96, "num_hidden_layers": 1, "num_attention_heads": 32, "num_key_value_heads": 8,
+    "head_dim": 32, "intermediate_size": 112, "vocab_size": 300, "rms_norm_eps": 2e-5,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 16.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 1024},
+    "max_position_embeddings": 8192, "tie_word_embeddings": True, "hidden_act": "silu",
+}
+
 
 def _family(hidden, heads, kv_heads, head_dim, inter, vocab, factor, tied):
     return {
@@ -54,4 +66,4 @@ FAMILY_3B = _family(3072, 24, 8, 128, 8192, 16033, 32.0, True)
 FAMILY_8B = _family(4096, 32, 8, 128, 14336, 16033, 8.0, False)
 
 TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-ALL = {**TINY, "1B": FAMILY_1B, "3B": FAMILY_3B, "8B": FAMILY_8B}
+ALL = {**TINY, "D": TINY_D, "1B": FAMILY_1B, "3B": FAMILY_3B, "8B": FAMILY_8B}
