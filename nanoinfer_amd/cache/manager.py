@@ -119,16 +119,22 @@ class ReservationPlan:
 class KVCacheManager:
     """Pages and state slots for the caches of one model.
 
-    ``needs[c]`` is what cache ``c`` wants.  ``num_pages`` is the size of every group's pool, in
-    pages of ``page_size`` tokens.  ``device=None`` keeps the books without allocating pools.
+    ``needs[c]`` is what cache ``c`` wants.  ``num_pages`` is the size of the pool of a group that
+    keeps all keys, in pages of ``page_size`` tokens.  A group that keeps a window of n keys never
+    holds more of a request than its window and the tokens of one step: when ``max_step_tokens``
+    (the most tokens one request brings to one step) is given, such a group's pool is only as
+    large as ``max_requests`` requests can fill, and no larger than ``num_pages``; without it every
+    group gets ``num_pages``.  ``device=None`` keeps the books without allocating pools.
     """
 
     def __init__(self, needs: Dict[int, CacheNeed], page_size: int, num_pages: int, max_requests: int,
-                 dtype: torch.dtype = torch.float32, device: Optional[torch.device] = None):
+                 dtype: torch.dtype = torch.float32, device: Optional[torch.device] = None,
+                 max_step_tokens: Optional[int] = None):
         if page_size < 1:
             raise ValueError(f"page_size must be at least 1, got {page_size}")
         self.page_size = int(page_size)
         self.num_pages = int(num_pages)
+        self.max_step_tokens = None if max_step_tokens is None else int(max_step_tokens)
         self.dtype = dtype
         self.device = device
         self.groups: List[KVGroup] = []
@@ -143,7 +149,7 @@ class KVCacheManager:
                 if gi is None:
                     gi = len(self.groups)
                     by_need[need.kv] = gi
-                    self.groups.append(KVGroup(need.kv, [], self.page_size, BlockManager(self.num_pages)))
+                    self.groups.append(KVGroup(need.kv, [], self.page_size, BlockManager(self.pages_of_group(need.kv, max_requests))))
                 self.groups[gi].cache_ids.append(cid)
                 self.group_of_cache[cid] = gi
             if need.state is not None:
@@ -152,12 +158,22 @@ class KVCacheManager:
         self._tokens: Dict[Hashable, int] = {}
         if device is not None:
             for g in self.groups:
-                shape = (self.num_pages, g.need.kv_heads, self.page_size, g.need.head_dim)
+                shape = (g.pages.num_pages, g.need.kv_heads, self.page_size, g.need.head_dim)
                 for cid in g.cache_ids:
                     g.kpools[cid] = torch.zeros(shape, dtype=dtype, device=device)
                     g.vpools[cid] = torch.zeros(shape, dtype=dtype, device=device)
             for cid, sn in self.state_needs.items():
                 self.state[cid] = torch.zeros((max_requests,) + tuple(sn.shape), dtype=sn.dtype, device=device)
+
+    def pages_of_group(self, need: KVNeed, max_requests: int) -> int:
+        """Pages in the pool of a group with this need.  A windowed group holds of one request at most
+        the pages that its window and one step's tokens touch: before a step the keys of the window,
+        during it the step's tokens as well, and a run of n keys touches at most
+        ``ceil(n / page_size) + 1`` pages."""
+        if need.window is None or self.max_step_tokens is None:
+            return self.num_pages
+        per_request = -(-(int(need.window) + self.max_step_tokens) // self.page_size) + 1
+        return min(self.num_pages, int(max_requests) * per_request)
 
     # ---------------------------------------------------------------- queries
     def has(self, request: Hashable) -> bool:
@@ -181,6 +197,12 @@ class KVCacheManager:
 
     def min_free_pages(self) -> int:
         return min((g.pages.num_free for g in self.groups), default=self.num_pages)
+
+    def pool_bytes(self) -> int:
+        """Bytes of all key and value pools together."""
+        el = torch.empty(0, dtype=self.dtype).element_size()
+        return sum(2 * len(g.cache_ids) * g.pages.num_pages * g.need.kv_heads * self.page_size * g.need.head_dim * el
+                   for g in self.groups)
 
     def utilization(self) -> float:
         return max((g.pages.utilization() for g in self.groups), default=0.0)
@@ -211,8 +233,12 @@ class KVCacheManager:
         return ReservationPlan(self)
 
     def max_tokens_per_request(self) -> int:
-        """The longest request the pools can ever hold (it then holds every page of a group)."""
-        return self.num_pages * self.page_size
+        """The longest request the pools can ever hold: it then holds every page of a group that keeps
+        all keys.  (A model whose groups all keep windows is bounded by its positions alone.)"""
+        full = [g.pages.num_pages for g in self.groups if g.need.window is None]
+        if full:
+            return min(full) * self.page_size
+        return self.num_pages * self.page_size if not self.groups else 1 << 60
 
     # ---------------------------------------------------------------- changes
     def reserve(self, request: Hashable, total_tokens: int) -> bool:

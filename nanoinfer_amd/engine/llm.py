@@ -43,7 +43,8 @@ class Engine:
             from .runner import ModelRunner
             runner = ModelRunner(model_dir, dtype=self.config.dtype, page_size=self.config.block_size,
                                  max_tokens=self.config.block_size * self.config.num_cache_blocks,
-                                 max_requests=self.config.max_sequences)
+                                 max_requests=self.config.max_sequences,
+                                 max_step_tokens=min(self.config.prefill_chunk_size, self.config.max_num_batched_tokens))
         if sampler is None:
             from ..sampling.sampler import Sampler
             sampler = Sampler(runner.device)

@@ -56,7 +56,7 @@ class Model:
         """Run the step described by ``ctx``; ``layer_cache(cache_id, writes)`` gives the
         :class:`LayerCache` of an entry of the order.  Returns float32 logits of ``ctx.logit_rows``
         (None when no row is wanted; the caches are filled all the same)."""
-        h = self.embedding.forward(ctx.token_ids)
+        h = self.embedding.forward(ctx.token_ids, ctx)
         pending = None
         for run in self.spec.order:
             cache: LayerCache = layer_cache(run.cache, run.writes_cache)

@@ -152,7 +152,7 @@ class ModelRunner:
 
     def __init__(self, model_dir: str, dtype: str = "bfloat16", page_size: int = 16, max_tokens: int = 4096,
                  max_requests: int = 64, device: Optional[torch.device] = None, use_graphs: bool = True,
-                 warm_up: bool = True):
+                 warm_up: bool = True, max_step_tokens: Optional[int] = None):
         self.device = device or K.require_gpu()
         torch_dtype = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
                        "float32": torch.float32, "fp32": torch.float32}.get(dtype)
@@ -166,8 +166,11 @@ class ModelRunner:
         del tensors
         self.page_size = int(page_size)
         num_pages = (int(max_tokens) + self.page_size - 1) // self.page_size
+        # with a bound on the tokens one request brings to a step, pools of windowed layers are only as
+        # large as their windows need; a longer portion is then refused
+        self.max_step_tokens = None if max_step_tokens is None else int(max_step_tokens)
         self.cache = KVCacheManager(self.model.cache_needs(), self.page_size, num_pages, max_requests,
-                                    dtype=torch_dtype, device=self.device)
+                                    dtype=torch_dtype, device=self.device, max_step_tokens=self.max_step_tokens)
         self.vocab_size = self.spec.vocab_size
         self.max_positions = self.model.max_positions
         self.eos_token_ids = tuple(self.spec.eos_token_ids)
@@ -181,7 +184,8 @@ class ModelRunner:
         """One short prompt and one decode step of a request of the runner's own, run eagerly and given
         back: the code objects of the kernels and the matrix library's set-up are loaded while the model
         is, not during the first request (on the 1B shape that is 0.2 s of its first step)."""
-        n = min(128, self.max_positions - 1, (self.cache.min_free_pages() - 1) * self.page_size)
+        n = min(128, self.max_positions - 1, (self.cache.min_free_pages() - 1) * self.page_size,
+                self.max_step_tokens or 128)
         if n < 2:
             return
         me = ("warm-up", id(self))
@@ -258,6 +262,7 @@ class ModelRunner:
         seen = set()
         vocab = self.vocab_size
         limit = self.model.max_positions
+        step_limit = getattr(self, "max_step_tokens", None)
         totals = []
         for e in entries:
             if e.request in seen:
@@ -267,6 +272,9 @@ class ModelRunner:
             n = len(toks)
             if n == 0:
                 raise StepError(f"request {e.request!r} brings no tokens")
+            if step_limit is not None and n > step_limit:
+                raise StepError(f"request {e.request!r} brings {n} tokens; the pools were sized for at most "
+                                f"{step_limit} of one request in a step")
             if not (0 <= min(toks) and max(toks) < vocab):
                 bad = next(t for t in toks if not 0 <= int(t) < vocab)
                 raise StepError(f"token id {bad} of request {e.request!r} is outside the vocabulary of {vocab}")

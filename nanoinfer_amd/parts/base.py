@@ -4,7 +4,7 @@ A part is built from its :class:`~nanoinfer_amd.config.spec.PartSpec` (kind, con
 names), the checkpoint tensors it asked for, and a :class:`Runtime` (compute type, device).  It
 knows nothing of the model it sits in.  Interfaces, by family:
 
-``embedding``     ``forward(token_ids[T] int32) -> h[T, d] float32``
+``embedding``     ``forward(token_ids[T] int32, ctx) -> h[T, d] float32`` (``ctx.positions`` for a learned position table)
 ``norm``          ``forward(h float32, pending | None, rows=None) -> x`` in the compute type;
                   without ``rows`` it first adds ``pending`` into ``h`` (the residual sum)
 ``position``      ``tables() -> (cos, sin) | None`` for the mixer that owns it

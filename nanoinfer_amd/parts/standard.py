@@ -18,10 +18,20 @@ from ..registry import get_part, register_part
 from .base import CacheNeed, KVNeed, LayerCache, Part, Runtime, WeightRequest, pending_for
 
 
+class PartWeights(dict):
+    """The tensors a part asked for, by their logical names; ``checkpoint`` is the whole set by
+    checkpoint name, which a part hands on to :func:`build_part` for a part it holds inside
+    itself (an attention's position encoding)."""
+
+    def __init__(self, own: Dict[str, torch.Tensor], checkpoint: Dict[str, torch.Tensor]):
+        super().__init__(own)
+        self.checkpoint = checkpoint
+
+
 def build_part(family: str, spec: PartSpec, tensors: Dict[str, torch.Tensor], rt: Runtime) -> Part:
     """Instantiate the registered class for ``spec.kind`` with the tensors it asked for."""
     cls = get_part(family, spec.kind)
-    return cls(spec, {logical: tensors[name] for logical, name in spec.weights.items()}, rt)
+    return cls(spec, PartWeights({logical: tensors[name] for logical, name in spec.weights.items()}, tensors), rt)
 
 
 def requests_of(family: str, spec: PartSpec) -> List[WeightRequest]:
@@ -47,7 +57,7 @@ class TableEmbedding(Part):
         self.hidden_size = int(spec.params["hidden_size"])
         self.weight = rt.matrix(spec.weights["weight"], weights["weight"])
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+    def forward(self, token_ids: torch.Tensor, ctx=None) -> torch.Tensor:
         out = torch.empty(token_ids.shape[0], self.hidden_size, dtype=torch.float32, device=self.rt.device)
         return K.embedding(token_ids, self.weight, out)
 
@@ -196,7 +206,8 @@ class Attention(Part):
         p, w = spec.params, spec.weights
         d, H, KVH, hd = p["hidden_size"], p["num_heads"], p["num_kv_heads"], p["head_dim"]
         return [WeightRequest(w["q"], (H * hd, d)), WeightRequest(w["k"], (KVH * hd, d)),
-                WeightRequest(w["v"], (KVH * hd, d)), WeightRequest(w["o"], (d, H * hd))]
+                WeightRequest(w["v"], (KVH * hd, d)), WeightRequest(w["o"], (d, H * hd))] + \
+            requests_of("position", p["position"])       # a position encoding may have tensors of its own
 
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
@@ -211,7 +222,7 @@ class Attention(Part):
         self.window = None if p.get("window") is None else int(p["window"])
         K.attention_lib(self.hd)  # refuses an unsupported head size now, not at the first step
         pos_spec: PartSpec = p["position"]
-        self.position = get_part("position", pos_spec.kind)(pos_spec, {}, rt)
+        self.position = build_part("position", pos_spec, getattr(weights, "checkpoint", {}), rt)
         names = spec.weights
         self.w_qkv = rt.weight("|".join((names["q"], names["k"], names["v"])),
                                torch.cat([weights["q"], weights["k"], weights["v"]], dim=0))

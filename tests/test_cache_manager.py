@@ -198,3 +198,37 @@ def test_random_orders_keep_the_books(seed):
         m.release(rid)
     m.check()
     assert all(g.pages.num_free == g.pages.num_pages for g in m.groups) and m.slots.num_free == 4
+
+
+def test_a_windowed_group_s_pool_is_sized_by_its_window_and_is_never_the_one_that_runs_out():
+    """With a bound on the tokens one request brings to a step, the pool of a windowed group holds
+    what ``max_requests`` windows and steps need, not the whole context: every request can then
+    always take its step's pages there, however long it grows, if the pages the window has passed
+    are given back after every step."""
+    import random
+
+    from nanoinfer_amd.parts.base import CacheNeed, KVNeed
+    page, window, step_tokens, requests = 4, 10, 7, 3
+    m = KVCacheManager({0: CacheNeed(kv=KVNeed(2, 16)), 1: CacheNeed(kv=KVNeed(2, 16, window=window))}, page, 400, requests,
+                       max_step_tokens=step_tokens)
+    full = next(g for g in m.groups if g.need.window is None)
+    windowed = next(g for g in m.groups if g.need.window == window)
+    assert full.pages.num_pages == 400
+    assert windowed.pages.num_pages == requests * (-(-(window + step_tokens) // page) + 1) == 18
+    assert m.max_tokens_per_request() == 400 * page
+    rng = random.Random(3)
+    held = {r: 0 for r in "abc"}
+    for _ in range(600):
+        r = rng.choice("abc")
+        n = rng.randint(1, step_tokens)
+        if held[r] + n > 120 * page // 3:          # stay inside the pool that keeps all keys
+            m.release(r)
+            held[r] = 0
+            continue
+        assert m.reserve(r, held[r] + n), "the windowed pool ran out"
+        held[r] += n
+        m.release_passed(r, held[r])
+        m.check()
+    # without the bound every group gets the whole pool
+    m2 = KVCacheManager({0: CacheNeed(kv=KVNeed(2, 16, window=window))}, page, 400, requests)
+    assert m2.groups[0].pages.num_pages == 400 and m2.max_tokens_per_request() == 1 << 60
