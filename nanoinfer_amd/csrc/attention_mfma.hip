@@ -213,8 +213,11 @@ void mfma_attention_kernel(
         constexpr int TBL_MAX = 1024;
         __shared__ int32_t tbl[TBL_MAX];
         int key_lo = 0, key_hi = 0, lp0 = 0;              // keys of the current segment, and its first page
+        // the first key any row of the tile may read: keys before it (the steps start at a multiple of
+        // KSTEP) may lie in pages that a window has passed and given back, and are never loaded
+        const int tile_lo = window > 0 ? max(0, tile.pos0 + 1 - window) : 0;
         auto row_address = [&](int key) -> size_t {       // offset of key's row for kv head g, key clamped into the segment
-            const int kc = min(max(key, key_lo), key_hi);
+            const int kc = min(max(key, max(key_lo, tile_lo)), key_hi);
             const int page = tbl[page_of(kc) - lp0];
             // the row's number fits 32 bits (the host checks the pool's size); one widening multiply makes the offset
             const uint32_t row = (static_cast<uint32_t>(max(page, 0)) * KVH + g) * page_size + slot_of(kc);
@@ -519,7 +522,8 @@ __global__ __launch_bounds__(DEC_WAVES * WAVE) void mfma_decode_kernel(
     __shared__ int32_t tbl[TBL_MAX];
     int key_lo = 0, key_hi = 0, lp0 = 0;
     auto row_address = [&](int key) -> size_t {
-        const int kc = min(max(key, key_lo), key_hi);
+        // clamped to keys the token may read: those before `lo` may lie in pages already given back
+        const int kc = min(max(key, max(key_lo, lo)), key_hi);
         const int page = tbl[page_of(kc) - lp0];
         // the row's number fits 32 bits (the host checks the pool's size); one widening multiply makes the offset
         const uint32_t row = (static_cast<uint32_t>(max(page, 0)) * KVH + g) * page_size + slot_of(kc);

@@ -8,7 +8,7 @@
 // upper set still holds the mass top_p (sums).  Equal logits at a
 // threshold are kept together.  The draw walks the kept tokens in vocabulary order and takes
 // the first whose cumulative mass reaches u * total (src/op/kernels/cuda/sampling_kernel.cu:330-398);
-// u in (0, 1] comes from the host, which derives it from (seed, request, step).
+// u in (0, 1] comes from the host, which derives it from (seed, tokens the request has generated so far).
 #include "common.h"
 
 #include <type_traits>

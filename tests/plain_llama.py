@@ -1,7 +1,7 @@
 """A plain, slow Llama forward: whole sequences, no cache, float64, one function per part.
 
 This is the oracle of the test-suite.  It is written from the formulas of the
-reference (file:line of /root/reference cited at every function), shares no code
+reference (cited at every function as file:line from the reference's root), shares no code
 with ``nanoinfer_amd`` and reads a model folder with the ``safetensors`` package
 and ``json`` only.
 

@@ -231,6 +231,12 @@ def paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, window, seed, nsplit, boo
             vpool[ids[at], :, :hi - lo] = v[lo:hi].transpose(0, 1)
             at += 1
         ks.append(k), vs.append(v), qs.append(q)
+        if window:
+            # keys that the window of the step's first query has passed: their pages may have been given
+            # back and hold anything; here NaN, so that a kernel that as much as multiplies them by zero shows
+            for i in range(max(0, n - q_lens[b] + 1 - window)):
+                kpool[int(table[b, i // ps]), :, i % ps] = float("nan")
+                vpool[int(table[b, i // ps]), :, i % ps] = float("nan")
         for i in range(n - q_lens[b], n):
             seq_of.append(b), positions.append(i)
     T = len(seq_of)
