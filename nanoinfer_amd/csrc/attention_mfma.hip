@@ -38,8 +38,26 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));    // 16 bytes tha
 #define KSTEP 32
 #define MA_WAVES 4
 #define NEG_BIG (-1.0e30f)
-#define KPAD 8   // elements of padding per staged row of K, for the same reason as VPAD
-#define VPAD 8   // elements of padding per staged row of V^T: the sixteen rows of a 16-byte read fall on different banks
+#define KPAD 8   // elements of padding per staged row of K: the sixteen rows of a 16-byte read fall on different banks
+#define VPAD 8   // elements of padding per staged row of V: the eight rows that half a wavefront reads at a time in a
+                 // transposing read (32 bytes of each) fall on different banks
+
+// V^T as the A operand of the second product, read from a V tile that lies in LDS as it lies in the
+// cache ([key][dim], rows of `row_elems` elements): gfx950's transposing read hands lane (r, kg) the
+// four elements V[key0 + 4*kg + i][dim0 + r], i = 0..3, when lane (r, kg) gives the address of
+// V[key0 + 4*kg + r/4][dim0 + 4*(r%4)] (within sixteen lanes it transposes the 4 x 16 block that four
+// rows of 32 bytes make).  Two reads, for the 16-key halves of a step, give the eight keys of a lane
+// in the order of its eight scores.  (Before, V was turned round on its way into LDS, with eight
+// 2-byte writes for every 16 bytes loaded: a third of the prompt kernel's LDS time.)
+typedef short shortx4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 read_v_operand(const uint16_t* tile, int row_elems, int dim0, int r, int kg) {
+    typedef __attribute__((address_space(3))) shortx4_t* lds_ptr;
+    const uint16_t* at = tile + (4 * kg + (r >> 2)) * row_elems + dim0 + 4 * (r & 3);
+    const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(at));
+    const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(at + 16 * row_elems));
+    const uint2 a = __builtin_bit_cast(uint2, lo), b = __builtin_bit_cast(uint2, hi);
+    return make_uint4(a.x, a.y, b.x, b.y);
+}
 
 struct QTile { int32_t seq, row0, ntok, pos0; };   // tokens row0..row0+ntok-1 of the batch, positions pos0..
 
@@ -147,10 +165,10 @@ void mfma_attention_kernel(
     constexpr int MA_THREADS = MA_WAVES * WAVE;
     constexpr int KK = HD / 32;              // k steps of the first product
     constexpr int DT = HD / 16;              // 16-wide tiles of the head dimension in the output
-    constexpr int VROW = KSTEP + VPAD;
+    constexpr int VROW = HD + VPAD;
     constexpr int KROW = HD + KPAD;
     __shared__ __attribute__((aligned(16))) uint16_t ksm[2][KSTEP][KROW];  // K of a step: [key][dim]
-    __shared__ __attribute__((aligned(16))) uint16_t vs[2][HD][VROW];      // V^T of a step: [dim][key, in the lanes' order]
+    __shared__ __attribute__((aligned(16))) uint16_t vs[2][KSTEP][VROW];   // V of a step, as it lies in the cache: [key][dim]
 
     // The launch has as many workgroups as the chip holds at once, and the tiles come sorted by the
     // number of keys they have to walk, longest first.  Workgroup w takes tiles w, 2P-1-w, 2P+w, ...
@@ -248,11 +266,9 @@ void mfma_attention_kernel(
         }
 
         // Staging of a step's 32 keys: a thread loads 8 dims (16 bytes) of one key's K row and of its V
-        // row.  K goes to LDS as it is, rows padded so that the sixteen rows of a 16-byte read fall on
-        // different banks.  V is written transposed, at the column where the lanes of the second
-        // product expect that key: lane group kg reads the eight keys {t*16 + kg*4 + i} as one 16-byte
-        // row piece [kg*8 + t*4 + i].  A wavefront covers all 32 keys and two 8-dim pieces, which
-        // spreads its 2-byte writes over the banks.
+        // row, neighbouring threads neighbouring pieces of a row.  Both go to LDS as they are, rows
+        // padded against bank conflicts of the reads; the second product's operand is taken from the V
+        // tile by transposing reads (read_v_operand).
         constexpr int PIECES = HD / 8;
         constexpr int ITEMS = KSTEP * PIECES;
         constexpr int PER_THREAD = (ITEMS + MA_THREADS - 1) / MA_THREADS;
@@ -262,33 +278,29 @@ void mfma_attention_kernel(
 #pragma unroll
             for (int i = 0; i < PER_THREAD; ++i) {
                 const int item = (tid + i * MA_THREADS) % ITEMS;
-                at[i] = row_address(ks + item % KSTEP) + (item / KSTEP) * 8;
+                at[i] = row_address(ks + item / PIECES) + (item % PIECES) * 8;
             }
         };
-        auto load_at = [&](const size_t (&at)[PER_THREAD], u32x4_t (&kdst)[PER_THREAD], uint4 (&vdst)[PER_THREAD]) {
+        auto load_at = [&](const size_t (&at)[PER_THREAD], u32x4_t (&kdst)[PER_THREAD], u32x4_t (&vdst)[PER_THREAD]) {
 #pragma unroll
             for (int i = 0; i < PER_THREAD; ++i) {
                 kdst[i] = *reinterpret_cast<const u32x4_t*>(kpool + at[i]);
-                vdst[i] = *reinterpret_cast<const uint4*>(vpool + at[i]);
+                vdst[i] = *reinterpret_cast<const u32x4_t*>(vpool + at[i]);
             }
         };
-        auto load_kv = [&](int ks, u32x4_t (&kdst)[PER_THREAD], uint4 (&vdst)[PER_THREAD]) {
+        auto load_kv = [&](int ks, u32x4_t (&kdst)[PER_THREAD], u32x4_t (&vdst)[PER_THREAD]) {
             size_t at[PER_THREAD];
             addresses(ks, at);
             load_at(at, kdst, vdst);
         };
-        auto store_kv = [&](int buf, const u32x4_t (&ksrc)[PER_THREAD], const uint4 (&vsrc)[PER_THREAD]) {
+        auto store_kv = [&](int buf, const u32x4_t (&ksrc)[PER_THREAD], const u32x4_t (&vsrc)[PER_THREAD]) {
 #pragma unroll
             for (int i = 0; i < PER_THREAD; ++i) {
                 const int item = tid + i * MA_THREADS;
                 if (item < ITEMS) {
-                    const int key = item % KSTEP, dim0 = (item / KSTEP) * 8;
+                    const int key = item / PIECES, dim0 = (item % PIECES) * 8;
                     *reinterpret_cast<u32x4_t*>(&ksm[buf][key][dim0]) = ksrc[i];
-                    const int col = ((key % 16) / 4) * 8 + (key / 16) * 4 + key % 4;
-                    const uint32_t w[4] = {vsrc[i].x, vsrc[i].y, vsrc[i].z, vsrc[i].w};
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        vs[buf][dim0 + e][col] = static_cast<uint16_t>(e & 1 ? w[e / 2] >> 16 : w[e / 2] & 0xffffu);
+                    *reinterpret_cast<u32x4_t*>(&vs[buf][key][dim0]) = vsrc[i];
                 }
             }
         };
@@ -298,7 +310,7 @@ void mfma_attention_kernel(
         // K and V of step s+1 are written to LDS during step s.
         constexpr int DEPTH = HD <= 64 ? 4 : HD <= 128 ? 3 : 2;
         u32x4_t kr[DEPTH][PER_THREAD];
-        uint4 vr[DEPTH][PER_THREAD];
+        u32x4_t vr[DEPTH][PER_THREAD];
         for (int seg0 = 0; seg0 < nsteps;) {
             key_lo = kfirst + seg0 * KSTEP;
             lp0 = page_of(key_lo);
@@ -316,7 +328,7 @@ void mfma_attention_kernel(
             // of the ring) to the other buffer.  The loop is unrolled DEPTH times so that a slot is a fixed
             // set of registers: rotating the ring by copies would wait for the newest loads.  A slot is
             // asked for its next rows as soon as it has been written to LDS.
-            auto step = [&](int s, u32x4_t (&knext)[PER_THREAD], uint4 (&vnext)[PER_THREAD]) {
+            auto step = [&](int s, u32x4_t (&knext)[PER_THREAD], u32x4_t (&vnext)[PER_THREAD]) {
                 const int ks = key_lo + s * KSTEP;
                 // where the rows asked for at the end of the step lie: looked up now, so that the table's answer
                 // has long come when the loads are issued
@@ -354,8 +366,7 @@ void mfma_attention_kernel(
                         uint4 vf_early[EARLY_V ? DT : 1];
                         if constexpr (EARLY_V) {
 #pragma unroll
-                            for (int dt = 0; dt < DT; ++dt)
-                                vf_early[dt] = *reinterpret_cast<const uint4*>(&vb[dt * 16 + r][kg * 8]);
+                            for (int dt = 0; dt < DT; ++dt) vf_early[dt] = read_v_operand(&vb[0][0], VROW, dt * 16, r, kg);
                         }
                         // S^T of block c for the two 16-key halves; this lane: row r of the block, keys ks + t*16 + kg*4 + i
                         auto scores = [&](int c, floatx4_t (&st)[2]) {
@@ -422,7 +433,7 @@ void mfma_attention_kernel(
                         for (int dt = 0; dt < DT; ++dt) {
                             uint4 vf;
                             if constexpr (EARLY_V) vf = vf_early[dt];
-                            else vf = *reinterpret_cast<const uint4*>(&vb[dt * 16 + r][kg * 8]);
+                            else vf = read_v_operand(&vb[0][0], VROW, dt * 16, r, kg);
 #pragma unroll
                             for (int c = 0; c < CB; ++c)
                                 o[c][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vf),
@@ -486,10 +497,10 @@ __global__ __launch_bounds__(DEC_WAVES * WAVE) void mfma_decode_kernel(
     constexpr int THREADS = NW * WAVE;
     constexpr int KK = HD / 32;
     constexpr int DT = HD / 16;
-    constexpr int VROW = KSTEP + VPAD;
-    __shared__ __attribute__((aligned(16))) uint16_t vs[NW][HD][VROW];     // per wavefront: V^T of its step
+    constexpr int VROW = HD + VPAD;
+    __shared__ __attribute__((aligned(16))) uint16_t vs[NW][KSTEP][VROW];  // per wavefront: V of its step, [key][dim]
     __shared__ float sm_ml[NW][16][2];
-    static_assert(HD * VROW * 2 >= 16 * HD * 4, "a wavefront's V tile is reused for its 16 x HD partial output");
+    static_assert(KSTEP * VROW * 2 >= 16 * HD * 4, "a wavefront's V tile is reused for its 16 x HD partial output");
 
     const int t = blockIdx.x;
     const int G = H / KVH;
@@ -546,25 +557,23 @@ __global__ __launch_bounds__(DEC_WAVES * WAVE) void mfma_decode_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-    // a lane loads 8 dims of one key (16 bytes) HD/16 times a step and writes them to LDS transposed
+    // a lane loads 8 dims of one key (16 bytes) HD/16 times a step, neighbouring lanes neighbouring pieces
+    // of a row, and writes them to LDS as they are; the second product takes its operand from there by
+    // transposing reads
     constexpr int V_PER_LANE = HD / 16;
-    auto load_v = [&](int ks, uint4 (&dst)[V_PER_LANE]) {
+    constexpr int PIECES = HD / 8;
+    auto load_v = [&](int ks, u32x4_t (&dst)[V_PER_LANE]) {
 #pragma unroll
         for (int i = 0; i < V_PER_LANE; ++i) {
             const int item = lane + i * WAVE;
-            dst[i] = *reinterpret_cast<const uint4*>(vpool + row_address(ks + item % KSTEP) + (item / KSTEP) * 8);
+            dst[i] = *reinterpret_cast<const u32x4_t*>(vpool + row_address(ks + item % KSTEP) + (item / KSTEP) * 8);
         }
     };
-    auto store_v = [&](const uint4 (&src)[V_PER_LANE]) {
+    auto store_v = [&](const u32x4_t (&src)[V_PER_LANE]) {
 #pragma unroll
         for (int i = 0; i < V_PER_LANE; ++i) {
             const int item = lane + i * WAVE;
-            const int key = item % KSTEP, dim0 = (item / KSTEP) * 8;
-            const int col = ((key % 16) / 4) * 8 + (key / 16) * 4 + key % 4;
-            const uint32_t w[4] = {src[i].x, src[i].y, src[i].z, src[i].w};
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                vs[wave][dim0 + e][col] = static_cast<uint16_t>(e & 1 ? w[e / 2] >> 16 : w[e / 2] & 0xffffu);
+            *reinterpret_cast<u32x4_t*>(&vs[wave][item % KSTEP][(item / KSTEP) * 8]) = src[i];
         }
     };
     auto load_k = [&](int ks, uint4 (&dst)[2][KK]) {
@@ -584,7 +593,7 @@ __global__ __launch_bounds__(DEC_WAVES * WAVE) void mfma_decode_kernel(
 
     constexpr int DEPTH = HD <= 64 ? 4 : HD <= 128 ? 3 : 2;
     uint4 kf[DEPTH][2][KK];
-    uint4 vr[DEPTH][V_PER_LANE];
+    u32x4_t vr[DEPTH][V_PER_LANE];
     for (int seg0 = 0; seg0 < nsteps;) {
         key_lo = kfirst + seg0 * KSTEP;
         lp0 = page_of(key_lo);
@@ -603,7 +612,7 @@ __global__ __launch_bounds__(DEC_WAVES * WAVE) void mfma_decode_kernel(
         // Step j lives in slot j % DEPTH of the ring; the loop is unrolled DEPTH times so that a slot
         // is a fixed set of registers (rotating the ring by copies would wait for the newest loads).
         // A slot is asked for its next rows as soon as its step has used it.
-        auto step = [&](int j, uint4 (&kslot)[2][KK], uint4 (&vslot)[V_PER_LANE]) {
+        auto step = [&](int j, uint4 (&kslot)[2][KK], u32x4_t (&vslot)[V_PER_LANE]) {
             const int ks = key_lo + (wave + j * NW) * KSTEP;
             if (j < mine) {
                 wave_sync();                       // the reads of the previous step are done
@@ -629,10 +638,10 @@ __global__ __launch_bounds__(DEC_WAVES * WAVE) void mfma_decode_kernel(
                 }
                 const uint4 pf = inner ? weights<false>(raw, scale2, m_run) : weights<true>(raw, scale2, m_run);
                 l_run = row_sum_step(pf, l_run);
-                wave_sync();                       // V^T of this step is in LDS
+                wave_sync();                       // V of this step is in LDS
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const uint4 vf = *reinterpret_cast<const uint4*>(&vs[wave][dt * 16 + r][kg * 8]);
+                    const uint4 vf = read_v_operand(&vs[wave][0][0], VROW, dt * 16, r, kg);
                     o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vf),
                                                                     __builtin_bit_cast(bf16x8_t, pf), o[dt], 0, 0, 0);
                 }

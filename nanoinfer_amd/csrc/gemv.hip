@@ -638,6 +638,16 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_rows_kernel(const T* __rest
     const int share = (pieces + splits - 1) / splits;
     const int p_begin = min(pieces, static_cast<int>(blockIdx.y) * share), p_end = min(pieces, p_begin + share);
     y += static_cast<size_t>(blockIdx.y) * M * N;
+    if constexpr (EPI == EPI_ROPE) {
+        // the rows may be dealt out to several workgroups (blockIdx.z), ROWS each: a workgroup then brings
+        // only its own rows of x into LDS, which is most of what it loads when the matrix has few tiles
+        const int row0 = static_cast<int>(blockIdx.z) * ROWS;
+        x += static_cast<size_t>(row0) * K;
+        y += static_cast<size_t>(row0) * rope.H * rope.hd;
+        rope.positions += row0;
+        if (rope.slot_mapping) rope.slot_mapping += row0;
+        M = min(M - row0, ROWS);
+    }
     unsigned char* slab = lds + wave * SLAB;
 
     const T* wrow[NT];      // first byte of this lane in piece 0 of each tile
@@ -819,9 +829,18 @@ static int launch_rows(const void* x, const void* W, void* y, int M, int N, int 
         constexpr int NTc = decltype(nt_tag)::value;
         constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
         const int grid = (tiles + NOUT - 1) / NOUT;
-        skinny_rows_kernel<T, TOUT, MB, NTc, EPI><<<dim3(grid, splits), GV_THREADS, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, splits);
+        skinny_rows_kernel<T, TOUT, MB, NTc, EPI><<<dim3(grid, splits, (M + MB * 16 - 1) / (MB * 16)), GV_THREADS, 0, stream>>>(
+            (const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, splits);
     };
-    if constexpr (EPI == EPI_SWIGLU || EPI == EPI_ROPE) {
+    if constexpr (EPI == EPI_SWIGLU) {
+        // two pairs of gate and up tiles a workgroup where asked for: half the workgroups, and with them
+        // half the loads of x (every workgroup brings all of x into its LDS); bfloat16 only, where the
+        // sixteen fragments of partial sums fit the registers beside two trips of W
+        if constexpr (sizeof(T) == 2) {
+            if (NT >= 4) { run(std::integral_constant<int, 4>{}); return NI_LAUNCH_RESULT(); }
+        }
+        run(std::integral_constant<int, 2>{});
+    } else if constexpr (EPI == EPI_ROPE) {
         run(std::integral_constant<int, 2>{});
     } else {
         if constexpr (MB <= 2) {
@@ -838,7 +857,8 @@ static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K,
                      hipStream_t stream, RopeArgs rope = RopeArgs{}) {
     if (M <= 16 && tiled) return launch_decode<T, TOUT, EPI, 0>(x, W, y, M, N, K, I, NT, stream, rope);
     if (tiled) {
-        if (M <= 32) return launch_rows<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
+        // (with the rotation epilogue the rows are dealt out 32 to a workgroup: see skinny_rows_kernel)
+        if (M <= 32 || EPI == EPI_ROPE) return launch_rows<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
         return launch_rows<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
     }
     if constexpr (EPI == EPI_RESIDUAL) {
