@@ -36,7 +36,7 @@ def main(argv: List[str] = None) -> int:
 
     runner = ModelRunner(args.model, dtype=args.dtype, page_size=args.page_size, max_tokens=args.max_tokens,
                          max_requests=args.max_requests)
-    print(f"[trace_run] model ready: {runner.config.architecture}, {args.dtype}, "
+    print(f"[trace_run] model ready: {runner.arch.name}, {args.dtype}, "
           f"{runner.cache.num_pages} pages of {runner.page_size}", file=sys.stderr, flush=True)
     import torch
 
