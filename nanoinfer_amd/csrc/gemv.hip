@@ -313,6 +313,15 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
                                                                    RopeArgs rope, NormArgs norm, int splits) {
     constexpr int EL = Piece<T>::ELEMS;
     constexpr int CH = 4 * EL;
+    // The rows that a staged prologue leaves in LDS are dead once every wavefront has picked its operands
+    // from them; where they are large enough, the partial sums of the end take their memory (float32 rows
+    // of 2,048 elements for eight rows are 66 KB: with the sums beside them one workgroup would fill a
+    // compute unit's LDS, sharing the memory two fit).
+    constexpr int STAGED_ROW = XP * WV * CH + 16 / static_cast<int>(sizeof(T));
+    constexpr int STAGED_BYTES = (XP > 0 && SR > 0) ? SR * STAGED_ROW * static_cast<int>(sizeof(T)) : 0;
+    constexpr int SUMS_BYTES = WV * NT * WAVE * 4 * static_cast<int>(sizeof(float));
+    constexpr bool SHARE_LDS = STAGED_BYTES >= SUMS_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char staged_rows[STAGED_BYTES > 0 ? STAGED_BYTES : 16];
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;      // the same in every lane: say so
     const int r = lane % 16, kg = lane / 16;
@@ -383,7 +392,8 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
             constexpr int KMAX = XP * WV * CH;                 // elements of a row that the compiled size covers
             constexpr int QPT = (KMAX / 4 + THREADS - 1) / THREADS;      // groups of four columns per thread
             constexpr int XROW = KMAX + 16 / sizeof(T);        // 16 bytes of padding: rows start on different banks
-            __shared__ __attribute__((aligned(16))) T xs[SR][XROW];
+            static_assert(XROW == STAGED_ROW, "the staged rows are sized at the top of the kernel");
+            T (*xs)[XROW] = reinterpret_cast<T (*)[XROW]>(staged_rows);
             if constexpr (PRO == PRO_MERGE) {
                 // x is the output of an attention whose keys were cut into runs: row m, head h is
                 // sum_s o[m,h,s,:] * w_s / sum_s l[m,h,s] * w_s with w_s = exp(max[m,h,s] - max over s), as the
@@ -604,7 +614,12 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
             multiply(c + STRIDE, wa_b, xb_b);
         }
     }
-    skinny_finish<T, TOUT, 1, NT, EPI, WV, false, HALVES>(acc, y, M, N, I, rope);
+    if constexpr (SHARE_LDS) {
+        __syncthreads();                   // every wavefront has taken its operands from the staged rows
+        skinny_finish<T, TOUT, 1, NT, EPI, WV, true, HALVES>(acc, y, M, N, I, rope, reinterpret_cast<float*>(staged_rows));
+    } else {
+        skinny_finish<T, TOUT, 1, NT, EPI, WV, false, HALVES>(acc, y, M, N, I, rope);
+    }
 }
 
 // 17 to 64 rows with re-tiled W.  The operand layout spreads a row of x over few lanes, so loaded
@@ -797,7 +812,7 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
                 return;
             }
         }
-        if constexpr (XP == 4 && NTc <= 2) {
+        if constexpr ((XP == 4 || (XP == 8 && std::is_same<T, float>::value)) && NTc <= 2) {
             // up to eight rows: the prologue staged through LDS (its rows and the partial sums both fit),
             // compiled for 1, 4 and 8 rows
             if (M == 1) { with_halves(Waves8{}, std::integral_constant<int, 1>{}); return; }
