@@ -342,12 +342,18 @@ def test_recorded_decode_steps_equal_eager_ones(dtype):
     compare(got, reqs, folder, dtype, "recorded decode")
 
 
-def test_recorded_steps_with_library_products_are_checked_before_use():
+@pytest.mark.parametrize("verdict", ["as it comes", "refused", "accepted"])
+def test_recorded_steps_with_library_products_are_checked_before_use(verdict, monkeypatch):
     """More than 16 rows go to the library's matrix product.  A recording that contains one is
-    replayed against eager runs before it is trusted; whatever that check decides, the logits of
-    every step equal those of a runner that records nothing."""
+    replayed against eager runs before it is trusted.  The check's answer is also forced both ways:
+    a refused shape is noted and runs eagerly from then on, an accepted one is replayed; either way
+    the logits of every step equal those of a runner that records nothing."""
     from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
     folder = model_folder("A", stored="bfloat16")
+    asked = []
+    if verdict != "as it comes":
+        monkeypatch.setattr(ModelRunner, "_replays_faithfully",
+                            lambda self, *a, **kw: (asked.append(1), verdict == "accepted")[1])
     recorded = ModelRunner(folder, dtype="bfloat16", page_size=16, max_tokens=2048, max_requests=24)
     eager = ModelRunner(folder, dtype="bfloat16", page_size=16, max_tokens=2048, max_requests=24, use_graphs=False)
     n = 20
@@ -364,6 +370,43 @@ def test_recorded_steps_with_library_products_are_checked_before_use():
         assert float((a - b).abs().max()) <= 2e-3 * float(b.abs().max()), step
         toks = a.argmax(-1).tolist()
     assert len(recorded._recorded) + len(recorded._unrecordable) == 1
+    if verdict == "refused":
+        assert asked == [1] and len(recorded._unrecordable) == 1 and not recorded._recorded      # asked once, never recorded again
+    if verdict == "accepted":
+        assert asked == [1] and len(recorded._recorded) == 1
+
+
+def test_a_recording_whose_replays_differ_from_the_eager_step_is_refused():
+    """The check itself: a graph whose replays leave other logits than the eager step (here: a
+    stand-in that spoils the logits after every replay, as a misbehaving recorded node would) is not
+    trusted; the same graph unspoiled is."""
+    from nanoinfer_amd.engine.runner import ModelRunner, StepContext, StepEntry
+    folder = model_folder("A")
+    runner = ModelRunner(folder, dtype="float32", page_size=16, max_tokens=512, max_requests=4)
+    for i in range(2):
+        runner.step([StepEntry(i, list(random_tokens(256, 9 + i, 30 + i)), [])])
+    entries = [StepEntry(i, [3 + i], [0]) for i in range(2)]
+    runner._check_and_reserve(entries)
+    key = runner._graph_shape(entries)
+    rec = runner._record(key, entries)
+    assert rec is not None
+    warm = StepContext(runner.device, scratch_owner=runner)
+    flat, layout, rows = runner._describe(entries, warm)
+    runner._bind(warm, torch.from_numpy(flat).to(runner.device), layout, rows)
+
+    class Spoiled:
+        def __init__(self, graph, logits, by):
+            self.graph, self.logits, self.by = graph, logits, by
+
+        def replay(self):
+            self.graph.replay()
+            self.logits.add_(self.by)
+
+    staging = rec.stagings[0]
+    assert runner._replays_faithfully(Spoiled(rec.graph, rec.logits, 0.0), rec.logits, warm, rec.meta, staging)
+    assert not runner._replays_faithfully(Spoiled(rec.graph, rec.logits, 0.5), rec.logits, warm, rec.meta, staging)
+    rec.logits.fill_(float("nan"))
+    assert not runner._replays_faithfully(Spoiled(rec.graph, rec.logits, float("nan")), rec.logits, warm, rec.meta, staging)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
