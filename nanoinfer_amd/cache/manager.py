@@ -23,7 +23,7 @@ from typing import Dict, Hashable, List, Optional, Tuple
 import torch
 
 from ..parts.base import CacheNeed, KVNeed, StateNeed
-from .block_manager import BlockManager, OutOfPages, PageError
+from .block_manager import BlockManager, OutOfPages
 
 
 class CacheError(RuntimeError):
@@ -203,6 +203,14 @@ class KVCacheManager:
         el = torch.empty(0, dtype=self.dtype).element_size()
         return sum(2 * len(g.cache_ids) * g.pages.num_pages * g.need.kv_heads * self.page_size * g.need.head_dim * el
                    for g in self.groups)
+
+    @staticmethod
+    def pages_for_bytes(needs: Dict[int, CacheNeed], page_size: int, budget_bytes: int, dtype: torch.dtype) -> int:
+        """The largest ``num_pages`` whose pools fit ``budget_bytes`` when every cache of ``needs`` that
+        holds keys and values gets that many pages (windowed groups may then be given fewer)."""
+        el = torch.empty(0, dtype=dtype).element_size()
+        per_page = sum(2 * n.kv.kv_heads * page_size * n.kv.head_dim * el for n in needs.values() if n.kv is not None)
+        return int(budget_bytes // per_page) if per_page else 0
 
     def utilization(self) -> float:
         return max((g.pages.utilization() for g in self.groups), default=0.0)

@@ -46,6 +46,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--max-num-batched-tokens", type=int, default=2048)
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--num-cache-blocks", type=int, default=1024)
+    ap.add_argument("--kv-cache-gb", type=float, default=None,
+                    help="size the page pool by device memory (GiB for all key and value pools) instead of --num-cache-blocks")
     ap.add_argument("--max-model-len", type=int, default=None)
     ap.add_argument("--max-decode-run", type=int, default=8,
                     help="decode steps run back to back on one scheduling decision (requests without a repetition penalty)")
@@ -75,7 +77,8 @@ def main(argv: List[str] = None) -> int:
     cfg = EngineConfig(max_batch_size=args.max_batch_size, max_sequences=args.max_sequences,
                        prefill_chunk_size=args.prefill_chunk_size, block_size=args.block_size,
                        num_cache_blocks=args.num_cache_blocks, max_num_batched_tokens=args.max_num_batched_tokens,
-                       max_model_len=args.max_model_len, max_decode_run=args.max_decode_run, dtype=_DTYPES[args.dtype])
+                       max_model_len=args.max_model_len, max_decode_run=args.max_decode_run, dtype=_DTYPES[args.dtype],
+                       kv_cache_bytes=None if args.kv_cache_gb is None else int(args.kv_cache_gb * (1 << 30)))
     print(f"Model: {model_dir}  dtype: {args.dtype}", file=sys.stderr)
     t0 = time.perf_counter()
     engine = Engine(model_dir, cfg, ignore_eos=args.ignore_eos)

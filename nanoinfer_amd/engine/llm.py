@@ -10,8 +10,7 @@ the scheduler books the result.  ``generate`` wraps the loop for a list of promp
 from __future__ import annotations
 
 import random
-import time
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence
 
 from ..sampling.params import SamplingParams
@@ -43,7 +42,7 @@ class Engine:
             from .runner import ModelRunner
             runner = ModelRunner(model_dir, dtype=self.config.dtype, page_size=self.config.block_size,
                                  max_tokens=self.config.block_size * self.config.num_cache_blocks,
-                                 max_requests=self.config.max_sequences,
+                                 max_requests=self.config.max_sequences, kv_cache_bytes=self.config.kv_cache_bytes,
                                  max_step_tokens=min(self.config.prefill_chunk_size, self.config.max_num_batched_tokens))
         if sampler is None:
             from ..sampling.sampler import Sampler

@@ -11,7 +11,7 @@ The scheduler and the trace-replay program both drive :meth:`ModelRunner.step`.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, Hashable, Iterable, List, Optional, Sequence
 
 import numpy as np
@@ -152,7 +152,7 @@ class ModelRunner:
 
     def __init__(self, model_dir: str, dtype: str = "bfloat16", page_size: int = 16, max_tokens: int = 4096,
                  max_requests: int = 64, device: Optional[torch.device] = None, use_graphs: bool = True,
-                 warm_up: bool = True, max_step_tokens: Optional[int] = None):
+                 warm_up: bool = True, max_step_tokens: Optional[int] = None, kv_cache_bytes: Optional[int] = None):
         self.device = device or K.require_gpu()
         torch_dtype = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
                        "float32": torch.float32, "fp32": torch.float32}.get(dtype)
@@ -166,6 +166,10 @@ class ModelRunner:
         del tensors
         self.page_size = int(page_size)
         num_pages = (int(max_tokens) + self.page_size - 1) // self.page_size
+        if kv_cache_bytes is not None:      # a byte budget for the pools takes the place of the token count
+            num_pages = KVCacheManager.pages_for_bytes(self.model.cache_needs(), self.page_size, int(kv_cache_bytes), torch_dtype)
+            if num_pages < 1:
+                raise ValueError(f"{kv_cache_bytes} bytes do not hold one page of {self.page_size} tokens of this model's cache")
         # with a bound on the tokens one request brings to a step, pools of windowed layers are only as
         # large as their windows need; a longer portion is then refused
         self.max_step_tokens = None if max_step_tokens is None else int(max_step_tokens)

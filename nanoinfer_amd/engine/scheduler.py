@@ -22,7 +22,7 @@ import enum
 import time
 from collections import deque
 from dataclasses import dataclass, field
-from typing import Deque, Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Deque, Dict, List, Optional, Sequence
 
 from ..sampling.params import SamplingParams
 
@@ -95,6 +95,7 @@ class EngineConfig:
     prefill_chunk_size: int = 2048    # longest prompt portion of one request in one step
     block_size: int = 16              # tokens per cache page
     num_cache_blocks: int = 1024      # pages in the pool
+    kv_cache_bytes: Optional[int] = None  # instead of num_cache_blocks: device memory for all key and value pools
     max_num_batched_tokens: int = 2048  # token budget of a step
     max_model_len: Optional[int] = None  # longest request (prompt + generated); None: what model and pool allow
     max_decode_run: int = 8           # decode steps run back to back on one scheduling decision (1: never more than one)

@@ -9,7 +9,6 @@ from __future__ import annotations
 
 import ctypes
 import functools
-import math
 from typing import Dict, Optional
 
 import torch

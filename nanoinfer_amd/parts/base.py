@@ -15,7 +15,7 @@ knows nothing of the model it sits in.  Interfaces, by family:
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Tuple
 
 import torch

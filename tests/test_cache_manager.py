@@ -232,3 +232,14 @@ def test_a_windowed_group_s_pool_is_sized_by_its_window_and_is_never_the_one_tha
     # without the bound every group gets the whole pool
     m2 = KVCacheManager({0: CacheNeed(kv=KVNeed(2, 16, window=window))}, page, 400, requests)
     assert m2.groups[0].pages.num_pages == 400 and m2.max_tokens_per_request() == 1 << 60
+
+
+def test_pages_that_a_byte_budget_buys():
+    from nanoinfer_amd.parts.base import CacheNeed, KVNeed, StateNeed
+    needs = {0: CacheNeed(kv=KVNeed(8, 64)), 1: CacheNeed(kv=KVNeed(8, 64)), 2: CacheNeed(state=StateNeed((4,)))}
+    per_page = 2 * (2 * 8 * 16 * 64 * 2)            # two caches, keys and values, 16 tokens of 8 heads of 64 bfloat16
+    assert KVCacheManager.pages_for_bytes(needs, 16, 10 * per_page + 5, torch.bfloat16) == 10
+    assert KVCacheManager.pages_for_bytes(needs, 16, 10 * per_page, torch.float32) == 5
+    assert KVCacheManager.pages_for_bytes({2: needs[2]}, 16, 1 << 30, torch.float32) == 0
+    m = KVCacheManager(needs, 16, 10, 2, dtype=torch.bfloat16)
+    assert m.pool_bytes() == 10 * per_page

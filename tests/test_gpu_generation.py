@@ -222,6 +222,19 @@ def test_command_line(tmp_path):
     assert (out_dir / "config.json").exists() and (out_dir / "model.safetensors").exists()
 
 
+def test_the_pool_can_be_sized_by_a_byte_budget():
+    from nanoinfer_amd.sampling.params import SamplingParams
+    folder = model_folder("A")
+    # configuration A: 2 layers x (keys + values) x 2 kv heads x 16 dims x 4 bytes = 512 bytes a token, 8 KiB a page of 16
+    eng = engine(folder, dtype="float32", block_size=16, kv_cache_bytes=5 * 8192 + 100, max_sequences=2)
+    assert eng.runner.cache.num_pages == 5 and eng.runner.cache.pool_bytes() == 5 * 8192
+    prompt = list(random_tokens(256, 30, 4))
+    got = eng.generate([prompt], max_new_tokens=8, params=SamplingParams.greedy())[0].tokens
+    assert got == plain_greedy(folder, prompt, 8)
+    with pytest.raises(ValueError, match="do not hold one page"):
+        engine(folder, dtype="float32", block_size=16, kv_cache_bytes=100)
+
+
 def test_smoke_entry():
     sys.path.insert(0, ROOT)
     import __graft_entry__

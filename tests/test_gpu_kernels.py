@@ -1,6 +1,5 @@
 """Each HIP kernel alone against its plain reference, at sizes other than the engine's tests use:
 widths and vocabularies that are no power of two, head sizes in steps of 16, odd page sizes."""
-import functools
 import math
 import random
 

@@ -13,7 +13,6 @@ import json
 import os
 from dataclasses import asdict, dataclass
 
-import numpy as np
 import pytest
 import torch
 
