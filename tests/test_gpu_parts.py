@@ -127,7 +127,7 @@ class SpecRunner:
     """A ModelRunner over a spec and tensors given directly (no folder): the same Model, cache manager
     and step function, reached through the constructor's pieces."""
 
-    def __new__(cls, spec, tensors, dtype, page_size=8, max_tokens=512):
+    def __new__(cls, spec, tensors, dtype, page_size=8, max_tokens=512, max_step_tokens=None):
         from nanoinfer_amd.cache.manager import KVCacheManager
         from nanoinfer_amd.engine.model import Model
         from nanoinfer_amd.engine.runner import ModelRunner
@@ -138,7 +138,9 @@ class SpecRunner:
         r.rt = runtime(dtype)
         r.model = Model(spec, tensors, r.rt)
         r.page_size = page_size
-        r.cache = KVCacheManager(r.model.cache_needs(), page_size, max_tokens // page_size, 4, dtype=DT[dtype], device=r.device)
+        r.max_step_tokens = max_step_tokens
+        r.cache = KVCacheManager(r.model.cache_needs(), page_size, max_tokens // page_size, 4, dtype=DT[dtype], device=r.device,
+                                 max_step_tokens=max_step_tokens)
         r.vocab_size, r.max_positions, r.eos_token_ids = spec.vocab_size, r.model.max_positions, ()
         r._done, r._scratch = {}, None
         r._init_graphs(True)
@@ -246,6 +248,46 @@ def test_windowed_layer_gives_pages_back_while_running():
     assert full.pages.num_taken == 25 and windowed.tables["w"][:20] == [-1] * 20
     assert rel(torch.cat(outs), want) < TOL["float32"]
     runner.release("w")
+
+
+def test_a_windowed_layer_s_pool_is_as_small_as_its_window_allows():
+    """With a bound on the tokens a request brings to a step, the windowed layer's pool holds four
+    requests' windows and steps, not their contexts: two requests run far past what that pool could
+    hold of whole contexts, and a portion longer than the bound is refused before anything is reserved."""
+    from nanoinfer_amd.engine.runner import StepEntry, StepError
+    spec = tiny_spec(["attention", "attention"], [(0, 0), (1, 1)], window=[None, 9])
+    tensors = random_tensors(spec, 5)
+    runner = SpecRunner(spec, tensors, "float32", page_size=4, max_tokens=512, max_step_tokens=12)
+    windowed = next(g for g in runner.cache.groups if g.need.window == 9)
+    full = next(g for g in runner.cache.groups if g.need.window is None)
+    assert full.pages.num_pages == 128 and windowed.pages.num_pages == 4 * (-(-(9 + 12) // 4) + 1) == 28
+    assert all(g.kpools[c].shape[0] == g.pages.num_pages for g in runner.cache.groups for c in g.cache_ids)
+    tokens = {r: list(random_tokens(128, 150, 20 + i)) for i, r in enumerate("ab")}
+    want = {r: plain_spec_forward(spec, tensors, t) for r, t in tokens.items()}
+    at = {r: 0 for r in tokens}
+    sizes = [12, 1, 5, 1, 1, 9, 2]
+    k = 0
+    while any(at[r] < 150 for r in tokens):
+        entries = []
+        for r in tokens:
+            n = min(sizes[k % len(sizes)], 150 - at[r])
+            k += 1
+            if n:
+                entries.append(StepEntry(r, tokens[r][at[r]:at[r] + n], list(range(n))))
+        out = runner.step(entries)
+        row = 0
+        for e in entries:
+            n = len(e.tokens)
+            assert rel(out[row:row + n], want[e.request][at[e.request]:at[e.request] + n]) < TOL["float32"], (e.request, at[e.request])
+            row += n
+            at[e.request] += n
+        assert windowed.pages.num_taken <= 2 * 6
+    with pytest.raises(StepError, match="sized for at most"):
+        runner.step([StepEntry("c", [1] * 13, [])])
+    assert not runner.cache.has("c")
+    for r in tokens:
+        runner.release(r)
+    runner.cache.check()
 
 
 # ------------------------------------------------------------------ a toy mixer with state
