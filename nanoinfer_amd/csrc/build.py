@@ -147,9 +147,19 @@ def attention_mfma_f32_target(head_dim: int):
     return (f"ni_attention_mfma_f32_hd{head_dim}", ["attention_mfma_f32.hip"], {"HEAD_DIM": head_dim})
 
 
-def build_all(head_dims: Iterable[int] = COMMON_HEAD_DIMS, force: bool = True, verbose: bool = True) -> List[str]:
+def build_all(head_dims: Iterable[int] = COMMON_HEAD_DIMS, force: bool = True, verbose: bool = True,
+              jobs: Optional[int] = None) -> List[str]:
     """Compile every library (attention for the given head sizes)."""
     targets = [CORE, SAMPLING, SKINNY] + [attention_target(h) for h in head_dims] + \
         [attention_mfma_target(h) for h in head_dims if h % 32 == 0] + \
         [attention_mfma_f32_target(h) for h in head_dims]
-    return [library_path(n, s, d, force=force, verbose=verbose) for n, s, d in targets]
+    # the compiler runs in processes of its own: a few at a time (the longest, the skinny product, first)
+    from concurrent.futures import ThreadPoolExecutor
+    workers = max(1, min(8, (os.cpu_count() or 2) // 2 if jobs is None else int(jobs)))
+    order = sorted(range(len(targets)), key=lambda i: targets[i] is not SKINNY)
+    paths: List[Optional[str]] = [None] * len(targets)
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        futures = {i: pool.submit(library_path, *targets[i], force=force, verbose=verbose) for i in order}
+        for i, f in futures.items():
+            paths[i] = f.result()
+    return paths
