@@ -108,6 +108,13 @@ class ReservationPlan:
         return all(g.pages.can_allocate(have + n)
                    for g, have, n in zip(c.groups, self.new_pages, self._needs(request, total_tokens)))
 
+    def free_after(self, request: Hashable, total_tokens: int) -> int:
+        """Pages that the fullest group would still have free with this reservation beside those added."""
+        c = self.cache
+        return min((g.pages.num_free - have - n
+                    for g, have, n in zip(c.groups, self.new_pages, self._needs(request, total_tokens))),
+                   default=c.num_pages)
+
     def add(self, request: Hashable, total_tokens: int) -> None:
         if request not in self.cache._tokens:
             self.new_requests += 1

@@ -8,8 +8,9 @@ tokens, so a portion may be of any length down to one token; pages are taken por
 portion, not for the whole prompt at admission (src/engine/engine.cpp:167-172 does the latter).
 
 When pages run out (the reference fails the whole step there, src/engine/engine.cpp:403-404):
-a waiting request simply waits; if a *running* request cannot get pages for its next tokens, the
-youngest running request is preempted: its pages go back, its tokens so far (prompt and what it
+a waiting request simply waits (and is admitted only while ``admission_headroom`` pages stay free for
+every request already running, so that it is not thrown out again at the next page edge); if a
+*running* request cannot get pages for its next tokens, the youngest running request is preempted: its pages go back, its tokens so far (prompt and what it
 generated) are kept, and it returns to the *front* of the waiting queue to be recomputed from
 position 0 when room appears.  A request that could never fit (longer than the whole pool or the
 model's positions) is refused when it is added.
@@ -99,6 +100,7 @@ class EngineConfig:
     max_num_batched_tokens: int = 2048  # token budget of a step
     max_model_len: Optional[int] = None  # longest request (prompt + generated); None: what model and pool allow
     max_decode_run: int = 8           # decode steps run back to back on one scheduling decision (1: never more than one)
+    admission_headroom: int = 1       # pages left free for every request already running when another is admitted
     dtype: str = "bfloat16"
     seed: int = 0
 
@@ -229,6 +231,11 @@ class Scheduler:
             count = min(req.remaining, cfg.prefill_chunk_size, budget)
             if not fits(req, count):
                 break                          # strict FCFS: nobody overtakes the head of the queue
+            # Those already running grow by a page now and then: a newcomer that takes the last pages is the
+            # youngest, and would be preempted at the next page edge with its prompt computed for nothing.
+            # It waits instead until the pool has a little room beside it (nobody running: it may fill the pool).
+            if plan.free_after(req.request_id, req.num_computed + count) < cfg.admission_headroom * len(self.running):
+                break
             self.waiting.popleft()
             req.state = RequestState.RUNNING
             self.running.append(req)

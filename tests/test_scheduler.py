@@ -178,7 +178,7 @@ def test_waiting_request_waits_for_pages():
 
 
 def test_running_out_of_pages_preempts_the_youngest():
-    eng, runner = make_engine(page_size=4, num_pages=4, max_num_batched_tokens=64)
+    eng, runner = make_engine(page_size=4, num_pages=4, max_num_batched_tokens=64, admission_headroom=0)
     a = eng.add_request([1, 2, 3, 4, 5, 6, 7], 9, SamplingParams.greedy())   # 7 -> 15 tokens: ends in 4 pages
     b = eng.add_request([11, 12, 13, 14, 15, 16, 17], 9, SamplingParams.greedy())
     eng.step()                                                # both admitted: 2 pages each, pool full
@@ -199,6 +199,44 @@ def test_running_out_of_pages_preempts_the_youngest():
     again = [s for s in runner.steps if any(x[0] == b and x[1] > 1 for x in s)]
     assert len(again) == 2 and again[1][0][1] == 9            # 7 prompt + 2 generated
     assert not runner.cache.live_requests() and runner.cache.free_pages() == 4
+
+
+def test_a_newcomer_is_not_admitted_into_the_last_pages():
+    """With headroom (the default: one page for every running request) the second request waits
+    until the first is done instead of being admitted and preempted; a request alone may fill the
+    pool; and fewer prompts are computed twice under random traffic."""
+    eng, runner = make_engine(page_size=4, num_pages=4, max_num_batched_tokens=64)
+    a = eng.add_request([1, 2, 3, 4, 5, 6, 7], 9, SamplingParams.greedy())
+    b = eng.add_request([11, 12, 13, 14, 15, 16, 17], 9, SamplingParams.greedy())
+    eng.step()
+    assert [x[0] for x in runner.steps[0]] == [a] and eng.get_request(b).state == RequestState.WAITING
+    eng.run()
+    assert eng.scheduler.num_preemptions == 0
+    assert eng.get_request(a).generated == list(range(8, 17)) and eng.get_request(b).generated == list(range(18, 27))
+    # alone, a request takes every page
+    eng, runner = make_engine(page_size=4, num_pages=4)
+    c = eng.add_request(list(range(1, 14)), 4, SamplingParams.greedy())           # 13 + 3 = 16 tokens: the whole pool
+    eng.run()
+    assert eng.get_request(c).finish_reason == "length" and eng.scheduler.num_preemptions == 0
+    # random traffic on a small pool: all finish either way, with headroom fewer are thrown out
+    import random
+    thrown = {}
+    for headroom in (0, 1):
+        rng = random.Random(5)
+        eng, runner = make_engine(page_size=4, num_pages=24, max_requests=8, max_sequences=8, max_batch_size=8,
+                                  max_num_batched_tokens=32, admission_headroom=headroom)
+        want = {}
+        for _ in range(60):
+            if rng.random() < 0.5:
+                prompt = [rng.randrange(VOCAB) for _ in range(rng.randint(4, 24))]
+                n = rng.randint(8, 24)
+                want[eng.add_request(prompt, n, SamplingParams.greedy())] = [(prompt[-1] + 1 + i) % VOCAB for i in range(n)]
+            eng.step()
+        eng.run()
+        assert all(eng.get_request(r).generated == t for r, t in want.items())
+        assert runner.cache.free_pages() == 24
+        thrown[headroom] = eng.scheduler.num_preemptions
+    assert thrown[1] < thrown[0], thrown
 
 
 def test_engine_never_plans_more_than_fits():
