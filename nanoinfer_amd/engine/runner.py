@@ -147,6 +147,8 @@ class ModelRunner:
     HISTORY_ROWS = 16             # decode steps launched back to back before the host reads their tokens
     GRAPH_MIN_PORTION = 64        # a shorter prompt portion is not worth a recording
     GRAPH_MAX_PORTIONS = 24       # recordings of prompt portions kept (each holds its activations)
+    GRAPH_MAX_DECODES = 256       # recordings of decode steps kept (each holds its logits: batch x vocabulary floats);
+                                  # beyond that the one used longest ago is dropped and its shape recorded again if it returns
     GRAPH_PORTION_SIGHTS = 2      # a portion's shape is recorded when it comes this many times: recording costs
                                   # seven runs of the step and gains a few per cent of a run (a lone length never pays)
 
@@ -206,7 +208,7 @@ class ModelRunner:
     def _init_graphs(self, use_graphs: bool) -> None:
         import os
         self.use_graphs = bool(use_graphs) and self.model.graph_safe() and not os.environ.get("NANOINFER_NO_GRAPHS")
-        self._recorded: Dict[tuple, _RecordedStep] = {}
+        self._recorded: Dict[tuple, _RecordedStep] = {}      # in the order of their last use
         self._unrecordable = set()
         self._portion_sights: Dict[tuple, int] = {}      # how often a prompt portion's shape has come without a recording
         self._staging = [(None, None)] * 3     # pinned host buffers for the tables of eager steps, and their uploads' events
@@ -517,12 +519,17 @@ class ModelRunner:
         this replay chooses are also copied to that row of ``self._history`` (pinned host memory),
         and its logits are not kept.  ``pick(logits, out)``: launched behind the replay, it puts other
         tokens than the largest logits where the step leaves its choice."""
-        rec = self._recorded.get(key)
+        rec = self._recorded.pop(key, None)
         if rec is None:
             rec = self._record(key, entries)
             if rec is None:
                 return False
+            decodes = [k for k in self._recorded if k[0] == "d"]
+            for old in decodes[:max(0, len(decodes) - self.GRAPH_MAX_DECODES)]:      # the ones used longest ago
+                del self._recorded[old]
             # the recording itself ran nothing: fall through to the first replay
+        else:
+            self._recorded[key] = rec          # moved to the end: the most recently used
         kind, B, width = key[0], key[1], key[2]
         ps = self.page_size
         order = tuple(e.request for e in entries)

@@ -172,3 +172,23 @@ def test_tokens_on_the_device_are_refused_before_anything_changes():
     with pytest.raises(StepError):
         r._replay(key, [StepEntry("c", [0], [0]), StepEntry("d", [0], [0])], tokens_from=rec, history_row=0)
     assert rec.turn == turn and r._done == books
+
+
+def test_decode_recordings_are_kept_up_to_a_limit_and_the_least_recently_used_goes_first():
+    r = make_runner(page_size=16)
+    r.GRAPH_MAX_DECODES = 2
+    for n in ("a", "b"):
+        start(r, n, 250)
+    run_wave(r, ("a", "b"), 250, [5, 6], steps=8, run=4)            # shapes for contexts up to 256 and up to 512
+    first, second = r.recordings_made
+    assert list(r._recorded) == [first, second]
+    start(r, "c", 10)
+    run_wave(r, ("c",), 10, [7], steps=2, run=2)                     # a third shape: the first, used longest ago, goes
+    third = r.recordings_made[-1]
+    assert list(r._recorded) == [second, third]
+    run_wave(r, ("a", "b"), 258, [1, 2], steps=2, run=2)             # the second is used again: now the newest
+    assert list(r._recorded) == [third, second]
+    for n in ("d", "e"):
+        start(r, n, 100)
+    run_wave(r, ("d", "e"), 100, [3, 4], steps=2, run=2)             # the first shape comes back: recorded again
+    assert r.recordings_made[-1] == first and list(r._recorded) == [second, first]
