@@ -131,6 +131,24 @@ template <int N> struct VecIO<bf16_t, N> {
     }
 };
 
+// N consecutive elements (4 floats, or 4 or 8 bfloat16) stored from floats in one access of 8 or 16
+// bytes; p is aligned to that access.  Rounding to bfloat16 is the hardware's, to nearest even.
+template <typename T, int N> __device__ __forceinline__ void store_packed(T* p, const float* in) {
+    typedef uint32_t u32x4_hw __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x2_hw __attribute__((ext_vector_type(2)));
+    typedef float floatx4_hw __attribute__((ext_vector_type(4)));
+    if constexpr (sizeof(T) == 4) {
+        static_assert(N == 4, "four floats are 16 bytes");
+        *reinterpret_cast<floatx4_hw*>(p) = floatx4_hw{in[0], in[1], in[2], in[3]};
+    } else if constexpr (N == 8) {
+        *reinterpret_cast<u32x4_hw*>(p) = u32x4_hw{pack_bf16x2(in[0], in[1]), pack_bf16x2(in[2], in[3]),
+                                                   pack_bf16x2(in[4], in[5]), pack_bf16x2(in[6], in[7])};
+    } else {
+        static_assert(N == 4, "four or eight bfloat16");
+        *reinterpret_cast<u32x2_hw*>(p) = u32x2_hw{pack_bf16x2(in[0], in[1]), pack_bf16x2(in[2], in[3])};
+    }
+}
+
 // N consecutive elements kept as loaded (no conversion yet), so that rows waiting in registers
 // for their turn cost as few registers as they cost bytes.
 template <typename T, int N> struct RawRow {

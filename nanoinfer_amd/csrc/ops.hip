@@ -86,6 +86,82 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TP* __restrict__
     }
 }
 
+// The same for rows whose width is a multiple of four: a thread holds G groups of four consecutive
+// elements, so that every access is 16 bytes of float32 or 8 bytes of bfloat16 a lane and neighbouring
+// lanes touch neighbouring groups (a third of the instructions, and the memory system sees whole lines).
+template <typename TP, typename TO, int G>
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TP* __restrict__ pending, int addends, size_t addend_stride,
+                                       const float* __restrict__ w, TO* __restrict__ out,
+                                       const int32_t* __restrict__ rows, int d, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
+    float* hrow = h + src * d;
+    const TP* prow = pending ? pending + src * d : nullptr;
+    const int groups = d / 4;
+    float v[G][4], wv[G][4];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int at = (threadIdx.x + g * blockDim.x) * 4;
+        if (at < d) {
+            VecIO<float, 4>::load(hrow + at, v[g]);
+            VecIO<float, 4>::load(w + at, wv[g]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[g][e] = wv[g][e] = 0.f;
+        }
+    }
+    if (prow) {
+        // the addends in their order, four asked for before any is added
+        for (int a0 = 0; a0 < addends; a0 += 4) {
+            float t[4][G][4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    const int at = (threadIdx.x + g * blockDim.x) * 4;
+                    if (a0 + b < addends && at < d) {
+                        VecIO<TP, 4>::load(prow + (a0 + b) * addend_stride + at, t[b][g]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) t[b][g][e] = 0.f;
+                    }
+                }
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+#pragma unroll
+                for (int g = 0; g < G; ++g)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[g][e] += t[b][g][e];
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ss += v[g][e] * v[g][e];
+    if (!rows && prow) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int at = (threadIdx.x + g * blockDim.x) * 4;
+            if (at < d) store_packed<float, 4>(hrow + at, v[g]);
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(d) + eps);
+    TO* orow = out + static_cast<size_t>(r) * d;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int at = (threadIdx.x + g * blockDim.x) * 4;
+        if (at < d) {
+            float y[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) y[e] = (v[g][e] * inv) * wv[g][e];
+            store_packed<TO, 4>(orow + at, y);
+        }
+    }
+}
+
 // Rows of any width: two passes over memory.
 template <typename TP, typename TO>
 __global__ void add_rmsnorm_wide_kernel(float* __restrict__ h, const TP* __restrict__ pending, int addends, size_t addend_stride,
@@ -203,6 +279,65 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
     st(out + idx, g / (1.0f + expf(-g)) * u);
 }
 
+// The same in accesses of 16 bytes, for head sizes and rotated halves that are multiples of 16 bytes
+// of elements: an item is one such piece of a pair of halves, of a key's unrotated dims, or of a value.
+template <typename T>
+__global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
+                                         const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                         const int32_t* __restrict__ slot_mapping, T* __restrict__ kpool,
+                                         T* __restrict__ vpool, int H, int KVH, int hd, int rot, int page_size) {
+    constexpr int V = 16 / sizeof(T);
+    typedef uint32_t u32x4_hw __attribute__((ext_vector_type(4)));
+    const int t = blockIdx.x;
+    const int half = rot / 2;
+    T* row = qkv + static_cast<size_t>(t) * (H + 2 * KVH) * hd;
+    const int pos = positions[t];
+    const float* c = cos_t + static_cast<size_t>(pos) * half;
+    const float* s = sin_t + static_cast<size_t>(pos) * half;
+    const int slot = slot_mapping ? slot_mapping[t] : -1;
+    const int page = slot >= 0 ? slot / page_size : 0;
+    const int off = slot >= 0 ? slot % page_size : 0;
+    const int rot_vecs = half / V, pass_vecs = (hd - rot) / V, head_vecs = hd / V;
+    const int n_rot = (H + KVH) * rot_vecs;
+    const int n_pass = slot >= 0 ? KVH * pass_vecs : 0;
+    const int n_val = slot >= 0 ? KVH * head_vecs : 0;
+    for (int item = threadIdx.x; item < n_rot + n_pass + n_val; item += blockDim.x) {
+        if (item < n_rot) {
+            const int head = item / rot_vecs, j = (item % rot_vecs) * V;
+            T* hp = row + static_cast<size_t>(head) * hd;
+            const bool is_k = head >= H;
+            if (is_k && slot < 0) continue;
+            T* dst = is_k ? kpool + ((static_cast<size_t>(page) * KVH + (head - H)) * page_size + off) * hd : hp;
+            float x0[V], x1[V], cs[V], sn[V], y0[V], y1[V];
+            VecIO<T, V>::load(hp + j, x0);
+            VecIO<T, V>::load(hp + j + half, x1);
+            VecIO<float, V>::load(c + j, cs);
+            VecIO<float, V>::load(s + j, sn);
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                y0[e] = x0[e] * cs[e] - x1[e] * sn[e];
+                y1[e] = x0[e] * sn[e] + x1[e] * cs[e];
+            }
+            if constexpr (sizeof(T) == 4) {
+                store_packed<T, 4>(dst + j, y0);
+                store_packed<T, 4>(dst + j + half, y1);
+            } else {
+                store_packed<T, 8>(dst + j, y0);
+                store_packed<T, 8>(dst + j + half, y1);
+            }
+        } else if (item < n_rot + n_pass) {
+            const int k = item - n_rot, g = k / pass_vecs, dim = rot + (k % pass_vecs) * V;
+            T* dst = kpool + ((static_cast<size_t>(page) * KVH + g) * page_size + off) * hd;
+            *reinterpret_cast<u32x4_hw*>(dst + dim) = *reinterpret_cast<const u32x4_hw*>(row + static_cast<size_t>(H + g) * hd + dim);
+        } else {
+            const int k = item - n_rot - n_pass, g = k / head_vecs, dim = (k % head_vecs) * V;
+            T* dst = vpool + ((static_cast<size_t>(page) * KVH + g) * page_size + off) * hd;
+            *reinterpret_cast<u32x4_hw*>(dst + dim) =
+                *reinterpret_cast<const u32x4_hw*>(row + static_cast<size_t>(H + KVH + g) * hd + dim);
+        }
+    }
+}
+
 // The same, 16 bytes of gate and of up per thread (rows whose width is a multiple of V elements).
 // The bfloat16 instantiation takes the exponential with the hardware's exp2: its error is far
 // below the rounding of the stored result.
@@ -288,6 +423,12 @@ __global__ void random_normal_kernel(T* __restrict__ out, size_t count, uint64_t
 // ================================================================ entry points
 // dtype codes: 0 = float32, 1 = bfloat16
 
+static inline bool aligned_to(size_t bytes, const void* a, const void* b = nullptr, const void* c = nullptr,
+                              const void* d = nullptr) {
+    return (reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c) |
+            reinterpret_cast<uintptr_t>(d)) % bytes == 0;
+}
+
 static inline unsigned blocks_for(size_t n, unsigned per) { return static_cast<unsigned>((n + per - 1) / per); }
 
 NI_EXPORT int ni_embedding(const void* ids, const void* table, void* out, int T, int d, int vocab,
@@ -306,6 +447,12 @@ static void launch_add_rmsnorm(float* h, const TP* pending, int addends, size_t 
     constexpr int NV = 8;
     if (d <= NV * 1024) {
         const int threads = d <= NV * 64 ? 64 : d <= NV * 128 ? 128 : d <= NV * 256 ? 256 : d <= NV * 512 ? 512 : 1024;
+        if (d % 4 == 0 && aligned_to(16, h, w) && aligned_to(4 * sizeof(TP), pending) && aligned_to(4 * sizeof(TO), out) &&
+            (addends <= 1 || addend_stride % 4 == 0)) {
+            add_rmsnorm_vec_kernel<TP, TO, NV / 4><<<n_rows, threads, 0, stream>>>(h, pending, addends, addend_stride, w, out,
+                                                                                  rows, d, eps);
+            return;
+        }
         add_rmsnorm_kernel<TP, TO, NV><<<n_rows, threads, 0, stream>>>(h, pending, addends, addend_stride, w, out, rows, d, eps);
     } else {
         add_rmsnorm_wide_kernel<TP, TO><<<n_rows, 1024, 0, stream>>>(h, pending, addends, addend_stride, w, out, rows, d, eps);
@@ -344,6 +491,19 @@ NI_EXPORT int ni_rope_kv_write(void* qkv, const void* positions, const void* cos
                                const void* slot_mapping, void* kpool, void* vpool, int T, int H, int KVH, int hd,
                                int rot, int page_size, int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
+    const int vec = dtype == 0 ? 4 : 8;           // elements of a 16-byte access
+    if (rot > 0 && hd % vec == 0 && (rot / 2) % vec == 0 && aligned_to(16, qkv, cos_t, sin_t) && aligned_to(16, kpool, vpool)) {
+        if (dtype == 0)
+            rope_kv_write_vec_kernel<float><<<T, 256, 0, stream>>>((float*)qkv, (const int32_t*)positions, (const float*)cos_t,
+                                                                   (const float*)sin_t, (const int32_t*)slot_mapping,
+                                                                   (float*)kpool, (float*)vpool, H, KVH, hd, rot, page_size);
+        else
+            rope_kv_write_vec_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)qkv, (const int32_t*)positions,
+                                                                    (const float*)cos_t, (const float*)sin_t,
+                                                                    (const int32_t*)slot_mapping, (bf16_t*)kpool,
+                                                                    (bf16_t*)vpool, H, KVH, hd, rot, page_size);
+        return NI_LAUNCH_RESULT();
+    }
     if (dtype == 0)
         rope_kv_write_kernel<float><<<T, 256, 0, stream>>>((float*)qkv, (const int32_t*)positions, (const float*)cos_t,
                                                            (const float*)sin_t, (const int32_t*)slot_mapping,

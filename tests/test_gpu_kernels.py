@@ -107,6 +107,15 @@ def test_add_rmsnorm(K, dtype, d):
     out2 = K.add_rmsnorm(hd2, dev(pending), dev(w), eps, torch.empty(4, d, device="cuda", dtype=DT[dtype]), dev(rows))
     assert torch.equal(hd2.cpu(), h)
     assert rel(out2, P.rmsnorm(total[rows.long()], w, eps)) < KTOL[dtype]
+    # five float32 addends (the shares of a product cut along K), added in their order
+    shares = torch.randn(5, T, d, generator=g)
+    hd3 = dev(h.clone())
+    out3 = K.add_rmsnorm(hd3, dev(shares), dev(w), eps, torch.empty(T, d, device="cuda", dtype=DT[dtype]))
+    in_order = h.clone()
+    for a in range(5):
+        in_order += shares[a]
+    assert torch.equal(hd3.cpu(), in_order)                          # bit for bit: the same additions in the same order
+    assert rel(out3, P.rmsnorm(in_order.double(), w, eps)) < KTOL[dtype]
 
 
 def test_rope_table_holds_the_sines_of_position_times_frequency(K):
@@ -137,7 +146,8 @@ def plain_rotate_half(x, sin, cos, rot):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("H,KVH,hd,rot,ps", [(4, 2, 16, 16, 4), (6, 1, 32, 32, 8), (5, 5, 48, 24, 5), (8, 2, 128, 128, 16)])
+@pytest.mark.parametrize("H,KVH,hd,rot,ps", [(4, 2, 16, 16, 4), (6, 1, 32, 32, 8), (5, 5, 48, 24, 5), (8, 2, 128, 128, 16),
+                                               (3, 3, 64, 32, 8), (2, 1, 80, 48, 4)])
 def test_rope_and_cache_write(K, dtype, H, KVH, hd, rot, ps):
     g = torch.Generator().manual_seed(hd)
     T, pages = 11, 9
