@@ -931,15 +931,22 @@ NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N
     return launch_mb<bf16_t, bf16_t, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
 }
 
-// Up to 64 rows of bfloat16, re-tiled W: the K range cut into `splits` shares of whole 128-byte pieces, the sums of
-// share s stored as float32 in y[s] ([splits, M, N]); whoever reads y adds the shares in their order.  A matrix of
-// few tiles then fills the chip: 128 tiles in two or four shares are 256 workgroups.
+// Up to 64 rows, re-tiled W: the K range cut into `splits` shares of whole 128-byte pieces, the sums of share s
+// stored as float32 in y[s] ([splits, M, N]); whoever reads y adds the shares in their order.  A matrix of few
+// tiles then fills the chip: 128 tiles in two or four shares are 256 workgroups.  dtype 0: float32, 1: bfloat16.
+template <typename T>
+static int launch_ksplit(const void* x, const void* W, void* y, int M, int N, int K, int tiles_per_group, int splits,
+                         hipStream_t stream) {
+    if (M <= 16) return launch_decode<T, float, EPI_STORE, 0>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, NormArgs{}, splits);
+    if (M <= 32) return launch_rows<T, float, 2, EPI_STORE>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, splits);
+    return launch_rows<T, float, 4, EPI_STORE>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, splits);
+}
+
 NI_EXPORT int ni_skinny_gemm_ksplit(const void* x, const void* W, void* y, int M, int N, int K, int tiles_per_group, int splits,
-                                    hipStream_t stream) {
-    if (M <= 0 || M > 64 || N <= 0 || K % 16 != 0 || splits < 1 || splits > 16) return -1;
-    if (M <= 16) return launch_decode<bf16_t, float, EPI_STORE, 0>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, NormArgs{}, splits);
-    if (M <= 32) return launch_rows<bf16_t, float, 2, EPI_STORE>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, splits);
-    return launch_rows<bf16_t, float, 4, EPI_STORE>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, splits);
+                                    int dtype, hipStream_t stream) {
+    if (M <= 0 || M > 64 || N <= 0 || K % (dtype == 0 ? 8 : 16) != 0 || splits < 1 || splits > 16) return -1;
+    if (dtype == 0) return launch_ksplit<float>(x, W, y, M, N, K, tiles_per_group, splits, stream);
+    return launch_ksplit<bf16_t>(x, W, y, M, N, K, tiles_per_group, splits, stream);
 }
 
 // Whether the normalising prologue takes M rows of K elements of this type (1) or not (0).  Every

@@ -642,7 +642,7 @@ def norm_prologue_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
 
 
 def skinny_ksplit(M: int, K: int, dtype: torch.dtype, weight):
-    """(shares, tiles per workgroup) for a product of bfloat16 rows onto the residual stream whose K
+    """(shares, tiles per workgroup) for a product of rows onto the residual stream whose K
     range is worth cutting: a matrix of few 16-row tiles (the [2048, K] matrices of the 1B shape have
     128) leaves half the chip idle with one workgroup a tile, and every compute unit that does work
     loads all of x.  Cut into shares the product runs on about 256 workgroups, each loading its share
@@ -651,8 +651,10 @@ def skinny_ksplit(M: int, K: int, dtype: torch.dtype, weight):
     32 rows 14.2 -> 9.1, at 16 rows 12.7 -> 8.1, at 9 rows 9.8 -> 7.5; [2048, 2048] at 64 rows 7.3 -> 5.5,
     at 32 rows 5.0 -> 4.0, at 16 rows 4.65 -> 4.4.  Up to 16 rows only rows of 4,096 elements or more are
     cut, and only where the norm that follows is a kernel of its own anyway (where the next product can
-    normalise in its prologue that is worth more than the cut).  (1, .): not cut."""
-    if not (SPLIT_K and isinstance(weight, Weight) and weight.tiles is not None and dtype == torch.bfloat16
+    normalise in its prologue that is worth more than the cut).  Float32 rows are cut by the same rule (a decode
+    step of the 1B shape in float32: 4.51 -> 4.23 ms at batch 64, 3.18 -> 2.86 at 32, 2.42 -> 2.27 at 16; before,
+    the [2048, 8192] matrix at more than 32 rows went to the library, 41.6 us a layer).  (1, .): not cut."""
+    if not (SPLIT_K and isinstance(weight, Weight) and weight.tiles is not None
             and 1 <= M <= SKINNY_MAX_ROWS and skinny_ok(M, K, dtype)):
         return 1, 1
     N = weight.rows.shape[0]
@@ -671,13 +673,13 @@ def skinny_gemm_ksplit(x: torch.Tensor, weight, shares: int, per_group: int) -> 
     M, Kd = x.shape
     rows, tiles = _rows_and_tiles(weight)
     N = rows.shape[0]
-    _gpu(x, "x", torch.bfloat16)
-    _gpu(rows, "weight", torch.bfloat16, (N, Kd))
+    _gpu(x, "x", rows.dtype)
+    _gpu(rows, "weight", None, (N, Kd))
     if not (tiles is not None and 1 <= M <= SKINNY_MAX_ROWS and skinny_ok(M, Kd, x.dtype) and 1 <= shares <= 16):
         raise KernelError(f"the product in shares does not take M={M}, K={Kd}, {shares} shares with this matrix")
     out = torch.empty(shares, M, N, dtype=torch.float32, device=x.device)
     _check(skinny_lib().ni_skinny_gemm_ksplit(_ptr(x), _ptr(tiles), _ptr(out), M, N, Kd, int(per_group), int(shares),
-                                              _stream()), "skinny_gemm_ksplit")
+                                              dtype_code(x.dtype), _stream()), "skinny_gemm_ksplit")
     return out
 
 
