@@ -846,6 +846,8 @@ def test_where_the_skinny_product_gives_way_to_the_library(K):
     assert K.skinny_ksplit(65, 8192, torch.bfloat16, W) == (1, 1) == K.skinny_ksplit(8, 8192, torch.bfloat16, W)
     Wf = K.Weight(dev(torch.zeros(32, 8192)))
     assert K.residual_epilogue_ok(40, 8192, torch.float32, Wf) and K.skinny_ksplit(40, 8192, torch.float32, Wf) == (8, 2)
+    assert K.skinny_ksplit(8, 8192, torch.float32, Wf) == (8, 1)      # float32 rows this long are cut at any batch
+    assert K.skinny_ksplit(8, 4096, torch.float32, K.Weight(dev(torch.zeros(32, 4096)))) == (1, 1)
     plain = dev(torch.zeros(32, 8192))          # not re-tiled: past 16 rows the library's product, which adds into nothing
     assert not K.residual_epilogue_ok(40, 8192, torch.float32, plain)
     with pytest.raises(K.KernelError):
