@@ -544,6 +544,14 @@ def skinny_wins(M: int, K: int, dtype: torch.dtype, weight=None) -> bool:
         return True
     if not (isinstance(weight, Weight) and weight.tiles is not None):
         return False
+    if dtype == torch.float32:
+        # float32 rows are twice the bytes and a workgroup holds half the tiles, so what the workgroups load of x is
+        # twice the matrix and more.  Measured in recorded steps (us, skinny : library, with the SwiGLU kernel where the
+        # fusion saves it), layer sizes of the 1B / 3B / 8B shapes: only rows of 2,048 elements gain or tie
+        # ([2048, 2048] at 32 rows 10.7 : 10.1, stacked [16384, 2048] 36.7 : 35.4; at 64 rows 17.0 : 13.2 and 57.8 : 44.2);
+        # [16384, 3072] at 32 rows 52.9 : 51.2, at 64 rows 81.9 : 60.7; [3072, 8192] 41.2 : 30.6 and 61.1 : 45.2;
+        # [28672, 4096] 122.8 : 103.6 and 197.7 : 141.9; [4096, 14336] 72.3 : 57.9 and 107.5 : 86.2
+        return K <= 2048 and (M <= 32 or weight.rows.shape[0] < 8192)
     return M <= 32 or K <= 4096
 FUSE_NORMS = True           # residual sums and norms ride on the skinny products of a decode step where they can
 MERGE_IN_PRODUCT = True     # the key runs of a decode step's attention are merged by the output product where it can
@@ -665,6 +673,10 @@ def skinny_ksplit(M: int, K: int, dtype: torch.dtype, weight):
                             and not (dtype == torch.float32 and K >= 8192))
         if K < 4096 or prologue_follows:
             return 1, 1
+    if dtype == torch.float32 and M > SKINNY_BEST_ROWS and N > 2048:
+        # float32 past 16 rows: only matrices of at most 128 tiles gain by the cut; the library's product is faster on the
+        # others ([3072, 8192] at 64 rows in two shares 54.6 us against 45.2, [4096, 4096] 33.5 : 26.8, [4096, 14336] 93.8 : 86.2)
+        return 1, 1
     per = 2 if (M > 32 and K >= 4096) else 1
     groups = -(-((N + 15) // 16) // per)
     pieces = (K + 63) // 64
@@ -807,6 +819,16 @@ def qkv_rope_ok(M: int, K: int, hd: int, rotary_dim: int, dtype: torch.dtype) ->
     """Whether the product with a stacked [q; k; v] matrix can rotate and store in its epilogue:
     few rows, a head size that splits into pairs of 16-wide tiles, the whole head rotated."""
     return skinny_ok(M, K, dtype) and hd % 32 == 0 and rotary_dim == hd
+
+
+def qkv_rope_wins(M: int, K: int, dtype: torch.dtype) -> bool:
+    """Whether that fused product is also faster than the library's product and the rotation kernel behind it.
+    In bfloat16 always (17 to 64 rows of the 1B / 3B / 8B shapes: 7.2 : 12.9, 13.0 : 16.5, 20.7 : 21.8 us at 64 rows).
+    In float32 for rows of up to 2,048 elements, and for up to 16 rows of 4,096 or more: the 3B shape's
+    [5120, 3072] takes 29.5 : 22.4 at 8 rows and 41.2 : 33.1 at 64 (a float32 decode step of that shape at batch 8:
+    4.72 ms fused, 4.62 with the library), the 8B shape's [6144, 4096] 28.1 : 27.9 and 56.2 : 43.1 (a step at batch 8:
+    7.91 ms fused, 8.13 with the library; at batch 64 the library gains)."""
+    return dtype != torch.float32 or K <= 2048 or (M <= SKINNY_BEST_ROWS and K >= 4096)
 
 
 def skinny_qkv_rope(x, w_qkv, positions: torch.Tensor, cos: torch.Tensor,

@@ -236,7 +236,7 @@ class Attention(Part):
         tables = self.position.tables()
         d = self.w_qkv.shape[1]
         return (K.FUSE_NORMS and tables is not None and K.qkv_rope_ok(T, d, self.hd, 2 * tables[0].shape[1], self.rt.dtype)
-                and K.norm_prologue_ok(T, d, self.rt.dtype, self.w_qkv))
+                and K.qkv_rope_wins(T, d, self.rt.dtype) and K.norm_prologue_ok(T, d, self.rt.dtype, self.w_qkv))
 
     def adds_residual(self, T: int) -> bool:
         """Whether ``forward`` can take ``residual=h`` for T tokens: its output then goes into the residual
@@ -248,7 +248,8 @@ class Attention(Part):
         tables = self.position.tables()
         cos, sin = tables if tables is not None else (None, None)
         slots = cache.slot_mapping if cache.writes else None
-        if cos is not None and K.qkv_rope_ok(T, x.shape[1], self.hd, 2 * cos.shape[1], x.dtype):
+        if (cos is not None and K.qkv_rope_ok(T, x.shape[1], self.hd, 2 * cos.shape[1], x.dtype)
+                and K.qkv_rope_wins(T, x.shape[1], x.dtype)):
             # few rows: rotation and cache write ride on the product's epilogue
             qkv = K.skinny_qkv_rope(x, self.w_qkv, ctx.positions, cos, sin, slots, cache.kpool, cache.vpool,
                                     self.H, self.KVH, self.hd)

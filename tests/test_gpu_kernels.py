@@ -848,6 +848,17 @@ def test_where_the_skinny_product_gives_way_to_the_library(K):
     assert K.residual_epilogue_ok(40, 8192, torch.float32, Wf) and K.skinny_ksplit(40, 8192, torch.float32, Wf) == (8, 2)
     assert K.skinny_ksplit(8, 8192, torch.float32, Wf) == (8, 1)      # float32 rows this long are cut at any batch
     assert K.skinny_ksplit(8, 4096, torch.float32, K.Weight(dev(torch.zeros(32, 4096)))) == (1, 1)
+    # float32 past 16 rows: only rows of up to 2,048 elements are streamed by the skinny product, the stacked gate/up
+    # matrix only up to 32 rows; only matrices of at most 128 tiles are cut
+    narrow, stacked = K.Weight(dev(torch.zeros(48, 2048))), K.Weight(dev(torch.zeros(8192, 2048)))
+    assert K.skinny_wins(64, 2048, torch.float32, narrow) and K.skinny_wins(32, 2048, torch.float32, stacked)
+    assert not K.skinny_wins(33, 2048, torch.float32, stacked) and not K.skinny_wins(17, 3072, torch.float32, K.Weight(dev(torch.zeros(48, 3072))))
+    assert K.skinny_wins(16, 3072, torch.float32, narrow)          # up to 16 rows always
+    wide = K.Weight(dev(torch.zeros(2064, 8192)))
+    assert K.skinny_ksplit(40, 8192, torch.float32, wide) == (1, 1) and K.skinny_ksplit(40, 8192, torch.bfloat16, wide)[0] > 1
+    assert K.qkv_rope_wins(64, 8192, torch.bfloat16) and K.qkv_rope_wins(64, 2048, torch.float32)
+    assert not K.qkv_rope_wins(8, 3072, torch.float32) and not K.qkv_rope_wins(17, 4096, torch.float32)
+    assert K.qkv_rope_wins(16, 4096, torch.float32)
     plain = dev(torch.zeros(32, 8192))          # not re-tiled: past 16 rows the library's product, which adds into nothing
     assert not K.residual_epilogue_ok(40, 8192, torch.float32, plain)
     with pytest.raises(K.KernelError):
