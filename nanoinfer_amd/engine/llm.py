@@ -54,6 +54,7 @@ class Engine:
         self.scheduler.release = lambda req: runner.release(req.request_id)
         self._rng = random.Random(self.config.seed)
         self.num_steps = 0
+        self._stop = False
         self.last_prompt_tokens = 0   # tokens of the last step that belonged to prompt portions
 
     # ---------------------------------------------------------------- requests
@@ -75,8 +76,21 @@ class Engine:
     def get_request(self, request_id: int) -> Request:
         return self.scheduler.requests[request_id]
 
+    def get_request_result(self, request_id: int) -> List[int]:
+        """The tokens a request has generated so far (src/engine/engine.cpp: ``get_request_result`` gives their
+        text; token ids in and out here, a tokenizer is the caller's)."""
+        return list(self.get_request(request_id).generated)
+
+    def get_scheduler_stats(self) -> Dict[str, int]:
+        return self.scheduler.stats()
+
     def has_work(self) -> bool:
         return self.scheduler.has_work()
+
+    def stop(self) -> None:
+        """Make a ``run`` that is under way (on another thread, or from a callback between steps) return after
+        the step it is in; the requests stay where they are and a later ``run`` or ``step`` goes on with them."""
+        self._stop = True
 
     # ---------------------------------------------------------------- stepping
     def step(self) -> List[Request]:
@@ -139,7 +153,8 @@ class Engine:
     def run(self) -> List[Request]:
         """Step until nothing is left (src/engine/engine.cpp:191-198)."""
         finished: List[Request] = []
-        while self.has_work():
+        self._stop = False
+        while self.has_work() and not self._stop:
             finished.extend(self.step())
         return finished
 

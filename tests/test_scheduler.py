@@ -374,3 +374,27 @@ def test_what_keeps_a_decode_step_single():
     assert sched.config.max_decode_run == 8
     with pytest.raises(ValueError):
         EngineConfig(max_decode_run=0).validate()
+
+
+def test_a_run_can_be_stopped_and_taken_up_again():
+    """``stop`` (src/engine/engine.cpp: the flag that ``run`` looks at) ends the loop after the step under way;
+    what the requests have generated by then is theirs, and another ``run`` finishes them."""
+    eng, runner = make_engine(num_pages=32)
+    rid = eng.add_request([1, 2, 3], max_new_tokens=10)
+    steps = []
+    plain_step = eng.step
+
+    def step_then_stop():
+        out = plain_step()
+        steps.append(1)
+        if len(steps) == 4:
+            eng.stop()
+        return out
+
+    eng.step = step_then_stop
+    assert eng.run() == [] and len(steps) == 4 and eng.has_work()
+    assert eng.get_request_result(rid) == [4, 5, 6, 7]          # the prompt's step gave the first, three steps more
+    assert eng.get_scheduler_stats()["num_running"] == 1 and eng.get_scheduler_stats()["num_finished"] == 0
+    done = eng.run()
+    assert [r.request_id for r in done] == [rid] and eng.get_request_result(rid) == list(range(4, 14))
+    assert eng.get_scheduler_stats()["num_finished"] == 1 and not eng.has_work()
