@@ -13,7 +13,8 @@ the host instead of a recorded step), the decode step's fraction of the HBM roof
 ``points`` decode at batch 1 and 64.  The default line (1B shape, bfloat16) adds further points, each
 timed over 96 steps: decode at batch 8 from contexts of 8,192 and 32,768 tokens, the same model in
 true float32 (``decode_b8_fp32``, ``prefill_fp32``: the reference's own precision), and the 3B shape
-(``decode_b8_3b``), with the roofline fraction of each.  Peaks are MI355X's published ones: HBM
+(``decode_b8_3b``), with the roofline fraction of each, and prompts of 8,192 and 32,768 tokens
+(``prefill_8k``, ``prefill_32k``, in portions of 2,048).  Peaks are MI355X's published ones: HBM
 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s.  The reference publishes no numbers for
 this model, so ``vs_baseline`` is null.  ``--workload serving`` measures requests through the
 scheduler instead and prints a line of its own.
@@ -442,6 +443,11 @@ def main() -> int:
             points[f"decode_b8_ctx{n // 1024}k"] = round(8 / sec, 1)
             more[f"roofline_ctx{n // 1024}k"] = round(decode_bytes(cfg, 8, ctx, elem) / sec / HBM_PEAK, 4)
             log(f"decode batch 8 at context {n}: {sec * 1e3:.3f} ms a step")
+        for n in LONG_CONTEXTS:      # long prompts, where the attention is the larger part, in portions of the token budget
+            sec = rig.prefill(n, ENGINE_CHUNK)
+            more[f"prefill_{n // 1024}k"] = {"value": round(n / sec, 1), "tokens": n, "ms": round(sec * 1e3, 3),
+                                            "frac": round(prefill_flops(cfg, n) / sec / FLOP_PEAK[args.dtype], 4)}
+            log(f"prefill of {n} in portions of {ENGINE_CHUNK}: {sec * 1e3:.2f} ms")
         rig.close()
         # the reference's own precision: the same model in true float32
         rig32 = Rig(cfg, "fp32", 8 * CONTEXT_LEN, 8, args.decode_run)
