@@ -137,6 +137,44 @@ def test_preemption_does_not_change_the_tokens():
     assert tight.runner.cache.free_pages() == 30
 
 
+@pytest.mark.parametrize("name", ["A", "D"])
+def test_random_scheduling_settings_do_not_change_the_tokens(name, monkeypatch):
+    """Float32 generation, greedy or with seeded draws, under a dozen random settings of pool, page, portion,
+    token budget, sequences at once, decode run and recorded steps on or off (most of them preempt): the tokens
+    are those of an engine with room for everything."""
+    import random
+    from nanoinfer_amd.sampling.params import SamplingParams
+    folder = model_folder(name)
+    vocab, maxpos = ALL[name]["vocab_size"], ALL[name]["max_position_embeddings"]
+    preempted = 0
+    for seed in range(12):
+        rng = random.Random(seed * 31 + len(name))
+        new = rng.randint(5, 40)
+        prompts = [list(random_tokens(vocab, rng.randint(1, min(120, maxpos - new - 1)), seed * 100 + i))
+                   for i in range(rng.randint(2, 7))]
+        page = rng.choice([4, 8, 16])
+        need = sum(-(-(len(p) + new) // page) for p in prompts)
+        params = SamplingParams.greedy() if seed % 2 else SamplingParams(
+            temperature=rng.choice([0.5, 0.8, 1.3]), top_k=rng.choice([0, 5, 50]), top_p=rng.choice([1.0, 0.9, 0.5]),
+            repetition_penalty=rng.choice([1.0, 1.2]), seed=seed)
+        roomy = engine(folder, dtype="float32", block_size=page, num_cache_blocks=need + 8, max_sequences=8)
+        want = [r.tokens for r in roomy.generate(prompts, max_new_tokens=new, params=params)]
+        longest = max(-(-(len(p) + new) // page) for p in prompts)
+        if rng.random() < 0.3:
+            monkeypatch.setenv("NANOINFER_NO_GRAPHS", "1")
+        else:
+            monkeypatch.delenv("NANOINFER_NO_GRAPHS", raising=False)
+        tight = engine(folder, dtype="float32", block_size=page, num_cache_blocks=rng.randint(longest + 1, max(longest + 2, need)),
+                       max_sequences=rng.randint(1, 8), prefill_chunk_size=rng.choice([2, 5, 16, 64, 512]),
+                       max_num_batched_tokens=rng.choice([8, 33, 256, 2048]), max_decode_run=rng.choice([1, 2, 8]))
+        got = [r.tokens for r in tight.generate(prompts, max_new_tokens=new, params=params)]
+        assert got == want, (seed, tight.config)
+        preempted += tight.scheduler.num_preemptions > 0
+        tight.runner.cache.check()
+        assert tight.runner.cache.free_pages() == tight.runner.cache.num_pages
+    assert preempted >= 3
+
+
 def test_seeded_sampling_is_reproducible_and_follows_the_plain_pipeline():
     from nanoinfer_amd.sampling.params import SamplingParams
     from nanoinfer_amd.sampling.sampler import uniform_from_counter
