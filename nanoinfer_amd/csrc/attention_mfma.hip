@@ -23,6 +23,7 @@
 // softmax subtracts the maximum, divides by the plain sum; probabilities are rounded to bfloat16
 // for the second product and summed as rounded, in float32.
 #include "common.h"
+#include <type_traits>
 
 #include <algorithm>
 
@@ -328,13 +329,18 @@ void mfma_attention_kernel(
             // of the ring) to the other buffer.  The loop is unrolled DEPTH times so that a slot is a fixed
             // set of registers: rotating the ring by copies would wait for the newest loads.  A slot is
             // asked for its next rows as soon as it has been written to LDS.
-            auto step = [&](int s, u32x4_t (&knext)[PER_THREAD], u32x4_t (&vnext)[PER_THREAD]) {
+            // (A step is compiled twice.  INTERIOR: the step's 32 keys lie inside the key range of every row of
+            // every block of this wavefront, known before the loop, so it has no flags to work out, no masks and
+            // no branch but the one for a risen row, and the scores stay in the registers the matrix cores left
+            // them in.  Most steps of a long key range are of this kind.)
+            auto step = [&](auto interior_tag, int s, u32x4_t (&knext)[PER_THREAD], u32x4_t (&vnext)[PER_THREAD]) {
+                constexpr bool INTERIOR = decltype(interior_tag)::value;
                 const int ks = key_lo + s * KSTEP;
                 // where the rows asked for at the end of the step lie: looked up now, so that the table's answer
                 // has long come when the loads are issued
                 size_t at_next[PER_THREAD];
                 addresses(ks + (DEPTH + 1) * KSTEP, at_next);
-                if (s < seg_steps) {
+                if (INTERIOR || s < seg_steps) {
                     // The tiles of this step are in buffer s & 1; nobody still reads the other one.  Only LDS is
                     // ordered here: a full barrier would also wait for every row load in flight for later steps.
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
@@ -342,11 +348,11 @@ void mfma_attention_kernel(
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
                     // A block takes part in a step unless all its rows lie before the step's keys.  Steps whose 32
                     // keys lie inside the key range of every row of a block need no masking for it.
-                    bool act[CB], inner[CB], any_act = false, all_inner = true;
+                    bool act[CB], inner[CB], any_act = INTERIOR, all_inner = true;
 #pragma unroll
                     for (int c = 0; c < CB; ++c) {
-                        act[c] = blk_ok[c] && ks <= blk_pmax[c];
-                        inner[c] = act[c] && ks >= blk_lo_max[c] && ks + KSTEP - 1 <= blk_pmin[c];
+                        act[c] = INTERIOR || (blk_ok[c] && ks <= blk_pmax[c]);
+                        inner[c] = INTERIOR || (act[c] && ks >= blk_lo_max[c] && ks + KSTEP - 1 <= blk_pmin[c]);
                         any_act = any_act || act[c];
                         all_inner = all_inner && inner[c];
                     }
@@ -445,9 +451,33 @@ void mfma_attention_kernel(
                 }
                 load_at(at_next, knext, vnext);
             };
-            for (int s0 = 0; s0 < seg_steps; s0 += DEPTH) {
+            // the steps [in_lo, in_hi) of the segment, whole turns of the ring, are interior for this wavefront
+            int in_lo = seg_steps, in_hi = seg_steps;
+            {
+                bool every = true;
+                int lo_max = 0, p_min = blk_pmin[0];
 #pragma unroll
-                for (int d = 0; d < DEPTH; ++d) step(s0 + d, kr[(d + 1) % DEPTH], vr[(d + 1) % DEPTH]);
+                for (int c = 0; c < CB; ++c) {
+                    every = every && blk_ok[c];
+                    lo_max = max(lo_max, blk_lo_max[c]);
+                    p_min = min(p_min, blk_pmin[c]);
+                }
+                const int first = lo_max > key_lo ? (lo_max - key_lo + KSTEP - 1) / KSTEP : 0;       // ks >= lo_max
+                const int past = p_min - (KSTEP - 1) >= key_lo ? (p_min - (KSTEP - 1) - key_lo) / KSTEP + 1 : 0;   // ks + 31 <= p_min
+                const int a = (first + DEPTH - 1) / DEPTH * DEPTH;
+                const int b = min(past, seg_steps);
+                if (every && b - a >= DEPTH) { in_lo = a; in_hi = a + (b - a) / DEPTH * DEPTH; }
+            }
+            for (int s0 = 0; s0 < seg_steps; s0 += DEPTH) {
+                if (s0 >= in_lo && s0 < in_hi) {
+#pragma unroll
+                    for (int d = 0; d < DEPTH; ++d)
+                        step(std::true_type{}, s0 + d, kr[(d + 1) % DEPTH], vr[(d + 1) % DEPTH]);
+                } else {
+#pragma unroll
+                    for (int d = 0; d < DEPTH; ++d)
+                        step(std::false_type{}, s0 + d, kr[(d + 1) % DEPTH], vr[(d + 1) % DEPTH]);
+                }
             }
             seg0 += seg_steps;
         }

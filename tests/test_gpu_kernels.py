@@ -418,6 +418,13 @@ def test_mfma_attention_window_and_far_key(K, blocks):
             got = out.double().cpu()[-1].reshape(8, 64)
             expect = vs[0][key_at].double().repeat_interleave(4, 0)
             assert float((got - expect).abs().max()) < 0.05, key_at
+    # a window long enough that whole turns of the step ring lie inside every row's key range (the steps that run
+    # without masks), its start and the rows' own positions at their edges; the passed pages hold no finite number
+    for window, lens, q_lens in ((400, [900, 40], [90, 40]), (300, [901], [5]), (129, [700, 333], [64, 33]), (600, [777], [1])):
+        out, want, _ = paged_case(K, "bfloat16", 8, 2, 64, 16, lens, q_lens, window, window + lens[0], 1, kernel="mfma",
+                                  blocks=blocks)
+        assert not torch.isnan(out).any()
+        assert rel(out, want) < KTOL["bfloat16"], window
     with pytest.raises(Exception):
         K.attention_mfma_lib(48)
     assert not K.mfma_token_ok(torch.float32, 64) and not K.mfma_attention_ok(torch.bfloat16, 48)
