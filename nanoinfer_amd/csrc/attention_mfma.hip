@@ -176,8 +176,13 @@ void mfma_attention_kernel(
     // (P workgroups in x): to and fro through the sorted list, so that every workgroup gets about
     // the same number of keys and none is left working alone at the end.
     for (int round = 0;; ++round) {
-        const int tile_at = (round & 1) ? (round + 1) * gridDim.x - 1 - blockIdx.x : round * gridDim.x + blockIdx.x;
-        if (tile_at >= n_tiles) break;                // later rounds lie further on in the list
+        int tile_at = (round & 1) ? (round + 1) * gridDim.x - 1 - blockIdx.x : round * gridDim.x + blockIdx.x;
+        // With one round only nothing pairs long tiles with short ones inside a workgroup.  The chip then holds the
+        // whole grid at once, two workgroups a compute unit, and hands them out in the order of their numbers: unit u
+        // gets workgroups u and u + half the grid, which is the same x in the lower and the upper half of y.  The
+        // upper half walks the list backwards, so that every unit gets a long and a short tile.
+        if (n_tiles <= static_cast<int>(gridDim.x) && 2 * blockIdx.y >= gridDim.y && gridDim.y > 1) tile_at = n_tiles - 1 - tile_at;
+        if (tile_at >= n_tiles || tile_at < 0) break;                // later rounds lie further on in the list
         const QTile tile = tiles[tile_at];
         const int G = H / KVH;
         const int hpt = 1 << hpt_shift;                      // heads of a tile: a power of two up to 16
@@ -773,11 +778,13 @@ NI_EXPORT int ni_mfma_attention(const void* q, int q_stride, const void* kpool, 
             units[pow2] = cus;                                                                                      \
             slots[pow2] = cus * per_cu;                                                                             \
         }                                                                                                           \
-        /* an even number of rounds pairs long tiles with short ones; with few tiles every one gets a workgroup  */  \
+        /* with no more tiles than the chip holds workgroups every tile gets one (the kernel pairs them over the */  \
+        /* compute units); else two rounds pair long tiles with short ones, or more, as few as fit the chip:      */  \
+        /* three rounds leave more workgroups on the chip than four, and their shares differ by less than a tile  */  \
         int rounds = 1;                                                                                             \
-        if (n_tiles * per_tile >= 4 * units[pow2]) {                                                                \
+        if (n_tiles * per_tile > slots[pow2]) {                                                                     \
             rounds = 2;                                                                                             \
-            while ((n_tiles + rounds - 1) / rounds * per_tile > slots[pow2] && rounds < n_tiles) rounds += 2;       \
+            while ((n_tiles + rounds - 1) / rounds * per_tile > slots[pow2] && rounds < n_tiles) rounds += 1;       \
         }                                                                                                           \
         const int in_x = (n_tiles + rounds - 1) / rounds;                                                           \
         dim3 grid(in_x, KVH * chunks, nsplit);                                                                      \

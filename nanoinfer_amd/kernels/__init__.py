@@ -337,11 +337,12 @@ def mfma_tile_tokens(hd: int, group: int, n_tokens: Optional[int] = None, kv_hea
     """Tokens of one tile of the matrix-core attention kernel for ``group`` query heads per kv head.
     A wavefront owns one block of 16 rows, or two where the head size leaves registers for them.
     More blocks share every staged key among more rows and give a wavefront more independent work,
-    but the kernel pairs long tiles with short ones, two to a workgroup, and wants two workgroups on
-    every compute unit: the largest number of blocks is taken that leaves a step of ``n_tokens``
-    tokens four tiles for every compute unit (measured at head size 64: 2,048 tokens 57 us with one
-    block, 63 with two; 4,096 tokens 197 and 134).  Without ``n_tokens``: the smallest tile.  The
-    float32 kernel has one tile size."""
+    but fewer tiles fill the chip less evenly (the kernel pairs long tiles with short ones, in a workgroup
+    or over the two workgroups of a compute unit): two blocks are taken where a step of ``n_tokens``
+    tokens still has one and a half such tiles for every compute unit (measured at head size 64, one
+    block : two blocks in us: 1,024 tokens 19.8 : 24.0, 1,536 tokens 41.8 : 37.0, 2,048 tokens 44.2 : 43.2,
+    2,560 tokens 100.4 : 78.6, 3,072 tokens 117.2 : 95.3, 4,096 tokens 150.8 : 108.0).  Without ``n_tokens``:
+    the smallest tile.  The float32 kernel has one tile size."""
     if dtype == torch.float32:
         return int(attention_mfma_f32_lib(hd).ni_mfma_attention_f32_tile_tokens(int(group)))
     lib = attention_mfma_lib(hd)
@@ -351,7 +352,7 @@ def mfma_tile_tokens(hd: int, group: int, n_tokens: Optional[int] = None, kv_hea
         chunks = (group + hpt - 1) // hpt
         for b in (2,):
             if b <= int(lib.ni_mfma_attention_max_blocks()) and \
-                    (n_tokens // (4 * b * 16 // hpt)) * kv_heads * chunks >= 4 * COMPUTE_UNITS:
+                    2 * (n_tokens // (4 * b * 16 // hpt)) * kv_heads * chunks >= 3 * COMPUTE_UNITS:
                 blocks = b
                 break
     return int(lib.ni_mfma_attention_tile_tokens(int(group), blocks))
@@ -404,11 +405,14 @@ def mfma_splits(n_tiles: int, kv_heads: int, group: int, max_keys: int) -> int:
     """Into how many runs the matrix-core kernel cuts the keys of every tile.  Cutting costs a
     second kernel that merges the runs, and float32 partial results in between: a step with many
     tiles is cut only into runs of 2,048 keys or more, up to about a thousand workgroups (measured
-    for portions of 512 tokens at contexts of 512 to 8,192); a step with fewer tiles than the chip
-    has compute units, into runs of 512 keys or more until every unit has one."""
+    for portions of 512 tokens at contexts of 512 to 8,192), and not at all once it has two tiles for
+    every compute unit (2,048 tokens in tiles of 32 at contexts of 4,096 / 8,192 / 32,768: 88 / 180 / 721 us
+    uncut, 99 / 192 / 741 in two runs; 1,024 tokens, one tile a unit: 75 / 142 uncut, 64 / 114 in two);
+    a step with fewer tiles than the chip has compute units, into runs of 512 keys or more until
+    every unit has one."""
     hpt = _heads_per_tile(group)
     items = max(1, n_tiles * kv_heads * ((group + hpt - 1) // hpt))
-    many = min(1024 // items, max_keys // 2048)
+    many = min(1024 // items if items < 2 * COMPUTE_UNITS else 1, max_keys // 2048)
     few = min(COMPUTE_UNITS // items, max_keys // 512)
     return int(max(1, min(max(many, few), 16)))
 

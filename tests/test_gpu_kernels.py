@@ -351,15 +351,18 @@ def mfma_max_blocks(K, hd):
 
 
 def test_mfma_tile_size_and_splits_follow_the_step(K):
-    # 32 query heads on 8 kv heads, head size 64: tiles of 16 tokens, or of 32 where that leaves 1,024 tiles
+    # 32 query heads on 8 kv heads, head size 64: tiles of 16 tokens, or of 32 where that leaves 384 tiles (one and a
+    # half for every compute unit)
     assert K.mfma_tile_tokens(64, 4) == 16
-    assert K.mfma_tile_tokens(64, 4, 2048, 8) == 16
+    assert K.mfma_tile_tokens(64, 4, 1535, 8) == 16 and K.mfma_tile_tokens(64, 4, 1536, 8) == 32
+    assert K.mfma_tile_tokens(64, 4, 2048, 8) == 32
     assert K.mfma_tile_tokens(64, 4, 4096, 8) == 32
     assert K.mfma_tile_tokens(64, 4, 100, 8) == 16
     assert K.mfma_tile_tokens(128, 4, 8192, 8) == 16        # head size 128 leaves registers for one block only
     assert K.mfma_tile_tokens(256, 1, 8192, 8) == 64        # one head a tile: 4 wavefronts x 16 tokens, one block
     # many tiles: runs of 2,048 keys or more; fewer tiles than compute units: runs of 512 or more
     assert K.mfma_splits(128, 8, 4, 2048) == 1
+    assert K.mfma_splits(64, 8, 4, 32768) == 1 and K.mfma_splits(63, 8, 4, 32768) == 2     # two tiles a compute unit: uncut
     assert K.mfma_splits(32, 8, 4, 8192) == 4
     assert K.mfma_splits(8, 8, 4, 2048) == 4
     assert K.mfma_splits(8, 8, 4, 300) == 1
@@ -371,7 +374,8 @@ def test_mfma_tile_size_and_splits_follow_the_step(K):
     assert K.mfma_plan(64, 4, 8, 512, 512, 2048) == (32, 4) == K.mfma_plan(64, 4, 8, 512, 512, 1100)
     assert K.mfma_plan(64, 4, 8, 512, 512, 1024) == (16, None)        # the keys before it may be as few as its own
     assert K.mfma_plan(64, 4, 8, 512, 512, 5000) == (32, 4)
-    assert K.mfma_plan(64, 4, 8, 2048, 2048, 2048) == (16, None)      # a whole prompt: short and long tiles, paired
+    assert K.mfma_plan(64, 4, 8, 1024, 1024, 1024) == (16, None)      # a whole prompt: short and long tiles, paired
+    assert K.mfma_plan(64, 4, 8, 2048, 2048, 2048) == (32, None)
     assert K.mfma_plan(64, 4, 8, 4096, 4096, 4096) == (32, None)
     assert K.mfma_plan(64, 4, 8, 512, 300, 2048) == (16, None)        # several portions in the step
     assert K.mfma_plan(128, 4, 8, 512, 512, 2048) == (16, None)       # head size 128 has one block only
