@@ -61,7 +61,10 @@ __global__ __launch_bounds__(THREADS) void token_attention_kernel(
     constexpr int WAVES = THREADS / WAVE;
     constexpr bool FAST = sizeof(T) == 2;
 
-    const int t = blockIdx.x;
+    // (uncut key ranges of many tokens: a compute unit holds workgroups u and u + half the grid, the same x in the
+    // lower and the upper half of y; the upper half takes the tokens from the far end, so that tokens that come in the
+    // order of their contexts put a long and a short one on every unit)
+    const int t = (gridDim.z == 1 && gridDim.y > 1 && 2 * blockIdx.y >= gridDim.y) ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
     const int G = H / KVH;
     const int chunks = (G + GT - 1) / GT;
     const int g = blockIdx.y / chunks;

@@ -537,7 +537,10 @@ __global__ __launch_bounds__(DEC_WAVES * WAVE) void mfma_decode_kernel(
     __shared__ float sm_ml[NW][16][2];
     static_assert(KSTEP * VROW * 2 >= 16 * HD * 4, "a wavefront's V tile is reused for its 16 x HD partial output");
 
-    const int t = blockIdx.x;
+    // Uncut key ranges of many tokens: the chip holds the grid two workgroups a compute unit, u and u + half the grid,
+    // which is the same x in the lower and the upper half of y.  The upper half takes the tokens from the far end, so
+    // that a caller who brings the tokens in the order of their contexts gets a long and a short one on every unit.
+    const int t = (gridDim.z == 1 && gridDim.y > 1 && 2 * blockIdx.y >= gridDim.y) ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
     const int G = H / KVH;
     const int chunks = (G + 15) / 16;
     const int g = blockIdx.y / chunks;

@@ -101,6 +101,10 @@ class Engine:
         batch: ScheduledBatch = self.scheduler.schedule()
         if not batch:
             return []
+        if len(batch.items) > 1 and all(i.count == 1 and i.samples for i in batch.items):
+            # a decode step: longest context first (the order stays as the contexts grow together).  The attention
+            # kernels give a compute unit the tokens b and B - 1 - b of an uncut batch, a long and a short one.
+            batch.items.sort(key=lambda i: -i.start)
         entries = []
         sampling = []
         for item in batch.items:

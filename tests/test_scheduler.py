@@ -398,3 +398,17 @@ def test_a_run_can_be_stopped_and_taken_up_again():
     done = eng.run()
     assert [r.request_id for r in done] == [rid] and eng.get_request_result(rid) == list(range(4, 14))
     assert eng.get_scheduler_stats()["num_finished"] == 1 and not eng.has_work()
+
+
+def test_decode_steps_bring_the_longest_context_first():
+    """A step of single tokens is handed to the runner longest context first, whatever the order of arrival (the
+    attention kernels pair the ends of that order on a compute unit); the tokens are each request's own."""
+    eng, runner = make_engine(num_pages=64)
+    short = eng.add_request([1, 2, 3], max_new_tokens=4)
+    long = eng.add_request(list(range(10, 19)), max_new_tokens=4)
+    middle = eng.add_request([30, 31, 32, 33, 34], max_new_tokens=4)
+    eng.run()
+    decode_steps = [st for st in runner.steps if all(n == 1 for _, n, _ in st)]
+    assert decode_steps and all([r for r, _, _ in st] == [long, middle, short] for st in decode_steps)
+    assert eng.get_request_result(short) == [4, 5, 6, 7] and eng.get_request_result(long) == [19, 20, 21, 22]
+    assert eng.get_request_result(middle) == [35, 36, 37, 38]
