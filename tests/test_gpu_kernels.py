@@ -435,6 +435,44 @@ def test_mfma_attention_window_and_far_key(K, blocks):
     assert K.mfma_attention_ok(torch.float32, 48) and not K.mfma_attention_ok(torch.float32, 40)
 
 
+@pytest.mark.parametrize("blocks", [1, 2])
+def test_mfma_attention_more_tiles_than_the_chip_holds(K, blocks):
+    """A prompt of 4,200 tokens, 16 query heads on 8 kv heads: with tiles of 32 tokens more tiles than the chip holds
+    workgroups, dealt out in three rounds (with 64 tokens: two); with 1,100 tokens every tile has a workgroup of its
+    own and the upper half of the grid walks the list backwards.  Rows picked from the start, the end and the middle of
+    the prompt against the plain formula."""
+    H, KVH, hd, ps = 16, 8, 64, 16
+    for n in (4200, 1100):
+        g = torch.Generator().manual_seed(n + blocks)
+        q = torch.randn(n, H, hd, generator=g).bfloat16().float()
+        k = torch.randn(n, KVH, hd, generator=g).bfloat16().float()
+        v = torch.randn(n, KVH, hd, generator=g).bfloat16().float()
+        pages = -(-n // ps)
+        order = torch.randperm(pages, generator=g)
+        kpool = torch.full((pages + 2, KVH, ps, hd), float("nan"))
+        vpool = torch.full((pages + 2, KVH, ps, hd), float("nan"))
+        pad = pages * ps - n
+        kp = torch.cat([k, torch.zeros(pad, KVH, hd)]).view(pages, ps, KVH, hd).transpose(1, 2)
+        vp = torch.cat([v, torch.zeros(pad, KVH, hd)]).view(pages, ps, KVH, hd).transpose(1, 2)
+        kpool[order], vpool[order] = kp, vp
+        table = order.to(torch.int32).view(1, pages)
+        qkv = torch.cat([q.reshape(n, H * hd), torch.zeros(n, 2 * KVH * hd)], dim=1)
+        tile_tokens = K.mfma_tile_tokens(hd, H // KVH) * blocks
+        tiles = dev(torch.tensor(K.build_q_tiles([0], [n], [n], tile_tokens), dtype=torch.int32).view(-1, 4))
+        out = torch.empty(n, H * hd, device="cuda", dtype=torch.bfloat16)
+        K.mfma_attention(dev(qkv, torch.bfloat16), dev(kpool, torch.bfloat16), dev(vpool, torch.bfloat16), dev(table), tiles, out,
+                         H, KVH, hd, 1.0 / math.sqrt(hd), None, 1, None, tile_tokens)
+        got = out.float().cpu().view(n, H, hd)
+        assert not torch.isnan(got).any()
+        rows = sorted(set([0, 1, 15, 16, 31, 32, 33, 63, 64, 65, n // 2, n // 2 + 17, n - 65, n - 33, n - 2, n - 1]
+                          + torch.randint(0, n, (24,), generator=g).tolist()))
+        for t in rows:
+            for h in (0, 3, H - 1):
+                kk, vv = k[:t + 1, h // (H // KVH)].double(), v[:t + 1, h // (H // KVH)].double()
+                w = torch.softmax(kk @ q[t, h].double() / math.sqrt(hd), dim=0)
+                assert float((got[t, h].double() - w @ vv).abs().max()) < 2e-2, (n, t, h)
+
+
 # ---- the matrix-core kernel for prompt portions in float32
 
 @pytest.mark.parametrize("H,KVH,hd,ps", [(4, 2, 16, 16), (6, 1, 32, 8), (5, 5, 48, 5), (32, 8, 64, 16), (3, 3, 80, 16),
