@@ -73,8 +73,11 @@ __global__ __launch_bounds__(MA_WAVES * WAVE) void mfma_attention_f32_kernel(
     // As many workgroups as the chip holds at once; the tiles come sorted by the keys they walk,
     // longest first, and workgroup w takes tiles w, 2P-1-w, 2P+w, ... (P workgroups in x).
     for (int round = 0;; ++round) {
-        const int tile_at = (round & 1) ? (round + 1) * gridDim.x - 1 - blockIdx.x : round * gridDim.x + blockIdx.x;
-        if (tile_at >= n_tiles) break;
+        int tile_at = (round & 1) ? (round + 1) * gridDim.x - 1 - blockIdx.x : round * gridDim.x + blockIdx.x;
+        // one round only: the chip holds the whole grid, and a compute unit gets workgroups of the same x from the lower
+        // and the upper half of y; the upper half walks the sorted list backwards, so that long tiles meet short ones there
+        if (n_tiles <= static_cast<int>(gridDim.x) && 2 * blockIdx.y >= gridDim.y && gridDim.y > 1) tile_at = n_tiles - 1 - tile_at;
+        if (tile_at >= n_tiles || tile_at < 0) break;
         const QTile tile = tiles[tile_at];
         const int G = H / KVH;
         const int hpt = 1 << hpt_shift;
@@ -319,11 +322,12 @@ NI_EXPORT int ni_mfma_attention_f32(const void* q, int q_stride, const void* kpo
         units[pow2] = cus;
         slots[pow2] = cus * per_cu;
     }
-    // an even number of rounds pairs long tiles with short ones; with few tiles every one gets a workgroup
+    // with no more tiles than the chip holds workgroups every tile gets one (paired over the compute units, see the
+    // kernel); else two rounds pair long tiles with short ones, or more, as few as fit the chip
     int rounds = 1;
-    if (n_tiles * per_tile >= 4 * units[pow2]) {
+    if (n_tiles * per_tile > slots[pow2]) {
         rounds = 2;
-        while ((n_tiles + rounds - 1) / rounds * per_tile > slots[pow2] && rounds < n_tiles) rounds += 2;
+        while ((n_tiles + rounds - 1) / rounds * per_tile > slots[pow2] && rounds < n_tiles) rounds += 1;
     }
     const int in_x = (n_tiles + rounds - 1) / rounds;
     dim3 grid(in_x, KVH * chunks, nsplit);
