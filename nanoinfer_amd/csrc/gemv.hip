@@ -32,8 +32,11 @@
 // workgroup then normalises the rows itself (sums of squares over the wavefronts' K slices, met in
 // LDS) while its first pieces of W are already on their way, and keeps the normalised operand in
 // registers (K up to XP * 8 pieces).  With that prologue and the residual epilogue a block of a
-// decoder needs no kernel of its own for the residual sum or the norm.  The kernel for 17 to 64
-// rows brings x through LDS (see there).
+// decoder needs no kernel of its own for the residual sum or the norm.  Both also take float32
+// addends that h has not received yet (the shares of a product whose K range was cut to fill the
+// chip): the prologue normalises h plus the addends, the next residual epilogue brings them into
+// h with its own product, so the cut costs no kernel either.  The kernel for 17 to 64 rows brings
+// x through LDS (see there).
 // float32 inputs are multiplied in true float32 (no reduced-precision MFMA).
 #include <type_traits>
 
@@ -97,7 +100,14 @@ struct NormArgs {
     const float* part_o = nullptr;     // [M, heads, runs, hd]
     const float* part_ml = nullptr;    // [M, heads, runs, 2]: maximum (base e) and sum of each run
     int runs = 0, heads = 0, hd = 0;
+    // Addends that the residual stream has not received yet (the shares of a product whose K range was cut):
+    // float32 [n_pend, M, width of h].  The normalising prologue takes its rows as (h + pend[0]) + pend[1];
+    // the residual epilogue stores ((h + pend[0]) + pend[1]) + product.  The kernel that normalises does not
+    // write h, so between the two nothing has to be ordered.
+    const float* pend = nullptr;
+    int n_pend = 0;
 };
+#define PROLOGUE_ADDENDS_MAX 2        // addends the normalising prologue holds in registers beside its rows of h
 #define PRO_NORM 0      // the prologue computes RMSNorm(h)
 #define PRO_MERGE 1     // the prologue merges the key runs of an attention
 #define MERGE_RUNS_MAX 16         // key runs the merging prologue takes for one row
@@ -121,7 +131,8 @@ struct RopeArgs {
 // columns of every tile, the second the others (each has multiplied only its own rows of W).
 template <typename T, typename TOUT, int MB, int NT, int EPI, int WV = GV_WAVES, bool EXT = false, int HALVES = 1>
 __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TOUT* __restrict__ y, int M, int N, int I,
-                                              const RopeArgs& rope, float* ext = nullptr) {
+                                              const RopeArgs& rope, float* ext = nullptr, const float* pend = nullptr,
+                                              int n_pend = 0) {
     const int tid = threadIdx.x;
     const int wave = tid / WAVE, lane = tid % WAVE;
     const int wg = blockIdx.x / HALVES;
@@ -216,8 +227,19 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
             for (int w = 0; w < WV; ++w) v += red[w][ot * MB + mb][src];
         }
         TOUT* dst = y + static_cast<size_t>(m) * out_width + n;
-        if constexpr (EPI == EPI_RESIDUAL) *dst += v;      // float32 residual stream, this workgroup's own columns
-        else st(dst, v);
+        if constexpr (EPI == EPI_RESIDUAL) {      // float32 residual stream, this workgroup's own columns
+            float sum = *dst;
+            if (n_pend > 0) {       // what the stream has not received yet, in its order, then the product
+                const float* p = pend + static_cast<size_t>(m) * N + n;
+                const size_t stride = static_cast<size_t>(M) * N;
+                const float p0 = p[0], p1 = n_pend > 1 ? p[stride] : 0.f;      // asked for together
+                sum = (sum + p0) + p1;
+                for (int a = 2; a < n_pend; ++a) sum += p[a * stride];
+            }
+            *dst = sum + v;
+        } else {
+            st(dst, v);
+        }
     }
 }
 
@@ -307,7 +329,11 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
 // memory traffic, and their columns of the product are not stored).  A compute unit alone draws
 // about 37 GB/s from memory, so a launch of fewer workgroups than compute units cannot stream at
 // the chip's rate.
-template <typename T, typename TOUT, int NT, int EPI, int XP, int WV, int SR, int HALVES = 1, int PRO = PRO_NORM>
+// PEND (staged normalising prologue only): h comes with addends it has not received yet, which the prologue
+// adds to its rows.  A kernel of its own, because the addends wait in registers beside the rows of h while the
+// first pieces of W are asked for: for eight rows that is 172 registers instead of 120, one workgroup a compute
+// unit instead of two, which the products without addends should not pay.
+template <typename T, typename TOUT, int NT, int EPI, int XP, int WV, int SR, int HALVES = 1, int PRO = PRO_NORM, bool PEND = false>
 __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                                    TOUT* __restrict__ y, int M, int N, int K, int I,
                                                                    RopeArgs rope, NormArgs norm, int splits) {
@@ -479,10 +505,38 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
                     hv[m][q] = (m < M && in) ? *reinterpret_cast<const float4*>(norm.h + static_cast<size_t>(m) * K + k)
                                              : make_float4(0.f, 0.f, 0.f, 0.f);
             }
-            // loads come back in the order they went out: the few of the prologue first, W right behind
-            __builtin_amdgcn_sched_barrier(0);
-            load_w(wave, wa_a);
-            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (PEND) {
+                // addends that h has not received yet: asked for with the rows, added in their order
+                float4 pv[PROLOGUE_ADDENDS_MAX][SR][QPT];
+#pragma unroll
+                for (int a = 0; a < PROLOGUE_ADDENDS_MAX; ++a)
+#pragma unroll
+                    for (int q = 0; q < QPT; ++q) {
+                        const int k = 4 * (tid + q * THREADS);
+#pragma unroll
+                        for (int m = 0; m < SR; ++m)
+                            pv[a][m][q] = (a < norm.n_pend && m < M && k < K)
+                                              ? *reinterpret_cast<const float4*>(norm.pend + (static_cast<size_t>(a) * M + m) * K + k)
+                                              : make_float4(0.f, 0.f, 0.f, 0.f);
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+                load_w(wave, wa_a);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int a = 0; a < PROLOGUE_ADDENDS_MAX; ++a)
+#pragma unroll
+                    for (int m = 0; m < SR; ++m)
+#pragma unroll
+                        for (int q = 0; q < QPT; ++q) {
+                            hv[m][q].x += pv[a][m][q].x; hv[m][q].y += pv[a][m][q].y;
+                            hv[m][q].z += pv[a][m][q].z; hv[m][q].w += pv[a][m][q].w;
+                        }
+            } else {
+                // loads come back in the order they went out: the few of the prologue first, W right behind
+                __builtin_amdgcn_sched_barrier(0);
+                load_w(wave, wa_a);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             // all SR rows go through the same straight code (rows that do not exist are zeros): the
             // reductions of the rows then overlap instead of waiting for one another behind branches
             float ss[SR];
@@ -616,9 +670,10 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
     }
     if constexpr (SHARE_LDS) {
         __syncthreads();                   // every wavefront has taken its operands from the staged rows
-        skinny_finish<T, TOUT, 1, NT, EPI, WV, true, HALVES>(acc, y, M, N, I, rope, reinterpret_cast<float*>(staged_rows));
+        skinny_finish<T, TOUT, 1, NT, EPI, WV, true, HALVES>(acc, y, M, N, I, rope, reinterpret_cast<float*>(staged_rows),
+                                                             norm.pend, norm.n_pend);
     } else {
-        skinny_finish<T, TOUT, 1, NT, EPI, WV, false, HALVES>(acc, y, M, N, I, rope);
+        skinny_finish<T, TOUT, 1, NT, EPI, WV, false, HALVES>(acc, y, M, N, I, rope, nullptr, norm.pend, norm.n_pend);
     }
 }
 
@@ -779,6 +834,17 @@ template <typename T, typename TOUT, int EPI, int XP>
 static int launch_decode(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream,
                          RopeArgs rope = RopeArgs{}, NormArgs norm = NormArgs{}, int splits = 1) {
     if (splits != 1 && (XP != 0 || EPI != EPI_STORE)) return -8;      // shares are stored, not finished
+    if (norm.n_pend > 0) {
+        // addends that the residual stream has not received: for the staged normalising prologue (up to
+        // eight rows, at most two tiles a workgroup), or for the residual epilogue
+        if (norm.pend == nullptr) return -10;
+        if (XP > 0) {
+            const bool staged = (XP == 4 || (XP == 8 && std::is_same<T, float>::value)) && M <= 8 && (EPI == EPI_ROPE || NT < 4);
+            if (!staged || norm.n_pend > PROLOGUE_ADDENDS_MAX) return -10;
+        } else if (EPI != EPI_RESIDUAL) {
+            return -10;
+        }
+    }
     const int out_width = (EPI == EPI_SWIGLU) ? I : N;
     const int tiles = (out_width + 15) / 16;
     auto run = [&](auto nt_tag) {
@@ -793,6 +859,14 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
         const bool halve = CAN_HALVE && grid <= HALVE_BELOW;
         auto launch = [&](auto wv_tag, auto sr_tag, auto halves_tag) {
             constexpr int WVc = decltype(wv_tag)::value, SRc = decltype(sr_tag)::value, Hc = decltype(halves_tag)::value;
+            if constexpr (XP > 0 && SRc > 0) {
+                if (norm.n_pend > 0) {
+                    skinny_decode_kernel<T, TOUT, NTc, EPI, XP, WVc, SRc, Hc, PRO_NORM, true>
+                        <<<dim3(grid * Hc, splits), WVc * WAVE, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I,
+                                                                              rope, norm, splits);
+                    return;
+                }
+            }
             skinny_decode_kernel<T, TOUT, NTc, EPI, XP, WVc, SRc, Hc><<<dim3(grid * Hc, splits), WVc * WAVE, 0, stream>>>(
                 (const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm, splits);
         };
@@ -869,8 +943,9 @@ static int launch_rows(const void* x, const void* W, void* y, int M, int N, int 
 
 template <typename T, typename TOUT, int EPI>
 static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, bool tiled,
-                     hipStream_t stream, RopeArgs rope = RopeArgs{}) {
-    if (M <= 16 && tiled) return launch_decode<T, TOUT, EPI, 0>(x, W, y, M, N, K, I, NT, stream, rope);
+                     hipStream_t stream, RopeArgs rope = RopeArgs{}, NormArgs addends = NormArgs{}) {
+    if (M <= 16 && tiled) return launch_decode<T, TOUT, EPI, 0>(x, W, y, M, N, K, I, NT, stream, rope, addends);
+    if (addends.n_pend > 0) return -10;      // only the kernel of the decode step proper adds them
     if (tiled) {
         // (with the rotation epilogue the rows are dealt out 32 to a workgroup: see skinny_rows_kernel)
         if (M <= 32 || EPI == EPI_ROPE) return launch_rows<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
@@ -911,8 +986,10 @@ static int launch_normed(const NormArgs& norm, const void* W, void* y, int M, in
 // 3 add into y, the float32 residual stream [M, N] (tiled W).
 // K must be a multiple of 16 bytes' worth of elements x 2 (bf16: 16, f32: 8); M <= 64.
 // tiled: W is in the re-tiled order described at the top (swiglu then needs N/2 to be a multiple of 16).
+// pend, n_pend (epilogue 3, at most 16 rows): float32 [n_pend, M, N] that y has not received yet and that are
+// added before the product, y = ((y + pend[0]) + pend[1] ...) + x . W^T; null, 0: none.
 NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N, int K, int epilogue, int tiles_per_group,
-                             int tiled, int dtype, hipStream_t stream) {
+                             int tiled, int dtype, const void* pend, int n_pend, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64) return -1;
     const int el = dtype == 0 ? 8 : 16;
@@ -920,12 +997,16 @@ NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N
     const int I = N / 2;
     if (epilogue == 2 && (N % 2)) return -3;
     if (epilogue == 2 && tiled && (I % 16)) return -4;
+    if (n_pend < 0 || n_pend > 16 || (n_pend > 0 && (epilogue != 3 || !pend))) return -10;
+    NormArgs addends{nullptr, nullptr, 0.f};
+    addends.pend = (const float*)pend;
+    addends.n_pend = n_pend;
     if (dtype == 0) {
-        if (epilogue == 3) return launch_mb<float, float, EPI_RESIDUAL>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
+        if (epilogue == 3) return launch_mb<float, float, EPI_RESIDUAL>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream, RopeArgs{}, addends);
         if (epilogue == 2) return launch_mb<float, float, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
         return launch_mb<float, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
     }
-    if (epilogue == 3) return launch_mb<bf16_t, float, EPI_RESIDUAL>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
+    if (epilogue == 3) return launch_mb<bf16_t, float, EPI_RESIDUAL>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream, RopeArgs{}, addends);
     if (epilogue == 2) return launch_mb<bf16_t, bf16_t, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
     if (epilogue == 1) return launch_mb<bf16_t, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
     return launch_mb<bf16_t, bf16_t, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
@@ -958,16 +1039,24 @@ NI_EXPORT int ni_skinny_prologue_ok(int M, int K, int dtype) {
     return (dtype == 0 ? prologue_pieces<float>(K) : prologue_pieces<bf16_t>(K)) != 0;
 }
 
+NI_EXPORT int ni_skinny_prologue_addends() { return PROLOGUE_ADDENDS_MAX; }
+
 // The same product on RMSNorm(h) instead of a given x: h float32 [M <= 8, K], norm_weight float32 [K],
 // W re-tiled.  epilogue 0 (store in the compute type) or 2 (SwiGLU).
+// pend, n_pend: float32 [n_pend <= 2, M, K] that h has not received yet; the rows are normalised as
+// (h + pend[0]) + pend[1] and h itself is left as it is (at most two tiles a workgroup).
 NI_EXPORT int ni_skinny_gemm_normed(const void* h, const void* norm_weight, float eps, const void* W, void* y, int M, int N,
-                                    int K, int epilogue, int tiles_per_group, int dtype, hipStream_t stream) {
+                                    int K, int epilogue, int tiles_per_group, int dtype, const void* pend, int n_pend,
+                                    hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (!ni_skinny_prologue_ok(M, K, dtype)) return -5;
     if (epilogue != 0 && epilogue != 2) return -6;
     const int I = N / 2;
     if (epilogue == 2 && ((N % 2) || (I % 16))) return -4;
-    const NormArgs norm{(const float*)h, (const float*)norm_weight, eps};
+    if (n_pend < 0 || (n_pend > 0 && !pend)) return -10;
+    NormArgs norm{(const float*)h, (const float*)norm_weight, eps};
+    norm.pend = (const float*)pend;
+    norm.n_pend = n_pend;
     if (dtype == 0) {
         if (epilogue == 2) return launch_normed<float, EPI_SWIGLU>(norm, W, y, M, N, K, I, tiles_per_group, stream);
         return launch_normed<float, EPI_STORE>(norm, W, y, M, N, K, I, tiles_per_group, stream);
@@ -1002,12 +1091,17 @@ static int launch_merged(const NormArgs& merge, const void* W, void* y, int M, i
     return NI_LAUNCH_RESULT();
 }
 
+// pend, n_pend (epilogue 3): as for ni_skinny_gemm.
 NI_EXPORT int ni_skinny_gemm_merged(const void* part_o, const void* part_ml, int runs, int heads, int hd, const void* W,
-                                    void* y, int M, int N, int epilogue, int dtype, hipStream_t stream) {
+                                    void* y, int M, int N, int epilogue, int dtype, const void* pend, int n_pend,
+                                    hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (!part_o || !part_ml || !ni_skinny_merge_ok(M, heads, hd, runs, dtype)) return -5;
     if (epilogue != 0 && epilogue != 3) return -6;
+    if (n_pend < 0 || n_pend > 16 || (n_pend > 0 && (epilogue != 3 || !pend))) return -10;
     NormArgs merge{nullptr, nullptr, 0.f};
+    merge.pend = (const float*)pend;
+    merge.n_pend = n_pend;
     merge.part_o = (const float*)part_o;
     merge.part_ml = (const float*)part_ml;
     merge.runs = runs; merge.heads = heads; merge.hd = hd;
@@ -1018,11 +1112,12 @@ NI_EXPORT int ni_skinny_gemm_merged(const void* part_o, const void* part_ml, int
 // Product with the stacked [q; k; v] matrix ((H + 2 KVH) * hd rows), rotation of query and key
 // heads by the rows' positions, queries to q_out [M, H * hd], keys and values into the pools at
 // slot_mapping (null: not stored).  hd must be a multiple of 32 and fully rotated.
-// With x null the product is taken on RMSNorm(h): h float32 [M <= 8, K], norm_weight [K], W re-tiled.
+// With x null the product is taken on RMSNorm(h): h float32 [M <= 8, K], norm_weight [K], W re-tiled; pend, n_pend as
+// for ni_skinny_gemm_normed.
 NI_EXPORT int ni_skinny_qkv_rope(const void* x, const void* h, const void* norm_weight, float eps, const void* W,
                                  void* q_out, const void* positions, const void* cos_t, const void* sin_t,
                                  const void* slot_mapping, void* kpool, void* vpool, int M, int K, int H, int KVH, int hd,
-                                 int page_size, int tiled, int dtype, hipStream_t stream) {
+                                 int page_size, int tiled, int dtype, const void* pend, int n_pend, hipStream_t stream) {
     if (M <= 0) return 0;
     if (M > 64) return -1;
     if (K % (dtype == 0 ? 8 : 16) != 0) return -2;
@@ -1033,10 +1128,14 @@ NI_EXPORT int ni_skinny_qkv_rope(const void* x, const void* h, const void* norm_
     // the grid is sized from the output width: one workgroup per two tiles
     if (!x) {
         if (!h || !norm_weight || !tiled || !ni_skinny_prologue_ok(M, K, dtype)) return -5;
-        const NormArgs norm{(const float*)h, (const float*)norm_weight, eps};
+        if (n_pend < 0 || (n_pend > 0 && !pend)) return -10;
+        NormArgs norm{(const float*)h, (const float*)norm_weight, eps};
+        norm.pend = (const float*)pend;
+        norm.n_pend = n_pend;
         if (dtype == 0) return launch_normed<float, EPI_ROPE>(norm, W, q_out, M, N, K, 0, 2, stream, rope);
         return launch_normed<bf16_t, EPI_ROPE>(norm, W, q_out, M, N, K, 0, 2, stream, rope);
     }
+    if (n_pend != 0) return -10;      // addends go with the normalising prologue only
     if (dtype == 0) return launch_mb<float, float, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, tiled != 0, stream, rope);
     return launch_mb<bf16_t, bf16_t, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, tiled != 0, stream, rope);
 }

@@ -558,6 +558,7 @@ def skinny_wins(M: int, K: int, dtype: torch.dtype, weight=None) -> bool:
         return K <= 2048 and (M <= 32 or weight.rows.shape[0] < 8192)
     return M <= 32 or K <= 4096
 FUSE_NORMS = True           # residual sums and norms ride on the skinny products of a decode step where they can
+ADDENDS_IN_PROLOGUE = True  # the shares of a cut product are added by the next normalising prologue and residual epilogue
 MERGE_IN_PRODUCT = True     # the key runs of a decode step's attention are merged by the output product where it can
 SPLIT_K = True              # products of 17 to 64 rows on matrices of few tiles are cut along K, the next norm adds the shares
 
@@ -624,12 +625,17 @@ def _tiles_per_group(n_out: int) -> int:
 class NormedInput:
     """The input of a product given as the float32 residual stream ``h`` [M, K] together with the
     weight and eps of the RMSNorm that stands before the product: the skinny product normalises the
-    rows in its prologue instead of a kernel of its own (:func:`norm_prologue_ok` says when)."""
+    rows in its prologue instead of a kernel of its own (:func:`norm_prologue_ok` says when).
+    ``pending``: float32 addends [S, M, K] that ``h`` has not received yet (the shares of a product
+    whose K range was cut); the rows are normalised as ``(h + pending[0]) + pending[1]`` and ``h``
+    is left as it is: whoever adds into ``h`` next (the residual epilogue of a later product, given
+    the same addends) brings them in."""
 
-    __slots__ = ("h", "weight", "eps", "dtype")
+    __slots__ = ("h", "weight", "eps", "dtype", "pending")
 
-    def __init__(self, h: torch.Tensor, weight: torch.Tensor, eps: float, dtype: torch.dtype):
-        self.h, self.weight, self.eps, self.dtype = h, weight, float(eps), dtype
+    def __init__(self, h: torch.Tensor, weight: torch.Tensor, eps: float, dtype: torch.dtype,
+                 pending: Optional[torch.Tensor] = None):
+        self.h, self.weight, self.eps, self.dtype, self.pending = h, weight, float(eps), dtype, pending
 
     @property
     def shape(self):
@@ -645,12 +651,35 @@ def _prologue_sizes_ok(M: int, K: int, code: int) -> bool:
     return bool(skinny_lib().ni_skinny_prologue_ok(M, K, code))
 
 
-def norm_prologue_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
+@functools.lru_cache(maxsize=None)
+def prologue_addends() -> int:
+    """How many pending addends the normalising prologue can add to its rows of h."""
+    return int(skinny_lib().ni_skinny_prologue_addends())
+
+
+def norm_prologue_ok(M: int, K: int, dtype: torch.dtype, weight, addends: int = 0, swiglu: bool = False) -> bool:
     """Whether the skinny product can take RMSNorm(h) for its input: at most eight rows (every
     workgroup normalises all of them: beyond that the norm as a kernel of its own is faster), a
-    re-tiled matrix, rows short enough for the normalised operand to stay in registers."""
-    return (isinstance(weight, Weight) and weight.tiles is not None and dtype in _DTYPE_CODE
-            and _prologue_sizes_ok(int(M), int(K), dtype_code(dtype)))
+    re-tiled matrix, rows short enough for the normalised operand to stay in registers.  With
+    ``addends`` pending addends of h (:class:`NormedInput`): at most :func:`prologue_addends`, and a
+    matrix of whose tiles a workgroup takes at most two (``swiglu``: a stacked gate/up matrix)."""
+    if not (isinstance(weight, Weight) and weight.tiles is not None and dtype in _DTYPE_CODE
+            and _prologue_sizes_ok(int(M), int(K), dtype_code(dtype))):
+        return False
+    if addends == 0:
+        return True
+    n_out = weight.rows.shape[0] // 2 if swiglu else weight.rows.shape[0]
+    return addends <= prologue_addends() and _tiles_per_group(n_out) <= 2
+
+
+def _check_addends(pending: Optional[torch.Tensor], M: int, width: int):
+    """(pointer, count) of pending addends [S, M, width] in float32, for a kernel's arguments."""
+    if pending is None:
+        return None, 0
+    _gpu(pending, "pending addends", torch.float32)
+    if not (pending.dim() == 3 and pending.shape[1] == M and pending.shape[2] == width and 1 <= pending.shape[0] <= 16):
+        raise KernelError(f"pending addends {tuple(pending.shape)} against [S <= 16, {M}, {width}]")
+    return pending, int(pending.shape[0])
 
 
 def skinny_ksplit(M: int, K: int, dtype: torch.dtype, weight):
@@ -662,21 +691,27 @@ def skinny_ksplit(M: int, K: int, dtype: torch.dtype, weight):
     stream.  Measured at the 1B shape (us): [2048, 8192] at 64 rows 20.9 -> 12.0 (the library 20.4), at
     32 rows 14.2 -> 9.1, at 16 rows 12.7 -> 8.1, at 9 rows 9.8 -> 7.5; [2048, 2048] at 64 rows 7.3 -> 5.5,
     at 32 rows 5.0 -> 4.0, at 16 rows 4.65 -> 4.4.  Up to 16 rows only rows of 4,096 elements or more are
-    cut, and only where the norm that follows is a kernel of its own anyway (where the next product can
-    normalise in its prologue that is worth more than the cut).  Float32 rows are cut by the same rule (a decode
-    step of the 1B shape in float32: 4.51 -> 4.23 ms at batch 64, 3.18 -> 2.86 at 32, 2.42 -> 2.27 at 16; before,
-    the [2048, 8192] matrix at more than 32 rows went to the library, 41.6 us a layer).  (1, .): not cut."""
+    cut.  Up to eight rows the next product normalises in its prologue, which is worth more than the cut:
+    there the product goes in the two shares that this prologue can add to its rows of h by itself
+    (:class:`NormedInput` with ``pending``; the residual epilogue that follows brings them into h), which
+    needs no kernel for the sum ([2048, 8192] at 8 rows 11.7 -> 8.3 us, at one row 9.6 -> 8.0; a decode
+    step of the 1B shape 1.011 -> 0.982 ms at batch 8, 0.802 -> 0.776 at batch 1).  Float32 rows are cut by
+    the same rule (a decode step of the 1B shape in float32: 4.51 -> 4.23 ms at batch 64, 3.18 -> 2.86 at
+    32, 2.42 -> 2.27 at 16; before, the [2048, 8192] matrix at more than 32 rows went to the library,
+    41.6 us a layer).  (1, .): not cut."""
     if not (SPLIT_K and isinstance(weight, Weight) and weight.tiles is not None
             and 1 <= M <= SKINNY_MAX_ROWS and skinny_ok(M, K, dtype)):
         return 1, 1
     N = weight.rows.shape[0]
+    most = 16
     if M <= SKINNY_BEST_ROWS:
-        # float32 rows of 8,192 elements are cut even so: the matrix is twice the bytes, the cut gains more than the
-        # prologue (a float32 decode step of the 1B shape: 1.89 -> 1.82 ms at batch 8, 1.58 -> 1.55 at batch 1)
-        prologue_follows = (_prologue_sizes_ok(int(M), int(N), dtype_code(dtype))
-                            and not (dtype == torch.float32 and K >= 8192))
-        if K < 4096 or prologue_follows:
+        if K < 4096:
             return 1, 1
+        if _prologue_sizes_ok(int(M), int(N), dtype_code(dtype)):
+            # the next product can normalise in its prologue: cut into as many shares as that prologue adds
+            # to its rows of h (where it cannot, float32 rows of 8,192 elements are cut even so: the matrix
+            # is twice the bytes, the cut gains more than the prologue)
+            most = prologue_addends() if ADDENDS_IN_PROLOGUE else (16 if dtype == torch.float32 and K >= 8192 else 1)
     if dtype == torch.float32 and M > SKINNY_BEST_ROWS and N > 2048:
         # float32 past 16 rows: only matrices of at most 128 tiles gain by the cut; the library's product is faster on the
         # others ([3072, 8192] at 64 rows in two shares 54.6 us against 45.2, [4096, 4096] 33.5 : 26.8, [4096, 14336] 93.8 : 86.2)
@@ -686,7 +721,8 @@ def skinny_ksplit(M: int, K: int, dtype: torch.dtype, weight):
     pieces = (K + 63) // 64
     # as many shares as keep the workgroups within one to a compute unit (192 groups in two shares are one and a
     # half rounds: measured slower), each share at least sixteen pieces
-    return max(1, min(COMPUTE_UNITS // groups, pieces // 16, 16)), per
+    shares = max(1, min(COMPUTE_UNITS // groups, pieces // 16, most))
+    return shares, (per if shares > 1 else 1)
 
 
 def skinny_gemm_ksplit(x: torch.Tensor, weight, shares: int, per_group: int) -> torch.Tensor:
@@ -712,6 +748,14 @@ def residual_epilogue_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
     return skinny_wins(M, K, dtype, weight) or skinny_ksplit(M, K, dtype, weight)[0] > 1
 
 
+def residual_takes_addends(M: int, K: int, dtype: torch.dtype, weight) -> bool:
+    """Whether the product that goes into the residual stream can bring pending addends of the
+    stream in with it (``linear(..., residual=h, pending=...)``): the decode step's kernel with the
+    residual epilogue, not the product in shares."""
+    return (isinstance(weight, Weight) and weight.tiles is not None and M <= SKINNY_BEST_ROWS
+            and skinny_wins(M, K, dtype, weight) and skinny_ksplit(M, K, dtype, weight)[0] == 1)
+
+
 def _check_normed(x: NormedInput, Kd: int) -> None:
     _gpu(x.h, "h", torch.float32)
     if not (x.h.dim() == 2 and x.h.shape[1] == Kd):
@@ -719,12 +763,14 @@ def _check_normed(x: NormedInput, Kd: int) -> None:
     _gpu(x.weight, "norm weight", torch.float32, (Kd,))
 
 
-def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bool = False) -> torch.Tensor:
+def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bool = False,
+                pending: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x . weight^T`` for at most 64 rows of ``x``, streaming ``weight`` once (MFMA).  ``out``
     may be float32 for bfloat16 inputs.  With ``swiglu`` the weight is a stacked [2I, K] matrix
     (gate rows, then up rows) and ``out`` [M, I] receives ``silu(gate) * up``.  With ``residual``
-    ``out`` is the float32 residual stream [M, N] and the product is added into it.  ``x`` may be a
-    :class:`NormedInput`."""
+    ``out`` is the float32 residual stream [M, N] and the product is added into it, after the
+    ``pending`` addends [S, M, N] that the stream has not received yet (at most 16 rows).  ``x`` may
+    be a :class:`NormedInput`."""
     normed = isinstance(x, NormedInput)
     M, Kd = x.shape
     dtype = x.dtype
@@ -754,22 +800,27 @@ def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bo
             raise KernelError(f"out must be {dtype} or float32")
         _gpu(out, "out", None, (M, N))
         epi = 1 if (out.dtype == torch.float32 and dtype != torch.float32) else 0
+    if pending is not None and not (residual and M <= SKINNY_BEST_ROWS):
+        raise KernelError("pending addends go with the residual epilogue of at most 16 rows")
+    pend, n_pend = _check_addends(pending, M, N)
     per_group = _tiles_per_group(N // 2 if swiglu else N)
     if swiglu and M > 32 and tiles is not None:
         # past 32 rows a workgroup that multiplies two pairs of gate and up tiles halves the loads of x,
         # which every workgroup brings in whole (measured at [16384, 2048]: 64 rows 22.0 -> 20.9 us, 17 and 32 rows lose)
         per_group = max(per_group, 4)
     if normed:
-        if not (tiles is not None and norm_prologue_ok(M, Kd, dtype, weight) and epi in (0, 2)):
+        h_pend, h_n = _check_addends(x.pending, M, Kd)
+        if not (tiles is not None and norm_prologue_ok(M, Kd, dtype, weight, h_n, swiglu) and epi in (0, 2)):
             raise KernelError(f"the normalising prologue does not take M={M}, K={Kd} in {dtype} with this matrix and epilogue")
         _check_normed(x, Kd)
         _check(skinny_lib().ni_skinny_gemm_normed(_ptr(x.h), _ptr(x.weight), ctypes.c_float(x.eps), _ptr(tiles), _ptr(out),
-                                                  M, N, Kd, epi, per_group, dtype_code(dtype), _stream()),
+                                                  M, N, Kd, epi, per_group, dtype_code(dtype), _ptr(h_pend), h_n, _stream()),
                "skinny_gemm_normed")
         return out
     _gpu(x, "x")
     _check(skinny_lib().ni_skinny_gemm(_ptr(x), _ptr(rows if tiles is None else tiles), _ptr(out), M, N, Kd, epi,
-                                       per_group, 0 if tiles is None else 1, dtype_code(dtype), _stream()), "skinny_gemm")
+                                       per_group, 0 if tiles is None else 1, dtype_code(dtype), _ptr(pend), n_pend,
+                                       _stream()), "skinny_gemm")
     return out
 
 
@@ -792,12 +843,12 @@ def skinny_merge_wins(M: int, H: int, hd: int, nsplit: int, dtype: torch.dtype, 
 
 
 def skinny_gemm_merged(workspace: torch.Tensor, nsplit: int, M: int, H: int, hd: int, weight, out: torch.Tensor,
-                       residual: bool = False) -> torch.Tensor:
+                       residual: bool = False, pending: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``attn . weight^T`` where ``attn`` [M, H*hd] is still in the pieces that an attention kernel
     left in ``workspace`` for ``nsplit`` key runs (float32: outputs [M, H, nsplit, hd], then
     (maximum, sum) pairs [M, H, nsplit, 2]): the runs are merged in the product's prologue, with the
     numbers the merge kernel gives.  ``out`` as for :func:`skinny_gemm`, with ``residual`` the
-    float32 residual stream."""
+    float32 residual stream (and ``pending`` what it has not received yet)."""
     rows, tiles = _rows_and_tiles(weight)
     N = rows.shape[0]
     dtype = rows.dtype
@@ -814,8 +865,12 @@ def skinny_gemm_merged(workspace: torch.Tensor, nsplit: int, M: int, H: int, hd:
         _gpu(out, "out", torch.float32, (M, N))
     else:
         _gpu(out, "out", dtype, (M, N))
+    if pending is not None and not residual:
+        raise KernelError("pending addends go with the residual epilogue")
+    pend, n_pend = _check_addends(pending, M, N)
     _check(skinny_lib().ni_skinny_gemm_merged(_ptr(part_o), _ptr(part_ml), nsplit, H, hd, _ptr(tiles), _ptr(out), M, N,
-                                              3 if residual else 0, dtype_code(dtype), _stream()), "skinny_gemm_merged")
+                                              3 if residual else 0, dtype_code(dtype), _ptr(pend), n_pend, _stream()),
+           "skinny_gemm_merged")
     return out
 
 
@@ -859,9 +914,11 @@ def skinny_qkv_rope(x, w_qkv, positions: torch.Tensor, cos: torch.Tensor,
         if not (kpool.dim() == 4 and kpool.shape[1] == KVH and kpool.shape[3] == hd):
             raise KernelError(f"pool must be [pages, {KVH}, page_size, {hd}], is {tuple(kpool.shape)}")
         page_size = kpool.shape[2]
+    pend, n_pend = None, 0
     if normed:
-        if not (norm_prologue_ok(M, Kd, dtype, w_qkv)):
-            raise KernelError(f"the normalising prologue does not take M={M}, K={Kd} in {dtype}")
+        pend, n_pend = _check_addends(x.pending, M, Kd)
+        if not (norm_prologue_ok(M, Kd, dtype, w_qkv, min(n_pend, prologue_addends()))) or n_pend > prologue_addends():
+            raise KernelError(f"the normalising prologue does not take M={M}, K={Kd} in {dtype} with {n_pend} addends")
         _check_normed(x, Kd)
         x_ptr, h_ptr, nw_ptr, eps = None, _ptr(x.h), _ptr(x.weight), x.eps
         device = x.h.device
@@ -873,11 +930,12 @@ def skinny_qkv_rope(x, w_qkv, positions: torch.Tensor, cos: torch.Tensor,
     _check(skinny_lib().ni_skinny_qkv_rope(x_ptr, h_ptr, nw_ptr, ctypes.c_float(eps), _ptr(rows if tiles is None else tiles),
                                            _ptr(q), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping), _ptr(kpool),
                                            _ptr(vpool), M, Kd, H, KVH, hd, page_size, 0 if tiles is None else 1,
-                                           dtype_code(dtype), _stream()), "skinny_qkv_rope")
+                                           dtype_code(dtype), _ptr(pend), n_pend, _stream()), "skinny_qkv_rope")
     return q
 
 
-def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optional[torch.Tensor] = None):
+def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optional[torch.Tensor] = None,
+           pending: Optional[torch.Tensor] = None):
     """``x . weight^T`` with ``weight`` stored [out, in].  Few rows go to the hand-written skinny
     product; many rows to the library (rocBLAS/hipBLASLt), where float32 inputs are multiplied in
     true float32 (the reduced-precision matrix modes of the library are switched off at import).
@@ -885,7 +943,9 @@ def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optiona
     :class:`NormedInput` where :func:`norm_prologue_ok` holds.  With ``residual`` (the float32
     residual stream, where :func:`residual_epilogue_ok` holds) the product is added into it and
     nothing is returned, or (17 to 64 rows on a matrix of few tiles, :func:`skinny_ksplit`) it is
-    returned as float32 addends [S, M, N] that the next norm adds to the stream."""
+    returned as float32 addends [S, M, N] that the next norm adds to the stream.  ``pending``: addends
+    that ``residual`` has not received yet and that the product brings in with it (where
+    :func:`residual_takes_addends` holds)."""
     rows, _ = _rows_and_tiles(weight)
     if isinstance(x, NormedInput):
         if not (residual is None):
@@ -901,11 +961,15 @@ def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optiona
     if residual is not None:
         if not (residual_epilogue_ok(x.shape[0], x.shape[1], x.dtype, weight)):
             raise KernelError("the residual epilogue does not take this product")
+        if pending is not None and not residual_takes_addends(x.shape[0], x.shape[1], x.dtype, weight):
+            raise KernelError("this product cannot bring the residual stream's pending addends in")
         shares, per = skinny_ksplit(x.shape[0], x.shape[1], x.dtype, weight)
         if shares > 1:
             return skinny_gemm_ksplit(x, weight, shares, per)      # addends for the next norm
-        skinny_gemm(x, weight, residual, residual=True)
+        skinny_gemm(x, weight, residual, residual=True, pending=pending)
         return None
+    if pending is not None:
+        raise KernelError("pending addends go with a residual output")
     out_dtype = out_dtype or x.dtype
     if skinny_wins(x.shape[0], x.shape[1], x.dtype, weight):
         out = torch.empty(x.shape[0], rows.shape[0], dtype=out_dtype, device=x.device)

@@ -87,9 +87,10 @@ class RMSNorm(Part):
         out = torch.empty(n, self.size, dtype=self.rt.dtype, device=self.rt.device)
         return K.add_rmsnorm(h, pending, self.weight, self.eps, out, rows)
 
-    def as_prologue(self, h: torch.Tensor):
-        """This norm of ``h`` (nothing pending) as an input that a product can normalise itself."""
-        return K.NormedInput(h, self.weight, self.eps, self.rt.dtype)
+    def as_prologue(self, h: torch.Tensor, pending: Optional[torch.Tensor] = None):
+        """This norm of ``h`` as an input that a product can normalise itself; ``pending`` (float32
+        addends [S, T, size] that ``h`` has not received) goes along for a part that ``carries_addends``."""
+        return K.NormedInput(h, self.weight, self.eps, self.rt.dtype, pending)
 
 
 # ------------------------------------------------------------------ position
@@ -243,8 +244,20 @@ class Attention(Part):
         stream without a kernel for the sum (added by the product itself, or left as float32 addends)."""
         return K.FUSE_NORMS and K.residual_epilogue_ok(T, self.H * self.hd, self.rt.dtype, self.w_o)
 
+    def carries_addends(self, T: int, addends: int) -> bool:
+        """Whether ``forward`` can be given, for T tokens, a normed input that holds ``addends`` pending
+        addends of ``h``, together with ``residual=h``: its first product normalises ``h`` plus the addends,
+        its last one adds them into ``h`` with its own output."""
+        d = self.w_qkv.shape[1]
+        return (self.takes_normed(T) and self.adds_residual(T)
+                and K.norm_prologue_ok(T, d, self.rt.dtype, self.w_qkv, addends)
+                and K.residual_takes_addends(T, self.H * self.hd, self.rt.dtype, self.w_o))
+
     def forward(self, x, ctx, cache: LayerCache, residual: Optional[torch.Tensor] = None):
         T = x.shape[0]
+        carried = getattr(x, "pending", None)       # addends of the residual stream that came with a normed input
+        if carried is not None and residual is None:
+            raise K.KernelError("pending addends of the residual stream need residual=h to go into")
         tables = self.position.tables()
         cos, sin = tables if tables is not None else (None, None)
         slots = cache.slot_mapping if cache.writes else None
@@ -270,7 +283,7 @@ class Attention(Part):
             ws = ctx.workspace(T * self.H * nsplit * (self.hd + 2)) if nsplit > 1 else None
             K.mfma_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, out, self.H, self.KVH, self.hd,
                              self.scale, self.window, nsplit, ws, tile_tokens)
-            return K.linear(out, self.w_o, residual=residual)
+            return K.linear(out, self.w_o, residual=residual, pending=carried)
         # single tokens and short portions, token by token
         max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window)
         on_matrix_cores = K.mfma_token_ok(x.dtype, self.hd)
@@ -282,14 +295,14 @@ class Attention(Part):
             K.mfma_token_attention(qkv, cache.kpool, cache.vpool, cache.block_table, ctx.seq_of_token, ctx.positions,
                                    out, self.H, self.KVH, self.hd, self.scale, self.window, nsplit, ws, merge=False)
             if residual is not None:
-                K.skinny_gemm_merged(ws, nsplit, T, self.H, self.hd, self.w_o, residual, residual=True)
+                K.skinny_gemm_merged(ws, nsplit, T, self.H, self.hd, self.w_o, residual, residual=True, pending=carried)
                 return None
             y = torch.empty(T, self.w_o.rows.shape[0], dtype=x.dtype, device=x.device)
             return K.skinny_gemm_merged(ws, nsplit, T, self.H, self.hd, self.w_o, y)
         attend = K.mfma_token_attention if on_matrix_cores else K.token_attention
         attend(qkv, cache.kpool, cache.vpool, cache.block_table, ctx.seq_of_token, ctx.positions, out,
                self.H, self.KVH, self.hd, self.scale, self.window, nsplit, ws)
-        return K.linear(out, self.w_o, residual=residual)
+        return K.linear(out, self.w_o, residual=residual, pending=carried)
 
 
 # ------------------------------------------------------------------ feed-forward
@@ -323,8 +336,17 @@ class SwiGLU(Part):
     def adds_residual(self, T: int) -> bool:
         return K.FUSE_NORMS and K.residual_epilogue_ok(T, self.intermediate_size, self.rt.dtype, self.w_down)
 
+    def carries_addends(self, T: int, addends: int) -> bool:
+        d = self.w_gate_up.shape[1]
+        return (self.takes_normed(T) and self.adds_residual(T)
+                and K.norm_prologue_ok(T, d, self.rt.dtype, self.w_gate_up, addends, swiglu=True)
+                and K.residual_takes_addends(T, self.intermediate_size, self.rt.dtype, self.w_down))
+
     def forward(self, x, ctx, residual: Optional[torch.Tensor] = None):
-        return K.linear(K.linear_swiglu(x, self.w_gate_up), self.w_down, residual=residual)
+        carried = getattr(x, "pending", None)       # addends of the residual stream that came with a normed input
+        if carried is not None and residual is None:
+            raise K.KernelError("pending addends of the residual stream need residual=h to go into")
+        return K.linear(K.linear_swiglu(x, self.w_gate_up), self.w_down, residual=residual, pending=carried)
 
 
 # ------------------------------------------------------------------ block
@@ -338,8 +360,11 @@ class PreNormBlock:
     abilities of a mixer or feed-forward shorten this for steps of few tokens: ``adds_residual(T)``
     (given ``residual=h`` its last product adds into ``h`` itself and nothing is pending, or it
     returns float32 addends [S, T, d] for the next norm to sum) and ``takes_normed(T)`` (its first
-    product normalises ``h`` itself, given the norm's ``as_prologue(h)``).  A part without them is
-    run the plain way.
+    product normalises ``h`` itself, given the norm's ``as_prologue(h)``).  A part that has both may
+    also say ``carries_addends(T, S)``: given ``as_prologue(h, pending)`` with S float32 addends that
+    ``h`` has not received, and ``residual=h``, its first product normalises ``h`` plus the addends and
+    its last one brings them into ``h`` with its own output, so the shares of a cut product need no
+    kernel that sums them.  A part without these is run the plain way.
     """
 
     family = "block"
@@ -365,12 +390,19 @@ class PreNormBlock:
         return all(p.graph_safe is True for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn))
 
     def _normed_input(self, norm, part, h, pending):
-        """What ``part`` is given for ``norm(h + pending)``: the norm as a prologue where both sides can, else its output."""
+        """What ``part`` is given for ``norm(h + pending)``: the norm as a prologue where both sides can, else its
+        output.  Float32 addends go along with the prologue where the part ``carries_addends``: its first product
+        normalises ``h`` plus the addends, its last one adds them into ``h`` (it is then run with ``residual=h``)."""
         T = h.shape[0]
         takes = getattr(part, "takes_normed", None)
         prologue = getattr(norm, "as_prologue", None)
-        if pending is None and takes is not None and prologue is not None and takes(T):
-            return prologue(h)
+        if takes is not None and prologue is not None and takes(T):
+            if pending is None:
+                return prologue(h)
+            carries = getattr(part, "carries_addends", None)
+            if (carries is not None and getattr(norm, "takes_addends", False) and pending.dim() == 3
+                    and pending.dtype == torch.float32 and carries(T, pending.shape[0])):
+                return prologue(h, pending)
         return norm.forward(h, pending_for(norm, pending, self.rt.dtype))
 
     def forward(self, h, pending, ctx, cache: LayerCache):

@@ -58,3 +58,41 @@ def test_family_layer_sizes(name, dtype):
         want = plain_logits(folder, tuple(tokens), dtype)
         idx = sorted(got)
         assert_close(torch.stack([got[i] for i in idx]), want[idx], dtype, f"{name} {dtype} request {rid}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_whose_cut_products_are_added_by_the_next_layer(dtype, monkeypatch):
+    """At the 1B sizes a decode step's down product goes in two shares of K.  Up to eight rows the next
+    layer's first product adds them to its rows in its normalising prologue and its output product brings
+    them into the residual stream (no kernel sums them); the last layer's go to the final norm.  Steps of
+    eight, three and one token, recorded and not, against the plain implementation."""
+    from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
+    from nanoinfer_amd.parts import standard
+
+    folder = model_folder("1B", stored="bfloat16" if dtype == "bfloat16" else "float32")
+    vocab = ALL["1B"]["vocab_size"]
+    prompts = [random_tokens(vocab, 30 + 7 * i, 40 + i) for i in range(8)]
+    carried = []
+    carries = standard.Attention.carries_addends
+
+    def spy(self, T, addends):
+        carried.append((T, addends, carries(self, T, addends)))
+        return carried[-1][2]
+    monkeypatch.setattr(standard.Attention, "carries_addends", spy)
+    for graphs in (False, True):
+        runner = ModelRunner(folder, dtype=dtype, page_size=16, max_tokens=1024, max_requests=8, use_graphs=graphs)
+        for i, p in enumerate(prompts):
+            runner.step([StepEntry(i, p[:-4], [])])
+        got = {}
+        for k, live in ((4, 8), (3, 8), (2, 3), (1, 1)):        # the eight twice: the second time as a recorded step
+            out = runner.step([StepEntry(i, [prompts[i][-k]], [0]) for i in range(live)])
+            for i in range(live):
+                got[(i, len(prompts[i]) - k)] = out[i].clone()
+        for i in range(8):
+            runner.release(i)
+        runner.cache.check()
+        for i, p in enumerate(prompts):
+            want = plain_logits(folder, tuple(p), dtype)
+            at = sorted(pos for (r, pos) in got if r == i)
+            assert_close(torch.stack([got[(i, pos)] for pos in at]), want[at], dtype, f"1B {dtype} request {i} graphs {graphs}")
+    assert {(T, S) for T, S, _ in carried} == {(8, 2), (3, 2), (1, 2)} and all(ok for _, _, ok in carried)

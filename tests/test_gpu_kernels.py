@@ -758,8 +758,15 @@ def test_skinny_product_with_norm_prologue_and_residual_epilogue(K, dtype, M, N,
     stream = torch.randn(M + 2, N, generator=g)
     buf = dev(stream.clone())
     assert K.residual_epilogue_ok(M, Kd, DT[dtype], W) and not K.residual_epilogue_ok(M, Kd, DT[dtype], dev(w))
-    assert K.linear(dev(x), W, residual=buf[:M]) is None
-    assert rel(buf[:M], stream[:M].double() + x.double() @ w.double().t()) < 3e-6
+    shares = K.skinny_ksplit(M, Kd, DT[dtype], W)[0]
+    assert (shares > 1) == (Kd >= 4096), "long rows on a matrix of few tiles go in shares, for the next norm or prologue to add"
+    addends = K.linear(dev(x), W, residual=buf[:M])
+    if shares > 1:
+        assert addends.shape == (shares, M, N) and addends.dtype == torch.float32 and torch.equal(buf.cpu(), stream)
+        assert rel(addends.double().sum(0), x.double() @ w.double().t()) < 3e-6
+    else:
+        assert addends is None
+        assert rel(buf[:M], stream[:M].double() + x.double() @ w.double().t()) < 3e-6
     assert torch.equal(buf[M:].cpu(), stream[M:])
     with pytest.raises(K.KernelError):
         K.skinny_gemm(normed, dev(w), torch.empty(M, N, device="cuda", dtype=DT[dtype]))       # needs the re-tiled matrix
@@ -808,13 +815,15 @@ def test_skinny_product_of_17_to_64_rows_adds_into_the_residual_stream(K, dtype,
     assert rel(K.linear(dev(x), W), x.double() @ w.double().t()) < KTOL[dtype]
 
 
-@pytest.mark.parametrize("M,N,Kd,shares", [(9, 2048, 8192, 2), (16, 96, 4096, 4), (12, 272, 4112, 4), (8, 2048, 8192, 1),
-                                           (8, 3072, 8192, 1), (1, 4096, 14336, 1), (12, 3072, 8192, 1), (16, 2048, 2048, 1)])
-def test_long_products_of_up_to_16_rows_are_cut_where_a_norm_kernel_follows(K, M, N, Kd, shares):
+@pytest.mark.parametrize("M,N,Kd,shares", [(9, 2048, 8192, 2), (16, 96, 4096, 4), (12, 272, 4112, 4), (8, 2048, 8192, 2),
+                                           (1, 2048, 8192, 2), (8, 96, 4096, 2), (8, 3072, 8192, 1), (1, 4096, 14336, 1),
+                                           (12, 3072, 8192, 1), (16, 2048, 2048, 1), (8, 2048, 2048, 1)])
+def test_long_products_of_up_to_16_rows_are_cut_where_the_chip_has_room(K, M, N, Kd, shares):
     """Up to 16 bfloat16 rows of 4,096 elements or more onto the residual stream go in shares of K
-    where the norm that follows is a kernel of its own (past eight rows; up to eight the next product
-    normalises in its prologue, which is worth more) and the shares still make no more workgroups
-    than the chip has compute units (not the 192 tiles of the 3B shape in two shares)."""
+    where the shares still make no more workgroups than the chip has compute units (not the 192
+    tiles of the 3B shape in two shares): as many as fit past eight rows, where the norm that
+    follows is a kernel of its own; two up to eight rows, which the next product's normalising
+    prologue adds to its rows itself."""
     g = torch.Generator().manual_seed(M + N + Kd)
     w = (torch.randn(N, Kd, generator=g) / math.sqrt(Kd)).to(torch.bfloat16)
     W = K.Weight(dev(w))
@@ -864,6 +873,91 @@ def test_skinny_product_merges_the_key_runs_of_an_attention(K, M, H, hd, N, runs
     assert rel(got, want) < KTOL["bfloat16"], (M, H, hd, N, runs)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("M,N,Kd,S", [(1, 64, 2048, 2), (8, 96, 2048, 2), (4, 1000, 528, 1), (5, 64, 192, 2), (7, 3072, 2048, 2),
+                                      (2, 32, 48, 1), (8, 128, 1024, 2)])
+def test_pending_addends_of_the_residual_stream_ride_on_the_products(K, dtype, M, N, Kd, S):
+    """The shares of a cut product, which h has not received yet: the normalising prologue normalises
+    (h + p0) + p1 and leaves h alone, the residual epilogue stores ((h + p0) + p1) + product.  Both
+    give the very numbers of the same kernels run on a stream that a plain sum has updated before."""
+    g = torch.Generator().manual_seed(M * 31 + N + Kd + S)
+    h = torch.randn(M, Kd, generator=g) * 3
+    pend = torch.randn(S, M, Kd, generator=g) * 2
+    summed = h.clone()
+    for a in range(S):
+        summed += pend[a]
+    nw = 1 + 0.1 * torch.randn(Kd, generator=g)
+    eps = 3e-6
+    w = (torch.randn(N, Kd, generator=g) / math.sqrt(Kd)).to(DT[dtype])
+    W = K.Weight(dev(w))
+    assert K.prologue_addends() == 2
+    assert K.norm_prologue_ok(M, Kd, DT[dtype], W, S) and not K.norm_prologue_ok(M, Kd, DT[dtype], W, 3)
+    h_dev = dev(h)
+    with_addends = K.NormedInput(h_dev, dev(nw), eps, DT[dtype], dev(pend))
+    plain = K.NormedInput(dev(summed), dev(nw), eps, DT[dtype])
+    out = lambda n: torch.empty(M, n, device="cuda", dtype=DT[dtype])
+    got, want = K.skinny_gemm(with_addends, W, out(N)), K.skinny_gemm(plain, W, out(N))
+    assert torch.equal(got, want), "normed with addends, store"
+    assert rel(got, P.rmsnorm(summed.double(), nw, eps).to(DT[dtype]).double() @ w.double().t()) < KTOL[dtype]
+    assert torch.equal(K.linear(with_addends, W), want)
+    if N % 32 == 0:
+        assert K.norm_prologue_ok(M, Kd, DT[dtype], W, S, swiglu=True)
+        assert torch.equal(K.linear_swiglu(with_addends, W), K.linear_swiglu(plain, W)), "normed with addends, swiglu"
+    assert torch.equal(h_dev.cpu(), h), "the prologue leaves h as it is"
+    # the residual epilogue: the stream's own addends [S, M, N] first, then the product
+    x = torch.randn(M, Kd, generator=g).to(DT[dtype])
+    stream = torch.randn(M + 1, N, generator=g)
+    owed = torch.randn(S, M, N, generator=g)
+    assert K.residual_takes_addends(M, Kd, DT[dtype], W)
+    got = dev(stream.clone())
+    assert K.linear(dev(x), W, residual=got[:M], pending=dev(owed)) is None
+    want = stream.clone()
+    for a in range(S):
+        want[:M] += owed[a]
+    want = dev(want)
+    K.linear(dev(x), W, residual=want[:M])
+    assert torch.equal(got, want), "residual with addends"
+    with pytest.raises(K.KernelError):
+        K.linear(dev(x), W, pending=dev(owed))                                    # nothing to add them into
+    with pytest.raises(K.KernelError):
+        K.linear(dev(x), W, residual=got[:M], pending=dev(owed[:, :, :N - 16]))   # of another width
+    with pytest.raises(K.KernelError):
+        K.skinny_gemm(K.NormedInput(h_dev, dev(nw), eps, DT[dtype], dev(torch.zeros(3, M, Kd))), W, out(N))   # more than it holds
+
+
+def test_pending_addends_with_rotation_and_with_merged_key_runs(K):
+    """The same for the product that rotates and writes the cache (normalising prologue) and for the output
+    product that merges an attention's key runs (residual epilogue)."""
+    g = torch.Generator().manual_seed(5)
+    for dtype, M, H, KVH, hd, Kd in (("bfloat16", 8, 32, 8, 64, 2048), ("float32", 3, 4, 2, 32, 192), ("bfloat16", 1, 6, 1, 32, 528)):
+        h = torch.randn(M, Kd, generator=g) * 2
+        pend = torch.randn(2, M, Kd, generator=g)
+        summed = (h + pend[0]) + pend[1]
+        nw = 1 + 0.1 * torch.randn(Kd, generator=g)
+        W = K.Weight(dev((torch.randn((H + 2 * KVH) * hd, Kd, generator=g) / math.sqrt(Kd)).to(DT[dtype])))
+        positions = dev(torch.randint(0, 500, (M,), generator=g).to(torch.int32))
+        slots = dev(torch.tensor(random.Random(2).sample(range(32), M), dtype=torch.int32))
+        cos, sin = K.rope_table(dev(torch.from_numpy(P.rope_frequencies(hd, 10000.0, None))), 512)
+        results = []
+        for x in (K.NormedInput(dev(h), dev(nw), 1e-5, DT[dtype], dev(pend)), K.NormedInput(dev(summed), dev(nw), 1e-5, DT[dtype])):
+            kp = torch.zeros(2, KVH, 16, hd, dtype=DT[dtype], device="cuda")
+            vp = torch.zeros_like(kp)
+            results.append((K.skinny_qkv_rope(x, W, positions, cos, sin, slots, kp, vp, H, KVH, hd), kp, vp))
+        for a, b in zip(*results):
+            assert torch.equal(a, b), dtype
+    M, H, hd, N, runs = 2, 32, 64, 2048, 8
+    part_o = torch.randn(M, H, runs, hd, generator=g)
+    ml = torch.stack([torch.randn(M, H, runs, generator=g), torch.rand(M, H, runs, generator=g) + 1], -1)
+    ws = dev(torch.cat([part_o.reshape(-1), ml.reshape(-1)]))
+    wt = K.Weight(dev(torch.randn(N, H * hd, generator=g) / 45, torch.bfloat16))
+    stream, owed = torch.randn(M, N, generator=g), torch.randn(2, M, N, generator=g)
+    got = dev(stream.clone())
+    K.skinny_gemm_merged(ws, runs, M, H, hd, wt, got, residual=True, pending=dev(owed))
+    want = dev((stream + owed[0]) + owed[1])
+    K.skinny_gemm_merged(ws, runs, M, H, hd, wt, want, residual=True)
+    assert torch.equal(got, want)
+
+
 def test_what_the_merging_prologue_refuses(K):
     wt = K.Weight(dev(torch.zeros(64, 2048), torch.bfloat16))
     assert K.skinny_merge_ok(8, 32, 64, 4, torch.bfloat16, wt)
@@ -892,11 +986,17 @@ def test_where_the_skinny_product_gives_way_to_the_library(K):
     assert not K.skinny_wins(65, 2048, torch.bfloat16, W) and not K.skinny_wins(8, 2040, torch.bfloat16, W)
     # with the next norm to add them, 40 rows of 8,192 go in eight shares of K instead
     assert K.residual_epilogue_ok(40, 8192, torch.bfloat16, W) and K.skinny_ksplit(40, 8192, torch.bfloat16, W) == (8, 2)
-    assert K.skinny_ksplit(65, 8192, torch.bfloat16, W) == (1, 1) == K.skinny_ksplit(8, 8192, torch.bfloat16, W)
+    assert K.skinny_ksplit(65, 8192, torch.bfloat16, W) == (1, 1)
+    # up to eight rows the next product normalises in its prologue, which adds two shares to its rows: two then
+    assert K.skinny_ksplit(8, 8192, torch.bfloat16, W) == (2, 1) and K.skinny_ksplit(9, 8192, torch.bfloat16, W) == (8, 1)
+    assert K.skinny_ksplit(8, 2048, torch.bfloat16, K.Weight(dev(torch.zeros(32, 2048), torch.bfloat16))) == (1, 1)
+    full = K.Weight(dev(torch.zeros(4096, 8192), torch.bfloat16))      # 256 tiles fill the chip uncut
+    assert K.skinny_ksplit(8, 8192, torch.bfloat16, full) == (1, 1) and K.residual_takes_addends(8, 8192, torch.bfloat16, full)
+    assert not K.residual_takes_addends(8, 8192, torch.bfloat16, W)     # goes in shares itself
     Wf = K.Weight(dev(torch.zeros(32, 8192)))
     assert K.residual_epilogue_ok(40, 8192, torch.float32, Wf) and K.skinny_ksplit(40, 8192, torch.float32, Wf) == (8, 2)
-    assert K.skinny_ksplit(8, 8192, torch.float32, Wf) == (8, 1)      # float32 rows this long are cut at any batch
-    assert K.skinny_ksplit(8, 4096, torch.float32, K.Weight(dev(torch.zeros(32, 4096)))) == (1, 1)
+    assert K.skinny_ksplit(8, 8192, torch.float32, Wf) == (2, 1)
+    assert K.skinny_ksplit(8, 4096, torch.float32, K.Weight(dev(torch.zeros(32, 4096)))) == (2, 1)
     # float32 past 16 rows: only rows of up to 2,048 elements are streamed by the skinny product, the stacked gate/up
     # matrix only up to 32 rows; only matrices of at most 128 tiles are cut
     narrow, stacked = K.Weight(dev(torch.zeros(48, 2048))), K.Weight(dev(torch.zeros(8192, 2048)))
