@@ -1,7 +1,8 @@
-// Attention of prompt portions over the paged key/value cache on the matrix cores of gfx950, in
-// true float32: both products by v_mfma_f32_16x16x4_f32, softmax with the accurate exponential.
-// Compiled once per head size (-DHEAD_DIM=n, a multiple of 16 up to 256).  The float32 twin of the
-// bfloat16 kernel of attention_mfma.hip, with the same tiles and the same interface.
+// Attention over the paged key/value cache on the matrix cores of gfx950, in true float32: both
+// products by v_mfma_f32_16x16x4_f32, softmax with the accurate exponential.  Compiled once per
+// head size (-DHEAD_DIM=n, a multiple of 16 up to 256).  The float32 twins of the bfloat16 kernels
+// of attention_mfma.hip, with the same tiles and the same interfaces: first the kernel for prompt
+// portions, described here; at the end of the file the one for single tokens.
 //
 // A workgroup of four wavefronts owns one tile of consecutive tokens of one sequence and the query
 // heads of one kv head (up to 16 at a time).  A "row" is one (token, head) pair; a wavefront owns
@@ -335,5 +336,222 @@ NI_EXPORT int ni_mfma_attention_f32(const void* q, int q_stride, const void* kpo
                                                  (const int32_t*)block_table, table_stride, (const QTile*)tiles, n_tiles,
                                                  (float*)out, (float*)part_o, (float*)part_ml, H, KVH, page_size, page_shift,
                                                  hpt_shift, window, scale, nsplit);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Single tokens (decode steps, short prompt portions) in true float32: one workgroup per (token,
+// kv head, sixteen query heads of its group, run of the key range).  The rows of the products are
+// the query heads that share the kv head; the wavefronts of the workgroup take the 16-key steps
+// of the run in turn, each with a running (reference, sum, output) of its own, and meet in LDS at
+// the end.  Both operands that come from the cache are loaded from global memory straight in the
+// layout the matrix instructions want, so nothing is staged and no barrier stands in the loop:
+//   K as the A operand of S^T = K . Q^T: lane (r, kg) holds dims kg*HD/4 .. +HD/4 of key r, 64
+//     bytes in a row at head size 64 (four lanes read one row between them);
+//   V^T as the A operand of O^T += V^T . P^T: for the keys {4*kg + i} of MFMA i, lane (r, kg)
+//     holds dims r*HD/16 .. +HD/16 of key 4*kg + i (sixteen lanes read one row between them).
+// The rows of a step wait in registers, DEC_DEPTH steps ahead of the arithmetic.
+#define DEC_WAVES 4
+#define DEC_KEYS 16
+#define DEC_DEPTH (HEAD_DIM <= 64 ? 4 : HEAD_DIM <= 128 ? 3 : 2)
+
+template <bool POW2>
+__global__ __launch_bounds__(DEC_WAVES * WAVE) void mfma_decode_f32_kernel(
+    const float* __restrict__ q, int q_stride, const float* __restrict__ kpool, const float* __restrict__ vpool,
+    const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ seq_of_token,
+    const int32_t* __restrict__ positions, float* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int H, int KVH, int page_size, int page_shift, int window, float scale, int nsplit) {
+    constexpr int HD = HEAD_DIM;
+    constexpr int NW = DEC_WAVES;
+    constexpr int THREADS = NW * WAVE;
+    constexpr int KS = DEC_KEYS;
+    constexpr int QK = HD / 4;                     // MFMAs of the first product per step; floats of Q and of a key a lane holds
+    constexpr int DB = HD / 16;                    // MFMAs of the second product per 4 keys
+    constexpr int DEPTH = DEC_DEPTH;
+    __shared__ __attribute__((aligned(16))) float so[NW][16][HD];      // the wavefronts' outputs, met at the end
+    __shared__ float sm_ml[NW][16][2];
+    constexpr int TBL_MAX = 1024;
+    __shared__ int32_t tbl[TBL_MAX];
+
+    // (uncut key ranges of many tokens: a compute unit holds workgroups u and u + half the grid, the same x in the
+    // lower and the upper half of y; the upper half takes the tokens from the far end, so that tokens that come in
+    // the order of their contexts put a long and a short one on every unit)
+    const int t = (gridDim.z == 1 && gridDim.y > 1 && 2 * blockIdx.y >= gridDim.y) ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
+    const int G = H / KVH;
+    const int chunks = (G + 15) / 16;
+    const int g = blockIdx.y / chunks;
+    const int chunk = blockIdx.y % chunks;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
+    const int r = lane % 16, kg = lane / 16;
+    const int hh = chunk * 16 + r;                 // this lane's row: a query head of the group
+    const bool row_ok = hh < G;
+    const int head = g * G + hh;
+
+    const int pos = positions[t];
+    const int seq = seq_of_token[t];
+    const int hi = pos + 1;
+    const int lo = window > 0 ? max(0, hi - window) : 0;
+    const int kbeg = lo / KS * KS;
+    const int nsteps_all = (hi - kbeg + KS - 1) / KS;
+    const int per_split = (nsteps_all + nsplit - 1) / nsplit;
+    const int s_begin = blockIdx.z * per_split;
+    const int nsteps = max(0, min(nsteps_all, s_begin + per_split) - s_begin);
+    const int kfirst = kbeg + s_begin * KS;
+
+    const int32_t* table = block_table + static_cast<size_t>(seq) * table_stride;
+    auto page_of = [&](int key) { return POW2 ? (key >> page_shift) : key / page_size; };
+    auto slot_of = [&](int key) { return POW2 ? (key & (page_size - 1)) : key % page_size; };
+    int key_lo = 0, key_hi = 0, lp0 = 0;
+    auto row_address = [&](int key) -> size_t {
+        // clamped to keys the token may read: those before `lo` may lie in pages already given back
+        const int kc = min(max(key, max(key_lo, lo)), key_hi);
+        const int page = tbl[page_of(kc) - lp0];
+        return ((static_cast<size_t>(max(page, 0)) * KVH + g) * page_size + slot_of(kc)) * HD;
+    };
+
+    // Q, scaled, as the B operand: lane (row r, group kg) holds dims kg*HD/4 .. +HD/4
+    float qf[QK];
+    if (row_ok) {
+        VecIO<float, QK>::load(q + static_cast<size_t>(t) * q_stride + static_cast<size_t>(head) * HD + kg * QK, qf);
+#pragma unroll
+        for (int j = 0; j < QK; ++j) qf[j] *= scale;
+    } else {
+#pragma unroll
+        for (int j = 0; j < QK; ++j) qf[j] = 0.f;
+    }
+
+    float m_ref = NEG_BIG, l_lane = 0.f;       // the row's reference; the sum of this lane's own weights
+    floatx4_t o[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) o[db] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    struct StepRows { float k[QK]; float v[4][DB]; };
+    auto load_rows = [&](int ks, StepRows& rows) {
+        VecIO<float, QK>::load(kpool + row_address(ks + r) + kg * QK, rows.k);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) VecIO<float, DB>::load(vpool + row_address(ks + 4 * kg + i) + r * DB, rows.v[i]);
+    };
+
+    StepRows ring[DEPTH];
+    for (int seg0 = 0; seg0 < nsteps;) {
+        key_lo = kfirst + seg0 * KS;
+        lp0 = page_of(max(key_lo, lo));
+        const int seg_steps = min(nsteps - seg0, ((lp0 + TBL_MAX) * page_size - key_lo) / KS);
+        key_hi = min(key_lo + seg_steps * KS, hi) - 1;
+        __syncthreads();
+        for (int i = tid; i <= page_of(key_hi) - lp0; i += THREADS) tbl[i] = table[lp0 + i];
+        __syncthreads();
+        // this wavefront's steps of the segment: wave, wave + NW, ...
+        const int mine = seg_steps > wave ? (seg_steps - wave + NW - 1) / NW : 0;
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) load_rows(key_lo + (wave + d * NW) * KS, ring[d]);
+        // Step j lives in slot j % DEPTH of the ring; the loop is unrolled DEPTH times so that a slot is a
+        // fixed set of registers, asked for its next rows as soon as its step has used it.
+        auto step = [&](int j, StepRows& rows) {
+            const int ks = key_lo + (wave + j * NW) * KS;
+            if (j < mine) {
+                // 1. scores: this lane gets row r, keys ks + 4*kg + i
+                floatx4_t st = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j1 = 0; j1 < QK; ++j1) st = __builtin_amdgcn_mfma_f32_16x16x4f32(rows.k[j1], qf[j1], st, 0, 0, 0);
+                const bool inner = ks >= lo && ks + KS - 1 <= pos;
+                float sc[4];
+                float lane_max = NEG_BIG;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float v = st[i];
+                    if (!inner) {
+                        const int key = ks + 4 * kg + i;
+                        v = (key <= pos && key >= lo) ? v : NEG_BIG;
+                    }
+                    sc[i] = v;
+                    lane_max = fmaxf(lane_max, v);
+                }
+                // 2. a row whose scores have risen far above its reference: move it, rescale what was summed
+                if (__any(lane_max - REF_SLACK > m_ref)) {
+                    const float mx = lanes4(lane_max, true);
+                    const bool move = mx > 0.5f * NEG_BIG && mx > m_ref + REF_SLACK;
+                    const float m_new = move ? mx : m_ref;
+                    const float corr = move ? expf(m_ref - m_new) : 1.0f;
+                    m_ref = m_new;
+                    l_lane *= corr;
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) o[db] *= corr;
+                }
+                // 3. weights, and O^T += V^T . P^T for the keys {4*kg + i} of MFMA i
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float p = expf(sc[i] - m_ref);
+                    if (!inner) p = sc[i] > 0.5f * NEG_BIG ? p : 0.f;
+                    l_lane += p;
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(rows.v[i][db], p, o[db], 0, 0, 0);
+                }
+            }
+            load_rows(ks + DEPTH * NW * KS, rows);
+        };
+        for (int j0 = 0; j0 < mine; j0 += DEPTH) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) step(j0 + d, ring[d]);
+        }
+        seg0 += seg_steps;
+    }
+
+    // wavefronts meet: every one leaves (reference, sum) of its rows and its 16 x HD output in LDS; this lane
+    // holds dims (4*kg + i)*DB + db of its row in o[db][i]
+    const float l = lanes4(l_lane, false);
+    if (kg == 0) { sm_ml[wave][r][0] = m_ref; sm_ml[wave][r][1] = l; }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) so[wave][r][(4 * kg + i) * DB + db] = o[db][i];
+    __syncthreads();
+    const int rows_here = min(16, G - chunk * 16);
+    for (int idx = tid; idx < rows_here * HD; idx += THREADS) {
+        const int row = idx / HD, dim = idx % HD;
+        float M = sm_ml[0][row][0];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) M = fmaxf(M, sm_ml[w][row][0]);
+        float Lsum = 0.f, O = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const float f = expf(sm_ml[w][row][0] - M);
+            Lsum += sm_ml[w][row][1] * f;
+            O += so[w][row][dim] * f;
+        }
+        const int h = g * G + chunk * 16 + row;
+        if (nsplit == 1) {
+            out[static_cast<size_t>(t) * H * HD + static_cast<size_t>(h) * HD + dim] = O / Lsum;
+        } else {
+            const size_t p = (static_cast<size_t>(t) * H + h) * nsplit + blockIdx.z;
+            part_o[p * HD + dim] = O;
+            if (dim == 0) { part_ml[p * 2] = M; part_ml[p * 2 + 1] = Lsum; }
+        }
+    }
+}
+
+// Attention of single tokens on the matrix cores in float32: same arguments and partial-result layout as the
+// token-at-a-time kernel (`out` is left to its merge kernel when nsplit > 1).
+NI_EXPORT int ni_mfma_token_attention_f32(const void* q, int q_stride, const void* kpool, const void* vpool,
+                                          const void* block_table, int table_stride, const void* seq_of_token,
+                                          const void* positions, void* out, void* part_o, void* part_ml, int T_tokens,
+                                          int H, int KVH, int page_size, int window, float scale, int nsplit,
+                                          hipStream_t stream) {
+    if (T_tokens <= 0) return 0;
+    if (H < 1 || KVH < 1 || H % KVH != 0 || page_size < 1 || nsplit < 1 || nsplit > 65535 || !(scale > 0.f)) return -1;
+    if (nsplit > 1 && (!part_o || !part_ml)) return -2;
+    if (q_stride % 4 != 0) return -3;
+    const int G = H / KVH;
+    const int chunks = (G + 15) / 16;
+    const bool pow2 = (page_size & (page_size - 1)) == 0;
+    int page_shift = 0;
+    while (pow2 && (1 << page_shift) < page_size) ++page_shift;
+    dim3 grid(T_tokens, KVH * chunks, nsplit);
+    auto kernel = pow2 ? mfma_decode_f32_kernel<true> : mfma_decode_f32_kernel<false>;
+    kernel<<<grid, DEC_WAVES * WAVE, 0, stream>>>(
+        (const float*)q, q_stride, (const float*)kpool, (const float*)vpool, (const int32_t*)block_table, table_stride,
+        (const int32_t*)seq_of_token, (const int32_t*)positions, (float*)out, (float*)part_o, (float*)part_ml, H, KVH,
+        page_size, page_shift, window, scale, nsplit);
     return NI_LAUNCH_RESULT();
 }

@@ -290,22 +290,25 @@ def mfma_token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Te
                          seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, H: int, KVH: int,
                          hd: int, scale: float, window: Optional[int], nsplit: int,
                          workspace: Optional[torch.Tensor] = None, merge: bool = True) -> torch.Tensor:
-    """:func:`token_attention` on the matrix cores (bfloat16, head sizes that :func:`mfma_token_ok`
+    """:func:`token_attention` on the matrix cores (types and head sizes that :func:`mfma_token_ok`
     takes): the query heads of a kv head are the rows of the products, the wavefronts of a
     workgroup share out the keys.  With ``nsplit > 1`` and ``merge=False`` the partial results of
     the key runs are left in ``workspace`` for :func:`skinny_gemm_merged` and ``out`` is not written."""
     if not (mfma_token_ok(qkv.dtype, hd)):
         raise KernelError(f"mfma_token_attention does not take {qkv.dtype} with head size {hd}")
-    if not (qkv.shape[1] % 8 == 0):
+    if not (qkv.shape[1] % (16 // qkv.element_size()) == 0):
         raise KernelError("rows of qkv are not aligned to 16 bytes")
     T, part_o, part_ml = _token_attention_checks(qkv, kpool, vpool, block_table, seq_of_token, positions, out,
                                                  H, KVH, hd, nsplit, workspace)
-    if not (kpool.numel() // hd < 2 ** 32):
-        raise KernelError("the matrix-core attention kernels number the rows of a pool in 32 bits")
-    _check(attention_mfma_lib(hd).ni_mfma_token_attention(
-        _ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table), block_table.shape[1],
-        _ptr(seq_of_token), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), T, H, KVH, kpool.shape[2],
-        int(window) if window else 0, ctypes.c_float(scale), nsplit, _stream()), "mfma_token_attention")
+    if qkv.dtype == torch.float32:
+        launch = attention_mfma_f32_lib(hd).ni_mfma_token_attention_f32
+    else:
+        if not (kpool.numel() // hd < 2 ** 32):
+            raise KernelError("the matrix-core attention kernels number the rows of a pool in 32 bits")
+        launch = attention_mfma_lib(hd).ni_mfma_token_attention
+    _check(launch(_ptr(qkv), qkv.shape[1], _ptr(kpool), _ptr(vpool), _ptr(block_table), block_table.shape[1],
+                  _ptr(seq_of_token), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), T, H, KVH, kpool.shape[2],
+                  int(window) if window else 0, ctypes.c_float(scale), nsplit, _stream()), "mfma_token_attention")
     if nsplit > 1 and merge:
         _check(attention_lib(hd).ni_merge_splits(_ptr(part_o), _ptr(part_ml), _ptr(out), T, H, nsplit,
                                                  dtype_code(out.dtype), _stream()), "merge_splits")
@@ -321,8 +324,11 @@ def mfma_attention_ok(dtype: torch.dtype, hd: int) -> bool:
 
 
 def mfma_token_ok(dtype: torch.dtype, hd: int) -> bool:
-    """Whether the matrix-core kernel for single tokens takes this type and head size (bfloat16 only)."""
-    return dtype == torch.bfloat16 and hd % 32 == 0 and 32 <= hd <= 256
+    """Whether a matrix-core kernel for single tokens takes this type and head size: bfloat16 with
+    head sizes in steps of 32, float32 in steps of 16."""
+    if dtype == torch.bfloat16:
+        return hd % 32 == 0 and 32 <= hd <= 256
+    return dtype == torch.float32 and hd % 16 == 0 and 16 <= hd <= 256
 
 
 COMPUTE_UNITS = 256      # of an MI355X

@@ -386,21 +386,38 @@ def test_mfma_tile_size_and_splits_follow_the_step(K):
 def test_mfma_token_attention_head_sizes_and_groups(K, H, KVH, hd, ps):
     # the kernel for single tokens: rows are the query heads of a kv head (20 of them: two chunks of 16)
     lens, q_lens = [1, 37, 130, 64, 300, 33], [1, 37, 2, 1, 3, 1]
-    for nsplit in (1, 3):
-        out, want, _ = paged_case(K, "bfloat16", H, KVH, hd, ps, lens, q_lens, None, hd + H, nsplit, kernel="mfma_token")
+    for dtype in ("bfloat16", "float32"):
+        for nsplit in (1, 3):
+            out, want, _ = paged_case(K, dtype, H, KVH, hd, ps, lens, q_lens, None, hd + H, nsplit, kernel="mfma_token")
+            assert not torch.isnan(out).any(), "a key outside the sequence's own pages took part"
+            assert rel(out, want) < KTOL[dtype], (dtype, H, KVH, hd, ps, nsplit)
+
+
+@pytest.mark.parametrize("H,KVH,hd,ps", [(4, 2, 16, 16), (5, 5, 48, 5), (3, 3, 80, 16), (2, 1, 112, 16), (24, 8, 128, 16), (34, 2, 64, 8)])
+def test_mfma_token_attention_in_float32_at_its_own_head_sizes(K, H, KVH, hd, ps):
+    # head sizes in steps of 16, which the bfloat16 kernel does not take; 17 heads a group: two chunks of 16
+    lens, q_lens = [1, 37, 130, 64, 300, 33, 17], [1, 37, 2, 1, 3, 1, 1]
+    assert K.mfma_token_ok(torch.float32, hd) and K.mfma_token_ok(torch.bfloat16, hd) == (hd % 32 == 0)
+    for nsplit in (1, 2, 5):
+        out, want, _ = paged_case(K, "float32", H, KVH, hd, ps, lens, q_lens, None, hd + H, nsplit, kernel="mfma_token")
         assert not torch.isnan(out).any(), "a key outside the sequence's own pages took part"
-        assert rel(out, want) < KTOL["bfloat16"], (H, KVH, hd, ps, nsplit)
+        assert rel(out, want) < KTOL["float32"], (H, KVH, hd, ps, nsplit)
 
 
-def test_mfma_token_attention_window_and_far_key(K):
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_mfma_token_attention_window_and_far_key(K, dtype):
     for window in (1, 7, 16, 33, 100):
-        out, want, _ = paged_case(K, "bfloat16", 4, 2, 32, 8, [150, 9, 33], [150, 9, 2], window, window, 1, kernel="mfma_token")
+        out, want, _ = paged_case(K, dtype, 4, 2, 32, 8, [150, 9, 33], [150, 9, 2], window, window, 1, kernel="mfma_token")
         assert not torch.isnan(out).any()
-        assert rel(out, want) < KTOL["bfloat16"], window
+        assert rel(out, want) < KTOL[dtype], window
+    for window, nsplit in ((300, 3), (129, 2), (600, 4)):      # windows cut into runs: the first run starts inside a step
+        out, want, _ = paged_case(K, dtype, 8, 2, 64, 16, [901, 333], [2, 1], window, window, nsplit, kernel="mfma_token")
+        assert not torch.isnan(out).any()
+        assert rel(out, want) < KTOL[dtype], window
     for key_at in (37, 16, 15, 0, 31, 32, 127, 128, 698):
-        out, want, (qs, ks, vs) = paged_case(K, "bfloat16", 8, 2, 64, 16, [700], [1], None, 9, 1 + key_at % 4,
+        out, want, (qs, ks, vs) = paged_case(K, dtype, 8, 2, 64, 16, [700], [1], None, 9, 1 + key_at % 4,
                                              boost=(0, key_at, 699, 6.0), kernel="mfma_token")
-        assert rel(out, want) < KTOL["bfloat16"]
+        assert rel(out, want) < KTOL[dtype]
         got = out.double().cpu()[-1].reshape(8, 64)
         expect = vs[0][key_at].double().repeat_interleave(4, 0)
         assert float((got - expect).abs().max()) < 0.05, key_at
@@ -431,7 +448,7 @@ def test_mfma_attention_window_and_far_key(K, blocks):
         assert rel(out, want) < KTOL["bfloat16"], window
     with pytest.raises(Exception):
         K.attention_mfma_lib(48)
-    assert not K.mfma_token_ok(torch.float32, 64) and not K.mfma_attention_ok(torch.bfloat16, 48)
+    assert K.mfma_token_ok(torch.float32, 48) and not K.mfma_token_ok(torch.bfloat16, 48) and not K.mfma_attention_ok(torch.bfloat16, 48)
     assert K.mfma_attention_ok(torch.float32, 48) and not K.mfma_attention_ok(torch.float32, 40)
 
 
