@@ -350,10 +350,12 @@ NI_EXPORT int ni_mfma_attention_f32(const void* q, int q_stride, const void* kpo
 //     bytes in a row at head size 64 (four lanes read one row between them);
 //   V^T as the A operand of O^T += V^T . P^T: for the keys {4*kg + i} of MFMA i, lane (r, kg)
 //     holds dims r*HD/16 .. +HD/16 of key 4*kg + i (sixteen lanes read one row between them).
-// The rows of a step wait in registers, DEC_DEPTH steps ahead of the arithmetic.
+// The rows of a step wait in registers, DEC_DEPTH steps ahead of the arithmetic: two, which leaves the registers
+// for two workgroups a compute unit up to head size 128 (with three or four steps ahead a decode batch of mixed
+// context lengths ran slower: one workgroup a unit cannot pair a long token with a short one).
 #define DEC_WAVES 4
 #define DEC_KEYS 16
-#define DEC_DEPTH (HEAD_DIM <= 64 ? 4 : HEAD_DIM <= 128 ? 3 : 2)
+#define DEC_DEPTH 2
 
 template <bool POW2>
 __global__ __launch_bounds__(DEC_WAVES * WAVE) void mfma_decode_f32_kernel(
