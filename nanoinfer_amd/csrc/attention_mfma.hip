@@ -629,7 +629,8 @@ __global__ __launch_bounds__(DEC_WAVES * WAVE) void mfma_decode_kernel(
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     };
 
-    constexpr int DEPTH = HD <= 64 ? 4 : HD <= 128 ? 3 : 2;
+    constexpr int DEPTH = 2;      // steps whose rows wait in registers ahead of the arithmetic: more (four at head size 64, three at 128) left
+                                  // fewer workgroups on a compute unit and were slower at every batch, most of all where the context lengths differ
     uint4 kf[DEPTH][2][KK];
     u32x4_t vr[DEPTH][V_PER_LANE];
     for (int seg0 = 0; seg0 < nsteps;) {
