@@ -810,6 +810,11 @@ def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bo
         raise KernelError("pending addends go with the residual epilogue of at most 16 rows")
     pend, n_pend = _check_addends(pending, M, N)
     per_group = _tiles_per_group(N // 2 if swiglu else N)
+    if tiles is None and per_group == 4 and M <= 12:
+        # the widest matrices as stored (the head over the vocabulary): few rows stream fastest with fewer tiles a
+        # workgroup (measured at [128256, 2048], us for 1 / 2 / 4 tiles: one row 83.9 / 87.4 / 90.3, four rows
+        # 86.0 / 87.3 / 94.3, eight rows 97.9 / 90.5 / 94.1, twelve 109.9 / 98.8 / 100.0, sixteen 118.6 / 103.2 / 100.5)
+        per_group = 1 if M <= 4 else 2
     if swiglu and M > 32 and tiles is not None:
         # past 32 rows a workgroup that multiplies two pairs of gate and up tiles halves the loads of x,
         # which every workgroup brings in whole (measured at [16384, 2048]: 64 rows 22.0 -> 20.9 us, 17 and 32 rows lose)
