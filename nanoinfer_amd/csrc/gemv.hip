@@ -883,8 +883,8 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
             launch(wv_tag, sr_tag, One{});
         };
         if constexpr (XP == 0 && NTc == 1) {
-            // rows of 4,096 elements or more in few workgroups: sixteen wavefronts each
-            if (grid <= HALVE_BELOW && K >= 4096) {
+            // rows of 2,048 elements or more in few workgroups: sixteen wavefronts each
+            if (grid <= HALVE_BELOW && K >= 2048) {
                 with_halves(std::integral_constant<int, 16>{}, std::integral_constant<int, 0>{});
                 return;
             }
