@@ -125,6 +125,57 @@ struct RopeArgs {
     int H, KVH, hd, page_size;
 };
 
+// What an epilogue reads from memory, asked for while W is still streaming instead of at the end, where every
+// load is a round trip that nothing hides (the rotation's are two in a row: the position, then its angle).
+// For the first item of a thread (item == threadIdx.x), which with at most 16 rows and few tiles is its only one.
+struct EpiEarly {
+    bool have = false;       // the values below are those of item threadIdx.x
+    int pos = 0, slot = -1;  // rotation: the row's position and cache slot
+    float a = 0.f, b = 0.f;  // rotation: cos and sin; residual: the stream's value and its first addend
+    float c = 0.f;           // residual: the second addend
+};
+
+// The first half for the rotation epilogue (position and slot of the thread's row), the whole for the residual one.
+template <int EPI, int NT, int HALVES>
+__device__ __forceinline__ void epi_early_first(EpiEarly& e, const void* y, int M, int N, const RopeArgs& rope,
+                                                const float* pend, int n_pend) {
+    const int item = threadIdx.x;
+    const int wg = blockIdx.x / HALVES, wg_half = blockIdx.x % HALVES;
+    if constexpr (EPI == EPI_ROPE) {
+        const int n_local = item % 16, m = item / 16;
+        if (item >= 16 * 16 || m >= M || (HALVES == 2 && (n_local >> 3) != wg_half)) return;
+        e.have = true;
+        e.pos = rope.positions[m];
+        if (rope.slot_mapping) e.slot = rope.slot_mapping[m];
+    } else if constexpr (EPI == EPI_RESIDUAL) {
+        const int n_in = item % (NT * 16), m = item / (NT * 16);
+        const int n = wg * NT * 16 + n_in;
+        if (item >= 16 * NT * 16 || m >= M || n >= N || (HALVES == 2 && ((n_in % 16) >> 3) != wg_half)) return;
+        e.have = true;
+        const float* dst = static_cast<const float*>(y) + static_cast<size_t>(m) * N + n;
+        e.a = *dst;
+        if (n_pend > 0) {
+            const float* p = pend + static_cast<size_t>(m) * N + n;
+            e.b = p[0];
+            e.c = n_pend > 1 ? p[static_cast<size_t>(M) * N] : 0.f;
+        }
+    }
+}
+// The second half for the rotation epilogue, once the position has arrived: cos and sin of the thread's pair.
+template <int EPI, int HALVES>
+__device__ __forceinline__ void epi_early_second(EpiEarly& e, const RopeArgs& rope) {
+    if constexpr (EPI == EPI_ROPE) {
+        if (!e.have) return;
+        const int wg = blockIdx.x / HALVES;
+        const int per_head = rope.hd / 32;
+        if (wg / per_head >= rope.H + rope.KVH) return;       // values do not turn
+        const int j = (wg % per_head) * 16 + static_cast<int>(threadIdx.x) % 16;
+        const size_t at = static_cast<size_t>(e.pos) * (rope.hd / 2) + j;
+        e.a = rope.cos_t[at];
+        e.b = rope.sin_t[at];
+    }
+}
+
 // What follows the main loop of both kernels: the wavefronts' partial sums meet in LDS and the
 // epilogue stores them.
 // HALVES == 2: two workgroups share the tiles that one would own; the first stores the first eight
@@ -132,7 +183,7 @@ struct RopeArgs {
 template <typename T, typename TOUT, int MB, int NT, int EPI, int WV = GV_WAVES, bool EXT = false, int HALVES = 1>
 __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TOUT* __restrict__ y, int M, int N, int I,
                                               const RopeArgs& rope, float* ext = nullptr, const float* pend = nullptr,
-                                              int n_pend = 0) {
+                                              int n_pend = 0, const EpiEarly* early = nullptr) {
     const int tid = threadIdx.x;
     const int wave = tid / WAVE, lane = tid % WAVE;
     const int wg = blockIdx.x / HALVES;
@@ -174,10 +225,16 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
                 x1 += red[w][1 * MB + mb][src];
             }
             const int j = j0 + n_local;
+            const bool ready = early != nullptr && early->have && item == tid;      // asked for while W was streaming
             if (head < rope.H + rope.KVH) {             // queries and keys turn, values do not
-                const int pos = rope.positions[m];
-                const float c = rope.cos_t[static_cast<size_t>(pos) * half + j];
-                const float sn = rope.sin_t[static_cast<size_t>(pos) * half + j];
+                float c, sn;
+                if (ready) {
+                    c = early->a; sn = early->b;
+                } else {
+                    const int pos = rope.positions[m];
+                    c = rope.cos_t[static_cast<size_t>(pos) * half + j];
+                    sn = rope.sin_t[static_cast<size_t>(pos) * half + j];
+                }
                 const float y0 = x0 * c - x1 * sn;
                 const float y1 = x0 * sn + x1 * c;
                 x0 = y0; x1 = y1;
@@ -187,7 +244,7 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
                 st(dst + j, x0);
                 st(dst + j + half, x1);
             } else if (rope.slot_mapping) {
-                const int slot = rope.slot_mapping[m];
+                const int slot = ready ? early->slot : rope.slot_mapping[m];
                 if (slot >= 0) {
                     const bool is_k = head < rope.H + rope.KVH;
                     const int g = is_k ? head - rope.H : head - rope.H - rope.KVH;
@@ -228,11 +285,17 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
         }
         TOUT* dst = y + static_cast<size_t>(m) * out_width + n;
         if constexpr (EPI == EPI_RESIDUAL) {      // float32 residual stream, this workgroup's own columns
-            float sum = *dst;
+            const bool ready = early != nullptr && early->have && item == tid;      // asked for while W was streaming
+            float sum = ready ? early->a : *dst;
             if (n_pend > 0) {       // what the stream has not received yet, in its order, then the product
                 const float* p = pend + static_cast<size_t>(m) * N + n;
                 const size_t stride = static_cast<size_t>(M) * N;
-                const float p0 = p[0], p1 = n_pend > 1 ? p[stride] : 0.f;      // asked for together
+                float p0, p1;
+                if (ready) {
+                    p0 = early->b; p1 = early->c;
+                } else {
+                    p0 = p[0]; p1 = n_pend > 1 ? p[stride] : 0.f;      // asked for together
+                }
                 sum = (sum + p0) + p1;
                 for (int a = 2; a < n_pend; ++a) sum += p[a * stride];
             }
@@ -360,6 +423,9 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
     const int share = (pieces + splits - 1) / splits;
     const int p_begin = min(pieces, static_cast<int>(blockIdx.y) * share), p_end = min(pieces, p_begin + share);
     y += static_cast<size_t>(blockIdx.y) * M * N;
+    EpiEarly early;         // what the epilogue will read, asked for before W (not behind the merging prologue's many
+                            // loads, where it gained nothing: the o product of one row 6.6 -> 7.3 us)
+    if constexpr (PRO == PRO_NORM) epi_early_first<EPI, NT, HALVES>(early, y, M, N, rope, norm.pend, norm.n_pend);
 
     const T* wrow[NT];      // first byte of this lane in piece 0 of each tile
 #pragma unroll
@@ -647,6 +713,7 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
                 xn[p / PT][p % PT][0].from_floats(f);
             }
         }
+        epi_early_second<EPI, HALVES>(early, rope);      // behind the first trip of W; the position has arrived long ago
 #pragma unroll
         for (int t = 0; t < TRIPS; t += 2) {
             const int c = wave + t * STRIDE;
@@ -664,6 +731,7 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
         };
         Piece<T> xb_a[PT][1], xb_b[PT][1];
         load_x(p_begin + wave, xb_a);
+        epi_early_second<EPI, HALVES>(early, rope);      // behind the first trip of W and x (waits for the position only)
         for (int c = p_begin + wave; c < p_end; c += 2 * STRIDE) {
             if (c + STRIDE < p_end) { load_w(c + STRIDE, wa_b); load_x(c + STRIDE, xb_b); }
             multiply(c, wa_a, xb_a);
@@ -674,9 +742,9 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
     if constexpr (SHARE_LDS) {
         __syncthreads();                   // every wavefront has taken its operands from the staged rows
         skinny_finish<T, TOUT, 1, NT, EPI, WV, true, HALVES>(acc, y, M, N, I, rope, reinterpret_cast<float*>(staged_rows),
-                                                             norm.pend, norm.n_pend);
+                                                             norm.pend, norm.n_pend, &early);
     } else {
-        skinny_finish<T, TOUT, 1, NT, EPI, WV, false, HALVES>(acc, y, M, N, I, rope, nullptr, norm.pend, norm.n_pend);
+        skinny_finish<T, TOUT, 1, NT, EPI, WV, false, HALVES>(acc, y, M, N, I, rope, nullptr, norm.pend, norm.n_pend, &early);
     }
 }
 
