@@ -521,8 +521,11 @@ void mfma_attention_kernel(
 // workgroup barrier inside the loop.
 #define DEC_WAVES (HEAD_DIM <= 128 ? 4 : 2)
 
+// (Asked for four wavefronts a SIMD at head size 64, the compiler fits the kernel into 122 registers instead of 148
+// without spilling, and a compute unit holds four workgroups instead of three: 11.5 -> 10.8 us at batch 8.)
 template <bool POW2>
-__global__ __launch_bounds__(DEC_WAVES * WAVE) void mfma_decode_kernel(
+__global__ __launch_bounds__(DEC_WAVES * WAVE) __attribute__((amdgpu_waves_per_eu(HEAD_DIM <= 64 ? 4 : 2)))
+void mfma_decode_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ positions, bf16_t* __restrict__ out, float* __restrict__ part_o,
