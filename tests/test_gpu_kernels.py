@@ -736,7 +736,7 @@ def test_skinny_product(K, dtype, M, N, Kd):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("M,N,Kd", [(1, 32, 64), (5, 50, 192), (16, 1000, 528), (8, 4096, 2048), (3, 778, 1024), (16, 96, 48),
-                                    (2, 64, 4096), (6, 1000, 528), (7, 96, 48), (9, 64, 256)])
+                                    (2, 64, 4096), (6, 1000, 528), (7, 96, 48), (9, 64, 256), (5, 33008, 48)])
 def test_skinny_product_with_norm_prologue_and_residual_epilogue(K, dtype, M, N, Kd):
     """RMSNorm(h) as the input of a product (store and SwiGLU epilogues), and a product added into
     the residual stream, against the plain steps in float64.  Row widths that are no multiple of a
