@@ -10,11 +10,18 @@ is decoded tokens per second.  The same line carries the prefill of one 2,048-to
 portions of 512 (``prefill``; ``--prefill-chunk`` changes the cut), in one portion, the engine's
 default (``prefill_one_portion``, and ``prefill_one_portion_eager`` with every kernel launched from
 the host instead of a recorded step), the decode step's fraction of the HBM roofline, and in
-``points`` decode at batch 1 and 64.  The default line (1B shape, bfloat16) adds further points, each
-timed over 96 steps: decode at batch 8 from contexts of 8,192 and 32,768 tokens, the same model in
-true float32 (``decode_b8_fp32``, ``prefill_fp32``: the reference's own precision), and the 3B shape
-(``decode_b8_3b``), with the roofline fraction of each, and prompts of 8,192 and 32,768 tokens
-(``prefill_8k``, ``prefill_32k``, in portions of 2,048).  Peaks are MI355X's published ones: HBM
+``points`` decode at batch 1 and 64 (``rooflines`` holds the roofline fraction of every point by
+its name).  The default line (1B shape, bfloat16) adds further points, each timed over 96 steps:
+decode at batch 8 and 64 from contexts of 8,192 and 32,768 tokens; prompts of 8,192 and 32,768
+tokens (``prefill_8k``, ``prefill_32k``, in portions of 2,048); the same model in true float32
+(``decode_b8_fp32``, ``decode_b8_ctx8k_fp32``, ``prefill_fp32``: the reference's own precision); the
+3B shape in bfloat16 at batch 1, 8 and 64; requests through the scheduler (``serving_1b_bf16``,
+``serving_1b_bf16_128req_half_pool`` with half the pages its 128 requests need, and
+``serving_3b_fp32``: 64 concurrent requests of the 3B shape in float32, prompts uniform in
+[128, 2048], 256 new tokens each); and the 8B shape at its full 32 layers in float32
+(``prefill_8b_fp32`` of 2,048 tokens in portions of 512, ``decode_b1/b8/b64_8b_fp32``) and in
+bfloat16.  A further point that fails is named in ``errors`` and costs the line nothing else.
+Peaks are MI355X's published ones: HBM
 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s.  The reference publishes no numbers for
 this model, so ``vs_baseline`` is null.  ``--workload serving`` measures requests through the
 scheduler instead and prints a line of its own.
@@ -217,14 +224,17 @@ def percentile(values, q: float) -> float:
     return values[min(len(values) - 1, int(q * len(values)))]
 
 
-def serving(args) -> int:
-    """``--workload serving``: requests through the engine's own scheduler, as a user's program
-    drives it (``Engine.add_request`` / ``Engine.step``): 64 requests arrive at once, prompts of
-    uniform random length in [128, 2048] (seeded), 256 new tokens each, greedy, continuous
-    batching with prompt portions beside decode tokens.  The report follows the reference's demo
-    (demo/batched_infer_multi_prompts.cpp:356-362: prefill and decode tokens a second) and adds
-    the step times, the share of the HBM roofline of the decode steps, and the host's share of
-    the wall time (wall minus the spans between the GPU events around every step's launches)."""
+def serving_measure(args) -> dict:
+    """Requests through the engine's own scheduler, as a user's program drives it
+    (``Engine.add_request`` / ``Engine.step``): ``args.requests`` requests arrive at once, prompts of
+    uniform random length in [``min_prompt``, ``max_prompt``] (seeded), ``new_tokens`` new tokens each,
+    greedy, continuous batching with prompt portions beside decode tokens.  The report follows the
+    reference's demo (demo/batched_infer_multi_prompts.cpp:356-362: prefill and decode tokens a
+    second) and adds the step times, the share of the HBM roofline of the decode steps, and the
+    host's share of the wall time (wall minus the spans between the GPU events around every
+    step's launches).  Returns the result line as a dict."""
+    import gc
+
     import torch
 
     import nanoinfer_amd  # noqa: F401
@@ -293,7 +303,9 @@ def serving(args) -> int:
     one_pass(False)
     log("measured pass ...")
     rows, total = one_pass(True)
+    preempted_before = engine.scheduler.num_preemptions
     plain_rows, plain_total = one_pass(False)      # without events and their synchronisation: the figure that counts
+    preempted = engine.scheduler.num_preemptions - preempted_before
 
     generated = n_req * new_tokens
     prefill_s = sum(w * (p / (p + d)) for w, _, _, p, d, _ in plain_rows if p + d)
@@ -335,10 +347,28 @@ def serving(args) -> int:
         "host_share": {"all_steps": round(1.0 - gpu_sum / wall_sum, 4) if wall_sum else None,
                        "decode_steps": round(host_share_decode, 4),
                        "measured_pass_ms": round(total * 1e3, 1)},
-        "preemptions": engine.scheduler.num_preemptions,
+        "preemptions": preempted,          # of the pass that ``value`` is from
     }
-    print(json.dumps(result))
+    del engine, runner
+    gc.collect()
+    torch.cuda.empty_cache()
+    return result
+
+
+def serving(args) -> int:
+    """``--workload serving``: a result line of its own for :func:`serving_measure`."""
+    print(json.dumps(serving_measure(args)))
     return 0
+
+
+def serving_brief(full: dict) -> dict:
+    """The figures of a serving result that go onto the default line, flat."""
+    return {"value": full["value"], "total_ms": full["total_ms"], "requests": full["config"]["requests"],
+            "new_tokens": full["config"]["new_tokens"], "prefill_tok_s": full["prefill"]["value"],
+            "decode_tok_s": full["decode"]["value"], "decode_step_ms": full["decode_step_ms"]["mean"],
+            "decode_step_p99_ms": full["decode_step_ms"]["p99"], "roofline_frac": full["roofline"]["frac"],
+            "host_share": full["host_share"]["all_steps"], "preemptions": full["preemptions"],
+            "cache_pages": full["config"]["cache_pages"]}
 
 
 def main() -> int:
@@ -404,7 +434,7 @@ def main() -> int:
     max_batch = max(args.batch, 64) if extras else args.batch
     pool = max_batch * CONTEXT_LEN
     if further:
-        pool = max(pool, 8 * (LONG_CONTEXTS[-1] + 512))
+        pool = max(pool, 64 * (LONG_CONTEXTS[-1] + 512))
     rig = Rig(cfg, args.dtype, pool, max_batch, args.decode_run)
 
     if args.phase == "prefill":
@@ -432,48 +462,111 @@ def main() -> int:
     log(f"decode batch {args.batch}: {step_s * 1e3:.3f} ms a step")
     points = {}
     more = {}
+    errors = []
+
+    def attempt(what: str, fn) -> None:
+        """A further point must not cost the line its contract: what fails is named in ``errors``."""
+        try:
+            fn()
+        except Exception as e:      # noqa: BLE001
+            log(f"{what} failed: {type(e).__name__}: {e}")
+            errors.append(f"{what}: {type(e).__name__}: {str(e)[:200]}")
+
+    def decode_point(r, c, name: str, batch: int, context: int, el: int, label: str) -> None:
+        sec, ctx = r.decode(batch, context, POINT_STEPS, POINT_WARMUP)
+        points[name] = round(batch / sec, 1)
+        more.setdefault("rooflines", {})[name] = round(decode_bytes(c, batch, ctx, el) / sec / HBM_PEAK, 4)
+        log(f"{label}: decode batch {batch} at context {context}: {sec * 1e3:.3f} ms a step")
+
     if extras:
         for b in (1, 64):
-            sec, _ = rig.decode(b, PROMPT_LEN, POINT_STEPS, POINT_WARMUP)
-            points[f"decode_b{b}"] = round(b / sec, 1)
-            log(f"decode batch {b}: {sec * 1e3:.3f} ms a step")
+            decode_point(rig, cfg, f"decode_b{b}", b, PROMPT_LEN, elem, f"{args.shape} {args.dtype}")
     if further:
-        for n in LONG_CONTEXTS:
-            sec, ctx = rig.decode(8, n, POINT_STEPS, POINT_WARMUP)
-            points[f"decode_b8_ctx{n // 1024}k"] = round(8 / sec, 1)
-            more[f"roofline_ctx{n // 1024}k"] = round(decode_bytes(cfg, 8, ctx, elem) / sec / HBM_PEAK, 4)
-            log(f"decode batch 8 at context {n}: {sec * 1e3:.3f} ms a step")
-        for n in LONG_CONTEXTS:      # long prompts, where the attention is the larger part, in portions of the token budget
-            sec = rig.prefill(n, ENGINE_CHUNK)
-            more[f"prefill_{n // 1024}k"] = {"value": round(n / sec, 1), "tokens": n, "ms": round(sec * 1e3, 3),
-                                            "frac": round(prefill_flops(cfg, n) / sec / FLOP_PEAK[args.dtype], 4)}
-            log(f"prefill of {n} in portions of {ENGINE_CHUNK}: {sec * 1e3:.2f} ms")
+        def long_contexts():
+            for n in LONG_CONTEXTS:
+                sec, ctx = rig.decode(8, n, POINT_STEPS, POINT_WARMUP)
+                points[f"decode_b8_ctx{n // 1024}k"] = round(8 / sec, 1)
+                more[f"roofline_ctx{n // 1024}k"] = round(decode_bytes(cfg, 8, ctx, elem) / sec / HBM_PEAK, 4)
+                log(f"decode batch 8 at context {n}: {sec * 1e3:.3f} ms a step")
+            for n in LONG_CONTEXTS:
+                decode_point(rig, cfg, f"decode_b64_ctx{n // 1024}k", 64, n, elem, "1B bf16")
+            for n in LONG_CONTEXTS:      # long prompts, where the attention is the larger part, in portions of the token budget
+                sec = rig.prefill(n, ENGINE_CHUNK)
+                more[f"prefill_{n // 1024}k"] = {"value": round(n / sec, 1), "tokens": n, "ms": round(sec * 1e3, 3),
+                                                "frac": round(prefill_flops(cfg, n) / sec / FLOP_PEAK[args.dtype], 4)}
+                log(f"prefill of {n} in portions of {ENGINE_CHUNK}: {sec * 1e3:.2f} ms")
+        attempt("long contexts", long_contexts)
         rig.close()
-        # the reference's own precision: the same model in true float32
-        rig32 = Rig(cfg, "fp32", 8 * CONTEXT_LEN, 8, args.decode_run)
-        sec = rig32.prefill(PROMPT_LEN, args.prefill_chunk)
-        more["prefill_fp32"] = prefill_record(sec, "fp32")
-        more["prefill_fp32_one_portion"] = prefill_record(rig32.prefill(PROMPT_LEN, ENGINE_CHUNK), "fp32")
-        log(f"float32: prefill of {PROMPT_LEN} in portions of {args.prefill_chunk}: {sec * 1e3:.2f} ms")
-        sec, ctx = rig32.decode(8, PROMPT_LEN, POINT_STEPS, POINT_WARMUP)
-        points["decode_b8_fp32"] = round(8 / sec, 1)
-        more["roofline_fp32"] = round(decode_bytes(cfg, 8, ctx, 4) / sec / HBM_PEAK, 4)
-        log(f"float32: decode batch 8: {sec * 1e3:.3f} ms a step")
-        rig32.close()
-        # the next size of the family
-        cfg3 = dict(SHAPES["3b"][2])
-        rig3 = Rig(cfg3, "bf16", 8 * CONTEXT_LEN, 8, args.decode_run)
-        sec = rig3.prefill(PROMPT_LEN, ENGINE_CHUNK)
-        more["prefill_3b_one_portion"] = prefill_record(sec, "bf16", prefill_flops(cfg3, PROMPT_LEN))
-        sec, ctx = rig3.decode(8, PROMPT_LEN, POINT_STEPS, POINT_WARMUP)
-        points["decode_b8_3b"] = round(8 / sec, 1)
-        more["roofline_3b"] = round(decode_bytes(cfg3, 8, ctx, 2) / sec / HBM_PEAK, 4)
-        log(f"3B shape: decode batch 8: {sec * 1e3:.3f} ms a step")
-        rig3.close()
+
+        def float32_1b():
+            # the reference's own precision: the same model in true float32
+            rig32 = Rig(cfg, "fp32", 8 * (LONG_CONTEXTS[0] + 2048), 8, args.decode_run)
+            try:
+                sec = rig32.prefill(PROMPT_LEN, args.prefill_chunk)
+                more["prefill_fp32"] = prefill_record(sec, "fp32")
+                more["prefill_fp32_one_portion"] = prefill_record(rig32.prefill(PROMPT_LEN, ENGINE_CHUNK), "fp32")
+                log(f"float32: prefill of {PROMPT_LEN} in portions of {args.prefill_chunk}: {sec * 1e3:.2f} ms")
+                sec, ctx = rig32.decode(8, PROMPT_LEN, POINT_STEPS, POINT_WARMUP)
+                points["decode_b8_fp32"] = round(8 / sec, 1)
+                more["roofline_fp32"] = round(decode_bytes(cfg, 8, ctx, 4) / sec / HBM_PEAK, 4)
+                log(f"float32: decode batch 8: {sec * 1e3:.3f} ms a step")
+                decode_point(rig32, cfg, "decode_b8_ctx8k_fp32", 8, LONG_CONTEXTS[0], 4, "1B fp32")
+            finally:
+                rig32.close()
+        attempt("float32", float32_1b)
+
+        def shape_3b():
+            # the next size of the family
+            cfg3 = dict(SHAPES["3b"][2])
+            rig3 = Rig(cfg3, "bf16", 64 * CONTEXT_LEN, 64, args.decode_run)
+            try:
+                sec = rig3.prefill(PROMPT_LEN, ENGINE_CHUNK)
+                more["prefill_3b_one_portion"] = prefill_record(sec, "bf16", prefill_flops(cfg3, PROMPT_LEN))
+                sec, ctx = rig3.decode(8, PROMPT_LEN, POINT_STEPS, POINT_WARMUP)
+                points["decode_b8_3b"] = round(8 / sec, 1)
+                more["roofline_3b"] = round(decode_bytes(cfg3, 8, ctx, 2) / sec / HBM_PEAK, 4)
+                log(f"3B shape: decode batch 8: {sec * 1e3:.3f} ms a step")
+                for b in (1, 64):
+                    decode_point(rig3, cfg3, f"decode_b{b}_3b", b, PROMPT_LEN, 2, "3B bf16")
+            finally:
+                rig3.close()
+        attempt("3B shape", shape_3b)
+
+        def serving_points():
+            # through the scheduler (the benchmark configuration of the 3B shape: float32, 64 concurrent requests,
+            # prompts uniform in [128, 2048], 256 new tokens each), and the 1B shape in bfloat16 beside it
+            import copy
+            for key, shape, dt, n_req, share in (("serving_1b_bf16", "1b", "bf16", 64, 1.0),
+                                                 ("serving_1b_bf16_128req_half_pool", "1b", "bf16", 128, 0.5),
+                                                 ("serving_3b_fp32", "3b", "fp32", 64, 1.0)):
+                a = copy.copy(args)
+                a.shape, a.dtype, a.layers, a.prefill_chunk, a.requests, a.pool_share = shape, dt, None, None, n_req, share
+                full_line = serving_measure(a)
+                more[key] = serving_brief(full_line)
+                log(f"{key}: {full_line['value']} generated tok/s, decode steps of {full_line['decode_step_ms']['mean']} ms "
+                    f"at {full_line['roofline']['frac']} of the roofline, {full_line['preemptions']} preemptions")
+        attempt("serving", serving_points)
+
+        def shape_8b(dt: str, el: int, prefill_too: bool):
+            # the 8B shape at full depth (in float32: 32 GB of weights)
+            cfg8 = dict(SHAPES["8b"][2])
+            rig8 = Rig(cfg8, dt, 64 * CONTEXT_LEN, 64, args.decode_run)
+            try:
+                if prefill_too:
+                    sec = rig8.prefill(PROMPT_LEN, PREFILL_CHUNK)
+                    more[f"prefill_8b_{dt}"] = prefill_record(sec, dt, prefill_flops(cfg8, PROMPT_LEN))
+                    log(f"8B shape, {dt}: prefill of {PROMPT_LEN} in portions of {PREFILL_CHUNK}: {sec * 1e3:.2f} ms")
+                for b in (1, 8, 64):
+                    decode_point(rig8, cfg8, f"decode_b{b}_8b_{dt}", b, PROMPT_LEN, el, f"8B {dt}")
+            finally:
+                rig8.close()
+        attempt("8B shape, float32", lambda: shape_8b("fp32", 4, True))
+        attempt("8B shape, bfloat16", lambda: shape_8b("bf16", 2, False))
 
     achieved = decode_bytes(cfg, args.batch, mean_ctx, elem) / step_s
     result = {
-        "metric": f"decode tok/s at batch {args.batch} ({shown_name} shape, context {CONTEXT_LEN})",
+        "metric": f"decode tok/s at batch {args.batch} ({shown_name} shape, prompts of {PROMPT_LEN} tokens, "
+                  f"decode context ~{round(mean_ctx)}, pool for {CONTEXT_LEN})",
         "value": round(args.batch / step_s, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -495,6 +588,8 @@ def main() -> int:
         "points": points,
     }
     result.update(more)
+    if errors:
+        result["errors"] = errors
     print(json.dumps(result))
     return 0
 

@@ -28,8 +28,7 @@ def build_spec(cfg: LlamaConfig) -> ModelSpec:
     blocks = []
     for i in range(cfg.num_hidden_layers):
         pre = f"model.layers.{i}."
-        blocks.append(BlockSpec(
-            kind="prenorm",
+        blocks.append(BlockSpec(kind="prenorm", parts=dict(
             mixer_norm=PartSpec("rmsnorm", {"size": d, "eps": cfg.rms_norm_eps},
                                 {"weight": pre + "input_layernorm.weight"}),
             mixer=PartSpec("attention",
@@ -43,7 +42,7 @@ def build_spec(cfg: LlamaConfig) -> ModelSpec:
             ffn=PartSpec("swiglu", {"hidden_size": d, "intermediate_size": cfg.intermediate_size},
                          {"gate": pre + "mlp.gate_proj.weight", "up": pre + "mlp.up_proj.weight",
                           "down": pre + "mlp.down_proj.weight"}),
-        ))
+        )))
     embed_name = "model.embed_tokens.weight"
     head_name = embed_name if cfg.tie_word_embeddings else "lm_head.weight"
     return ModelSpec(

@@ -23,17 +23,26 @@ class PartSpec:
 
 @dataclass
 class BlockSpec:
-    """A residual block: how a mixer and a feed-forward are arranged around the residual stream.
+    """A residual block: which arrangement (``kind``, a key of the block registry) of which parts.
 
-    ``kind`` chooses the arrangement (``"prenorm"``: x + mixer(norm(x)), then x + ffn(norm(x)),
-    src/model/llama.cpp:324-379).
+    ``parts`` maps the role a part plays in the block to its spec; which roles a kind of block has,
+    and of which family each is, is that block class's own knowledge (the ``prenorm`` block, x +
+    mixer(norm(x)) then x + ffn(norm(x)), src/model/llama.cpp:324-379, has ``mixer_norm``,
+    ``mixer``, ``ffn_norm`` and ``ffn``).  Another arrangement (more norms, a mixer beside the
+    feed-forward) is another block class with other roles; nothing else changes.  ``params``
+    holds constants of the arrangement itself.  A role reads as an attribute: ``spec.mixer``.
     """
 
     kind: str
-    mixer_norm: PartSpec
-    mixer: PartSpec
-    ffn_norm: PartSpec
-    ffn: PartSpec
+    parts: Dict[str, PartSpec] = field(default_factory=dict)
+    params: Dict[str, Any] = field(default_factory=dict)
+
+    def __getattr__(self, role: str) -> PartSpec:
+        parts = self.__dict__.get("parts")
+        if parts is not None and role in parts:
+            return parts[role]
+        raise AttributeError(f"block of kind {self.__dict__.get('kind')!r} has no part {role!r}; "
+                             f"it has {sorted(parts or ())}")
 
 
 @dataclass

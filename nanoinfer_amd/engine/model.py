@@ -12,7 +12,7 @@ from typing import Dict, Optional
 import torch
 
 from ..config.spec import ModelSpec
-from ..parts.base import CacheNeed, LayerCache, Runtime, pending_for
+from ..parts.base import CacheNeed, LayerCache, Runtime, flag_of, pending_for
 from ..parts.standard import build_part
 from ..registry import get_part
 
@@ -42,12 +42,18 @@ class Model:
                 raise ValueError(f"block {run.block} reads cache {run.cache} before any block has written it")
         self.max_positions = spec.max_positions
 
+    def _all_parts(self):
+        return [self.embedding, self.final_norm, self.head] + list(self.blocks)
+
     def graph_safe(self) -> bool:
         """Whether a step of this model may be recorded into a HIP graph: every part says of itself
         that its launches depend on device data only (``graph_safe``), never on the host lists."""
-        parts = [self.embedding, self.final_norm, self.head] + list(self.blocks)
-        return all(getattr(p, "graph_safe", False) is True or (callable(getattr(p, "graph_safe", None)) and p.graph_safe())
-                   for p in parts)
+        return all(flag_of(p, "graph_safe", False) for p in self._all_parts())
+
+    def idempotent(self) -> bool:
+        """Whether running the same step twice leaves the caches as running it once does: true of keys
+        and values written to their places, not of a per-request state that a part updates in place."""
+        return all(flag_of(p, "idempotent", True) for p in self._all_parts())
 
     def cache_needs(self) -> Dict[int, CacheNeed]:
         return dict(self._needs)

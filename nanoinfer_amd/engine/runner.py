@@ -45,6 +45,31 @@ class GroupView:
     page_size: int
 
 
+@dataclass
+class SeqTables:
+    """What the step knows of each of its sequences, on the device (int32 [B] each, batch order):
+    the first row of its portion, the portion's length, the tokens in the cache after the step, and
+    the request's state slot.  A part whose launches may be recorded reads these, never the host lists."""
+
+    q_start: torch.Tensor
+    q_len: torch.Tensor
+    context_len: torch.Tensor
+    state_slot: torch.Tensor
+
+
+@dataclass
+class _Layout:
+    """Where the parts of a step's flat integer table lie: per cache group (offset of the slot
+    mapping, offset of the block table, table width), and the offset of the per-sequence table
+    (four rows of B entries: first row, length, context length, state slot)."""
+
+    groups: list
+    seq: int
+
+
+_HOST_LISTS = ("requests", "q_start", "q_len", "context_len", "state_slot")
+
+
 class StepContext:
     """Everything a part may want to know about the step it is running in.
 
@@ -60,23 +85,36 @@ class StepContext:
         self.device = device
         self.n_tokens = 0
         self.n_seqs = 0
-        self.requests: List[Hashable] = []
-        self.q_start: List[int] = []
-        self.q_len: List[int] = []
-        self.context_len: List[int] = []
-        self.state_slot: List[int] = []
+        self._host = {name: [] for name in _HOST_LISTS}
+        self._sealed = False
         self.max_context = 0
         self.max_q_len = 0
         self.token_ids: torch.Tensor = None
         self.positions: torch.Tensor = None
         self.seq_of_token: torch.Tensor = None
         self.logit_rows: Optional[torch.Tensor] = None
+        self.per_seq: Optional[SeqTables] = None
         self.groups: List[GroupView] = []
         self.recording = recording
         self._scratch_owner = scratch_owner
         self._scratch: Optional[torch.Tensor] = None
         self._q_tiles: Dict[int, torch.Tensor] = {}
         self.tile_sizes_asked = set()
+
+    def __getattr__(self, name: str):
+        # the host lists: one entry per sequence, in batch order.  While a step is being recorded they
+        # are not there to read: the recording would keep what they said at that moment for every replay.
+        if name in _HOST_LISTS:
+            if self.__dict__.get("_sealed"):
+                raise StepError(f"ctx.{name} is a host list, and this step is being recorded: its replays "
+                                f"would run with the values of now.  Read ctx.per_seq (the same per sequence, "
+                                f"on the device), or declare the part graph_safe = False")
+            return self.__dict__["_host"][name]
+        raise AttributeError(name)
+
+    def seal(self) -> None:
+        """From here on the host lists cannot be read (the runner calls this before it records)."""
+        self._sealed = True
 
     def q_tiles(self, tile_tokens: int) -> Optional[torch.Tensor]:
         """The portions of the step cut into tiles of at most ``tile_tokens`` tokens, int32 [n, 4]
@@ -88,7 +126,8 @@ class StepContext:
             self.tile_sizes_asked.add(tile_tokens)
             if self.recording:
                 return None
-            flat = K.build_q_tiles(self.q_start, self.q_len, self.context_len, tile_tokens)
+            host = self._host
+            flat = K.build_q_tiles(host["q_start"], host["q_len"], host["context_len"], tile_tokens)
             upload = getattr(self._scratch_owner, "_upload", None)
             if upload is not None:       # through the runner's pinned buffers: the host does not wait for the GPU
                 t = upload(flat).view(-1, 4)
@@ -151,18 +190,42 @@ class ModelRunner:
                                   # beyond that the one used longest ago is dropped and its shape recorded again if it returns
     GRAPH_PORTION_SIGHTS = 2      # a portion's shape is recorded when it comes this many times: recording costs
                                   # seven runs of the step and gains a few per cent of a run (a lone length never pays)
+    GRAPH_MAX_BYTES = 8 << 30     # device memory that all recordings together may hold (their logits, activations and
+                                  # tables: what the allocator's reserved memory grew by while each was made);
+                                  # beyond that the ones used longest ago are dropped, of either kind
 
     def __init__(self, model_dir: str, dtype: str = "bfloat16", page_size: int = 16, max_tokens: int = 4096,
                  max_requests: int = 64, device: Optional[torch.device] = None, use_graphs: bool = True,
-                 warm_up: bool = True, max_step_tokens: Optional[int] = None, kv_cache_bytes: Optional[int] = None):
+                 warm_up: bool = True, max_step_tokens: Optional[int] = None, kv_cache_bytes: Optional[int] = None,
+                 graph_memory_bytes: Optional[int] = None):
+        arch, config, spec = read_model_folder(model_dir)
+        tensors = load_tensors(model_dir, spec)
+        self._setup(spec, tensors, dtype, page_size, max_tokens, max_requests, device, use_graphs, warm_up,
+                    max_step_tokens, kv_cache_bytes, graph_memory_bytes, arch=arch, config=config)
+
+    @classmethod
+    def from_spec(cls, spec, tensors: Dict[str, torch.Tensor], dtype: str = "bfloat16", page_size: int = 16,
+                  max_tokens: int = 4096, max_requests: int = 64, device: Optional[torch.device] = None,
+                  use_graphs: bool = True, warm_up: bool = False, max_step_tokens: Optional[int] = None,
+                  kv_cache_bytes: Optional[int] = None, graph_memory_bytes: Optional[int] = None) -> "ModelRunner":
+        """A runner over a model given as data (a :class:`~nanoinfer_amd.config.spec.ModelSpec`) and its
+        tensors by checkpoint name (CPU tensors), without a folder: the same model, cache manager and
+        step function.  The tensors are checked against what the parts of the spec ask for."""
+        from ..weights.loader import check_tensors
+        self = cls.__new__(cls)
+        self._setup(spec, check_tensors(spec, tensors), dtype, page_size, max_tokens, max_requests, device, use_graphs,
+                    warm_up, max_step_tokens, kv_cache_bytes, graph_memory_bytes)
+        return self
+
+    def _setup(self, spec, tensors, dtype, page_size, max_tokens, max_requests, device, use_graphs, warm_up,
+               max_step_tokens, kv_cache_bytes, graph_memory_bytes, arch=None, config=None) -> None:
         self.device = device or K.require_gpu()
         torch_dtype = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
                        "float32": torch.float32, "fp32": torch.float32}.get(dtype)
         if torch_dtype is None:
             raise ValueError(f"dtype {dtype!r} is not one of bfloat16, float32")
         self.dtype = torch_dtype
-        self.arch, self.config, self.spec = read_model_folder(model_dir)
-        tensors = load_tensors(model_dir, self.spec)
+        self.arch, self.config, self.spec = arch, config, spec
         self.rt = Runtime(torch_dtype, self.device)
         self.model = Model(self.spec, tensors, self.rt)
         del tensors
@@ -182,6 +245,8 @@ class ModelRunner:
         self.eos_token_ids = tuple(self.spec.eos_token_ids)
         self._done: Dict[Hashable, int] = {}   # tokens of each live request already in the cache
         self._scratch: Optional[torch.Tensor] = None
+        if graph_memory_bytes is not None:
+            self.GRAPH_MAX_BYTES = int(graph_memory_bytes)
         self._init_graphs(use_graphs)
         if warm_up:
             self._warm_up()

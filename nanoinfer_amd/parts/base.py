@@ -10,7 +10,7 @@ knows nothing of the model it sits in.  Interfaces, by family:
 ``position``      ``tables() -> (cos, sin) | None`` for the mixer that owns it
 ``mixer``         ``cache_need() -> CacheNeed``; ``forward(x, ctx, cache) -> y[T, d]``
 ``feed_forward``  ``forward(x, ctx) -> y[T, d]``
-``block``         ``forward(h, pending, ctx, cache) -> (h, pending)``
+``block``         ``forward(h, pending, ctx, cache) -> (h, pending)``; its parts by role (:class:`Block`)
 ``head``          ``forward(x[R, d]) -> logits[R, vocab] float32``
 """
 from __future__ import annotations
@@ -104,6 +104,11 @@ class Part:
     # True when a part's launches depend only on device data and on the sizes of the step, so that
     # a step may be recorded once and replayed; a part that reads the step's host lists says False
     graph_safe = False
+    # False when running the same step a second time changes what the part leaves behind (a state
+    # updated in place: keys and values written again at the same places are the same).  Whoever runs
+    # a step more than once (the recording of a step into a HIP graph does) then puts the
+    # per-request state back in between.
+    idempotent = True
 
     @classmethod
     def weight_requests(cls, spec: PartSpec) -> List[WeightRequest]:
@@ -112,6 +117,67 @@ class Part:
     def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
         self.spec = spec
         self.rt = rt
+
+
+def flag_of(part, name: str, default: bool) -> bool:
+    """A yes/no property of a part (``graph_safe``, ``idempotent``) that a simple part states as a
+    class attribute and a part made of parts (a block) as a method."""
+    value = getattr(part, name, default)
+    return bool(value() if callable(value) else value)
+
+
+class Block:
+    """Base of the blocks: an arrangement of parts around the residual stream.
+
+    A block class names its roles and the family of each in ``ROLES`` (role -> family); the base
+    asks every role's part for its tensors, builds the parts as attributes of those names, and
+    answers for the whole block what each part answers for itself.  ``forward(h, pending, ctx,
+    cache) -> (h, pending)`` is the subclass's: ``h`` is the float32 residual stream [T, d],
+    ``pending`` an addend that the stream has not received yet (or None), which the next norm sums
+    in; the cache goes to the block's ``mixer``."""
+
+    family = "block"
+    kind = ""
+    ROLES: Dict[str, str] = {}
+
+    @classmethod
+    def _roles(cls, spec):
+        missing = [r for r in cls.ROLES if r not in spec.parts]
+        extra = [r for r in spec.parts if r not in cls.ROLES]
+        if missing or extra:
+            raise ValueError(f"a block of kind {spec.kind!r} has the parts {sorted(cls.ROLES)}; "
+                             f"missing: {missing}, not known: {extra}")
+        return cls.ROLES.items()
+
+    @classmethod
+    def weight_requests(cls, spec) -> List[WeightRequest]:
+        from ..registry import get_part
+        out: List[WeightRequest] = []
+        for role, family in cls._roles(spec):
+            out += get_part(family, spec.parts[role].kind).weight_requests(spec.parts[role])
+        return out
+
+    def __init__(self, spec, tensors: Dict[str, torch.Tensor], rt: Runtime):
+        from .standard import build_part
+        self.spec = spec
+        self.rt = rt
+        self.roles = []
+        for role, family in self._roles(spec):
+            setattr(self, role, build_part(family, spec.parts[role], tensors, rt))
+            self.roles.append(role)
+
+    def parts(self):
+        return [getattr(self, r) for r in self.roles]
+
+    def cache_need(self) -> "CacheNeed":
+        """What the block wants of the cache: what its mixer wants."""
+        return self.mixer.cache_need()
+
+    def graph_safe(self) -> bool:
+        return all(flag_of(p, "graph_safe", False) for p in self.parts())
+
+    def idempotent(self) -> bool:
+        return all(flag_of(p, "idempotent", True) for p in self.parts())
 
 
 def pending_for(norm, pending: Optional[torch.Tensor], dtype: torch.dtype) -> Optional[torch.Tensor]:

@@ -13,9 +13,9 @@ import numpy as np
 import torch
 
 from .. import kernels as K
-from ..config.spec import BlockSpec, PartSpec
+from ..config.spec import PartSpec
 from ..registry import get_part, register_part
-from .base import CacheNeed, KVNeed, LayerCache, Part, Runtime, WeightRequest, pending_for
+from .base import Block, CacheNeed, KVNeed, LayerCache, Part, Runtime, WeightRequest, pending_for
 
 
 class PartWeights(dict):
@@ -232,12 +232,26 @@ class Attention(Part):
     def cache_need(self) -> CacheNeed:
         return CacheNeed(kv=KVNeed(self.KVH, self.hd, self.window))
 
+    # The pass is four stages, each a method of its own, so that a variant of attention replaces the stage
+    # it changes and keeps the others: project (x -> stacked q, k, v), rotate_and_write (position encoding,
+    # keys and values into the cache pages), attend (queries over the cache), output (the o product, onto the
+    # residual stream where it can).  The first two also exist fused in one kernel for steps of few rows; the
+    # fused kernel stands in only for a class that has left both stages as they are here.
+
+    def _fused_projection(self, T: int, d: int, dtype) -> bool:
+        """Whether the product with the stacked matrix rotates and stores in its own epilogue for T rows."""
+        cls = type(self)
+        if cls.project is not Attention.project or cls.rotate_and_write is not Attention.rotate_and_write:
+            return False
+        tables = self.position.tables()
+        return (tables is not None and K.qkv_rope_ok(T, d, self.hd, 2 * tables[0].shape[1], dtype)
+                and K.qkv_rope_wins(T, d, dtype))
+
     def takes_normed(self, T: int) -> bool:
         """Whether ``forward`` takes the norm before it as a prologue of its first product for T tokens."""
-        tables = self.position.tables()
         d = self.w_qkv.shape[1]
-        return (K.FUSE_NORMS and tables is not None and K.qkv_rope_ok(T, d, self.hd, 2 * tables[0].shape[1], self.rt.dtype)
-                and K.qkv_rope_wins(T, d, self.rt.dtype) and K.norm_prologue_ok(T, d, self.rt.dtype, self.w_qkv))
+        return (K.FUSE_NORMS and self._fused_projection(T, d, self.rt.dtype)
+                and K.norm_prologue_ok(T, d, self.rt.dtype, self.w_qkv))
 
     def adds_residual(self, T: int) -> bool:
         """Whether ``forward`` can take ``residual=h`` for T tokens: its output then goes into the residual
@@ -253,29 +267,42 @@ class Attention(Part):
                 and K.norm_prologue_ok(T, d, self.rt.dtype, self.w_qkv, addends)
                 and K.residual_takes_addends(T, self.H * self.hd, self.rt.dtype, self.w_o))
 
-    def forward(self, x, ctx, cache: LayerCache, residual: Optional[torch.Tensor] = None):
-        T = x.shape[0]
-        carried = getattr(x, "pending", None)       # addends of the residual stream that came with a normed input
-        if carried is not None and residual is None:
-            raise K.KernelError("pending addends of the residual stream need residual=h to go into")
+    def project(self, x, ctx) -> torch.Tensor:
+        """Stage 1: ``x`` [T, d] -> [T, (H + 2 KVH) * hd], the query heads, then the key heads, then the
+        value heads, as projected."""
+        return K.linear(x, self.w_qkv)
+
+    def rotate_and_write(self, qkv: torch.Tensor, ctx, cache: LayerCache) -> torch.Tensor:
+        """Stage 2: the position encoding on the query and key heads of ``qkv`` (in place), and the keys and
+        values of the step's tokens into their places in the cache pages (where this entry of the order writes)."""
         tables = self.position.tables()
         cos, sin = tables if tables is not None else (None, None)
         slots = cache.slot_mapping if cache.writes else None
-        if (cos is not None and K.qkv_rope_ok(T, x.shape[1], self.hd, 2 * cos.shape[1], x.dtype)
-                and K.qkv_rope_wins(T, x.shape[1], x.dtype)):
-            # few rows: rotation and cache write ride on the product's epilogue
-            qkv = K.skinny_qkv_rope(x, self.w_qkv, ctx.positions, cos, sin, slots, cache.kpool, cache.vpool,
-                                    self.H, self.KVH, self.hd)
-        else:
-            qkv = K.linear(x, self.w_qkv)
-            K.rope_kv_write(qkv, ctx.positions, cos, sin, slots, cache.kpool, cache.vpool, self.H, self.KVH, self.hd)
-        out = torch.empty(T, self.H * self.hd, dtype=x.dtype, device=x.device)
+        K.rope_kv_write(qkv, ctx.positions, cos, sin, slots, cache.kpool, cache.vpool, self.H, self.KVH, self.hd)
+        return qkv
+
+    def project_rotate_write(self, x, ctx, cache: LayerCache) -> torch.Tensor:
+        """Stages 1 and 2: by one kernel where few rows allow it and neither stage has been replaced."""
+        T = x.shape[0]
+        if self._fused_projection(T, x.shape[1], x.dtype):
+            cos, sin = self.position.tables()
+            return K.skinny_qkv_rope(x, self.w_qkv, ctx.positions, cos, sin, cache.slot_mapping if cache.writes else None,
+                                     cache.kpool, cache.vpool, self.H, self.KVH, self.hd)
+        return self.rotate_and_write(self.project(x, ctx), ctx, cache)
+
+    def attend(self, qkv: torch.Tensor, ctx, cache: LayerCache, leave_runs: bool = False):
+        """Stage 3: every query of ``qkv`` over the keys and values of its sequence in the cache, up to its own
+        position (inside the window, if there is one).  Returns ``out`` [T, H * hd]; or, with ``leave_runs``
+        where the key ranges were cut into runs that the output product can merge itself, ``(workspace, runs)``."""
+        T = qkv.shape[0]
+        dtype = qkv.dtype
+        out = torch.empty(T, self.H * self.hd, dtype=dtype, device=qkv.device)
         tiles = None
-        if ctx.max_q_len >= self.MFMA_MIN_PORTION and K.mfma_attention_ok(x.dtype, self.hd):
+        if ctx.max_q_len >= self.MFMA_MIN_PORTION and K.mfma_attention_ok(dtype, self.hd):
             # prompt portions: tiles of tokens on the matrix cores (a recorded step has them only if
             # it was recorded with them)
             max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window + ctx.max_q_len)
-            tile_tokens, nsplit = K.mfma_plan(self.hd, self.H // self.KVH, self.KVH, T, ctx.max_q_len, max_keys, x.dtype)
+            tile_tokens, nsplit = K.mfma_plan(self.hd, self.H // self.KVH, self.KVH, T, ctx.max_q_len, max_keys, dtype)
             tiles = ctx.q_tiles(tile_tokens)
         if tiles is not None:
             if nsplit is None:
@@ -283,26 +310,45 @@ class Attention(Part):
             ws = ctx.workspace(T * self.H * nsplit * (self.hd + 2)) if nsplit > 1 else None
             K.mfma_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, out, self.H, self.KVH, self.hd,
                              self.scale, self.window, nsplit, ws, tile_tokens)
-            return K.linear(out, self.w_o, residual=residual, pending=carried)
+            return out
         # single tokens and short portions, token by token
         max_keys = ctx.max_context if self.window is None else min(ctx.max_context, self.window)
-        on_matrix_cores = K.mfma_token_ok(x.dtype, self.hd)
+        on_matrix_cores = K.mfma_token_ok(dtype, self.hd)
         choose = K.mfma_token_splits if on_matrix_cores else K.choose_splits
         nsplit = choose(T, self.KVH, self.H // self.KVH, max_keys)
         ws = ctx.workspace(T * self.H * nsplit * (self.hd + 2)) if nsplit > 1 else None
-        if on_matrix_cores and nsplit > 1 and K.MERGE_IN_PRODUCT and K.skinny_merge_wins(T, self.H, self.hd, nsplit, x.dtype, self.w_o):
+        if (leave_runs and on_matrix_cores and nsplit > 1 and K.MERGE_IN_PRODUCT
+                and K.skinny_merge_wins(T, self.H, self.hd, nsplit, dtype, self.w_o)):
             # one or two rows: the output product merges the key runs in its prologue, no kernel of its own does
             K.mfma_token_attention(qkv, cache.kpool, cache.vpool, cache.block_table, ctx.seq_of_token, ctx.positions,
                                    out, self.H, self.KVH, self.hd, self.scale, self.window, nsplit, ws, merge=False)
-            if residual is not None:
-                K.skinny_gemm_merged(ws, nsplit, T, self.H, self.hd, self.w_o, residual, residual=True, pending=carried)
-                return None
-            y = torch.empty(T, self.w_o.rows.shape[0], dtype=x.dtype, device=x.device)
-            return K.skinny_gemm_merged(ws, nsplit, T, self.H, self.hd, self.w_o, y)
+            return ws, nsplit
         attend = K.mfma_token_attention if on_matrix_cores else K.token_attention
         attend(qkv, cache.kpool, cache.vpool, cache.block_table, ctx.seq_of_token, ctx.positions, out,
                self.H, self.KVH, self.hd, self.scale, self.window, nsplit, ws)
-        return K.linear(out, self.w_o, residual=residual, pending=carried)
+        return out
+
+    def output(self, attended, T: int, residual: Optional[torch.Tensor] = None, carried: Optional[torch.Tensor] = None):
+        """Stage 4: the o product of what :meth:`attend` returned.  With ``residual`` (the float32 stream) the
+        product goes into it (None is returned) or comes back as float32 addends for the next norm; ``carried``
+        are addends that the stream has not received and that go in with it."""
+        if isinstance(attended, tuple):
+            ws, nsplit = attended
+            if residual is not None:
+                K.skinny_gemm_merged(ws, nsplit, T, self.H, self.hd, self.w_o, residual, residual=True, pending=carried)
+                return None
+            y = torch.empty(T, self.w_o.rows.shape[0], dtype=self.rt.dtype, device=ws.device)
+            return K.skinny_gemm_merged(ws, nsplit, T, self.H, self.hd, self.w_o, y)
+        return K.linear(attended, self.w_o, residual=residual, pending=carried)
+
+    def forward(self, x, ctx, cache: LayerCache, residual: Optional[torch.Tensor] = None):
+        T = x.shape[0]
+        carried = getattr(x, "pending", None)       # addends of the residual stream that came with a normed input
+        if carried is not None and residual is None:
+            raise K.KernelError("pending addends of the residual stream need residual=h to go into")
+        qkv = self.project_rotate_write(x, ctx, cache)
+        leave_runs = type(self).output is Attention.output      # a replaced output stage gets the merged rows
+        return self.output(self.attend(qkv, ctx, cache, leave_runs=leave_runs), T, residual, carried)
 
 
 # ------------------------------------------------------------------ feed-forward
@@ -352,7 +398,7 @@ class SwiGLU(Part):
 # ------------------------------------------------------------------ block
 
 @register_part("block", "prenorm")
-class PreNormBlock:
+class PreNormBlock(Block):
     """``h += mixer(norm1(h)); h += ffn(norm2(h))`` (src/model/llama.cpp:324-379).
 
     The residual stream ``h`` is float32.  The last addend is handed on as ``pending`` and is
@@ -367,27 +413,7 @@ class PreNormBlock:
     kernel that sums them.  A part without these is run the plain way.
     """
 
-    family = "block"
-    kind = "prenorm"
-
-    @classmethod
-    def weight_requests(cls, spec: BlockSpec) -> List[WeightRequest]:
-        return (requests_of("norm", spec.mixer_norm) + requests_of("mixer", spec.mixer)
-                + requests_of("norm", spec.ffn_norm) + requests_of("feed_forward", spec.ffn))
-
-    def __init__(self, spec: BlockSpec, tensors: Dict[str, torch.Tensor], rt: Runtime):
-        self.spec = spec
-        self.rt = rt
-        self.mixer_norm = build_part("norm", spec.mixer_norm, tensors, rt)
-        self.mixer = build_part("mixer", spec.mixer, tensors, rt)
-        self.ffn_norm = build_part("norm", spec.ffn_norm, tensors, rt)
-        self.ffn = build_part("feed_forward", spec.ffn, tensors, rt)
-
-    def cache_need(self) -> CacheNeed:
-        return self.mixer.cache_need()
-
-    def graph_safe(self) -> bool:
-        return all(p.graph_safe is True for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn))
+    ROLES = {"mixer_norm": "norm", "mixer": "mixer", "ffn_norm": "norm", "ffn": "feed_forward"}
 
     def _normed_input(self, norm, part, h, pending):
         """What ``part`` is given for ``norm(h + pending)``: the norm as a prologue where both sides can, else its
