@@ -51,6 +51,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--max-model-len", type=int, default=None)
     ap.add_argument("--max-decode-run", type=int, default=8,
                     help="decode steps run back to back on one scheduling decision (requests without a repetition penalty)")
+    ap.add_argument("--one-weight-copy", action="store_true",
+                    help="keep every layer matrix once on the device (no re-tiled copy for decode steps: less memory, slower decoding)")
     ap.add_argument("--json", action="store_true", help="print the generated ids as one JSON line per request")
     return ap
 
@@ -78,11 +80,15 @@ def main(argv: List[str] = None) -> int:
                        prefill_chunk_size=args.prefill_chunk_size, block_size=args.block_size,
                        num_cache_blocks=args.num_cache_blocks, max_num_batched_tokens=args.max_num_batched_tokens,
                        max_model_len=args.max_model_len, max_decode_run=args.max_decode_run, dtype=_DTYPES[args.dtype],
-                       kv_cache_bytes=None if args.kv_cache_gb is None else int(args.kv_cache_gb * (1 << 30)))
+                       kv_cache_bytes=None if args.kv_cache_gb is None else int(args.kv_cache_gb * (1 << 30)),
+                       one_weight_copy=args.one_weight_copy)
     print(f"Model: {model_dir}  dtype: {args.dtype}", file=sys.stderr)
     t0 = time.perf_counter()
     engine = Engine(model_dir, cfg, ignore_eos=args.ignore_eos)
     print(f"Loaded in {time.perf_counter() - t0:.2f} s", file=sys.stderr)
+    mem = engine.runner.memory_report()
+    print(f"Device memory: weights {mem['weights'] / 2**30:.3f} GiB ({mem['weights'] / max(mem['checkpoint'], 1):.2f} x the "
+          f"checkpoint's {mem['checkpoint'] / 2**30:.3f} GiB), key/value pools {mem['kv_pools'] / 2**30:.3f} GiB", file=sys.stderr)
 
     prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
     rng = random.Random(args.prompt_seed)

@@ -1,5 +1,6 @@
 // Attention of prompt portions over the paged key/value cache on the matrix cores of gfx950.
-// bfloat16 only; compiled once per head size (-DHEAD_DIM=n, a multiple of 32 up to 256).
+// bfloat16 only; compiled once per head size (-DHEAD_DIM=n, a multiple of 16 up to 256; the kernel for
+// single tokens takes the multiples of 32 among them).
 //
 // A workgroup of four wavefronts owns one tile of consecutive tokens of one sequence and the
 // query heads of one kv head (up to 16 of them at a time).  A "row" is one (token, head) pair; a
@@ -30,7 +31,15 @@
 #ifndef HEAD_DIM
 #error "HEAD_DIM must be defined"
 #endif
-static_assert(HEAD_DIM % 32 == 0 && HEAD_DIM >= 32 && HEAD_DIM <= 256, "head size: multiple of 32, at most 256");
+static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256, "head size: multiple of 16, at most 256");
+// A head size that is an odd multiple of 16 leaves the first product 16 dims after its steps of 32.  A lane
+// then holds 4 dims of its key (or of its row of Q) instead of 8, in the first half of its operand; the
+// second half is zero in both operands (the k index of a matrix instruction is only a label, so the four
+// real dims of every lane meet their partners and the zeros meet zeros).  No lane reads past its row.
+// (One instruction of half the depth, v_mfma_f32_16x16x16_bf16, behind the chain of v_mfma_f32_16x16x32_bf16
+// into the same accumulator gave wrong scores now and then at head sizes 48 and 80: one kind of matrix
+// instruction per chain is kept.)
+#define HEAD_HALF (HEAD_DIM % 32 != 0)
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
@@ -164,7 +173,8 @@ void mfma_attention_kernel(
     int page_size, int page_shift, int hpt_shift, int window, float scale, int nsplit) {
     constexpr int HD = HEAD_DIM;
     constexpr int MA_THREADS = MA_WAVES * WAVE;
-    constexpr int KK = HD / 32;              // k steps of the first product
+    constexpr int KK = HD / 32;              // k steps of 32 dims of the first product (and 16 dims more where HEAD_HALF)
+    constexpr int KKA = KK > 0 ? KK : 1;     // (an array's length)
     constexpr int DT = HD / 16;              // 16-wide tiles of the head dimension in the output
     constexpr int VROW = HD + VPAD;
     constexpr int KROW = HD + KPAD;
@@ -248,18 +258,22 @@ void mfma_attention_kernel(
             return static_cast<size_t>(row) * HD;
         };
 
-        // Q as the B operand: lane (row r, group kg) holds dims kk*32 + kg*8 .. +8
-        uint4 qf[CB][KK];
+        // Q as the B operand: lane (row r, group kg) holds dims kk*32 + kg*8 .. +8 (and of the last 16 dims
+        // of an odd head size, dims KK*32 + kg*4 .. +4)
+        uint4 qf[CB][KKA];
+        uint2 qh[CB];
 #pragma unroll
-        for (int c = 0; c < CB; ++c)
+        for (int c = 0; c < CB; ++c) {
+            const bf16_t* qrow = q + static_cast<size_t>(tile.row0 + (row_ok[c] ? tt[c] : 0)) * q_stride +
+                                 static_cast<size_t>(row_ok[c] ? head : 0) * HD;
 #pragma unroll
-            for (int kk = 0; kk < KK; ++kk) {
-                if (row_ok[c])
-                    qf[c][kk] = *reinterpret_cast<const uint4*>(q + static_cast<size_t>(tile.row0 + tt[c]) * q_stride +
-                                                                static_cast<size_t>(head) * HD + kk * 32 + kg * 8);
-                else
-                    qf[c][kk] = make_uint4(0, 0, 0, 0);
+            for (int kk = 0; kk < KK; ++kk)
+                qf[c][kk] = row_ok[c] ? *reinterpret_cast<const uint4*>(qrow + kk * 32 + kg * 8) : make_uint4(0, 0, 0, 0);
+            qh[c] = make_uint2(0, 0);
+            if constexpr (HEAD_HALF) {
+                if (row_ok[c]) qh[c] = *reinterpret_cast<const uint2*>(qrow + KK * 32 + kg * 4);
             }
+        }
 
         float m_run[CB];
         floatx4_t o[CB][DT], l_run[CB];
@@ -365,12 +379,15 @@ void mfma_attention_kernel(
                         // K as the A operand: lane (key r of a 16-key half, group kg) holds dims kk*32 + kg*8 .. +8
                         const uint16_t (*kb)[KROW] = ksm[s & 1];
                         const uint16_t (*vb)[VROW] = vs[s & 1];
-                        uint4 ka[2][KK];
+                        uint4 ka[2][KKA];
+                        uint2 kh[2];
 #pragma unroll
-                        for (int t = 0; t < 2; ++t)
+                        for (int t = 0; t < 2; ++t) {
 #pragma unroll
                             for (int kk = 0; kk < KK; ++kk)
                                 ka[t][kk] = *reinterpret_cast<const uint4*>(&kb[t * 16 + r][kk * 32 + kg * 8]);
+                            if constexpr (HEAD_HALF) kh[t] = *reinterpret_cast<const uint2*>(&kb[t * 16 + r][KK * 32 + kg * 4]);
+                        }
                         // V^T as the A operand of the second product, asked for now where registers allow: the
                         // answer comes while the first product and the exponentials run
                         constexpr bool EARLY_V = HD * CB <= 128;
@@ -389,6 +406,13 @@ void mfma_attention_kernel(
                                     st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ka[t][kk]),
                                                                                     __builtin_bit_cast(bf16x8_t, qf[c][kk]),
                                                                                     st[t], 0, 0, 0);
+                                if constexpr (HEAD_HALF) {
+                                    const uint4 ka_half = make_uint4(kh[t].x, kh[t].y, 0u, 0u);
+                                    const uint4 qf_half = make_uint4(qh[c].x, qh[c].y, 0u, 0u);
+                                    st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ka_half),
+                                                                                    __builtin_bit_cast(bf16x8_t, qf_half),
+                                                                                    st[t], 0, 0, 0);
+                                }
                             }
                         };
                         // 1. scores of every block, masked where the step lies at the edge of a block's key range (the
@@ -520,6 +544,7 @@ void mfma_attention_kernel(
 // end, so a whole key range needs no second kernel.  Each wavefront stages its own V tile: no
 // workgroup barrier inside the loop.
 #define DEC_WAVES (HEAD_DIM <= 128 ? 4 : 2)
+#if !HEAD_HALF
 
 // (Asked for four wavefronts a SIMD at head size 64, the compiler fits the kernel into 122 registers instead of 148
 // without spilling, and a compute unit holds four workgroups instead of three: 11.5 -> 10.8 us at batch 8.)
@@ -730,6 +755,8 @@ void mfma_decode_kernel(
     }
 }
 
+#endif   // !HEAD_HALF
+
 NI_EXPORT int ni_mfma_attention_head_dim() { return HEAD_DIM; }
 
 // Blocks of 16 rows that a wavefront can own at this head size.  Registers set the limit: two
@@ -815,6 +842,9 @@ NI_EXPORT int ni_mfma_token_attention(const void* q, int q_stride, const void* k
                                       const void* positions, void* out, void* part_o, void* part_ml, int T_tokens,
                                       int H, int KVH, int page_size, int window, float scale, int nsplit,
                                       hipStream_t stream) {
+#if HEAD_HALF
+    return -5;          // single tokens at this head size are the token-at-a-time kernel's
+#else
     if (T_tokens <= 0) return 0;
     if (H % KVH != 0 || page_size < 1 || nsplit < 1 || nsplit > 65535 || !(scale > 0.f)) return -1;
     if (nsplit > 1 && (!part_o || !part_ml)) return -2;
@@ -830,4 +860,5 @@ NI_EXPORT int ni_mfma_token_attention(const void* q, int q_stride, const void* k
         (const int32_t*)seq_of_token, (const int32_t*)positions, (bf16_t*)out, (float*)part_o, (float*)part_ml, H, KVH,
         page_size, page_shift, window, scale, nsplit);
     return NI_LAUNCH_RESULT();
+#endif
 }

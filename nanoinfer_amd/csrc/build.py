@@ -134,9 +134,9 @@ def attention_target(head_dim: int):
 
 
 def attention_mfma_target(head_dim: int):
-    if head_dim % 32 or not 32 <= head_dim <= 256:
+    if head_dim % 16 or not 16 <= head_dim <= 256:
         raise BuildError(f"head size {head_dim} is not supported by the matrix-core attention kernel: "
-                         "it must be a multiple of 32 between 32 and 256")
+                         "it must be a multiple of 16 between 16 and 256")
     return (f"ni_attention_mfma_hd{head_dim}", ["attention_mfma.hip"], {"HEAD_DIM": head_dim})
 
 
@@ -151,7 +151,7 @@ def build_all(head_dims: Iterable[int] = COMMON_HEAD_DIMS, force: bool = True, v
               jobs: Optional[int] = None) -> List[str]:
     """Compile every library (attention for the given head sizes)."""
     targets = [CORE, SAMPLING, SKINNY] + [attention_target(h) for h in head_dims] + \
-        [attention_mfma_target(h) for h in head_dims if h % 32 == 0] + \
+        [attention_mfma_target(h) for h in head_dims] + \
         [attention_mfma_f32_target(h) for h in head_dims]
     # the compiler runs in processes of its own: a few at a time (the longest, the skinny product, first)
     from concurrent.futures import ThreadPoolExecutor

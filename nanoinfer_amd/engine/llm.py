@@ -43,7 +43,9 @@ class Engine:
             runner = ModelRunner(model_dir, dtype=self.config.dtype, page_size=self.config.block_size,
                                  max_tokens=self.config.block_size * self.config.num_cache_blocks,
                                  max_requests=self.config.max_sequences, kv_cache_bytes=self.config.kv_cache_bytes,
-                                 max_step_tokens=min(self.config.prefill_chunk_size, self.config.max_num_batched_tokens))
+                                 max_step_tokens=min(self.config.prefill_chunk_size, self.config.max_num_batched_tokens),
+                                 one_weight_copy=self.config.one_weight_copy,
+                                 graph_memory_bytes=self.config.graph_memory_bytes)
         if sampler is None:
             from ..sampling.sampler import Sampler
             sampler = Sampler(runner.device)

@@ -169,6 +169,52 @@ class _RecordedStep:
     amax: torch.Tensor = None            # the same on the device, picked by the recording itself; a recorded decode step
                                          # writes it over its own token ids, where its next replay finds them without the host
     replayed: "torch.cuda.Event" = None  # the last replay has finished (and with it the copy into ``greedy``)
+    held_bytes: int = 0                  # device memory the recording holds (what the allocator's reserve grew by)
+
+
+class _Gpu:
+    """What recording a step needs from the device besides the model: kept apart so that the
+    runner's host side (tables, books, the order of runs while a step is recorded) can be driven
+    without a GPU by handing it other services."""
+
+    @staticmethod
+    def synchronize() -> None:
+        torch.cuda.synchronize()
+
+    @staticmethod
+    def pinned(t: torch.Tensor) -> torch.Tensor:
+        return t.pin_memory()
+
+    @staticmethod
+    def event():
+        return torch.cuda.Event()
+
+    @staticmethod
+    def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return K.argmax(logits, out=out)
+
+    @staticmethod
+    def reserved_bytes() -> int:
+        return int(torch.cuda.memory_reserved())
+
+    @staticmethod
+    def capture(run):
+        """Record what ``run()`` launches into a HIP graph (nothing is executed meanwhile); returns the
+        graph and what ``run`` returned.  Python's cycle collector is held off meanwhile: what it
+        finds may be an older runner with recordings of its own, and destroying a graph is one of
+        the calls that the runtime refuses while a stream is being captured (the refusal arrives in a
+        destructor and ends the process)."""
+        import gc
+        graph = torch.cuda.CUDAGraph()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                result = run()
+        finally:
+            if collecting:
+                gc.enable()
+        return graph, result
 
 
 class ModelRunner:
@@ -197,28 +243,30 @@ class ModelRunner:
     def __init__(self, model_dir: str, dtype: str = "bfloat16", page_size: int = 16, max_tokens: int = 4096,
                  max_requests: int = 64, device: Optional[torch.device] = None, use_graphs: bool = True,
                  warm_up: bool = True, max_step_tokens: Optional[int] = None, kv_cache_bytes: Optional[int] = None,
-                 graph_memory_bytes: Optional[int] = None):
+                 graph_memory_bytes: Optional[int] = None, one_weight_copy: bool = False):
         arch, config, spec = read_model_folder(model_dir)
         tensors = load_tensors(model_dir, spec)
         self._setup(spec, tensors, dtype, page_size, max_tokens, max_requests, device, use_graphs, warm_up,
-                    max_step_tokens, kv_cache_bytes, graph_memory_bytes, arch=arch, config=config)
+                    max_step_tokens, kv_cache_bytes, graph_memory_bytes, arch=arch, config=config,
+                    one_weight_copy=one_weight_copy)
 
     @classmethod
     def from_spec(cls, spec, tensors: Dict[str, torch.Tensor], dtype: str = "bfloat16", page_size: int = 16,
                   max_tokens: int = 4096, max_requests: int = 64, device: Optional[torch.device] = None,
                   use_graphs: bool = True, warm_up: bool = False, max_step_tokens: Optional[int] = None,
-                  kv_cache_bytes: Optional[int] = None, graph_memory_bytes: Optional[int] = None) -> "ModelRunner":
+                  kv_cache_bytes: Optional[int] = None, graph_memory_bytes: Optional[int] = None,
+                  one_weight_copy: bool = False) -> "ModelRunner":
         """A runner over a model given as data (a :class:`~nanoinfer_amd.config.spec.ModelSpec`) and its
         tensors by checkpoint name (CPU tensors), without a folder: the same model, cache manager and
         step function.  The tensors are checked against what the parts of the spec ask for."""
         from ..weights.loader import check_tensors
         self = cls.__new__(cls)
         self._setup(spec, check_tensors(spec, tensors), dtype, page_size, max_tokens, max_requests, device, use_graphs,
-                    warm_up, max_step_tokens, kv_cache_bytes, graph_memory_bytes)
+                    warm_up, max_step_tokens, kv_cache_bytes, graph_memory_bytes, one_weight_copy=one_weight_copy)
         return self
 
     def _setup(self, spec, tensors, dtype, page_size, max_tokens, max_requests, device, use_graphs, warm_up,
-               max_step_tokens, kv_cache_bytes, graph_memory_bytes, arch=None, config=None) -> None:
+               max_step_tokens, kv_cache_bytes, graph_memory_bytes, arch=None, config=None, one_weight_copy=False) -> None:
         self.device = device or K.require_gpu()
         torch_dtype = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
                        "float32": torch.float32, "fp32": torch.float32}.get(dtype)
@@ -226,7 +274,11 @@ class ModelRunner:
             raise ValueError(f"dtype {dtype!r} is not one of bfloat16, float32")
         self.dtype = torch_dtype
         self.arch, self.config, self.spec = arch, config, spec
-        self.rt = Runtime(torch_dtype, self.device)
+        # the products of decode steps stream a re-tiled copy of every layer matrix beside the rows that the
+        # library's product of prompt portions reads; ``one_weight_copy`` does without it (a slower decode step)
+        self.rt = Runtime(torch_dtype, self.device, tiled=not one_weight_copy)
+        el = 2 if torch_dtype == torch.bfloat16 else 4
+        self.checkpoint_bytes = sum(t.numel() * (el if t.dim() > 1 else 4) for t in tensors.values())
         self.model = Model(self.spec, tensors, self.rt)
         del tensors
         self.page_size = int(page_size)
@@ -251,6 +303,12 @@ class ModelRunner:
         if warm_up:
             self._warm_up()
 
+    def memory_report(self) -> Dict[str, int]:
+        """Bytes of device memory: the model's tensors, what the checkpoint is in the compute type (matrices; norm
+        weights in float32), the key and value pools, and what the recordings hold."""
+        return {"weights": self.rt.device_bytes(), "checkpoint": int(self.checkpoint_bytes),
+                "kv_pools": self.cache.pool_bytes(), "recordings": int(self._recorded_bytes)}
+
     def _warm_up(self) -> None:
         """One short prompt and one decode step of a request of the runner's own, run eagerly and given
         back: the code objects of the kernels and the matrix library's set-up are loaded while the model
@@ -264,16 +322,19 @@ class ModelRunner:
         try:
             self.step([StepEntry(me, [0] * n, [n - 1])])
             logits = self.step([StepEntry(me, [0], [0])])
-            K.argmax(logits)
-            torch.cuda.synchronize()
+            self.gpu.argmax(logits)
+            self.gpu.synchronize()
         finally:
             self.use_graphs = graphs
             self.release(me)
+
+    gpu = _Gpu
 
     def _init_graphs(self, use_graphs: bool) -> None:
         import os
         self.use_graphs = bool(use_graphs) and self.model.graph_safe() and not os.environ.get("NANOINFER_NO_GRAPHS")
         self._recorded: Dict[tuple, _RecordedStep] = {}      # in the order of their last use
+        self._recorded_bytes = 0                             # device memory the recordings hold, as measured when each was made
         self._unrecordable = set()
         self._portion_sights: Dict[tuple, int] = {}      # how often a prompt portion's shape has come without a recording
         self._staging = [(None, None)] * 3     # pinned host buffers for the tables of eager steps, and their uploads' events
@@ -294,11 +355,11 @@ class ModelRunner:
         if done is not None:
             done.synchronize()            # the upload that last used this buffer has read it
         if buf is None or buf.numel() < n:
-            buf = torch.empty(max(n, 4096, 2 * (buf.numel() if buf is not None else 0)), dtype=torch.int32).pin_memory()
+            buf = self.gpu.pinned(torch.empty(max(n, 4096, 2 * (buf.numel() if buf is not None else 0)), dtype=torch.int32))
         buf.numpy()[:n] = flat
         dev = torch.empty(n, dtype=torch.int32, device=self.device)
         dev.copy_(buf[:n], non_blocking=True)
-        done = done or torch.cuda.Event()
+        done = done or self.gpu.event()
         done.record()
         self._staging[i] = (buf, done)
         return dev
@@ -311,7 +372,7 @@ class ModelRunner:
             rec = held[1]
             rec.replayed.synchronize()
             return rec.greedy.tolist()
-        return K.argmax(logits).tolist()
+        return self.gpu.argmax(logits).tolist()
 
     # ---------------------------------------------------------------- bookkeeping
     def computed_tokens(self, request: Hashable) -> int:
@@ -365,20 +426,22 @@ class ModelRunner:
     def _describe(self, entries: List[StepEntry], ctx: StepContext, table_width: Optional[int] = None):
         """Fill the host side of ``ctx`` and return every integer table of the step as one flat
         int32 array, with the places of its parts: [token ids | positions | sequence of token |
-        logit rows | per group: slot mapping, block table]."""
+        logit rows | per group: slot mapping, block table | per sequence: first row, length,
+        context length, state slot]."""
         ps = self.page_size
         i32 = np.int32
         token_ids, positions, seq_of_token = [], [], []
         logit_rows: List[int] = []
         row = 0
+        host = ctx._host
         for si, e in enumerate(entries):
             n = len(e.tokens)
             done = self._done.get(e.request, 0)
-            ctx.requests.append(e.request)
-            ctx.q_start.append(row)
-            ctx.q_len.append(n)
-            ctx.context_len.append(done + n)
-            ctx.state_slot.append(self.cache.state_slot(e.request))
+            host["requests"].append(e.request)
+            host["q_start"].append(row)
+            host["q_len"].append(n)
+            host["context_len"].append(done + n)
+            host["state_slot"].append(self.cache.state_slot(e.request))
             token_ids.append(np.asarray(e.tokens, dtype=i32))
             positions.append(np.arange(done, done + n, dtype=i32))
             seq_of_token.append(np.full(n, si, dtype=i32))
@@ -387,8 +450,8 @@ class ModelRunner:
             row += n
         ctx.n_tokens = row
         ctx.n_seqs = len(entries)
-        ctx.max_context = max(ctx.context_len)
-        ctx.max_q_len = max(ctx.q_len)
+        ctx.max_context = max(host["context_len"])
+        ctx.max_q_len = max(host["q_len"])
         pieces = token_ids + positions + seq_of_token + [np.asarray(logit_rows, dtype=i32)]
         at = 3 * row + len(logit_rows)
         layout = []
@@ -409,7 +472,8 @@ class ModelRunner:
             pieces.append(block_table.reshape(-1))
             layout.append((off_slot, at, width))
             at += B * width
-        return np.concatenate(pieces), layout, len(logit_rows)
+        pieces.append(np.asarray(host["q_start"] + host["q_len"] + host["context_len"] + host["state_slot"], dtype=i32))
+        return np.concatenate(pieces), _Layout(layout, at), len(logit_rows)
 
     def _bind(self, ctx: StepContext, dev: torch.Tensor, layout, n_rows: int) -> None:
         T, B = ctx.n_tokens, ctx.n_seqs
@@ -419,7 +483,9 @@ class ModelRunner:
         ctx.logit_rows = dev[3 * T:3 * T + n_rows] if n_rows else None
         ctx.groups = [GroupView(block_table=dev[off_table:off_table + B * width].view(B, width),
                                 slot_mapping=dev[off_slot:off_slot + T], page_size=self.page_size)
-                      for (off_slot, off_table, width) in layout]
+                      for (off_slot, off_table, width) in layout.groups]
+        at = layout.seq
+        ctx.per_seq = SeqTables(dev[at:at + B], dev[at + B:at + 2 * B], dev[at + 2 * B:at + 3 * B], dev[at + 3 * B:at + 4 * B])
 
     def _layer_cache(self, ctx: StepContext):
         cache = self.cache
@@ -482,61 +548,97 @@ class ModelRunner:
         tiles = {}
         pieces, at = [flat], len(flat)
         for ts in sorted(tile_sizes):
-            rows = K.build_q_tiles(ctx.q_start, ctx.q_len, ctx.context_len, ts)
+            rows = K.build_q_tiles(ctx._host["q_start"], ctx._host["q_len"], ctx._host["context_len"], ts)
             tiles[ts] = (at, len(rows) // 4)        # where they start, how many
             pieces.append(np.asarray(rows, dtype=np.int32))
             at += len(rows)
         return (np.concatenate(pieces) if len(pieces) > 1 else flat), layout, n_rows, tiles
 
+    def _state_keeper(self):
+        """``rewind()``: puts the per-request state of every cache back to what it is now.  A step that
+        is being recorded runs several times (once the ordinary way first, then in trial replays beside
+        eager runs): keys and values land in the same places with the same values each time, but a
+        state that a part updates in place would move on with every run.  For a model whose parts are
+        all idempotent ``rewind`` does nothing."""
+        if not self.cache.state or self.model.idempotent():
+            return lambda: None
+        kept = {cid: t.clone() for cid, t in self.cache.state.items()}
+
+        def rewind() -> None:
+            for cid, t in kept.items():
+                self.cache.state[cid].copy_(t)
+        return rewind
+
     def _record(self, key, entries: List[StepEntry]) -> Optional[_RecordedStep]:
         kind, size, pages, bound, _ = key
+        gpu = self.gpu
         calls_before = K.library_calls()
+        rewind = self._state_keeper()
         # run the step once the ordinary way first: code objects get loaded and buffers sized outside
-        # the recording, and the model says which attention tiles it wants.  Running a step twice is
-        # harmless: it writes the same keys, values and logits again.
+        # the recording, and the model says which attention tiles it wants.  Keys, values and logits
+        # are simply written again by later runs; per-request state is put back (``rewind``).
         warm = StepContext(self.device, scratch_owner=self)
         flat_w, layout_w, rows_w = self._describe(entries, warm)
         self._bind(warm, torch.from_numpy(flat_w).to(self.device), layout_w, rows_w)
         warm_logits = self.model.forward(warm, self._layer_cache(warm))
         if warm_logits is not None:
-            K.argmax(warm_logits)
-        torch.cuda.synchronize()
+            gpu.argmax(warm_logits)
+        gpu.synchronize()
+        rewind()
+        held_before = gpu.reserved_bytes()
         ctx = StepContext(self.device, recording=True)
         flat, layout, n_rows, tiles = self._tables_of(entries, ctx, pages, warm.tile_sizes_asked)
         ctx.max_context = bound
-        staging = torch.from_numpy(flat).pin_memory()
-        meta = staging.to(self.device)
+        staging = gpu.pinned(torch.from_numpy(flat))
+        meta = staging.to(self.device, copy=True)
         self._bind(ctx, meta, layout, n_rows)
         for ts, (off, count) in tiles.items():
             ctx._q_tiles[ts] = meta[off:off + 4 * count].view(-1, 4)
-        greedy = torch.empty(max(n_rows, 1), dtype=torch.int32).pin_memory()
-        amax = None
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        ctx.seal()
+        greedy = gpu.pinned(torch.empty(max(n_rows, 1), dtype=torch.int32))
+
+        def run():
             logits = self.model.forward(ctx, self._layer_cache(ctx))
+            amax = None
             if logits is not None:
                 # greedy decoding needs only this: the recording picks the largest logit of every row, so
                 # that one copy brings the ids to the host.  A decode step writes them where its own token
                 # ids stand: replayed again for the same requests it decodes on, whether or not the host
                 # has looked at the tokens yet.
-                amax = K.argmax(logits, out=meta[0:size]) if kind == "d" else K.argmax(logits)
+                amax = gpu.argmax(logits, out=meta[0:size]) if kind == "d" else gpu.argmax(logits)
+            return logits, amax
+
+        graph, (logits, amax) = gpu.capture(run)
         if ctx.tile_sizes_asked - set(tiles):
             self._unrecordable.add(key)       # the recorded run asked for tiles the eager run did not: not the same step
             return None
-        if K.library_calls() != calls_before and not self._replays_faithfully(graph, logits, warm, meta, staging):
+        if K.library_calls() != calls_before and not self._replays_faithfully(graph, logits, warm, meta, staging, rewind):
             # a library routine ran inside and its recorded nodes do not reproduce the eager result
             # (some record memory-clearing nodes that misbehave on replay): this shape runs eagerly
             self._unrecordable.add(key)
             return None
         if kind == "d":
             meta.copy_(staging)               # the recording's trial replays have put their own tokens there
-        stagings = [staging] + [torch.empty_like(staging).pin_memory() for _ in range(self.STAGING_BUFFERS - 1)]
-        rec = _RecordedStep(graph, meta, stagings, logits, ctx, [torch.cuda.Event() for _ in stagings])
-        rec.greedy, rec.amax, rec.replayed, rec.tiles = greedy, amax, torch.cuda.Event(), tiles
+        stagings = [staging] + [gpu.pinned(torch.empty_like(staging)) for _ in range(self.STAGING_BUFFERS - 1)]
+        rec = _RecordedStep(graph, meta, stagings, logits, ctx, [gpu.event() for _ in stagings])
+        rec.greedy, rec.amax, rec.replayed, rec.tiles = greedy, amax, gpu.event(), tiles
+        rec.held_bytes = max(0, gpu.reserved_bytes() - held_before) + meta.numel() * 4
         for done in rec.copied:
             done.record()
         self._recorded[key] = rec
+        self._recorded_bytes += rec.held_bytes
         return rec
+
+    def _drop_recordings(self) -> None:
+        """Keep the recordings within their bounds: decode shapes by number, all of them together by the
+        device memory they hold; the ones used longest ago go first (the newest always stays)."""
+        decodes = [k for k in self._recorded if k[0] == "d"]
+        for old in decodes[:max(0, len(decodes) - self.GRAPH_MAX_DECODES)]:
+            self._recorded_bytes -= self._recorded.pop(old).held_bytes
+        for old in list(self._recorded)[:-1]:
+            if self._recorded_bytes <= self.GRAPH_MAX_BYTES:
+                break
+            self._recorded_bytes -= self._recorded.pop(old).held_bytes
 
     def _written_rows(self, ctx: StepContext) -> torch.Tensor:
         """The keys and values that a step has written, of every cache, gathered into one tensor:
@@ -551,26 +653,41 @@ class ModelRunner:
                 parts.append(g.vpools[cid][pages, :, offs].float().reshape(-1))
         return torch.cat(parts) if parts else torch.zeros(1, device=self.device)
 
+    def _state_rows(self, ctx: StepContext) -> List[torch.Tensor]:
+        """The per-request state of the step's sequences, of every cache that holds state."""
+        slots = ctx.per_seq.state_slot.long()
+        return [t[slots].float().reshape(-1) for _, t in sorted(self.cache.state.items())]
+
     def _replays_faithfully(self, graph, logits, warm: StepContext, meta: torch.Tensor, staging: torch.Tensor,
-                            rounds: int = 3) -> bool:
+                            rewind=lambda: None, rounds: int = 3) -> bool:
         """Replay a fresh recording several times, with the same step run eagerly and a
         synchronisation between the replays, and compare every replay with the eager run: the
-        logits, or for a step that returns none the keys and values it wrote.  A step may be run any
-        number of times: it writes the same keys and values again.  (Its tables are uploaded anew
-        each time: a recorded decode step overwrites its token ids with the ones it has chosen.)"""
+        logits, or for a step that returns none the keys and values it wrote; and the per-request
+        state it leaves, if the model has any.  Keys and values are simply written again by every
+        run; state is put back before each (``rewind``) and at the end.  (The tables are uploaded
+        anew each time: a recorded decode step overwrites its token ids with the ones it has chosen.)"""
+        gpu = self.gpu
+
+        def left_behind(out):
+            parts = [out.reshape(-1)] if out is not None else [self._written_rows(warm)]
+            return torch.cat(parts + self._state_rows(warm)).clone()
+
+        ok = True
         for _ in range(rounds):
             meta.copy_(staging)
+            rewind()
             graph.replay()
-            torch.cuda.synchronize()
-            got = logits.clone() if logits is not None else self._written_rows(warm)
-            want = self.model.forward(warm, self._layer_cache(warm))
-            if logits is None:
-                want = self._written_rows(warm)
-            torch.cuda.synchronize()
+            gpu.synchronize()
+            got = left_behind(logits)
+            rewind()
+            want = left_behind(self.model.forward(warm, self._layer_cache(warm)))
+            gpu.synchronize()
             scale = float(want.abs().max())
             if not bool(torch.isfinite(got).all()) or float((got - want).abs().max()) > 1e-3 * max(scale, 1e-30):
-                return False
-        return True
+                ok = False
+                break
+        rewind()
+        return ok
 
     def _replay(self, key, entries: List[StepEntry], tokens_from: Optional[_RecordedStep] = None,
                 history_row: Optional[int] = None, pick=None) -> bool:
@@ -589,10 +706,8 @@ class ModelRunner:
             rec = self._record(key, entries)
             if rec is None:
                 return False
-            decodes = [k for k in self._recorded if k[0] == "d"]
-            for old in decodes[:max(0, len(decodes) - self.GRAPH_MAX_DECODES)]:      # the ones used longest ago
-                del self._recorded[old]
-            # the recording itself ran nothing: fall through to the first replay
+            self._drop_recordings()
+            # the recording itself has left nothing behind: fall through to the first replay
         else:
             self._recorded[key] = rec          # moved to the end: the most recently used
         kind, B, width = key[0], key[1], key[2]
@@ -617,8 +732,10 @@ class ModelRunner:
                 st[b] = int(e.tokens[0])
                 st[B + b] = done
                 totals.append(done + 1)
+            off_ctx = rec.layout.seq + 2 * B
+            st[off_ctx:off_ctx + B] = totals
             for gi, g in enumerate(self.cache.groups):
-                off_slot, off_table, _ = rec.layout[gi]
+                off_slot, off_table, _ = rec.layout.groups[gi]
                 written = rec.pages_written[gi]
                 for b, e in enumerate(entries):
                     table = g.tables[e.request]
@@ -638,7 +755,7 @@ class ModelRunner:
             rec.layout = layout
             rec.order = order if kind == "d" else ()
             rec.pages_written = [[len(g.tables[e.request]) for e in entries] for g in self.cache.groups]
-            totals = ctx.context_len
+            totals = ctx._host["context_len"]
         if tokens_from is None:
             rec.meta.copy_(staging, non_blocking=True)
         else:
@@ -705,7 +822,7 @@ class ModelRunner:
                 flat, layout, n_rows = self._describe(entries, ctx)
                 self._bind(ctx, self._upload(flat), layout, n_rows)
                 logits = self.model.forward(ctx, self._layer_cache(ctx))
-                totals = ctx.context_len
+                totals = ctx._host["context_len"]
             close()
             self._book(entries, totals)
         for r in end:
@@ -733,8 +850,8 @@ class ModelRunner:
         last: Optional[_RecordedStep] = None
         self._greedy_of = None
         if self._history is None:
-            self._history = torch.zeros(self.HISTORY_ROWS, self.GRAPH_MAX_BATCH, dtype=torch.int32).pin_memory()
-            self._history_done = torch.cuda.Event()
+            self._history = self.gpu.pinned(torch.zeros(self.HISTORY_ROWS, self.GRAPH_MAX_BATCH, dtype=torch.int32))
+            self._history_done = self.gpu.event()
 
         def collect() -> None:
             nonlocal launched, tokens

@@ -101,6 +101,8 @@ class EngineConfig:
     max_model_len: Optional[int] = None  # longest request (prompt + generated); None: what model and pool allow
     max_decode_run: int = 8           # decode steps run back to back on one scheduling decision (1: never more than one)
     admission_headroom: int = 1       # pages left free for every request already running when another is admitted
+    one_weight_copy: bool = False     # keep every layer matrix once on the device (no re-tiled copy for decode steps: slower)
+    graph_memory_bytes: Optional[int] = None  # device memory that recorded steps may hold together (None: the runner's default)
     dtype: str = "bfloat16"
     seed: int = 0
 

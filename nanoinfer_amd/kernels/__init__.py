@@ -317,10 +317,8 @@ def mfma_token_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Te
 
 def mfma_attention_ok(dtype: torch.dtype, hd: int) -> bool:
     """Whether a matrix-core attention kernel for prompt portions takes this type and head size:
-    bfloat16 with head sizes in steps of 32, float32 in steps of 16."""
-    if dtype == torch.bfloat16:
-        return hd % 32 == 0 and 32 <= hd <= 256
-    return dtype == torch.float32 and hd % 16 == 0 and 16 <= hd <= 256
+    bfloat16 and float32, head sizes in steps of 16 up to 256."""
+    return dtype in (torch.bfloat16, torch.float32) and hd % 16 == 0 and 16 <= hd <= 256
 
 
 def mfma_token_ok(dtype: torch.dtype, hd: int) -> bool:
@@ -612,8 +610,17 @@ _library_calls = 0
 
 
 def library_calls() -> int:
-    """How many matrix products went to the library so far (a recorded step must contain none)."""
+    """How many library routines (matrix products) ran inside steps so far.  A step in whose recording
+    the count has moved is replayed against eager runs before the recording is used."""
     return _library_calls
+
+
+def note_library_call() -> None:
+    """For a part that calls a library routine of its own inside a step (a product, a reduction):
+    say so, so that a recording of the step is tried against eager runs before it is used (some
+    library routines record nodes that do not replay faithfully)."""
+    global _library_calls
+    _library_calls += 1
 
 
 

@@ -58,12 +58,25 @@ class Runtime:
     """Compute type and device of a model, and buffers that parts share (one rotation table for
     all layers with the same constants, one device copy of a tensor used twice)."""
 
-    def __init__(self, dtype: torch.dtype, device: torch.device):
+    def __init__(self, dtype: torch.dtype, device: torch.device, tiled: bool = True):
         if dtype not in (torch.float32, torch.bfloat16):
             raise ValueError(f"compute type {dtype} is not supported (float32 or bfloat16)")
         self.dtype = dtype
         self.device = device
+        # False: no layer matrix gets the second, re-tiled copy that the products of decode steps stream; they
+        # then read the rows as stored (slower), and device memory holds the checkpoint once
+        self.tiled = bool(tiled)
         self.shared: Dict[object, object] = {}
+
+    def device_bytes(self) -> int:
+        """Bytes of device memory that the model's tensors take (every shared buffer once)."""
+        seen, total = set(), 0
+        for value in self.shared.values():
+            for t in (value if isinstance(value, tuple) else (getattr(value, "rows", value), getattr(value, "tiles", None))):
+                if isinstance(t, torch.Tensor) and t.is_cuda and t.untyped_storage().data_ptr() not in seen:
+                    seen.add(t.untyped_storage().data_ptr())
+                    total += t.untyped_storage().nbytes()
+        return total
 
     def matrix(self, name: str, cpu: torch.Tensor) -> torch.Tensor:
         """A checkpoint matrix on the device in the compute type; the same name gives the same buffer."""
@@ -79,6 +92,7 @@ class Runtime:
         compute type (shared with :meth:`matrix`) plus, when ``tiled``, the copy that the skinny
         product of decoding streams."""
         from .. import kernels as K
+        tiled = tiled and self.tiled
         key = ("weight", name, self.dtype, tiled)
         w = self.shared.get(key)
         if w is None:

@@ -139,6 +139,19 @@ def load_tensors(folder: str, spec: ModelSpec) -> Dict[str, torch.Tensor]:
     return {n: _as_stored(f.tensor(n)) for n in want}
 
 
+def check_tensors(spec: ModelSpec, tensors: Dict[str, torch.Tensor], where: str = "the tensors given") -> Dict[str, torch.Tensor]:
+    """Tensors handed over directly (no file) checked as a checkpoint's are: every tensor the parts of
+    ``spec`` ask for is there with its shape and none besides, or ONE error names all that differ."""
+    want = expected_tensors(spec)
+    missing = sorted(n for n in want if n not in tensors)
+    unexpected = sorted(n for n in tensors if n not in want
+                        and not any(n.endswith(suffix) for suffix in spec.ignorable_suffixes))
+    wrong = sorted((n, want[n], tuple(tensors[n].shape)) for n in want if n in tensors and tuple(tensors[n].shape) != want[n])
+    if missing or unexpected or wrong:
+        raise WeightMismatchError(where, missing, unexpected, wrong)
+    return {n: _as_stored(tensors[n]) for n in want}
+
+
 def write_model_folder(folder: str, config_json: Dict[str, Any], tensors: Dict[str, torch.Tensor],
                        shards: int = 1) -> str:
     """``config.json`` and the checkpoint: one ``model.safetensors``, or ``shards`` files and their index."""

@@ -23,10 +23,11 @@ _folders = {}
 _root = None
 
 
-def model_folder(name: str, stored: str = "float32", seed: int = 7) -> str:
-    """A random-weights model folder for tiny configuration ``name`` (made once, in a temp folder)."""
+def model_folder(name: str, stored: str = "float32", seed: int = 7, **init) -> str:
+    """A random-weights model folder for tiny configuration ``name`` (made once, in a temp folder).
+    ``init`` replaces fields of the architecture's rule for drawing the weights (``overrides=...``)."""
     global _root
-    key = (name, stored, seed)
+    key = (name, stored, seed, repr(sorted(init.items())))
     if key not in _folders:
         import nanoinfer_amd  # noqa: F401
         from nanoinfer_amd.weights.loader import make_random_model
@@ -35,7 +36,8 @@ def model_folder(name: str, stored: str = "float32", seed: int = 7) -> str:
             _root = tempfile.mkdtemp(prefix="nanoinfer-tests-")
             import atexit
             atexit.register(shutil.rmtree, _root, ignore_errors=True)
-        _folders[key] = make_random_model(os.path.join(_root, f"{name}-{stored}-{seed}"), ALL[name], seed, dtype=stored)
+        _folders[key] = make_random_model(os.path.join(_root, f"{name}-{stored}-{seed}-{len(_folders)}"), ALL[name], seed,
+                                          dtype=stored, **init)
     return _folders[key]
 
 

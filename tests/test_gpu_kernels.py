@@ -330,7 +330,9 @@ def test_attention_block_table_longer_than_one_segment(K, kernel):
 # ---- the matrix-core kernel for prompt portions (bfloat16)
 
 @pytest.mark.parametrize("H,KVH,hd,ps", [(4, 2, 32, 8), (6, 1, 32, 8), (32, 8, 64, 16), (16, 2, 128, 16), (2, 2, 256, 16),
-                                         (3, 3, 96, 4), (32, 1, 64, 16), (5, 5, 64, 5), (12, 4, 64, 16)])
+                                         (3, 3, 96, 4), (32, 1, 64, 16), (5, 5, 64, 5), (12, 4, 64, 16),
+                                         # odd multiples of 16: the last 16 dims of a head go through a product of their own
+                                         (4, 2, 16, 16), (5, 5, 48, 5), (6, 2, 80, 16), (2, 1, 112, 16), (16, 1, 144, 8), (3, 3, 240, 16)])
 def test_mfma_attention_head_sizes_and_groups(K, H, KVH, hd, ps):
     # whole prompts, portions that start in the middle of a sequence, single tokens beside them, tile edges
     lens, q_lens = [1, 37, 130, 64, 200, 17], [1, 37, 2, 1, 77, 16]
@@ -447,9 +449,51 @@ def test_mfma_attention_window_and_far_key(K, blocks):
         assert not torch.isnan(out).any()
         assert rel(out, want) < KTOL["bfloat16"], window
     with pytest.raises(Exception):
-        K.attention_mfma_lib(48)
-    assert K.mfma_token_ok(torch.float32, 48) and not K.mfma_token_ok(torch.bfloat16, 48) and not K.mfma_attention_ok(torch.bfloat16, 48)
-    assert K.mfma_attention_ok(torch.float32, 48) and not K.mfma_attention_ok(torch.float32, 40)
+        K.attention_mfma_lib(40)
+    assert K.mfma_token_ok(torch.float32, 48) and not K.mfma_token_ok(torch.bfloat16, 48) and K.mfma_attention_ok(torch.bfloat16, 48)
+    assert K.mfma_attention_ok(torch.float32, 48) and not K.mfma_attention_ok(torch.float32, 40) and not K.mfma_attention_ok(torch.bfloat16, 40)
+    # the kernel for single tokens is not compiled for the odd multiples of 16: asked all the same, it refuses
+    with pytest.raises(K.KernelError):
+        K.mfma_token_attention(torch.zeros(1, 8 * 48, device="cuda", dtype=torch.bfloat16), *[None] * 6, 4, 2, 48, 1.0, None, 1)
+
+
+@pytest.mark.parametrize("hd,blocks", [(16, 1), (16, 2), (48, 1), (48, 2), (80, 1), (112, 1)])
+def test_mfma_attention_window_and_far_key_at_odd_multiples_of_16(K, hd, blocks):
+    """The bfloat16 kernel for prompt portions at head sizes 16, 48, 80 and 112: windows whose passed pages hold no
+    finite number, and one far key that takes all the weight of the last query (a key that differs from its
+    neighbours in its last 16 dims only would be lost by a kernel that forgot them: here every dim counts)."""
+    for window in (1, 7, 33, 100):
+        out, want, _ = paged_case(K, "bfloat16", 4, 2, hd, 8, [150, 9, 33], [150, 9, 2], window, window + hd, 1, kernel="mfma",
+                                  blocks=blocks)
+        assert not torch.isnan(out).any()
+        assert rel(out, want) < KTOL["bfloat16"], window
+    for key_at in (37, 16, 0, 31, 32, 698):
+        for n_q in (5, 90):
+            out, want, (qs, ks, vs) = paged_case(K, "bfloat16", 8, 2, hd, 16, [700], [n_q], None, 9 + hd, 1 + key_at % 4,
+                                                 boost=(0, key_at, 699, 6.0 if hd >= 48 else 10.0), kernel="mfma", blocks=blocks)
+            assert rel(out, want) < KTOL["bfloat16"]
+            got = out.double().cpu()[-1].reshape(8, hd)
+            expect = vs[0][key_at].double().repeat_interleave(4, 0)
+            assert float((got - expect).abs().max()) < 0.05, key_at
+    # the last 16 dims alone decide: two keys that agree everywhere else
+    g = torch.Generator().manual_seed(hd)
+    n, H, KVH = 64, 2, 1
+    k = torch.zeros(n, KVH, hd)
+    k[:, 0, hd - 16:] = torch.randn(n, 16, generator=g).to(torch.bfloat16).float()
+    v = torch.randn(n, KVH, hd, generator=g).to(torch.bfloat16).float()
+    q = torch.zeros(n, H, hd)
+    q[:, :, hd - 16:] = (k[:, :, hd - 16:] * 8).to(torch.bfloat16).float()
+    kpool, vpool = k.transpose(0, 1)[None].contiguous(), v.transpose(0, 1)[None].contiguous()       # one page of 64 slots
+    qkv = torch.zeros(n, (H + 2 * KVH) * hd)
+    qkv[:, :H * hd] = q.reshape(n, -1)
+    tile_tokens = K.mfma_tile_tokens(hd, H // KVH) * blocks
+    tiles = dev(torch.tensor(K.build_q_tiles([0], [n], [n], tile_tokens), dtype=torch.int32).view(-1, 4))
+    out = torch.empty(n, H * hd, device="cuda", dtype=torch.bfloat16)
+    K.mfma_attention(dev(qkv, torch.bfloat16), dev(kpool, torch.bfloat16), dev(vpool, torch.bfloat16),
+                     dev(torch.zeros(1, 1, dtype=torch.int32)), tiles, out, H, KVH, hd, 1.0 / math.sqrt(hd), None, 1, None, tile_tokens)
+    want = P.causal_attention(q, k, v, range(n)).reshape(n, H * hd)
+    assert rel(out, want) < KTOL["bfloat16"]
+    assert float((want - v.double().mean(0).reshape(1, hd).repeat(1, H)).abs().max()) > 0.3      # far from the plain mean of the values
 
 
 @pytest.mark.parametrize("blocks", [1, 2])
@@ -996,39 +1040,52 @@ def test_what_the_merging_prologue_refuses(K):
         K.skinny_gemm_merged(torch.zeros(100, device="cuda"), 4, 8, 32, 64, wt, torch.empty(8, 64, device="cuda", dtype=torch.bfloat16))
 
 
-def test_where_the_skinny_product_gives_way_to_the_library(K):
-    W = K.Weight(dev(torch.zeros(32, 8192, dtype=torch.bfloat16)))
-    assert K.skinny_wins(16, 8192, torch.bfloat16, W) and K.skinny_wins(32, 8192, torch.bfloat16, W)
-    assert not K.skinny_wins(33, 8192, torch.bfloat16, W) and K.skinny_wins(64, 4096, torch.bfloat16, W)
-    assert not K.skinny_wins(65, 2048, torch.bfloat16, W) and not K.skinny_wins(8, 2040, torch.bfloat16, W)
-    # with the next norm to add them, 40 rows of 8,192 go in eight shares of K instead
-    assert K.residual_epilogue_ok(40, 8192, torch.bfloat16, W) and K.skinny_ksplit(40, 8192, torch.bfloat16, W) == (8, 2)
-    assert K.skinny_ksplit(65, 8192, torch.bfloat16, W) == (1, 1)
-    # up to eight rows the next product normalises in its prologue, which adds two shares to its rows: two then
-    assert K.skinny_ksplit(8, 8192, torch.bfloat16, W) == (2, 1) and K.skinny_ksplit(9, 8192, torch.bfloat16, W) == (8, 1)
-    assert K.skinny_ksplit(8, 2048, torch.bfloat16, K.Weight(dev(torch.zeros(32, 2048), torch.bfloat16))) == (1, 1)
-    full = K.Weight(dev(torch.zeros(4096, 8192), torch.bfloat16))      # 256 tiles fill the chip uncut
-    assert K.skinny_ksplit(8, 8192, torch.bfloat16, full) == (1, 1) and K.residual_takes_addends(8, 8192, torch.bfloat16, full)
-    assert not K.residual_takes_addends(8, 8192, torch.bfloat16, W)     # goes in shares itself
-    Wf = K.Weight(dev(torch.zeros(32, 8192)))
-    assert K.residual_epilogue_ok(40, 8192, torch.float32, Wf) and K.skinny_ksplit(40, 8192, torch.float32, Wf) == (8, 2)
-    assert K.skinny_ksplit(8, 8192, torch.float32, Wf) == (2, 1)
-    assert K.skinny_ksplit(8, 4096, torch.float32, K.Weight(dev(torch.zeros(32, 4096)))) == (2, 1)
-    # float32 past 16 rows: only rows of up to 2,048 elements are streamed by the skinny product, the stacked gate/up
-    # matrix only up to 32 rows; only matrices of at most 128 tiles are cut
-    narrow, stacked = K.Weight(dev(torch.zeros(48, 2048))), K.Weight(dev(torch.zeros(8192, 2048)))
-    assert K.skinny_wins(64, 2048, torch.float32, narrow) and K.skinny_wins(32, 2048, torch.float32, stacked)
-    assert not K.skinny_wins(33, 2048, torch.float32, stacked) and not K.skinny_wins(17, 3072, torch.float32, K.Weight(dev(torch.zeros(48, 3072))))
-    assert K.skinny_wins(16, 3072, torch.float32, narrow)          # up to 16 rows always
-    wide = K.Weight(dev(torch.zeros(2064, 8192)))
-    assert K.skinny_ksplit(40, 8192, torch.float32, wide) == (1, 1) and K.skinny_ksplit(40, 8192, torch.bfloat16, wide)[0] > 1
-    assert K.qkv_rope_wins(64, 8192, torch.bfloat16) and K.qkv_rope_wins(64, 2048, torch.float32)
-    assert not K.qkv_rope_wins(8, 3072, torch.float32) and not K.qkv_rope_wins(17, 4096, torch.float32)
-    assert K.qkv_rope_wins(16, 4096, torch.float32)
-    plain = dev(torch.zeros(32, 8192))          # not re-tiled: past 16 rows the library's product, which adds into nothing
-    assert not K.residual_epilogue_ok(40, 8192, torch.float32, plain)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whichever_product_is_chosen_equals_the_plain_one(K, dtype):
+    """``K.linear`` and ``K.linear_swiglu`` choose between the skinny kernels (whole, or cut along K into
+    float32 shares) and the library by rules that were measured and may be measured again.  Whatever
+    they choose, for row counts and widths on both sides of every rule: the result is the plain product,
+    onto the residual stream as well as into a tensor of its own."""
+    g = torch.Generator().manual_seed(5)
+    dt = DT[dtype]
+    paths = set()
+    for N, Kd in ((32, 8192), (2048, 2048), (48, 3072), (4096, 4096), (40, 2040 if dtype == "float32" else 2032)):
+        w = (torch.randn(N, Kd, generator=g) / math.sqrt(Kd)).to(dt)
+        W = K.Weight(dev(w))
+        for M in (1, 8, 9, 16, 17, 32, 33, 40, 64, 65, 130):
+            x = torch.randn(M, Kd, generator=g).to(dt)
+            want = x.double() @ w.double().t()
+            calls = K.library_calls()
+            assert rel(K.linear(dev(x), W), want) < KTOL[dtype], (M, N, Kd)
+            paths.add("library" if K.library_calls() != calls else "skinny")
+            if K.residual_epilogue_ok(M, Kd, dt, W):
+                h0 = torch.randn(M, N, generator=g)
+                h = dev(h0.clone())
+                out = K.linear(dev(x), W, residual=h)
+                if out is None:
+                    total = h
+                    paths.add("residual")
+                else:       # float32 shares for the next norm to add
+                    assert out.dtype == torch.float32 and out.dim() == 3 and out.shape[0] == K.skinny_ksplit(M, Kd, dt, W)[0] > 1
+                    assert torch.equal(h.cpu(), h0)
+                    total = h + out.sum(0)
+                    paths.add("shares")
+                assert rel(total, h0.double() + want) < KTOL[dtype], (M, N, Kd)
+    for inter, Kd in ((8192, 2048), (136, 96)):
+        w = (torch.randn(2 * inter, Kd, generator=g) / math.sqrt(Kd)).to(dt)
+        W = K.Weight(dev(w))
+        for M in (8, 17, 32, 33, 64, 65):
+            x = torch.randn(M, Kd, generator=g).to(dt)
+            gu = x.double() @ w.double().t()
+            assert rel(K.linear_swiglu(dev(x), W), P.swiglu(gu[:, :inter], gu[:, inter:])) < KTOL[dtype], (M, inter, Kd)
+    assert paths == {"library", "skinny", "residual", "shares"}        # the cases did reach every way
+    # what no rule may change: more than 64 rows never go to the skinny kernels, and a matrix that is not
+    # re-tiled has no residual epilogue past 16 rows (the library's product adds into nothing)
+    assert not K.skinny_wins(65, 2048, dt, K.Weight(dev(torch.zeros(32, 2048)), tiled=True))
+    plain = dev(torch.zeros(32, 8192))
+    assert not K.residual_epilogue_ok(40, 8192, dt, plain)
     with pytest.raises(K.KernelError):
-        K.linear(dev(torch.zeros(40, 8192)), plain, residual=dev(torch.zeros(40, 32)))
+        K.linear(dev(torch.zeros(40, 8192)).to(dt), plain.to(dt), residual=dev(torch.zeros(40, 32)))
 
 
 def test_skinny_product_reference_vector(K):

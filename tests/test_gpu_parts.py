@@ -109,8 +109,10 @@ def tiny_spec(mixer_kinds, order, d=64, H=4, KVH=2, hd=16, I=96, V=128, window=N
         else:
             ffn = PartSpec(ffn_kinds[i], {"hidden_size": d, "intermediate_size": I, "experts": experts},
                            {"router": pre + "router", "w1": pre + "w1", "w2": pre + "w2"})
-        blocks.append(BlockSpec("prenorm", PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": pre + "n1"}), mixer,
-                                PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": pre + "n2"}), ffn))
+        blocks.append(BlockSpec("prenorm", {"mixer_norm": PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": pre + "n1"}),
+                                            "mixer": mixer,
+                                            "ffn_norm": PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": pre + "n2"}),
+                                            "ffn": ffn}))
     return ModelSpec(V, d, 256, PartSpec("table", {"vocab_size": V, "hidden_size": d}, {"weight": "emb"}), blocks,
                      [LayerRun(*o) for o in order], PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": "nf"}),
                      PartSpec("linear", {"vocab_size": V, "hidden_size": d}, {"weight": "emb"}))
@@ -123,28 +125,12 @@ def random_tensors(spec, seed):
             for n, s in expected_tensors(spec).items()}
 
 
-class SpecRunner:
-    """A ModelRunner over a spec and tensors given directly (no folder): the same Model, cache manager
-    and step function, reached through the constructor's pieces."""
-
-    def __new__(cls, spec, tensors, dtype, page_size=8, max_tokens=512, max_step_tokens=None):
-        from nanoinfer_amd.cache.manager import KVCacheManager
-        from nanoinfer_amd.engine.model import Model
-        from nanoinfer_amd.engine.runner import ModelRunner
-        r = ModelRunner.__new__(ModelRunner)
-        r.device = torch.device("cuda", 0)
-        r.dtype = DT[dtype]
-        r.spec = spec
-        r.rt = runtime(dtype)
-        r.model = Model(spec, tensors, r.rt)
-        r.page_size = page_size
-        r.max_step_tokens = max_step_tokens
-        r.cache = KVCacheManager(r.model.cache_needs(), page_size, max_tokens // page_size, 4, dtype=DT[dtype], device=r.device,
+def SpecRunner(spec, tensors, dtype, page_size=8, max_tokens=512, max_step_tokens=None):
+    """A runner over a spec and tensors given directly (no folder): the same model, cache manager and
+    step function, through the runner's own constructor for models given as data."""
+    from nanoinfer_amd.engine.runner import ModelRunner
+    return ModelRunner.from_spec(spec, tensors, dtype=dtype, page_size=page_size, max_tokens=max_tokens, max_requests=4,
                                  max_step_tokens=max_step_tokens)
-        r.vocab_size, r.max_positions, r.eos_token_ids = spec.vocab_size, r.model.max_positions, ()
-        r._done, r._scratch = {}, None
-        r._init_graphs(True)
-        return r
 
 
 def plain_spec_forward(spec, tensors, tokens, extra_mixers=None, extra_ffns=None, extra_positions=None):

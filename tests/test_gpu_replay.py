@@ -100,10 +100,11 @@ def max_live_tokens(steps, requests, page):
     return worst
 
 
-def run_in_process(folder, dtype, page, steps, max_tokens):
+def run_in_process(folder, dtype, page, steps, max_tokens, seen=None, **runner_options):
+    """Replay ``steps`` through a runner of its own; ``seen`` (a dict) is told which shapes were recorded."""
     from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
 
-    runner = ModelRunner(folder, dtype=dtype, page_size=page, max_tokens=max_tokens, max_requests=4)
+    runner = ModelRunner(folder, dtype=dtype, page_size=page, max_tokens=max_tokens, max_requests=4, **runner_options)
     got = {}
     given_back = set()      # pages that some finished request held
     reused = False
@@ -122,6 +123,9 @@ def run_in_process(folder, dtype, page, steps, max_tokens):
             runner.release(r)
     runner.cache.check()
     assert runner.cache.free_pages() == runner.cache.num_pages and not runner.cache.live_requests()
+    if seen is not None:
+        seen["recorded"], seen["unrecordable"] = list(runner._recorded), set(runner._unrecordable)
+        seen["memory"] = runner.memory_report()
     return got, reused
 
 
@@ -234,6 +238,25 @@ def test_first_tokens_of_a_sequence(name, dtype):
     steps = [([("g", list(toks[:1]), [0]), ("h", list(toks[:2]), [0, 1])], ["g", "h"])]
     got, _ = run_in_process(folder, dtype, PAGE[name], steps, 128)
     compare(got, {"g": toks[:1], "h": toks[:2]}, folder, dtype, "two short requests")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_copy_of_every_matrix_gives_the_same_logits(dtype):
+    """``one_weight_copy``: no layer matrix gets the re-tiled copy that the products of decode steps stream; they
+    read the rows as stored, and norms and residual sums run as kernels of their own.  Device memory then holds
+    the checkpoint once (by default nearly twice); the logits of every way of cutting stay the plain ones."""
+    name = "B"
+    folder, requests = model_folder(name), make_requests(name)
+    memory = {}
+    for one_copy in (True, False):
+        seen = {}
+        for steps in (tail_one_by_one(requests), mixed(requests, seed=4)):
+            got, _ = run_in_process(folder, dtype, PAGE[name], steps, max_live_tokens(steps, requests, PAGE[name]), seen=seen,
+                                    one_weight_copy=one_copy)
+            compare(got, requests, folder, dtype, f"{name}, one copy of the matrices: {one_copy}")
+        memory[one_copy] = seen["memory"]
+    assert memory[True]["weights"] <= 1.02 * memory[True]["checkpoint"] + (1 << 20)      # the rotation tables are the rest
+    assert memory[False]["weights"] >= 1.5 * memory[False]["checkpoint"]
 
 
 def test_stored_bfloat16_weights_give_the_same_logits_in_both_stores():
@@ -350,10 +373,14 @@ def test_recorded_steps_with_library_products_are_checked_before_use(verdict, mo
     the logits of every step equal those of a runner that records nothing."""
     from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
     folder = model_folder("A", stored="bfloat16")
-    asked = []
+    asked, said = [], []
+    check = ModelRunner._replays_faithfully
     if verdict != "as it comes":
         monkeypatch.setattr(ModelRunner, "_replays_faithfully",
                             lambda self, *a, **kw: (asked.append(1), verdict == "accepted")[1])
+    else:       # the check itself, looked over the shoulder
+        monkeypatch.setattr(ModelRunner, "_replays_faithfully",
+                            lambda self, *a, **kw: (asked.append(1), said.append(check(self, *a, **kw)), said[-1])[2])
     recorded = ModelRunner(folder, dtype="bfloat16", page_size=16, max_tokens=2048, max_requests=24)
     eager = ModelRunner(folder, dtype="bfloat16", page_size=16, max_tokens=2048, max_requests=24, use_graphs=False)
     n = 20
@@ -370,6 +397,22 @@ def test_recorded_steps_with_library_products_are_checked_before_use(verdict, mo
         assert float((a - b).abs().max()) <= 2e-3 * float(b.abs().max()), step
         toks = a.argmax(-1).tolist()
     assert len(recorded._recorded) + len(recorded._unrecordable) == 1
+    if verdict == "as it comes":
+        # asked once, and the shape went where the answer sent it; a shape that was accepted passes the same
+        # check again now, after the steps that have replayed it
+        assert asked == [1] and len(said) == 1
+        assert len(recorded._recorded) == (1 if said[0] else 0) and len(recorded._unrecordable) == (0 if said[0] else 1)
+        if said[0]:
+            from nanoinfer_amd.engine.runner import StepContext
+            (key, rec), = recorded._recorded.items()
+            entries = [StepEntry(i, [toks[i]], [0]) for i in range(n)]
+            recorded._check_and_reserve(entries)
+            warm = StepContext(recorded.device, scratch_owner=recorded)
+            flat, layout, rows = recorded._describe(entries, warm)
+            recorded._bind(warm, torch.from_numpy(flat).to(recorded.device), layout, rows)
+            staging = rec.stagings[0]
+            staging.numpy()[:] = recorded._tables_of(entries, StepContext(recorded.device), key[2], ())[0]
+            assert check(recorded, rec.graph, rec.logits, warm, rec.meta, staging)
     if verdict == "refused":
         assert asked == [1] and len(recorded._unrecordable) == 1 and not recorded._recorded      # asked once, never recorded again
     if verdict == "accepted":
@@ -603,3 +646,97 @@ def test_long_sequences_reach_the_larger_tiles_and_the_key_runs_of_prompt_attent
         assert by_tokens[512] == (4, 2 * small)
     else:
         assert by_tokens[4200][1] == small
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("name", ["E64", "E128"])
+def test_the_family_s_head_sizes_reach_the_larger_tiles_and_the_key_runs_through_the_engine(name, dtype, monkeypatch):
+    """Head sizes 64 (32 query heads on 8) and 128 (24 on 8) on one narrow layer: a prompt of 2,300 tokens
+    in one step (at head size 64 the tiles of two blocks a wavefront), a lone portion of 512 tokens
+    1,100 tokens into its sequence (two-block tiles with the keys cut into runs at head size 64), a
+    lone portion of 128 tokens there (few tiles: key runs at either head size), then tokens one by
+    one.  What the attention was asked for is noted, so that the test fails if these paths are no
+    longer the ones taken."""
+    from nanoinfer_amd import kernels as K
+    folder = model_folder(name)
+    cfg = ALL[name]
+    vocab, hd, group = cfg["vocab_size"], cfg["head_dim"], cfg["num_attention_heads"] // cfg["num_key_value_heads"]
+    asked, original = [], K.mfma_attention
+    monkeypatch.setattr(K, "mfma_attention", lambda *a, **kw: (asked.append((a[0].shape[0], a[11], a[13])), original(*a, **kw))[1])
+    small = K.mfma_tile_tokens(hd, group, dtype=torch.bfloat16 if dtype == "bfloat16" else torch.float32)
+    long_prompt = random_tokens(vocab, 2300, 51)
+    deep = random_tokens(vocab, 1100 + 512 + 128 + 20, 52)
+    steps = [([("long", list(long_prompt), [0, 1, 1023, 1024, 2047, 2048, 2299])], ["long"]),
+             ([("deep", list(deep[:1100]), [1099])], []),
+             ([("deep", list(deep[1100:1612]), [0, 255, 511])], []),
+             ([("deep", list(deep[1612:1740]), [0, 64, 127])], [])]
+    steps += [([("deep", [t], [0])], []) for t in deep[1740:]]
+    steps[-1] = (steps[-1][0], ["deep"])
+    got, _ = run_in_process(folder, dtype, 16, steps, 2304 + 64)
+    compare(got, {"long": long_prompt, "deep": deep}, folder, dtype, f"configuration {name}")
+    by_tokens = {t: (nsplit, tile) for t, nsplit, tile in asked}
+    if dtype == "bfloat16" and hd == 64:
+        assert by_tokens[2300] == (1, 2 * small) and by_tokens[512] == (4, 2 * small)
+    if dtype == "bfloat16":
+        assert by_tokens[128][0] > 1 and by_tokens[128][1] == small
+    else:
+        assert by_tokens[2300][1] == small
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_a_sequence_longer_than_one_segment_of_the_block_table(dtype):
+    """Configuration F (two heads on one, one layer) past 16,384 tokens at pages of 16: the block table
+    of the sequence no longer fits one segment of the table that the attention kernels keep in LDS.
+    The prompt goes in portions of 2,048, the last ones ending a little before the seam; then a
+    portion of 96 tokens across it, tokens one by one beyond it, and a portion of 40 further on.
+    Query and key matrices are drawn ten times larger than the others, so that a row's attention
+    rests on a handful of keys anywhere in the sequence and not on the mean of all of them."""
+    name = "F"
+    folder = model_folder(name, overrides=((".q_proj.weight", 0.0, 0.25), (".k_proj.weight", 0.0, 0.25)))
+    vocab = ALL[name]["vocab_size"]
+    n = 16384 + 200
+    toks = random_tokens(vocab, n, 61)
+    steps, at = [], 0
+    while at + 2048 <= 16384 - 64:
+        steps.append(([("s", list(toks[at:at + 2048]), [0, 2047])], []))
+        at += 2048
+    head = 16384 - 40 - at
+    steps.append(([("s", list(toks[at:at + head]), [head - 1])], []))           # up to 40 tokens before the seam
+    at += head
+    steps.append(([("s", list(toks[at:at + 96]), list(range(0, 96, 5)) + [95])], []))     # across it
+    at += 96
+    for t in toks[at:at + 24]:
+        steps.append(([("s", [t], [0])], []))                                        # single tokens beyond it
+    at += 24
+    steps.append(([("s", list(toks[at:at + 40]), list(range(40)))], []))
+    at += 40
+    for t in toks[at:]:
+        steps.append(([("s", [t], [0])], []))
+    steps[-1] = (steps[-1][0], ["s"])
+    got, _ = run_in_process(folder, dtype, 16, steps, n + 64)
+    assert max(p for _, p in got) == n - 1 and any(16300 < p < 16384 for _, p in got)
+    compare(got, {"s": toks}, folder, dtype, "past one table segment")
+    # the attention does rest on few keys: the largest softmax weight of a late row is far above 1 / context
+    config, tensors = P_read(folder)
+    assert peak_weight(config, tensors, toks, row=n - 1) > 50.0 / n
+
+
+def P_read(folder):
+    import plain_llama as P
+    return P.read_model_folder(folder)
+
+
+def peak_weight(config, tensors, toks, row):
+    """The largest softmax weight that head 0 of the (only) layer gives any key at ``row``."""
+    import math
+
+    import plain_llama as P
+    H, KVH, hd = config["num_attention_heads"], config["num_key_value_heads"], config["head_dim"]
+    T = len(toks)
+    x = P.rmsnorm(P.embedding(tensors["model.embed_tokens.weight"], toks), tensors["model.layers.0.input_layernorm.weight"],
+                  config["rms_norm_eps"])
+    sin, cos = P.rope_tables(range(T), P.rope_frequencies(hd, config["rope_theta"], config.get("rope_scaling")))
+    q = P.rope_interleaved(P.linear(x, P.permute_reverse(tensors["model.layers.0.self_attn.q_proj.weight"], H)).reshape(T, H, hd), sin, cos)
+    k = P.rope_interleaved(P.linear(x, P.permute_reverse(tensors["model.layers.0.self_attn.k_proj.weight"], KVH)).reshape(T, KVH, hd), sin, cos)
+    scores = (k[:row + 1, 0] @ q[row, 0]) / math.sqrt(hd)
+    return float(torch.softmax(scores, 0).max())

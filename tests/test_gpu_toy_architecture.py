@@ -56,14 +56,14 @@ def toy_spec(cfg: ToyConfig):
         pre = f"toy.{i}."
         position = PartSpec("toy_stored_rotation", {"rotary_dim": cfg.head_size, "max_positions": cfg.positions},
                             {"freqs": pre + "rotation"})
-        blocks.append(BlockSpec(
-            "prenorm", PartSpec("rmsnorm", {"size": d, "eps": cfg.eps}, {"weight": pre + "n1"}),
-            PartSpec("attention", {"hidden_size": d, "num_heads": cfg.heads, "num_kv_heads": cfg.kv_heads,
-                                   "head_dim": cfg.head_size, "scale": None, "window": None, "position": position},
-                     {"q": pre + "q", "k": pre + "k", "v": pre + "v", "o": pre + "o"}),
-            PartSpec("rmsnorm", {"size": d, "eps": cfg.eps}, {"weight": pre + "n2"}),
-            PartSpec("swiglu", {"hidden_size": d, "intermediate_size": cfg.inner},
-                     {"gate": pre + "g", "up": pre + "u", "down": pre + "d"})))
+        blocks.append(BlockSpec("prenorm", dict(
+            mixer_norm=PartSpec("rmsnorm", {"size": d, "eps": cfg.eps}, {"weight": pre + "n1"}),
+            mixer=PartSpec("attention", {"hidden_size": d, "num_heads": cfg.heads, "num_kv_heads": cfg.kv_heads,
+                                         "head_dim": cfg.head_size, "scale": None, "window": None, "position": position},
+                           {"q": pre + "q", "k": pre + "k", "v": pre + "v", "o": pre + "o"}),
+            ffn_norm=PartSpec("rmsnorm", {"size": d, "eps": cfg.eps}, {"weight": pre + "n2"}),
+            ffn=PartSpec("swiglu", {"hidden_size": d, "intermediate_size": cfg.inner},
+                         {"gate": pre + "g", "up": pre + "u", "down": pre + "d"}))))
     return ModelSpec(
         vocab_size=cfg.vocab, hidden_size=d, max_positions=cfg.positions,
         embedding=PartSpec("toy_learned_positions", {"vocab_size": cfg.vocab, "hidden_size": d, "positions": cfg.positions},

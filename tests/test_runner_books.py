@@ -8,7 +8,7 @@ import torch
 
 from nanoinfer_amd.cache.manager import KVCacheManager
 from nanoinfer_amd.engine.runner import ModelRunner, StepContext, StepEntry, StepError, _RecordedStep
-from nanoinfer_amd.parts.base import CacheNeed, KVNeed
+from nanoinfer_amd.parts.base import CacheNeed, KVNeed, StateNeed
 
 VOCAB = 97
 
@@ -36,7 +36,7 @@ class _Graph:
         rec = self.rec_of()
         r, B = self.runner, len(rec.order)
         meta = rec.meta
-        (off_slot, off_table, width) = rec.layout[0]
+        (off_slot, off_table, width) = rec.layout.groups[0]
         g = r.cache.groups[0]
         ps = r.page_size
         for b, request in enumerate(rec.order):
@@ -46,6 +46,8 @@ class _Graph:
             assert int(meta[off_slot + b]) == table[pos // ps] * ps + pos % ps
             row = meta[off_table + b * width: off_table + (b + 1) * width].tolist()
             assert row[:len(table)] == table and all(x == -1 for x in row[len(table):])
+            per_seq = meta[rec.layout.seq: rec.layout.seq + 4 * B].view(4, B)[:, b].tolist()
+            assert per_seq == [b, 1, pos + 1, r.cache.state_slot(request)], "the per-sequence table of the replay"
             meta[b] = next_token(int(meta[b]), pos)
         rec.logits.zero_()
         for b in range(B):
@@ -192,3 +194,128 @@ def test_decode_recordings_are_kept_up_to_a_limit_and_the_least_recently_used_go
         start(r, n, 100)
     run_wave(r, ("d", "e"), 100, [3, 4], steps=2, run=2)             # the first shape comes back: recorded again
     assert r.recordings_made[-1] == first and list(r._recorded) == [second, first]
+
+
+# ------------------------------------------------------------------ the real recording, over a model with state
+
+class _HostServices:
+    """The device services of the runner for a run without a GPU: nothing to wait for, ordinary memory,
+    and a "graph" that runs its step anew at every replay (as a HIP graph launches its kernels anew).
+    While a step is captured nothing is executed, as on the GPU: the model is told to give its buffers only."""
+
+    def __init__(self, model):
+        self.model = model
+
+    synchronize = staticmethod(lambda: None)
+    pinned = staticmethod(lambda t: t)
+    event = staticmethod(_Event)
+    reserved_bytes = staticmethod(lambda: 0)
+
+    @staticmethod
+    def argmax(logits, out=None):
+        ids = logits.argmax(dim=1).to(torch.int32)
+        if out is None:
+            return ids
+        out.copy_(ids)
+        return out
+
+    def capture(self, run):
+        self.model.dry = True
+        try:
+            result = run()
+        finally:
+            self.model.dry = False
+        return SimpleNamespace(replay=run), result
+
+
+class _CountingModel:
+    """Stands for a model with a mixer that updates a per-request state in place: every run of a step
+    adds one to the state of each of its sequences, and "chooses" the next token by the formula.  It
+    reads its step from the device tables only, and counts as a step with a library product inside,
+    so that a fresh recording is tried against eager runs before it is used."""
+
+    max_positions = 8192
+
+    def __init__(self, cache, idempotent_says):
+        self.cache, self.dry, self.says = cache, False, idempotent_says
+        self.buffers = {}
+
+    def graph_safe(self):
+        return True
+
+    def idempotent(self):
+        return self.says
+
+    def forward(self, ctx, layer_cache):
+        from nanoinfer_amd import kernels as K
+        B = ctx.n_seqs
+        logits = self.buffers.setdefault(id(ctx), torch.zeros(B, VOCAB))
+        K._library_calls += 1
+        if self.dry:
+            return logits
+        slots = ctx.per_seq.state_slot.long()
+        self.cache.state[0][slots] += 1.0
+        tokens = (ctx.token_ids[:B].long() * 31 + ctx.positions[:B].long() * 7 + 1) % VOCAB
+        logits.zero_()
+        logits[torch.arange(B), tokens] = 1.0
+        return logits
+
+
+def make_state_runner(idempotent_says):
+    r = object.__new__(ModelRunner)
+    r.device = torch.device("cpu")
+    r.page_size = 16
+    r.max_step_tokens = None
+    r.cache = KVCacheManager({0: CacheNeed(kv=KVNeed(1, 16), state=StateNeed((1,)))}, 16, 64, 8, device=r.device)
+    r.vocab_size = VOCAB
+    r.model = _CountingModel(r.cache, idempotent_says)
+    r.gpu = _HostServices(r.model)
+    r.max_positions = 8192
+    r._done = {}
+    r._scratch = None
+    r._init_graphs(True)
+    return r
+
+
+def test_a_state_advances_once_for_every_booked_step_also_while_steps_are_recorded():
+    """Recording a step runs it several times: once the ordinary way, then in trial replays beside eager
+    runs.  A model that says its step is not idempotent finds its per-request state put back in between,
+    so that after n booked steps the state has moved n times, whether a step was run eagerly, recorded
+    just then, or replayed; and the tokens are those of the formula."""
+    r = make_state_runner(idempotent_says=False)
+    names, first = ("a", "b", "c"), [3, 50, 7]
+    r.step([StepEntry(n, [1] * 5, []) for n in names])                  # prompts: an eager step
+    booked = 1
+    toks = list(first)
+    got = []
+    for _ in range(3):                                                  # single steps: the first one records
+        toks = r.greedy_tokens(r.step([StepEntry(n, [t], [0]) for n, t in zip(names, toks)]))
+        got.append(list(toks))
+        booked += 1
+        for n in names:
+            assert float(r.cache.state[0][r.cache.state_slot(n)]) == booked
+    assert len(r._recorded) == 1
+    rows = r.decode_run([StepEntry(n, [t], [0]) for n, t in zip(names, toks)], 6)     # and a run of replays
+    got.extend(rows)
+    booked += 6
+    assert got == expected(first, [5, 5, 5], 9)
+    for n in names:
+        assert float(r.cache.state[0][r.cache.state_slot(n)]) == booked
+
+
+def test_without_that_declaration_the_recording_would_move_the_state():
+    """The same model calling itself idempotent: the runs of the recording all land in the state.  (What
+    the test above guards against; here it shows that the stand-in can tell the difference.)"""
+    r = make_state_runner(idempotent_says=True)
+    r.step([StepEntry("a", [1] * 5, [])])
+    r.step([StepEntry("a", [3], [0])])
+    assert float(r.cache.state[0][r.cache.state_slot("a")]) > 2
+
+
+def test_host_lists_cannot_be_read_while_a_step_is_recorded():
+    ctx = StepContext(torch.device("cpu"), recording=True)
+    ctx._host["q_len"].append(1)
+    assert ctx.q_len == [1]
+    ctx.seal()
+    with pytest.raises(StepError, match="per_seq"):
+        ctx.q_len

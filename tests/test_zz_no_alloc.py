@@ -57,13 +57,24 @@ def _both(lib, n_tokens, context, nsplit, dtype, seed):
                                  nsplit, code, stream)
     assert err == 0
     torch.cuda.synchronize()
-    held = torch.cuda.memory_allocated()
-    err = lib.ni_token_attention_static(_ptr(q), H * HD, _ptr(kpool), _ptr(vpool), _ptr(table), table.shape[1],
-                                        _ptr(seq), _ptr(pos), _ptr(got), n_tokens, H, KVH, PAGE, 0, scale, nsplit,
-                                        code, stream)
-    assert err == 0
+
+    def static_call(out):
+        return lib.ni_token_attention_static(_ptr(q), H * HD, _ptr(kpool), _ptr(vpool), _ptr(table), table.shape[1],
+                                             _ptr(seq), _ptr(pos), _ptr(out), n_tokens, H, KVH, PAGE, 0, scale, nsplit,
+                                             code, stream)
+
+    # once first: the library's code object and its array come to the device with its first launch.  From
+    # then on a call must leave both the framework's allocator and the driver's count of free device
+    # memory where they were (the latter sees a hipMalloc that the former never hears of).
+    first = torch.full_like(want, float("nan"))
+    assert static_call(first) == 0
+    torch.cuda.synchronize()
+    held, free = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+    assert static_call(got) == 0
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == held
+    assert torch.cuda.mem_get_info()[0] == free, "device memory was taken or given back during the call"
+    assert torch.equal(first, got)
     assert bool(torch.isfinite(got.float()).all())
     assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
     return got

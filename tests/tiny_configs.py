@@ -45,6 +45,31 @@ TINY_D = {
 }
 
 
+# the head sizes and head counts of the family (64 with 32 heads on 8, 128 with 24 on 8) on one narrow layer,
+# with positions for prompts of thousands of tokens: what the attention kernels do at the sizes they meet in
+# use (tiles of two blocks, key runs), through the engine, at a cost the plain implementation can bear
+TINY_E64 = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 128, "num_hidden_layers": 1, "num_attention_heads": 32, "num_key_value_heads": 8,
+    "head_dim": 64, "intermediate_size": 144, "vocab_size": 211, "rms_norm_eps": 1e-5,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 1024},
+    "max_position_embeddings": 8192, "tie_word_embeddings": True, "hidden_act": "silu",
+}
+TINY_E128 = dict(TINY_E64, hidden_size=96, num_attention_heads=24, head_dim=128, intermediate_size=112, vocab_size=173)
+
+# two heads on one, a narrow layer, and positions past 16,384: a sequence whose block table no longer fits
+# one segment of the attention kernels' table in LDS (1,024 pages of 16 tokens)
+TINY_F = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 64, "num_hidden_layers": 1, "num_attention_heads": 2, "num_key_value_heads": 1,
+    "head_dim": 64, "intermediate_size": 80, "vocab_size": 61, "rms_norm_eps": 1e-5,
+    "rope_theta": 500000.0, "rope_scaling": None,
+    "max_position_embeddings": 17408, "tie_word_embeddings": True, "hidden_act": "silu",
+}
+
+
 def _family(hidden, heads, kv_heads, head_dim, inter, vocab, factor, tied):
     return {
         "architectures": ["LlamaForCausalLM"], "model_type": "llama",
@@ -66,4 +91,4 @@ FAMILY_3B = _family(3072, 24, 8, 128, 8192, 16033, 32.0, True)
 FAMILY_8B = _family(4096, 32, 8, 128, 14336, 16033, 8.0, False)
 
 TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-ALL = {**TINY, "D": TINY_D, "1B": FAMILY_1B, "3B": FAMILY_3B, "8B": FAMILY_8B}
+ALL = {**TINY, "D": TINY_D, "E64": TINY_E64, "E128": TINY_E128, "F": TINY_F, "1B": FAMILY_1B, "3B": FAMILY_3B, "8B": FAMILY_8B}
