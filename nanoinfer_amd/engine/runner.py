@@ -227,7 +227,7 @@ class ModelRunner:
     step then cost one call.
     """
 
-    GRAPH_MAX_BATCH = 64
+    GRAPH_MAX_BATCH = 256         # decode steps of more sequences run eagerly
     STAGING_BUFFERS = 4           # pinned copies of a recorded step's tables, used in turn
     HISTORY_ROWS = 16             # decode steps launched back to back before the host reads their tokens
     GRAPH_MIN_PORTION = 64        # a shorter prompt portion is not worth a recording

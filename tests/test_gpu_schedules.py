@@ -15,19 +15,23 @@ pytestmark = pytest.mark.gpu
 
 # ------------------------------------------------------------------ more than 64 sequences in a step
 
+@pytest.mark.parametrize("recorded_up_to", [64, 256])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_steps_of_more_than_64_sequences(dtype):
+def test_steps_of_more_than_64_sequences(dtype, recorded_up_to):
     """A hundred live requests of configuration B: their prompts in one step of a hundred portions, a
     pure decode step of a hundred tokens, a step of seventy tokens beside thirty portions of two, and
     the rest token by token, a hundred a step (the last steps shrink below 64 as requests end).
-    Every row of every step is compared with the plain implementation."""
+    Every row of every step is compared with the plain implementation.  More than 64 rows are past
+    what the skinny products take: such a decode step runs on the library's products and the kernels
+    between them, eagerly (``recorded_up_to`` 64) or as a recorded step."""
     from nanoinfer_amd.engine.runner import ModelRunner, StepEntry
     name, n = "B", 100
     folder = model_folder(name)
     vocab = ALL[name]["vocab_size"]
     requests = {i: random_tokens(vocab, 14 + (i * 7) % 29, 4000 + i) for i in range(n)}
     runner = ModelRunner(folder, dtype=dtype, page_size=8, max_tokens=n * 48, max_requests=128)
-    assert runner.GRAPH_MAX_BATCH == 64
+    assert runner.GRAPH_MAX_BATCH == 256
+    runner.GRAPH_MAX_BATCH = recorded_up_to
     done = {i: 0 for i in requests}
     got = {}
 
@@ -52,6 +56,7 @@ def test_steps_of_more_than_64_sequences(dtype):
         step(live)
     assert max(sizes) > 64 > min(sizes)                                # both sides of the recorded steps' limit
     assert not runner.cache.live_requests() and runner.cache.free_pages() == runner.cache.num_pages
+    assert (max(key[1] for key in runner._recorded if key[0] == "d") > 64) == (recorded_up_to > 64)
     for i, toks in requests.items():
         want = plain_logits(folder, tuple(toks), dtype)
         assert_close(torch.stack([got[(i, p)] for p in range(len(toks))]), want, dtype, f"request {i} of {n}")
