@@ -58,10 +58,12 @@ class Model:
     def cache_needs(self) -> Dict[int, CacheNeed]:
         return dict(self._needs)
 
-    def forward(self, ctx, layer_cache) -> Optional[torch.Tensor]:
+    def forward(self, ctx, layer_cache, logits_out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run the step described by ``ctx``; ``layer_cache(cache_id, writes)`` gives the
         :class:`LayerCache` of an entry of the order.  Returns float32 logits of ``ctx.logit_rows``
-        (None when no row is wanted; the caches are filled all the same)."""
+        (None when no row is wanted; the caches are filled all the same).  ``logits_out``: float32
+        [at least as many rows, vocab] whose first rows are to take the logits, for a head that
+        ``writes_into`` a given tensor (any other head returns a tensor of its own)."""
         h = self.embedding.forward(ctx.token_ids, ctx)
         pending = None
         for run in self.spec.order:
@@ -70,4 +72,6 @@ class Model:
         if ctx.logit_rows is None or ctx.logit_rows.shape[0] == 0:
             return None
         x = self.final_norm.forward(h, pending_for(self.final_norm, pending, self.rt.dtype), rows=ctx.logit_rows)
+        if logits_out is not None and getattr(self.head, "writes_into", False):
+            return self.head.forward(x, out=logits_out[:x.shape[0]])
         return self.head.forward(x)

@@ -232,7 +232,7 @@ class ModelRunner:
     HISTORY_ROWS = 16             # decode steps launched back to back before the host reads their tokens
     GRAPH_MIN_PORTION = 64        # a shorter prompt portion is not worth a recording
     GRAPH_MAX_PORTIONS = 24       # recordings of prompt portions kept (each holds its activations)
-    GRAPH_MAX_DECODES = 256       # recordings of decode steps kept (each holds its logits: batch x vocabulary floats);
+    GRAPH_MAX_DECODES = 1024      # recordings of decode steps kept (their logits go to one buffer that all share);
                                   # beyond that the one used longest ago is dropped and its shape recorded again if it returns
     GRAPH_PORTION_SIGHTS = 2      # a portion's shape is recorded when it comes this many times: recording costs
                                   # seven runs of the step and gains a few per cent of a run (a lone length never pays)
@@ -307,7 +307,8 @@ class ModelRunner:
         """Bytes of device memory: the model's tensors, what the checkpoint is in the compute type (matrices; norm
         weights in float32), the key and value pools, and what the recordings hold."""
         return {"weights": self.rt.device_bytes(), "checkpoint": int(self.checkpoint_bytes),
-                "kv_pools": self.cache.pool_bytes(), "recordings": int(self._recorded_bytes)}
+                "kv_pools": self.cache.pool_bytes(),
+                "recordings": int(self._recorded_bytes) + (0 if self._logits_buffer is None else self._logits_buffer.numel() * 4)}
 
     def _warm_up(self) -> None:
         """One short prompt and one decode step of a request of the runner's own, run eagerly and given
@@ -335,6 +336,7 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and self.model.graph_safe() and not os.environ.get("NANOINFER_NO_GRAPHS")
         self._recorded: Dict[tuple, _RecordedStep] = {}      # in the order of their last use
         self._recorded_bytes = 0                             # device memory the recordings hold, as measured when each was made
+        self._logits_buffer = None                           # float32 [GRAPH_MAX_BATCH, vocabulary]: where recorded steps leave their logits
         self._unrecordable = set()
         self._portion_sights: Dict[tuple, int] = {}      # how often a prompt portion's shape has come without a recording
         self._staging = [(None, None)] * 3     # pinned host buffers for the tables of eager steps, and their uploads' events
@@ -598,7 +600,9 @@ class ModelRunner:
         greedy = gpu.pinned(torch.empty(max(n_rows, 1), dtype=torch.int32))
 
         def run():
-            logits = self.model.forward(ctx, self._layer_cache(ctx))
+            # the logits of every recording go to one buffer of the runner's: a replay's are copied out before the
+            # next replay writes there, so a recording holds its activations only
+            logits = self.model.forward(ctx, self._layer_cache(ctx), logits_out=self._shared_logits())
             amax = None
             if logits is not None:
                 # greedy decoding needs only this: the recording picks the largest logit of every row, so
@@ -628,6 +632,11 @@ class ModelRunner:
         self._recorded[key] = rec
         self._recorded_bytes += rec.held_bytes
         return rec
+
+    def _shared_logits(self) -> torch.Tensor:
+        if self._logits_buffer is None:
+            self._logits_buffer = torch.empty(self.GRAPH_MAX_BATCH, self.vocab_size, dtype=torch.float32, device=self.device)
+        return self._logits_buffer
 
     def _drop_recordings(self) -> None:
         """Keep the recordings within their bounds: decode shapes by number, all of them together by the

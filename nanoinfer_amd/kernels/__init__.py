@@ -953,7 +953,7 @@ def skinny_qkv_rope(x, w_qkv, positions: torch.Tensor, cos: torch.Tensor,
 
 
 def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optional[torch.Tensor] = None,
-           pending: Optional[torch.Tensor] = None):
+           pending: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
     """``x . weight^T`` with ``weight`` stored [out, in].  Few rows go to the hand-written skinny
     product; many rows to the library (rocBLAS/hipBLASLt), where float32 inputs are multiplied in
     true float32 (the reduced-precision matrix modes of the library are switched off at import).
@@ -963,8 +963,11 @@ def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optiona
     nothing is returned, or (17 to 64 rows on a matrix of few tiles, :func:`skinny_ksplit`) it is
     returned as float32 addends [S, M, N] that the next norm adds to the stream.  ``pending``: addends
     that ``residual`` has not received yet and that the product brings in with it (where
-    :func:`residual_takes_addends` holds)."""
+    :func:`residual_takes_addends` holds).  ``out``: where a plain product is to be written ([M, N] of the
+    output type) instead of a new tensor."""
     rows, _ = _rows_and_tiles(weight)
+    if out is not None and (isinstance(x, NormedInput) or residual is not None):
+        raise KernelError("out= goes with a plain product")
     if isinstance(x, NormedInput):
         if not (residual is None):
             raise KernelError("a normed input and a residual output in one product are not compiled")
@@ -989,15 +992,19 @@ def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optiona
     if pending is not None:
         raise KernelError("pending addends go with a residual output")
     out_dtype = out_dtype or x.dtype
+    if out is not None:
+        _gpu(out, "out", out_dtype, (x.shape[0], rows.shape[0]))
     if skinny_wins(x.shape[0], x.shape[1], x.dtype, weight):
-        out = torch.empty(x.shape[0], rows.shape[0], dtype=out_dtype, device=x.device)
+        if out is None:
+            out = torch.empty(x.shape[0], rows.shape[0], dtype=out_dtype, device=x.device)
         return skinny_gemm(x, weight, out)
     rows_t = weight.rows_t if isinstance(weight, Weight) else rows.t()
     global _library_calls
     _library_calls += 1
     if out_dtype != x.dtype:
-        return torch.mm(x, rows_t, out_dtype=out_dtype)
-    return torch.mm(x, rows_t)
+        result = torch.mm(x, rows_t, out_dtype=out_dtype)
+        return result if out is None else out.copy_(result)
+    return torch.mm(x, rows_t) if out is None else torch.mm(x, rows_t, out=out)
 
 
 def linear_swiglu(x, weight_gate_up) -> torch.Tensor:

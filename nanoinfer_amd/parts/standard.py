@@ -457,6 +457,7 @@ class LinearHead(Part):
     shares its device buffer."""
 
     graph_safe = True
+    writes_into = True       # ``forward`` takes ``out=``: float32 [R, vocab] to write the logits into
 
     @classmethod
     def weight_requests(cls, spec):
@@ -468,5 +469,5 @@ class LinearHead(Part):
         # the large matrix is streamed as stored: re-tiling gains nothing at its size and would double it
         self.weight = rt.matrix(spec.weights["weight"], weights["weight"])
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return K.linear(x, self.weight, out_dtype=torch.float32)
+    def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return K.linear(x, self.weight, out_dtype=torch.float32, out=out)

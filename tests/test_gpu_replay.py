@@ -362,6 +362,11 @@ def test_recorded_decode_steps_equal_eager_ones(dtype):
         both([dec("g1")], end=["g1"] if done["g1"] == len(reqs["g1"]) - 1 else ())
     both([dec("g0"), dec("g2")])
     assert len(recorded._recorded) >= 3 and not eager._recorded
+    # every recording leaves its logits in the runner's one buffer (they are copied out after a replay), so a
+    # recording holds its activations only, not batch x vocabulary floats of its own
+    shared = recorded._logits_buffer
+    assert shared.shape == (recorded.GRAPH_MAX_BATCH, vocab)
+    assert all(rec.logits.data_ptr() == shared.data_ptr() for rec in recorded._recorded.values())
     compare(got, reqs, folder, dtype, "recorded decode")
 
 

@@ -246,7 +246,7 @@ class _CountingModel:
     def idempotent(self):
         return self.says
 
-    def forward(self, ctx, layer_cache):
+    def forward(self, ctx, layer_cache, logits_out=None):
         from nanoinfer_amd import kernels as K
         B = ctx.n_seqs
         logits = self.buffers.setdefault(id(ctx), torch.zeros(B, VOCAB))
