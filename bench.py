@@ -14,7 +14,9 @@ the host instead of a recorded step), the decode step's fraction of the HBM roof
 its name).  The default line (1B shape, bfloat16) adds further points, each timed over 96 steps:
 decode at batch 8 and 64 from contexts of 8,192 and 32,768 tokens; prompts of 8,192 and 32,768
 tokens (``prefill_8k``, ``prefill_32k``, in portions of 2,048); the same model in true float32
-(``decode_b8_fp32``, ``decode_b8_ctx8k_fp32``, ``prefill_fp32``: the reference's own precision); the
+(``decode_b8_fp32``, ``decode_b8_ctx8k_fp32``, ``prefill_fp32``: the reference's own precision);
+requests that draw instead of taking the largest logit (``decode_b8_temperature``,
+``decode_b8_top_k_top_p``); the
 3B shape in bfloat16 at batch 1, 8 and 64; requests through the scheduler (``serving_1b_bf16``,
 ``serving_1b_bf16_128req_half_pool`` with half the pages its 128 requests need, and
 ``serving_3b_fp32``: 64 concurrent requests of the 3B shape in float32, prompts uniform in
@@ -180,10 +182,12 @@ class Rig:
             runner.use_graphs = graphs
         return min(times[1:])
 
-    def decode(self, batch: int, context: int, steps: int, warmup: int):
+    def decode(self, batch: int, context: int, steps: int, warmup: int, sampling=None):
         """(seconds a step, mean context) of ``steps`` decode steps of ``batch`` requests whose
         prompts of ``context`` tokens are in the cache, as the engine decodes greedy requests: runs
-        of steps on one scheduling decision, the tokens passing from step to step on the device."""
+        of steps on one scheduling decision, the tokens passing from step to step on the device.
+        ``sampling`` (a ``SamplingParams`` without a repetition penalty): every request draws with
+        these options instead, as the engine runs such requests: the draw is part of the recorded step."""
         from nanoinfer_amd import kernels as K
         from nanoinfer_amd.engine.runner import StepEntry
 
@@ -198,10 +202,24 @@ class Rig:
             tokens.append(K.argmax(logits).tolist()[0])
         log(f"batch {batch}: prompts of {context} tokens are in the cache")
 
+        generated = [[] for _ in ids]
+        sampler = None
+        if sampling is not None:
+            from nanoinfer_amd.sampling.sampler import Sampler
+            sampler = Sampler(runner.device)
+
         def run(toks, n):
             while n > 0:
                 k = min(self.decode_run, n)
-                toks = runner.decode_run([StepEntry(i, [t], [0]) for i, t in zip(ids, toks)], k)[-1]
+                entries = [StepEntry(i, [t], [0]) for i, t in zip(ids, toks)]
+                if sampler is None:
+                    toks = runner.decode_run(entries, k)[-1]
+                else:
+                    rows = runner.decode_run(entries, k, draw=sampler.draw_tables([sampling] * batch, generated, k))
+                    for row in rows:
+                        for g, t in zip(generated, row):
+                            g.append(t)
+                    toks = rows[-1]
                 n -= k
             return toks
 
@@ -481,6 +499,16 @@ def main() -> int:
     if extras:
         for b in (1, 64):
             decode_point(rig, cfg, f"decode_b{b}", b, PROMPT_LEN, elem, f"{args.shape} {args.dtype}")
+
+        def sampled():
+            # requests that draw instead of taking the largest logit (the draw is part of the recorded step)
+            from nanoinfer_amd.sampling.params import SamplingParams
+            for name, params in (("decode_b8_temperature", SamplingParams(temperature=0.8, seed=1)),
+                                 ("decode_b8_top_k_top_p", SamplingParams(temperature=0.8, top_k=50, top_p=0.9, seed=1))):
+                sec, _ = rig.decode(args.batch, PROMPT_LEN, POINT_STEPS, POINT_WARMUP, sampling=params)
+                points[name.replace("b8", f"b{args.batch}")] = round(args.batch / sec, 1)
+                log(f"{name}: {sec * 1e3:.3f} ms a step")
+        attempt("sampled decoding", sampled)
     if further:
         def long_contexts():
             for n in LONG_CONTEXTS:

@@ -109,6 +109,38 @@ struct SampleArgs {
 #define SP_THREADS 256
 #define SP_WAVES (SP_THREADS / WAVE)
 
+// Sweeps over a slice of a row.  A load that waits for the one before it costs a round trip to memory
+// each, and a slice of some four thousand elements is sixteen of them for every thread: both sweeps ask
+// for eight elements before the first is used (an element past the end is read from the last one and
+// not used: no load is under a branch).
+//   sweep_strided: thread t takes lo + t, lo + t + SP_THREADS, ...
+//   sweep_run:     a thread's own run i0 .. i1 - 1, in order
+#define SP_AHEAD 8
+template <typename F>
+__device__ __forceinline__ void sweep_strided(const float* __restrict__ p, int lo, int hi, int tid, F&& f) {
+    for (int base = lo + tid; base < hi; base += SP_AHEAD * SP_THREADS) {
+        float v[SP_AHEAD];
+#pragma unroll
+        for (int k = 0; k < SP_AHEAD; ++k) v[k] = p[min(base + k * SP_THREADS, hi - 1)];
+#pragma unroll
+        for (int k = 0; k < SP_AHEAD; ++k) {
+            const int i = base + k * SP_THREADS;
+            if (i < hi) f(v[k], i);
+        }
+    }
+}
+template <typename F>
+__device__ __forceinline__ void sweep_run(const float* __restrict__ p, int i0, int i1, F&& f) {
+    for (int base = i0; base < i1; base += SP_AHEAD) {
+        float v[SP_AHEAD];
+#pragma unroll
+        for (int k = 0; k < SP_AHEAD; ++k) v[k] = p[min(base + k, i1 - 1)];
+#pragma unroll
+        for (int k = 0; k < SP_AHEAD; ++k)
+            if (base + k < i1) f(v[k], base + k);
+    }
+}
+
 struct Slice { int lo, hi; };
 __device__ __forceinline__ Slice slice_of(int part, int V, int P) {
     const int per = ((V + P - 1) / P + 3) & ~3;
@@ -130,10 +162,17 @@ __device__ int decide_level(const uint32_t* __restrict__ hist_row, int P, CT& re
     const int tid = threadIdx.x;                      // SP_THREADS == 256: thread t owns bin 255 - t
     const int bin = 255 - tid;
     CT mine = 0;
-    for (int p = 0; p < P; ++p) {
-        const uint32_t raw = hist_row[static_cast<size_t>(p) * 256 + bin];
-        if constexpr (std::is_same<CT, float>::value) mine += __uint_as_float(raw);
-        else mine += raw;
+    for (int p0 = 0; p0 < P; p0 += SP_AHEAD) {          // eight parts' bins asked for at a time, added in the order of the parts
+        uint32_t raw[SP_AHEAD];
+#pragma unroll
+        for (int k = 0; k < SP_AHEAD; ++k) raw[k] = hist_row[static_cast<size_t>(min(p0 + k, P - 1)) * 256 + bin];
+#pragma unroll
+        for (int k = 0; k < SP_AHEAD; ++k) {
+            if (p0 + k < P) {
+                if constexpr (std::is_same<CT, float>::value) mine += __uint_as_float(raw[k]);
+                else mine += raw[k];
+            }
+        }
     }
     // inclusive scan over the threads = sum of the bins from `bin` upwards
     CT incl = mine;
@@ -162,11 +201,14 @@ __device__ int decide_level(const uint32_t* __restrict__ hist_row, int P, CT& re
 }
 
 // Launch 1: penalty and temperature (src/op/kernels/cuda/sampling_kernel.cu:38-88), the slice's
-// largest value, and the counts of the first radix level for top-k.
-__global__ __launch_bounds__(SP_THREADS) void sample_prepare_kernel(SampleArgs a) {
+// largest value, and the counts of the first radix level for top-k.  `plain`: no row of the batch asks for
+// top-k or top-p, so every token is kept; the slice's sum of exp(w - its own maximum) is taken here as well,
+// and the draw, which scales it to the row's maximum, is the only other launch.
+__global__ __launch_bounds__(SP_THREADS) void sample_prepare_kernel(SampleArgs a, int plain) {
     __shared__ float s_val[SP_WAVES];
     __shared__ int s_idx[SP_WAVES];
     __shared__ uint32_t s_hist[256];
+    __shared__ float s_red[16];
     const int r = blockIdx.x, part = blockIdx.y, tid = threadIdx.x;
     const Slice sl = slice_of(part, a.V, a.P);
     const float* lrow = a.logits + static_cast<size_t>(r) * a.V;
@@ -174,10 +216,24 @@ __global__ __launch_bounds__(SP_THREADS) void sample_prepare_kernel(SampleArgs a
     const float T = a.temperature[r];
     const float inv_t = (T <= 0.f || T == 1.0f) ? 1.0f : 1.0f / T;
     const float pen = a.penalty[r];
-    for (int i = sl.lo + tid; i < sl.hi; i += SP_THREADS) w[i] = lrow[i] * inv_t;
+    const bool counts = row_top_k(a, r);
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
     s_hist[tid] = 0;
     __syncthreads();
-    if (pen != 1.0f) {
+    auto consider = [&](float v, int i) {
+        better(best, idx, v, i);
+        if (counts) atomicAdd(&s_hist[order_key(v) >> 24], 1u);
+    };
+    if (pen == 1.0f) {
+        sweep_strided(lrow, sl.lo, sl.hi, tid, [&](float l, int i) {
+            const float v = l * inv_t;
+            w[i] = v;
+            consider(v, i);
+        });
+    } else {
+        sweep_strided(lrow, sl.lo, sl.hi, tid, [&](float l, int i) { w[i] = l * inv_t; });
+        __syncthreads();
         const int first = a.pen_off[r];
         const int n_pen = a.pen_count ? a.pen_count[r] : a.pen_off[r + 1] - first;
         for (int j = tid; j < n_pen; j += SP_THREADS) {
@@ -189,14 +245,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_prepare_kernel(SampleArgs a
             }
         }
         __syncthreads();
-    }
-    const bool counts = row_top_k(a, r);
-    float best = -INFINITY;
-    int idx = 0x7fffffff;
-    for (int i = sl.lo + tid; i < sl.hi; i += SP_THREADS) {
-        const float v = w[i];
-        better(best, idx, v, i);
-        if (counts) atomicAdd(&s_hist[order_key(v) >> 24], 1u);
+        sweep_strided(w, sl.lo, sl.hi, tid, consider);
     }
 #pragma unroll
     for (int off = WAVE / 2; off > 0; off >>= 1) {
@@ -211,8 +260,17 @@ __global__ __launch_bounds__(SP_THREADS) void sample_prepare_kernel(SampleArgs a
         for (int wv = 1; wv < SP_WAVES; ++wv) better(best, idx, s_val[wv], s_idx[wv]);
         a.part_max[r * a.P + part] = best;
         a.part_arg[r * a.P + part] = idx;
+        s_val[0] = best;
     }
     if (counts) hist_of(a, 0, r, part)[tid] = s_hist[tid];
+    if (plain && row_samples(a, r)) {
+        __syncthreads();
+        const float m = s_val[0];           // the slice's largest value (every thread reads back what the workgroup wrote)
+        float z = 0.f;
+        sweep_strided(w, sl.lo, sl.hi, tid, [&](float v, int) { z += expf(v - m); });
+        z = block_sum(z, s_red);
+        if (tid == 0) a.part_z[r * a.P + part] = z;
+    }
 }
 
 // Launches 2 to 4 (level = 1, 2, 3): decide level `level` - 1 of the top-k descent from the counts the
@@ -236,10 +294,10 @@ __global__ __launch_bounds__(SP_THREADS) void sample_top_k_kernel(SampleArgs a, 
     __syncthreads();
     const Slice sl = slice_of(part, a.V, a.P);
     const float* w = a.work + static_cast<size_t>(r) * a.V;
-    for (int i = sl.lo + tid; i < sl.hi; i += SP_THREADS) {
-        const uint32_t key = order_key(w[i]);
+    sweep_strided(w, sl.lo, sl.hi, tid, [&](float v, int) {
+        const uint32_t key = order_key(v);
         if ((key & mask) == prefix) atomicAdd(&s_hist[(key >> shift) & 255u], 1u);
-    }
+    });
     __syncthreads();
     hist_of(a, level & 1, r, part)[tid] = s_hist[tid];
 }
@@ -253,10 +311,19 @@ __device__ uint32_t top_k_threshold(const SampleArgs& a, int r, uint32_t* s_scan
     return st[4] | static_cast<uint32_t>(b);
 }
 
+// The row's largest value from the slices' (at most 32 of them: one load each by the first threads, met in LDS).
+// Called by every thread of the workgroup.
 __device__ float row_max(const SampleArgs& a, int r) {
-    float M = a.part_max[r * a.P];
-    for (int p = 1; p < a.P; ++p) M = fmaxf(M, a.part_max[r * a.P + p]);
-    return M;
+    __shared__ float s_row_max;
+    const int tid = threadIdx.x;
+    if (tid < WAVE) {
+        float m = tid < a.P ? a.part_max[r * a.P + tid] : -INFINITY;
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, WAVE));
+        if (tid == 0) s_row_max = m;
+    }
+    __syncthreads();
+    return s_row_max;
 }
 
 // Launch 5: the softmax mass of the slice's kept tokens, and the sums of the first radix level for top-p.
@@ -276,14 +343,14 @@ __global__ __launch_bounds__(SP_THREADS) void sample_mass_kernel(SampleArgs a) {
     const Slice sl = slice_of(part, a.V, a.P);
     const float* w = a.work + static_cast<size_t>(r) * a.V;
     float z = 0.f;
-    for (int i = sl.lo + tid; i < sl.hi; i += SP_THREADS) {
-        const uint32_t key = order_key(w[i]);
+    sweep_strided(w, sl.lo, sl.hi, tid, [&](float v, int) {
+        const uint32_t key = order_key(v);
         if (key >= thr) {
-            const float e = expf(w[i] - M);
+            const float e = expf(v - M);
             z += e;
             if (sums) atomicAdd(&s_hist[key >> 24], e);
         }
-    }
+    });
     z = block_sum(z, s_red);
     if (tid == 0) a.part_z[r * a.P + part] = z;
     if (sums) hist_of(a, 0, r, part)[tid] = __float_as_uint(s_hist[tid]);
@@ -320,10 +387,10 @@ __global__ __launch_bounds__(SP_THREADS) void sample_top_p_kernel(SampleArgs a, 
     __syncthreads();
     const Slice sl = slice_of(part, a.V, a.P);
     const float* w = a.work + static_cast<size_t>(r) * a.V;
-    for (int i = sl.lo + tid; i < sl.hi; i += SP_THREADS) {
-        const uint32_t key = order_key(w[i]);
-        if (key >= thr && (key & mask) == prefix) atomicAdd(&s_hist[(key >> shift) & 255u], expf(w[i] - M));
-    }
+    sweep_strided(w, sl.lo, sl.hi, tid, [&](float v, int) {
+        const uint32_t key = order_key(v);
+        if (key >= thr && (key & mask) == prefix) atomicAdd(&s_hist[(key >> shift) & 255u], expf(v - M));
+    });
     __syncthreads();
     hist_of(a, level & 1, r, part)[tid] = __float_as_uint(s_hist[tid]);
 }
@@ -354,8 +421,9 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kept_kernel(SampleArgs a) {
     const int i0 = min(sl.hi, sl.lo + tid * seg), i1 = min(sl.hi, i0 + seg);
     float mine = 0.f;
     int last_kept = -1;
-    for (int i = i0; i < i1; ++i)
-        if (order_key(w[i]) >= thr) { mine += expf(w[i] - M); last_kept = i; }
+    sweep_run(w, i0, i1, [&](float v, int i) {
+        if (order_key(v) >= thr) { mine += expf(v - M); last_kept = i; }
+    });
     if (last_kept >= 0) atomicMax(&s_last, last_kept);
     const float mass = block_sum(mine, s_red);
     if (tid == 0) { a.part_mass[r * a.P + part] = mass; a.part_last[r * a.P + part] = s_last; }
@@ -363,14 +431,19 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kept_kernel(SampleArgs a) {
 
 // Launch 10, one workgroup per row: the slice in which the cumulative mass reaches u * total, and in
 // it the first token that does (src/op/kernels/cuda/sampling_kernel.cu:330-398); rows that do not
-// sample take the largest (penalised) logit.
-__global__ __launch_bounds__(SP_THREADS) void sample_draw_kernel(SampleArgs a) {
+// sample take the largest (penalised) logit.  `plain` (see the first launch): every token is kept, and a
+// slice's mass is its sum of exp(w - its own maximum) scaled to the row's maximum.
+__global__ __launch_bounds__(SP_THREADS) void sample_draw_kernel(SampleArgs a, int plain) {
     __shared__ float s_red[SP_WAVES];
     __shared__ int s_pick;
+    __shared__ float s_pmax[32], s_mass[32];
+    __shared__ int s_parg[32], s_plast[32];
     const int r = blockIdx.x, tid = threadIdx.x;
+    if (tid < a.P) { s_pmax[tid] = a.part_max[r * a.P + tid]; s_parg[tid] = a.part_arg[r * a.P + tid]; }
+    __syncthreads();
     float best_v = -INFINITY;
     int best = 0x7fffffff;
-    for (int p = 0; p < a.P; ++p) better(best_v, best, a.part_max[r * a.P + p], a.part_arg[r * a.P + p]);
+    for (int p = 0; p < a.P; ++p) better(best_v, best, s_pmax[p], s_parg[p]);
     if (best == 0x7fffffff) best = 0;        // a row of NaN or -inf: the first token
     // with pen_count the chosen token joins the row's penalised tokens: the next draw of a run sees it
     auto choose = [&](int token) {
@@ -386,10 +459,22 @@ __global__ __launch_bounds__(SP_THREADS) void sample_draw_kernel(SampleArgs a) {
         return;
     }
     const float M = best_v;
-    const uint32_t thr = a.state[static_cast<size_t>(r) * 16 + 7];
+    const uint32_t thr = plain ? 0u : a.state[static_cast<size_t>(r) * 16 + 7];
+    if (tid < a.P) {
+        if (plain) {
+            const Slice sp = slice_of(tid, a.V, a.P);
+            s_mass[tid] = sp.hi > sp.lo ? a.part_z[r * a.P + tid] * expf(s_pmax[tid] - M) : 0.f;
+            s_plast[tid] = sp.hi > sp.lo ? sp.hi - 1 : -1;
+        } else {
+            s_mass[tid] = a.part_mass[r * a.P + tid];
+            s_plast[tid] = a.part_last[r * a.P + tid];
+        }
+    }
+    if (tid == 0) s_pick = 0x7fffffff;
+    __syncthreads();
     float total = 0.f;
     int last = -1;
-    for (int p = 0; p < a.P; ++p) { total += a.part_mass[r * a.P + p]; last = max(last, a.part_last[r * a.P + p]); }
+    for (int p = 0; p < a.P; ++p) { total += s_mass[p]; last = max(last, s_plast[p]); }
     const float target = a.uniform[r] * total;
     // the first slice whose cumulative mass reaches the target
     int part = -1;
@@ -397,13 +482,11 @@ __global__ __launch_bounds__(SP_THREADS) void sample_draw_kernel(SampleArgs a) {
     {
         float cum = 0.f;
         for (int p = 0; p < a.P; ++p) {
-            const float m = a.part_mass[r * a.P + p];
+            const float m = s_mass[p];
             if (m > 0.f && cum < target && target <= cum + m) { part = p; before_part = cum; break; }
             cum += m;
         }
     }
-    if (tid == 0) s_pick = 0x7fffffff;
-    __syncthreads();
     if (part >= 0) {
         const Slice sl = slice_of(part, a.V, a.P);
         const float* w = a.work + static_cast<size_t>(r) * a.V;
@@ -411,8 +494,24 @@ __global__ __launch_bounds__(SP_THREADS) void sample_draw_kernel(SampleArgs a) {
         const int i0 = min(sl.hi, sl.lo + tid * seg), i1 = min(sl.hi, i0 + seg);
         float mine = 0.f;
         int last_kept = -1;
-        for (int i = i0; i < i1; ++i)
-            if (order_key(w[i]) >= thr) { mine += expf(w[i] - M); last_kept = i; }
+        // a thread's run is short where slices are (sixteen tokens at 128,256 of them in 32 slices): then the
+        // weights of its kept tokens stay in registers for the walk below (0 for a token that is not kept)
+        constexpr int KEEP = 16;
+        float kept_e[KEEP];
+#pragma unroll
+        for (int k = 0; k < KEEP; ++k) kept_e[k] = 0.f;
+        const bool in_registers = seg <= KEEP;
+        if (in_registers) {
+#pragma unroll
+            for (int k = 0; k < KEEP; ++k) {
+                const float v = w[min(i0 + k, sl.hi - 1)];
+                if (i0 + k < i1 && order_key(v) >= thr) { kept_e[k] = expf(v - M); mine += kept_e[k]; last_kept = i0 + k; }
+            }
+        } else {
+            sweep_run(w, i0, i1, [&](float v, int i) {
+                if (order_key(v) >= thr) { mine += expf(v - M); last_kept = i; }
+            });
+        }
         float incl = mine;
 #pragma unroll
         for (int off = 1; off < WAVE; off <<= 1) {
@@ -429,11 +528,23 @@ __global__ __launch_bounds__(SP_THREADS) void sample_draw_kernel(SampleArgs a) {
         if (mine > 0.f && excl < target && target <= incl) {
             float cum = excl;
             int pick = last_kept;
-            for (int i = i0; i < i1; ++i) {
-                if (order_key(w[i]) >= thr) {
-                    cum += expf(w[i] - M);
-                    if (cum >= target) { pick = i; break; }
+            bool found = false;
+            if (in_registers) {
+#pragma unroll
+                for (int k = 0; k < KEEP; ++k) {
+                    // (a kept token's weight may round to zero: it is passed over, as a token of no mass is never drawn)
+                    if (!found && kept_e[k] > 0.f) {
+                        cum += kept_e[k];
+                        if (cum >= target) { pick = i0 + k; found = true; }
+                    }
                 }
+            } else {
+                sweep_run(w, i0, i1, [&](float v, int i) {
+                    if (!found && order_key(v) >= thr) {
+                        cum += expf(v - M);
+                        if (cum >= target) { pick = i; found = true; }
+                    }
+                });
             }
             atomicMin(&s_pick, pick);
         }
@@ -442,7 +553,7 @@ __global__ __launch_bounds__(SP_THREADS) void sample_draw_kernel(SampleArgs a) {
     // rounding may leave the target a hair past every running sum: then the last kept token of the slice, or of the row
     if (tid == 0) {
         int pick = s_pick;
-        if (pick == 0x7fffffff && part >= 0) pick = a.part_last[r * a.P + part] >= 0 ? a.part_last[r * a.P + part] : 0x7fffffff;
+        if (pick == 0x7fffffff && part >= 0) pick = s_plast[part] >= 0 ? s_plast[part] : 0x7fffffff;
         choose(pick != 0x7fffffff ? pick : (last >= 0 ? last : best));
     }
 }
@@ -493,14 +604,19 @@ NI_EXPORT int ni_sample(const void* logits, void* work, const void* temperature,
     const dim3 grid(R, P);
     int err;
 #define SP_STEP(call) call; if ((err = NI_LAUNCH_RESULT()) != 0) return err;
-    SP_STEP((sample_prepare_kernel<<<grid, SP_THREADS, 0, stream>>>(a)))
-    if (uses_top_k)
-        for (int level = 1; level <= 3; ++level) { SP_STEP((sample_top_k_kernel<<<grid, SP_THREADS, 0, stream>>>(a, level))) }
-    SP_STEP((sample_mass_kernel<<<grid, SP_THREADS, 0, stream>>>(a)))
-    if (uses_top_p)
-        for (int level = 1; level <= 3; ++level) { SP_STEP((sample_top_p_kernel<<<grid, SP_THREADS, 0, stream>>>(a, level))) }
-    SP_STEP((sample_kept_kernel<<<grid, SP_THREADS, 0, stream>>>(a)))
-    SP_STEP((sample_draw_kernel<<<R, SP_THREADS, 0, stream>>>(a)))
+    // no row asks for top-k or top-p: every token is kept, and two launches do (the first also sums the slices' masses)
+    const int plain = !uses_top_k && !uses_top_p;
+    if (P > 32) return -1;
+    SP_STEP((sample_prepare_kernel<<<grid, SP_THREADS, 0, stream>>>(a, plain)))
+    if (!plain) {
+        if (uses_top_k)
+            for (int level = 1; level <= 3; ++level) { SP_STEP((sample_top_k_kernel<<<grid, SP_THREADS, 0, stream>>>(a, level))) }
+        SP_STEP((sample_mass_kernel<<<grid, SP_THREADS, 0, stream>>>(a)))
+        if (uses_top_p)
+            for (int level = 1; level <= 3; ++level) { SP_STEP((sample_top_p_kernel<<<grid, SP_THREADS, 0, stream>>>(a, level))) }
+        SP_STEP((sample_kept_kernel<<<grid, SP_THREADS, 0, stream>>>(a)))
+    }
+    SP_STEP((sample_draw_kernel<<<R, SP_THREADS, 0, stream>>>(a, plain)))
 #undef SP_STEP
     return 0;
 }

@@ -138,6 +138,11 @@ class Engine:
         requests = [item.request for item in batch.items]
         if all(r.params.use_greedy() and not r.params.use_repetition_penalty() for r in requests):
             chosen = self.runner.decode_run(entries, run)
+        elif (getattr(self.runner, "takes_draw_tables", False) and hasattr(self.sampler, "draw_tables")
+              and not any(r.params.use_repetition_penalty() for r in requests)):
+            # the draw is part of the recorded step: nothing is launched between a step and the next
+            tables = self.sampler.draw_tables([r.params for r in requests], [r.generated for r in requests], run)
+            chosen = self.runner.decode_run(entries, run, draw=tables)
         else:
             plan = self.sampler.plan([r.params for r in requests], [r.generated for r in requests], run)
             chosen = self.runner.decode_run(entries, run, pick=plan.launch)

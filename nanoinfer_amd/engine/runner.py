@@ -58,6 +58,16 @@ class SeqTables:
 
 
 @dataclass
+class DrawView:
+    """The options of a step's draw on the device, one entry per row in batch order."""
+
+    temperature: torch.Tensor     # float32 [B]
+    top_p: torch.Tensor           # float32 [B]
+    uniform: torch.Tensor         # float32 [B]: the number each row's draw is taken with
+    top_k: torch.Tensor           # int32 [B]
+
+
+@dataclass
 class _Layout:
     """Where the parts of a step's flat integer table lie: per cache group (offset of the slot
     mapping, offset of the block table, table width), and the offset of the per-sequence table
@@ -65,6 +75,7 @@ class _Layout:
 
     groups: list
     seq: int
+    draw: Optional[int] = None      # offset of the draw's table (temperature, top_p, uniform as float bits, top_k: B each), if the step has one
 
 
 _HOST_LISTS = ("requests", "q_start", "q_len", "context_len", "state_slot")
@@ -94,6 +105,7 @@ class StepContext:
         self.seq_of_token: torch.Tensor = None
         self.logit_rows: Optional[torch.Tensor] = None
         self.per_seq: Optional[SeqTables] = None
+        self.draw: Optional[DrawView] = None
         self.groups: List[GroupView] = []
         self.recording = recording
         self._scratch_owner = scratch_owner
@@ -196,6 +208,14 @@ class _Gpu:
     @staticmethod
     def reserved_bytes() -> int:
         return int(torch.cuda.memory_reserved())
+
+    @staticmethod
+    def draw(logits, work, view: "DrawView", ones, zeros, out, uses_top_k: bool, uses_top_p: bool) -> torch.Tensor:
+        """One token per row of ``logits`` into ``out`` by the sampling kernels, without a repetition penalty
+        (``ones``: a penalty of 1 per row; ``zeros``: the empty lists of penalised tokens)."""
+        R = logits.shape[0]
+        return K.sample(logits, work, view.temperature, view.top_k, view.top_p, ones[:R], zeros[:1], zeros[:R + 1],
+                        view.uniform, out, uses_top_k=uses_top_k, uses_top_p=uses_top_p)
 
     @staticmethod
     def capture(run):
@@ -337,6 +357,8 @@ class ModelRunner:
         self._recorded: Dict[tuple, _RecordedStep] = {}      # in the order of their last use
         self._recorded_bytes = 0                             # device memory the recordings hold, as measured when each was made
         self._logits_buffer = None                           # float32 [GRAPH_MAX_BATCH, vocabulary]: where recorded steps leave their logits
+        self._work_buffer = None
+        self._draw_consts = None
         self._unrecordable = set()
         self._portion_sights: Dict[tuple, int] = {}      # how often a prompt portion's shape has come without a recording
         self._staging = [(None, None)] * 3     # pinned host buffers for the tables of eager steps, and their uploads' events
@@ -425,11 +447,11 @@ class ModelRunner:
             raise OutOfPages(f"the step needs more pages or state slots than are free "
                              f"({self.cache.min_free_pages()} pages, {self.cache.slots.num_free} slots free)")
 
-    def _describe(self, entries: List[StepEntry], ctx: StepContext, table_width: Optional[int] = None):
+    def _describe(self, entries: List[StepEntry], ctx: StepContext, table_width: Optional[int] = None, draw_rows=None):
         """Fill the host side of ``ctx`` and return every integer table of the step as one flat
         int32 array, with the places of its parts: [token ids | positions | sequence of token |
         logit rows | per group: slot mapping, block table | per sequence: first row, length,
-        context length, state slot]."""
+        context length, state slot | the draw's table, if ``draw_rows`` (int32 [4 B]) is given]."""
         ps = self.page_size
         i32 = np.int32
         token_ids, positions, seq_of_token = [], [], []
@@ -475,7 +497,13 @@ class ModelRunner:
             layout.append((off_slot, at, width))
             at += B * width
         pieces.append(np.asarray(host["q_start"] + host["q_len"] + host["context_len"] + host["state_slot"], dtype=i32))
-        return np.concatenate(pieces), _Layout(layout, at), len(logit_rows)
+        off_draw = None
+        if draw_rows is not None:
+            if len(draw_rows) != 4 * B:
+                raise StepError(f"a draw's table has four entries a sequence: {len(draw_rows)} for {B} sequences")
+            off_draw = at + 4 * B
+            pieces.append(np.asarray(draw_rows, dtype=i32))
+        return np.concatenate(pieces), _Layout(layout, at, off_draw), len(logit_rows)
 
     def _bind(self, ctx: StepContext, dev: torch.Tensor, layout, n_rows: int) -> None:
         T, B = ctx.n_tokens, ctx.n_seqs
@@ -488,6 +516,10 @@ class ModelRunner:
                       for (off_slot, off_table, width) in layout.groups]
         at = layout.seq
         ctx.per_seq = SeqTables(dev[at:at + B], dev[at + B:at + 2 * B], dev[at + 2 * B:at + 3 * B], dev[at + 3 * B:at + 4 * B])
+        if layout.draw is not None:
+            at = layout.draw
+            as_float = dev[at:at + 3 * B].view(torch.float32)
+            ctx.draw = DrawView(as_float[0:B], as_float[B:2 * B], as_float[2 * B:3 * B], dev[at + 3 * B:at + 4 * B])
 
     def _layer_cache(self, ctx: StepContext):
         cache = self.cache
@@ -509,10 +541,11 @@ class ModelRunner:
         return get
 
     # ---------------------------------------------------------------- recorded decode steps
-    def _graph_shape(self, entries: List[StepEntry]):
+    def _graph_shape(self, entries: List[StepEntry], draw=None):
         """Key of the recorded step that can run these entries, or None when they must run eagerly.
-        Two kinds are recorded: single tokens only, each wanting its logits (``("d", batch, ...)``),
-        and one prompt portion alone that wants nothing or the logits of its last token
+        Two kinds are recorded: single tokens only, each wanting its logits (``("d", batch, ...)``; with
+        ``draw``, the (uses top-k, uses top-p) of a draw that the step makes itself, ``("s", batch, ...,
+        draw)``), and one prompt portion alone that wants nothing or the logits of its last token
         (``("p", tokens, ..., wanted rows)``).  Table width and context bound are rounded up to
         powers of two so that few recordings serve a growing context."""
         if not self.use_graphs or not 0 < len(entries) <= self.GRAPH_MAX_BATCH:
@@ -530,6 +563,8 @@ class ModelRunner:
                 return None
             longest = max(self._done.get(e.request, 0) for e in entries) + 1
             kind, size, rows = "d", len(entries), len(entries)
+            if draw is not None:
+                kind, rows = "s", (bool(draw[0]), bool(draw[1]))
         pages = max(16, 1 << (self.cache.pages_for(longest) - 1).bit_length())
         bound = max(256, 1 << (longest - 1).bit_length())
         key = (kind, size, pages, bound, rows)
@@ -543,10 +578,10 @@ class ModelRunner:
                 return None
         return key
 
-    def _tables_of(self, entries: List[StepEntry], ctx: StepContext, width: int, tile_sizes):
+    def _tables_of(self, entries: List[StepEntry], ctx: StepContext, width: int, tile_sizes, draw_rows=None):
         """Every integer table of a recorded step as one flat list: those of :meth:`_describe`, then
         the attention tiles of each tile size the model asked for."""
-        flat, layout, n_rows = self._describe(entries, ctx, table_width=width)
+        flat, layout, n_rows = self._describe(entries, ctx, table_width=width, draw_rows=draw_rows)
         tiles = {}
         pieces, at = [flat], len(flat)
         for ts in sorted(tile_sizes):
@@ -571,25 +606,29 @@ class ModelRunner:
                 self.cache.state[cid].copy_(t)
         return rewind
 
-    def _record(self, key, entries: List[StepEntry]) -> Optional[_RecordedStep]:
-        kind, size, pages, bound, _ = key
+    def _record(self, key, entries: List[StepEntry], draw_rows=None) -> Optional[_RecordedStep]:
+        kind, size, pages, bound, flags = key
         gpu = self.gpu
+        decode = kind in ("d", "s")
         calls_before = K.library_calls()
         rewind = self._state_keeper()
         # run the step once the ordinary way first: code objects get loaded and buffers sized outside
         # the recording, and the model says which attention tiles it wants.  Keys, values and logits
         # are simply written again by later runs; per-request state is put back (``rewind``).
         warm = StepContext(self.device, scratch_owner=self)
-        flat_w, layout_w, rows_w = self._describe(entries, warm)
+        flat_w, layout_w, rows_w = self._describe(entries, warm, draw_rows=draw_rows)
         self._bind(warm, torch.from_numpy(flat_w).to(self.device), layout_w, rows_w)
         warm_logits = self.model.forward(warm, self._layer_cache(warm))
         if warm_logits is not None:
             gpu.argmax(warm_logits)
+            if kind == "s":
+                gpu.draw(warm_logits, self._shared_work()[:size], warm.draw, *self._draw_constants(),
+                         torch.empty(size, dtype=torch.int32, device=self.device), *flags)
         gpu.synchronize()
         rewind()
         held_before = gpu.reserved_bytes()
         ctx = StepContext(self.device, recording=True)
-        flat, layout, n_rows, tiles = self._tables_of(entries, ctx, pages, warm.tile_sizes_asked)
+        flat, layout, n_rows, tiles = self._tables_of(entries, ctx, pages, warm.tile_sizes_asked, draw_rows=draw_rows)
         ctx.max_context = bound
         staging = gpu.pinned(torch.from_numpy(flat))
         meta = staging.to(self.device, copy=True)
@@ -609,7 +648,12 @@ class ModelRunner:
                 # that one copy brings the ids to the host.  A decode step writes them where its own token
                 # ids stand: replayed again for the same requests it decodes on, whether or not the host
                 # has looked at the tokens yet.
-                amax = gpu.argmax(logits, out=meta[0:size]) if kind == "d" else gpu.argmax(logits)
+                if kind == "s":
+                    # the step draws by itself: temperature, top-k, top-p and the uniform number of every row come
+                    # with the step's tables, and the token drawn lands where the largest logit's would
+                    amax = gpu.draw(logits, self._shared_work()[:size], ctx.draw, *self._draw_constants(), meta[0:size], *flags)
+                else:
+                    amax = gpu.argmax(logits, out=meta[0:size]) if decode else gpu.argmax(logits)
             return logits, amax
 
         graph, (logits, amax) = gpu.capture(run)
@@ -621,7 +665,7 @@ class ModelRunner:
             # (some record memory-clearing nodes that misbehave on replay): this shape runs eagerly
             self._unrecordable.add(key)
             return None
-        if kind == "d":
+        if decode:
             meta.copy_(staging)               # the recording's trial replays have put their own tokens there
         stagings = [staging] + [gpu.pinned(torch.empty_like(staging)) for _ in range(self.STAGING_BUFFERS - 1)]
         rec = _RecordedStep(graph, meta, stagings, logits, ctx, [gpu.event() for _ in stagings])
@@ -633,6 +677,20 @@ class ModelRunner:
         self._recorded_bytes += rec.held_bytes
         return rec
 
+    def _shared_work(self) -> torch.Tensor:
+        """Scratch of the sampling kernels of recorded steps, float32 [GRAPH_MAX_BATCH, vocabulary]: like the logits,
+        one buffer for all recordings."""
+        if self._work_buffer is None:
+            self._work_buffer = torch.empty(self.GRAPH_MAX_BATCH, self.vocab_size, dtype=torch.float32, device=self.device)
+        return self._work_buffer
+
+    def _draw_constants(self):
+        """(a penalty of 1 for every row, zeros: the empty lists of penalised tokens), for draws without a penalty."""
+        if self._draw_consts is None:
+            self._draw_consts = (torch.ones(self.GRAPH_MAX_BATCH, dtype=torch.float32, device=self.device),
+                                 torch.zeros(self.GRAPH_MAX_BATCH + 1, dtype=torch.int32, device=self.device))
+        return self._draw_consts
+
     def _shared_logits(self) -> torch.Tensor:
         if self._logits_buffer is None:
             self._logits_buffer = torch.empty(self.GRAPH_MAX_BATCH, self.vocab_size, dtype=torch.float32, device=self.device)
@@ -641,7 +699,7 @@ class ModelRunner:
     def _drop_recordings(self) -> None:
         """Keep the recordings within their bounds: decode shapes by number, all of them together by the
         device memory they hold; the ones used longest ago go first (the newest always stays)."""
-        decodes = [k for k in self._recorded if k[0] == "d"]
+        decodes = [k for k in self._recorded if k[0] in ("d", "s")]
         for old in decodes[:max(0, len(decodes) - self.GRAPH_MAX_DECODES)]:
             self._recorded_bytes -= self._recorded.pop(old).held_bytes
         for old in list(self._recorded)[:-1]:
@@ -699,7 +757,7 @@ class ModelRunner:
         return ok
 
     def _replay(self, key, entries: List[StepEntry], tokens_from: Optional[_RecordedStep] = None,
-                history_row: Optional[int] = None, pick=None) -> bool:
+                history_row: Optional[int] = None, pick=None, draw_rows=None) -> bool:
         """Run the entries through the recording of their shape (made now if there is none).  False:
         this shape cannot be recorded and the step has not run.  The logits are left in
         ``self._replayed_logits``.
@@ -709,10 +767,11 @@ class ModelRunner:
         chose, and are taken from where it left them on the device.  ``history_row``: the tokens
         this replay chooses are also copied to that row of ``self._history`` (pinned host memory),
         and its logits are not kept.  ``pick(logits, out)``: launched behind the replay, it puts other
-        tokens than the largest logits where the step leaves its choice."""
+        tokens than the largest logits where the step leaves its choice.  ``draw_rows``: the table of the
+        draw that a step of kind "s" makes itself (int32 [4 B])."""
         rec = self._recorded.pop(key, None)
         if rec is None:
-            rec = self._record(key, entries)
+            rec = self._record(key, entries, draw_rows=draw_rows)
             if rec is None:
                 return False
             self._drop_recordings()
@@ -720,9 +779,12 @@ class ModelRunner:
         else:
             self._recorded[key] = rec          # moved to the end: the most recently used
         kind, B, width = key[0], key[1], key[2]
+        decode = kind in ("d", "s")
+        if (kind == "s") != (draw_rows is not None):
+            raise StepError("a step that draws needs the draw's table, and only such a step takes one")
         ps = self.page_size
         order = tuple(e.request for e in entries)
-        if tokens_from is not None and not (kind == "d" and order == rec.order):
+        if tokens_from is not None and not (decode and order == rec.order):
             # refused before anything is changed: the caller's books and this recording's stay as they were
             raise StepError("tokens can stay on the device only between decode steps over the same requests")
         # the tables are written into the next staging buffer in turn, starting from those of the last replay
@@ -732,7 +794,7 @@ class ModelRunner:
         staging = rec.stagings[rec.turn]
         st = staging.numpy()                        # shares the pinned memory
         totals = []
-        if kind == "d" and order == rec.order:
+        if decode and order == rec.order:
             # the same requests in the same places as last time: tokens, positions and slots change,
             # block tables only grow at their ends
             st[:] = last.numpy()
@@ -743,6 +805,8 @@ class ModelRunner:
                 totals.append(done + 1)
             off_ctx = rec.layout.seq + 2 * B
             st[off_ctx:off_ctx + B] = totals
+            if draw_rows is not None:
+                st[rec.layout.draw:rec.layout.draw + 4 * B] = draw_rows
             for gi, g in enumerate(self.cache.groups):
                 off_slot, off_table, _ = rec.layout.groups[gi]
                 written = rec.pages_written[gi]
@@ -757,12 +821,12 @@ class ModelRunner:
                     st[off_slot + b] = table[done // ps] * ps + done % ps
         else:
             ctx = StepContext(self.device)
-            flat, layout, _, tiles = self._tables_of(entries, ctx, width, rec.tiles or ())
+            flat, layout, _, tiles = self._tables_of(entries, ctx, width, rec.tiles or (), draw_rows=draw_rows)
             if len(flat) != staging.numel() or tiles != (rec.tiles or {}):
                 raise StepError("a recorded step was asked to run another shape")
             st[:] = flat
             rec.layout = layout
-            rec.order = order if kind == "d" else ()
+            rec.order = order if decode else ()
             rec.pages_written = [[len(g.tables[e.request]) for e in entries] for g in self.cache.groups]
             totals = ctx._host["context_len"]
         if tokens_from is None:
@@ -838,12 +902,27 @@ class ModelRunner:
             self.release(r)
         return logits
 
-    def decode_run(self, entries: Sequence[StepEntry], steps: int, pick=None) -> List[List[int]]:
+    takes_draw_tables = True      # decode_run(..., draw=) exists: recorded decode steps can make the draw themselves
+
+    def _draw_eager(self, logits: torch.Tensor, draw, i: int) -> List[int]:
+        """Draw ``i`` of the tables ``draw`` over ``logits``, launched the ordinary way."""
+        B = logits.shape[0]
+        rows = torch.from_numpy(draw.rows(i)).to(self.device)
+        as_float = rows[:3 * B].view(torch.float32)
+        view = DrawView(as_float[0:B], as_float[B:2 * B], as_float[2 * B:3 * B], rows[3 * B:4 * B])
+        out = torch.empty(B, dtype=torch.int32, device=self.device)
+        self.gpu.draw(logits, torch.empty_like(logits), view, *self._draw_constants(), out, *draw.flags)
+        return out.tolist()
+
+    def decode_run(self, entries: Sequence[StepEntry], steps: int, pick=None, draw=None) -> List[List[int]]:
         """Decoding of ``steps`` tokens for every entry (one token each, wanting its logits):
         the first step takes the entries' tokens, every later one the tokens that the step before
-        chose: the index of the largest logit, lowest index on ties, or with ``pick`` what
+        chose: the index of the largest logit, lowest index on ties; or with ``pick`` what
         ``pick(i, logits, out)`` launches into ``out`` (int32 [entries], on the device) for step
-        ``i`` without waiting for anything.  Returns the chosen tokens,
+        ``i`` without waiting for anything; or with ``draw`` (a sampler's
+        :class:`~nanoinfer_amd.sampling.sampler.DrawTables`: temperature, top-k, top-p and the uniform
+        numbers of every step, no repetition penalty) what the sampling kernels draw, which are then part
+        of the recorded step itself.  Returns the chosen tokens,
         ``[step][entry]``: what ``steps`` calls of :meth:`step` with :meth:`greedy_tokens` between
         them return.  Where recordings of the steps' shapes exist, the steps are launched back to
         back, the tokens passing from one to the next on the device, and the host waits once at
@@ -852,6 +931,8 @@ class ModelRunner:
         entries = list(entries)
         if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
             raise StepError("decode_run takes entries of one token each that want its logits")
+        if pick is not None and draw is not None:
+            raise StepError("decode_run takes pick or draw, not both")
         B = len(entries)
         chosen: List[List[int]] = []
         tokens: Optional[List[int]] = [int(e.tokens[0]) for e in entries]     # None: still on the device
@@ -872,37 +953,50 @@ class ModelRunner:
                 tokens = rows[-1]
                 launched = 0
 
+        def the_ordinary_way(cur) -> None:
+            nonlocal tokens, last
+            logits = self.step(cur)
+            if draw is not None:
+                tokens = self._draw_eager(logits, draw, len(chosen))
+            elif pick is None:
+                tokens = self.greedy_tokens(logits)
+            else:
+                out = torch.empty(B, dtype=torch.int32, device=self.device)
+                pick(len(chosen), logits, out)
+                tokens = out.tolist()
+            chosen.append(list(tokens))
+            last = None
+
         order = tuple(e.request for e in entries)
+        flags = None if draw is None else draw.flags
         for _ in range(int(steps)):
             cur = [StepEntry(e.request, [tokens[b] if tokens is not None else 0], [0]) for b, e in enumerate(entries)]
-            key = self._graph_shape(cur) if B else None
+            key = self._graph_shape(cur, draw=flags) if B else None
             rec = self._recorded.get(key) if key is not None else None
+            # a step that draws by itself is recorded by its first replay here (the ordinary way records the other kind)
+            to_record = draw is not None and key is not None and rec is None
             if rec is None or rec.amax is None or launched == self.HISTORY_ROWS or \
                     (tokens is None and rec.order != order):
                 # also when the run passes into a recording of another shape (a longer context, a wider
                 # table) that last ran other requests: its tables are written anew, from tokens the host knows
                 collect()
                 cur = [StepEntry(e.request, [tokens[b]], [0]) for b, e in enumerate(entries)]
-            if rec is None or rec.amax is None:
-                logits = self.step(cur)
-                if pick is None:
-                    tokens = self.greedy_tokens(logits)
-                else:
-                    out = torch.empty(B, dtype=torch.int32, device=self.device)
-                    pick(len(chosen), logits, out)
-                    tokens = out.tolist()
-                chosen.append(list(tokens))
-                last = None
+            if (rec is None and not to_record) or (rec is not None and rec.amax is None):
+                the_ordinary_way(cur)
                 continue
             self._check_and_reserve(cur)
             at = len(chosen) + launched
             _, close = self._span()
-            self._replay(key, cur, tokens_from=last if tokens is None else None, history_row=launched,
-                         pick=None if pick is None else (lambda logits, out, at=at: pick(at, logits, out)))
+            ran = self._replay(key, cur, tokens_from=last if tokens is None else None, history_row=launched,
+                               pick=None if pick is None else (lambda logits, out, at=at: pick(at, logits, out)),
+                               draw_rows=None if draw is None else draw.rows(at))
             close()
+            if not ran:               # the shape cannot be recorded
+                the_ordinary_way(cur)
+                continue
             self._book(cur, self._last_context_len)
             launched += 1
             tokens = None
-            last = rec
+            last = self._recorded[key]
         collect()
         return chosen

@@ -77,6 +77,11 @@ class Sampler:
                  uses_top_p=any(p.use_top_p() and p.temperature > 0 for p in params))
         return out.tolist()
 
+    def draw_tables(self, params: Sequence[SamplingParams], generated: Sequence[Sequence[int]], steps: int) -> "DrawTables":
+        """The same draws as :meth:`plan` prepares, as host tables for a runner whose recorded decode steps
+        draw by themselves (requests without a repetition penalty)."""
+        return DrawTables(params, generated, steps)
+
     def plan(self, params: Sequence[SamplingParams], generated: Sequence[Sequence[int]], steps: int) -> "SamplingPlan":
         """The draws of ``steps`` successive tokens for the same rows, prepared in one upload: the
         uniform numbers of a seeded request do not depend on the tokens drawn before (they are keyed
@@ -84,6 +89,32 @@ class Sampler:
         without reading a token in between.  The tokens of a row with a repetition penalty are kept
         on the device, where every draw adds the token it chose."""
         return SamplingPlan(self.device, params, generated, steps)
+
+
+class DrawTables:
+    """The options of R rows and the uniform numbers of ``steps`` draws as host arrays, for a runner that has
+    the draw recorded into its decode steps: ``rows(i)`` is what step i's kernels read, as int32 words
+    [temperature | top_p | uniform of step i | top_k], R each.  For requests without a repetition penalty
+    (the tokens a penalty looks at grow with every draw; such requests go through :class:`SamplingPlan`)."""
+
+    def __init__(self, params: Sequence[SamplingParams], generated: Sequence[Sequence[int]], steps: int):
+        if any(p.use_repetition_penalty() for p in params):
+            raise ValueError("draw tables are for requests without a repetition penalty")
+        self.steps = int(steps)
+        self.uses_top_k = any(p.use_top_k() and p.temperature > 0 for p in params)
+        self.uses_top_p = any(p.use_top_p() and p.temperature > 0 for p in params)
+        self._head = np.array([[p.temperature for p in params],
+                               [p.top_p if p.use_top_p() else 1.0 for p in params]], dtype=np.float32).reshape(-1).view(np.int32)
+        self._uniform = np.array([[uniform_from_counter(max(p.seed, 0), len(g) + i) for p, g in zip(params, generated)]
+                                  for i in range(self.steps)], dtype=np.float32).view(np.int32)
+        self._top_k = np.array([p.top_k if p.use_top_k() else 0 for p in params], dtype=np.int32)
+
+    @property
+    def flags(self):
+        return (self.uses_top_k, self.uses_top_p)
+
+    def rows(self, i: int) -> np.ndarray:
+        return np.concatenate([self._head, self._uniform[i], self._top_k])
 
 
 class SamplingPlan:

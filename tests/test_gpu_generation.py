@@ -83,7 +83,7 @@ def test_decode_runs_with_planned_draws_give_the_tokens_of_single_steps():
     for run in (1, 8):
         eng = engine(folder, dtype="float32", block_size=8, num_cache_blocks=24, max_sequences=3, max_decode_run=run)
         asked, original = [], eng.runner.decode_run
-        eng.runner.decode_run = lambda entries, steps, pick=None: (asked.append((steps, pick is not None)), original(entries, steps, pick))[1]
+        eng.runner.decode_run = lambda entries, steps, pick=None, draw=None: (asked.append((steps, pick is not None)), original(entries, steps, pick, draw))[1]
         ids = [eng.add_request(p, n, o) for p, n, o in zip(prompts, (30, 11, 50, 17), options)]
         eng.run()
         outs.append([eng.get_request(i).generated for i in ids])
@@ -102,6 +102,36 @@ def test_decode_runs_with_planned_draws_give_the_tokens_of_single_steps():
         eng = engine(folder, dtype="float32", block_size=8, num_cache_blocks=24, max_decode_run=run)
         greedy.append(eng.generate([prompts[0]], 24, SamplingParams(temperature=0.0, repetition_penalty=1.5))[0].tokens)
     assert greedy[0] == greedy[1] and greedy[0] != outs[1][2][:24]
+
+
+def test_decode_runs_whose_steps_draw_by_themselves_give_the_tokens_of_single_steps(dtype="float32"):
+    """Requests that draw with temperature, top-k and top-p but without a repetition penalty decode in runs whose
+    recorded steps make the draw themselves (no kernel is launched between a step and the next): the tokens are
+    those of an engine that decides before every step and draws through the sampler.  Float32, so that the two
+    ways see the same logits but for the last bits (their batches differ where a request ends inside a run)."""
+    from nanoinfer_amd.sampling.params import SamplingParams
+    folder = model_folder("B")
+    prompts = [list(random_tokens(1000, n, 60 + n)) for n in (9, 40, 23, 3)]
+    options = [SamplingParams(temperature=0.8, seed=5), SamplingParams(temperature=1.3, top_k=40, top_p=0.9, seed=6),
+               SamplingParams.greedy(), SamplingParams(temperature=0.9, top_p=0.8, seed=7)]
+    outs, runs = [], []
+    for run in (1, 8):
+        eng = engine(folder, dtype=dtype, block_size=8, num_cache_blocks=24, max_sequences=3, max_decode_run=run)
+        asked, original = [], eng.runner.decode_run
+        eng.runner.decode_run = lambda entries, steps, pick=None, draw=None: (
+            asked.append((steps, pick is not None, draw is not None)), original(entries, steps, pick, draw))[1]
+        ids = [eng.add_request(p, n, o) for p, n, o in zip(prompts, (30, 11, 50, 17), options)]
+        eng.run()
+        outs.append([eng.get_request(i).generated for i in ids])
+        runs.append((asked, {key[0] for key in eng.runner._recorded}))
+        assert eng.runner.cache.free_pages() == 24
+    assert outs[0] == outs[1]
+    assert [len(t) for t in outs[1]] == [30, 11, 50, 17] and len({tuple(t) for t in outs[1]}) == 4
+    assert not runs[0][0] and "s" not in runs[0][1]
+    assert any(steps == 8 and draws and not picks for steps, picks, draws in runs[1][0]) and "s" in runs[1][1]
+    # and a seeded request alone draws the same tokens as in company
+    alone = engine(folder, dtype=dtype, block_size=8, num_cache_blocks=24, max_decode_run=8)
+    assert alone.generate([prompts[1]], 11, options[1])[0].tokens == outs[1][1]
 
 
 def test_stop_token_from_the_configuration():

@@ -160,7 +160,7 @@ def test_random_scheduling_settings_do_not_change_the_logits(name, dtype, monkey
                                           max_decode_run=rng.choice([1, 2, 8])), sampler=sampler, ignore_eos=True)
         planned = []
         decode_run = eng.runner.decode_run
-        eng.runner.decode_run = lambda entries, steps, pick=None: (planned.append(steps), decode_run(entries, steps, pick))[1]
+        eng.runner.decode_run = lambda entries, steps, pick=None, draw=None: (planned.append(steps), decode_run(entries, steps, pick, draw))[1]
         ids = [eng.add_request(p, new, SamplingParams(temperature=1.0, seed=i)) for i, p in enumerate(prompts)]
         eng.run()
         preempted += eng.scheduler.num_preemptions > 0

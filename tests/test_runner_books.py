@@ -70,9 +70,9 @@ def make_runner(page_size=8, num_pages=200, max_requests=8):
     r._history_done = _Event()
     r.recordings_made = []
 
-    def record(key, entries):
+    def record(key, entries, draw_rows=None):
         kind, size, pages, bound, _ = key
-        assert kind == "d"
+        assert kind == "d" and draw_rows is None
         ctx = StepContext(r.device, recording=True)
         flat, layout, n_rows, tiles = r._tables_of(entries, ctx, pages, ())
         staging = torch.tensor(flat, dtype=torch.int32)
@@ -219,6 +219,16 @@ class _HostServices:
         out.copy_(ids)
         return out
 
+    @staticmethod
+    def draw(logits, work, view, ones, zeros, out, uses_top_k, uses_top_p):
+        """Stands for the sampling kernels: the largest logit's index moved on by what the row's table says, so
+        that a test sees whether every step's own table has reached the step."""
+        R = logits.shape[0]
+        assert float(ones[:R].min()) == 1.0 and int(zeros[:R + 1].abs().max()) == 0 and not uses_top_p
+        shift = (view.uniform * 64).round().to(torch.int32) + view.top_k + (view.temperature * 8).round().to(torch.int32)
+        out.copy_((logits.argmax(dim=1).to(torch.int32) + shift) % VOCAB)
+        return out
+
     def capture(self, run):
         self.model.dry = True
         try:
@@ -319,3 +329,48 @@ def test_host_lists_cannot_be_read_while_a_step_is_recorded():
     ctx.seal()
     with pytest.raises(StepError, match="per_seq"):
         ctx.q_len
+
+
+def test_steps_that_draw_by_themselves_get_their_own_table_every_step():
+    """``decode_run(..., draw=tables)``: the draw is part of the recorded step, and what it reads (temperature,
+    top-k, top-p, and the uniform number of that very step) travels with the step's tables.  The stand-in draw
+    moves the token on by what its table says; the tokens follow, through the first steps that record the
+    shapes, a run across a context bound into another recording, and single eager steps when recording is off."""
+    from nanoinfer_amd.sampling.params import SamplingParams
+    from nanoinfer_amd.sampling.sampler import DrawTables
+    params = [SamplingParams(temperature=0.5, top_k=3, seed=11), SamplingParams(temperature=1.0, top_k=0, seed=12)]
+
+    def expect(first, context, generated, steps):
+        toks, out = list(first), []
+        for k in range(steps):
+            nxt = []
+            for b, (t, p) in enumerate(zip(toks, params)):
+                from nanoinfer_amd.sampling.sampler import uniform_from_counter
+                u = uniform_from_counter(p.seed, generated + k)
+                shift = round(float(torch.tensor(u, dtype=torch.float32) * 64)) + (p.top_k if p.top_k > 0 else 0) + round(p.temperature * 8)
+                nxt.append((next_token(t, context + k) + shift) % VOCAB)
+            toks = nxt
+            out.append(list(toks))
+        return out
+
+    for graphs in (True, False):
+        r = make_state_runner(idempotent_says=False)
+        r.use_graphs = graphs
+        names, first = ("a", "b"), [3, 50]
+        r.step([StepEntry(n, [1] * 250, []) for n in names])
+        generated = [[] for _ in names]
+        toks, got, done = list(first), [], 0
+        for k in (3, 8, 5):                    # the second run crosses the bound of 256 tokens
+            tables = DrawTables(params, generated, k)
+            assert tables.flags == (True, False)
+            rows = r.decode_run([StepEntry(n, [t], [0]) for n, t in zip(names, toks)], k, draw=tables)
+            assert rows == expect(toks, 250 + done, done, k), (graphs, done)
+            for row in rows:
+                for g, t in zip(generated, row):
+                    g.append(t)
+            toks, done = rows[-1], done + k
+        assert ({key[0] for key in r._recorded} == {"s"} and len(r._recorded) == 2) if graphs else not r._recorded
+        for n in names:                        # and the state moved once a step
+            assert float(r.cache.state[0][r.cache.state_slot(n)]) == 1 + done
+    with pytest.raises(ValueError, match="repetition penalty"):
+        DrawTables([SamplingParams(temperature=1.0, repetition_penalty=1.2)], [[]], 2)
