@@ -1019,7 +1019,9 @@ static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K,
     if (addends.n_pend > 0) return -10;      // only the kernel of the decode step proper adds them
     if (tiled) {
         // (with the rotation epilogue the rows are dealt out 32 to a workgroup: see skinny_rows_kernel)
+        // two, three or four blocks of sixteen rows: what a workgroup brings of x into its LDS grows with them
         if (M <= 32 || EPI == EPI_ROPE) return launch_rows<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
+        if (M <= 48) return launch_rows<T, TOUT, 3, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
         return launch_rows<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
     }
     if constexpr (EPI == EPI_RESIDUAL) {
@@ -1027,6 +1029,7 @@ static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K,
     } else {
         if (M <= 16) return launch_nt<T, TOUT, 1, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
         if (M <= 32) return launch_nt<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
+        if (M <= 48) return launch_nt<T, TOUT, 3, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
         return launch_nt<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
     }
 }
@@ -1091,6 +1094,7 @@ static int launch_ksplit(const void* x, const void* W, void* y, int M, int N, in
                          hipStream_t stream) {
     if (M <= 16) return launch_decode<T, float, EPI_STORE, 0>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, NormArgs{}, splits);
     if (M <= 32) return launch_rows<T, float, 2, EPI_STORE>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, splits);
+    if (M <= 48) return launch_rows<T, float, 3, EPI_STORE>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, splits);
     return launch_rows<T, float, 4, EPI_STORE>(x, W, y, M, N, K, 0, tiles_per_group, stream, RopeArgs{}, splits);
 }
 
