@@ -1002,8 +1002,7 @@ def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optiona
     global _library_calls
     _library_calls += 1
     if out_dtype != x.dtype:
-        result = torch.mm(x, rows_t, out_dtype=out_dtype)
-        return result if out is None else out.copy_(result)
+        return torch.mm(x, rows_t, out_dtype=out_dtype) if out is None else torch.mm(x, rows_t, out_dtype=out_dtype, out=out)
     return torch.mm(x, rows_t) if out is None else torch.mm(x, rows_t, out=out)
 
 
