@@ -125,6 +125,57 @@ struct RopeArgs {
     int H, KVH, hd, page_size;
 };
 
+// A norm done in two halves by the products on either side of it.  RMSNorm(h) . W^T = ((h * w) . W^T) / rms(h) row by
+// row, so the product that completes the residual stream (residual epilogue, `xn` set) also stores
+// xn[m, n] = h[m, n] * w[n] in the compute type and the sum of h[m, n]^2 over its own columns, ss_out[m * parts + wg]
+// (parts = its workgroups); and the product behind the norm (`ss_in` set) takes xn for its x and multiplies its sums
+// by 1 / sqrt(sum over the parts / width + eps) in its epilogue.  No kernel normalises and none reads h for it.
+// The sums of squares are float32 of the float32 stream, added in a fixed order.
+#define DEFER_PARTS_MAX 256       // workgroups whose sums of squares the product behind the norm adds up for a row
+struct DeferArgs {
+    void* xn = nullptr;            // [M, N] compute type: the stream times the next norm's weight
+    const float* w = nullptr;      // [N] that weight
+    float* ss_out = nullptr;       // [M, parts]
+    const float* ss_in = nullptr;  // [M, parts] of the product before
+    int parts = 0;
+    float eps = 0.f;
+    int width = 0;                 // elements of a row of the stream
+};
+
+// The taking side: wavefront w adds up the rows w, w + WV, ... (lane l the parts l, l + 64, ...), asked for before the
+// first trip of W and settled behind it, and leaves each row's factor in LDS for the epilogue.
+template <int WV, int MAXROWS>
+struct DeferTake {
+    static constexpr int RPW = (MAXROWS + WV - 1) / WV;
+    static constexpr int LPR = DEFER_PARTS_MAX / WAVE;
+    float v[RPW][LPR];
+    __device__ __forceinline__ void ask(const DeferArgs& d, int M, int wave, int lane) {
+        if (d.ss_in == nullptr) return;
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) {
+            const int m = wave + i * WV;
+#pragma unroll
+            for (int j = 0; j < LPR; ++j) {
+                const int part = lane + j * WAVE;
+                v[i][j] = (m < M && part < d.parts) ? d.ss_in[static_cast<size_t>(m) * d.parts + part] : 0.f;
+            }
+        }
+    }
+    __device__ __forceinline__ void settle(const DeferArgs& d, int M, int wave, int lane, float* factors) {
+        if (d.ss_in == nullptr) return;
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) {
+            const int m = wave + i * WV;
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < LPR; ++j) s += v[i][j];
+#pragma unroll
+            for (int off = WAVE / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
+            if (lane == 0 && m < M) factors[m] = 1.0f / sqrtf(s / static_cast<float>(d.width) + d.eps);
+        }
+    }
+};
+
 // What an epilogue reads from memory, asked for while W is still streaming instead of at the end, where every
 // load is a round trip that nothing hides (the rotation's are two in a row: the position, then its angle).
 // For the first item of a thread (item == threadIdx.x), which with at most 16 rows and few tiles is its only one.
@@ -133,12 +184,13 @@ struct EpiEarly {
     int pos = 0, slot = -1;  // rotation: the row's position and cache slot
     float a = 0.f, b = 0.f;  // rotation: cos and sin; residual: the stream's value and its first addend
     float c = 0.f;           // residual: the second addend
+    float d = 1.f;           // residual: the next norm's weight at the thread's column, where the epilogue leaves h * w behind
 };
 
 // The first half for the rotation epilogue (position and slot of the thread's row), the whole for the residual one.
 template <int EPI, int NT, int HALVES>
 __device__ __forceinline__ void epi_early_first(EpiEarly& e, const void* y, int M, int N, const RopeArgs& rope,
-                                                const float* pend, int n_pend) {
+                                                const float* pend, int n_pend, const float* next_w = nullptr) {
     const int item = threadIdx.x;
     const int wg = blockIdx.x / HALVES, wg_half = blockIdx.x % HALVES;
     if constexpr (EPI == EPI_ROPE) {
@@ -154,6 +206,7 @@ __device__ __forceinline__ void epi_early_first(EpiEarly& e, const void* y, int 
         e.have = true;
         const float* dst = static_cast<const float*>(y) + static_cast<size_t>(m) * N + n;
         e.a = *dst;
+        if (next_w != nullptr) e.d = next_w[n];
         if (n_pend > 0) {
             const float* p = pend + static_cast<size_t>(m) * N + n;
             e.b = p[0];
@@ -183,7 +236,8 @@ __device__ __forceinline__ void epi_early_second(EpiEarly& e, const RopeArgs& ro
 template <typename T, typename TOUT, int MB, int NT, int EPI, int WV = GV_WAVES, bool EXT = false, int HALVES = 1>
 __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TOUT* __restrict__ y, int M, int N, int I,
                                               const RopeArgs& rope, float* ext = nullptr, const float* pend = nullptr,
-                                              int n_pend = 0, const EpiEarly* early = nullptr) {
+                                              int n_pend = 0, const EpiEarly* early = nullptr,
+                                              const DeferArgs& defer = DeferArgs{}, const float* factors = nullptr) {
     const int tid = threadIdx.x;
     const int wave = tid / WAVE, lane = tid % WAVE;
     const int wg = blockIdx.x / HALVES;
@@ -205,6 +259,9 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
 #pragma unroll
             for (int i = 0; i < 4; ++i) red[wave][nt * MB + mb][lane * 4 + i] = acc[nt][mb][i];
     __syncthreads();
+    // the row's factor where the product stands behind a norm whose division it makes itself (1 otherwise)
+    const bool scaled = EPI != EPI_RESIDUAL && factors != nullptr && defer.ss_in != nullptr;
+    auto factor_of = [&](int m) { return scaled ? factors[m] : 1.0f; };
 
     // D[n_local][m_local] of a tile sits at lane = (n_local / 4) * 16 + m_local, register n_local % 4
     if constexpr (EPI == EPI_ROPE) {
@@ -224,6 +281,7 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
                 x0 += red[w][0 * MB + mb][src];
                 x1 += red[w][1 * MB + mb][src];
             }
+            if (scaled) { const float f = factor_of(m); x0 *= f; x1 *= f; }
             const int j = j0 + n_local;
             const bool ready = early != nullptr && early->have && item == tid;      // asked for while W was streaming
             if (head < rope.H + rope.KVH) {             // queries and keys turn, values do not
@@ -261,6 +319,57 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
     constexpr int NOUT = (EPI == EPI_SWIGLU) ? NT / 2 : NT;      // output tiles of the workgroup
     const int out_n0 = wg * NOUT * 16;
     const int out_width = (EPI == EPI_SWIGLU) ? I : N;
+    if constexpr (EPI == EPI_RESIDUAL && HALVES == 1) {
+        if (defer.xn != nullptr) {
+            // The stream's new values, and with them what the next norm needs of them: h * w in the compute type, and
+            // the sum of squares of each row over this workgroup's columns.  The items of a row are ROWW neighbouring
+            // lanes of one wavefront, which add their squares by shuffles: every lane of a wavefront that has items
+            // goes through the same code (lanes without a row or a column add zero and store nothing).
+            constexpr int ROWW = NT * 16;
+            static_assert(ROWW <= WAVE && WAVE % ROWW == 0, "the items of a row lie within a wavefront");
+            const int parts = gridDim.x;
+            for (int base = 0; base < MB * 16 * ROWW; base += WV * WAVE) {
+                const int item = base + tid;
+                if (item - lane >= MB * 16 * ROWW) break;           // the whole wavefront is past the items
+                const int n_in = item % ROWW, m = item / ROWW;
+                const int ot = n_in / 16, n_local = n_in % 16;
+                const int mb = m / 16, m_local = m % 16;
+                const int n = out_n0 + n_in;
+                const bool live = m < M && n < N;
+                float sq = 0.f;
+                if (live) {
+                    const int src = ((n_local / 4) * 16 + m_local) * 4 + (n_local % 4);
+                    float v = 0.f;
+#pragma unroll
+                    for (int w = 0; w < WV; ++w) v += red[w][ot * MB + mb][src];
+                    float* dst = reinterpret_cast<float*>(y) + static_cast<size_t>(m) * N + n;
+                    const bool ready = early != nullptr && early->have && item == tid;
+                    float sum = ready ? early->a : *dst;
+                    const float wn = ready ? early->d : defer.w[n];
+                    if (n_pend > 0) {
+                        const float* p = pend + static_cast<size_t>(m) * N + n;
+                        const size_t stride = static_cast<size_t>(M) * N;
+                        float p0, p1;
+                        if (ready) {
+                            p0 = early->b; p1 = early->c;
+                        } else {
+                            p0 = p[0]; p1 = n_pend > 1 ? p[stride] : 0.f;
+                        }
+                        sum = (sum + p0) + p1;
+                        for (int a = 2; a < n_pend; ++a) sum += p[a * stride];
+                    }
+                    const float hv = sum + v;
+                    *dst = hv;
+                    st(static_cast<T*>(defer.xn) + static_cast<size_t>(m) * N + n, hv * wn);
+                    sq = hv * hv;
+                }
+#pragma unroll
+                for (int off = ROWW / 2; off > 0; off >>= 1) sq += __shfl_xor(sq, off, WAVE);
+                if (n_in == 0 && m < M) defer.ss_out[static_cast<size_t>(m) * parts + wg] = sq;
+            }
+            return;
+        }
+    }
     for (int item = tid; item < MB * 16 * NOUT * 16; item += WV * WAVE) {
         const int n_in = item % (NOUT * 16);
         const int m = item / (NOUT * 16);
@@ -277,11 +386,13 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
                 g += red[w][(2 * ot) * MB + mb][src];
                 u += red[w][(2 * ot + 1) * MB + mb][src];
             }
+            if (scaled) { const float f = factor_of(m); g *= f; u *= f; }
             v = g / (1.0f + expf(-g)) * u;
         } else {
             v = 0.f;
 #pragma unroll
             for (int w = 0; w < WV; ++w) v += red[w][ot * MB + mb][src];
+            if (scaled) v *= factor_of(m);
         }
         TOUT* dst = y + static_cast<size_t>(m) * out_width + n;
         if constexpr (EPI == EPI_RESIDUAL) {      // float32 residual stream, this workgroup's own columns
@@ -399,9 +510,10 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_gemm_kernel(const T* __rest
 template <typename T, typename TOUT, int NT, int EPI, int XP, int WV, int SR, int HALVES = 1, int PRO = PRO_NORM, bool PEND = false>
 __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                                    TOUT* __restrict__ y, int M, int N, int K, int I,
-                                                                   RopeArgs rope, NormArgs norm, int splits) {
+                                                                   RopeArgs rope, NormArgs norm, int splits, DeferArgs defer) {
     constexpr int EL = Piece<T>::ELEMS;
     constexpr int CH = 4 * EL;
+    __shared__ float factors[16];      // of the rows, where the product makes the division of the norm before it
     // The rows that a staged prologue leaves in LDS are dead once every wavefront has picked its operands
     // from them; where they are large enough, the partial sums of the end take their memory (float32 rows
     // of 2,048 elements for eight rows are 66 KB: with the sums beside them one workgroup would fill a
@@ -425,7 +537,7 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
     y += static_cast<size_t>(blockIdx.y) * M * N;
     EpiEarly early;         // what the epilogue will read, asked for before W (not behind the merging prologue's many
                             // loads, where it gained nothing: the o product of one row 6.6 -> 7.3 us)
-    if constexpr (PRO == PRO_NORM) epi_early_first<EPI, NT, HALVES>(early, y, M, N, rope, norm.pend, norm.n_pend);
+    if constexpr (PRO == PRO_NORM) epi_early_first<EPI, NT, HALVES>(early, y, M, N, rope, norm.pend, norm.n_pend, defer.w);
 
     const T* wrow[NT];      // first byte of this lane in piece 0 of each tile
 #pragma unroll
@@ -723,6 +835,8 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
             if (t + 1 < TRIPS) multiply(c + STRIDE, wa_b, xn[t + 1 < TRIPS ? t + 1 : t]);
         }
     } else {
+        DeferTake<WV, 16> take;
+        if constexpr (EPI != EPI_RESIDUAL) take.ask(defer, M, wave, lane);      // a few cache hits, ahead of W
         load_w(p_begin + wave, wa_a);
         const T* xrow = x + static_cast<size_t>(row) * K;
         auto load_x = [&](int c, Piece<T> (&xb)[PT][1]) {
@@ -732,6 +846,7 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
         Piece<T> xb_a[PT][1], xb_b[PT][1];
         load_x(p_begin + wave, xb_a);
         epi_early_second<EPI, HALVES>(early, rope);      // behind the first trip of W and x (waits for the position only)
+        if constexpr (EPI != EPI_RESIDUAL) take.settle(defer, M, wave, lane, factors);
         for (int c = p_begin + wave; c < p_end; c += 2 * STRIDE) {
             if (c + STRIDE < p_end) { load_w(c + STRIDE, wa_b); load_x(c + STRIDE, xb_b); }
             multiply(c, wa_a, xb_a);
@@ -742,9 +857,10 @@ __global__ __launch_bounds__(WV * WAVE) void skinny_decode_kernel(const T* __res
     if constexpr (SHARE_LDS) {
         __syncthreads();                   // every wavefront has taken its operands from the staged rows
         skinny_finish<T, TOUT, 1, NT, EPI, WV, true, HALVES>(acc, y, M, N, I, rope, reinterpret_cast<float*>(staged_rows),
-                                                             norm.pend, norm.n_pend, &early);
+                                                             norm.pend, norm.n_pend, &early, defer, factors);
     } else {
-        skinny_finish<T, TOUT, 1, NT, EPI, WV, false, HALVES>(acc, y, M, N, I, rope, nullptr, norm.pend, norm.n_pend, &early);
+        skinny_finish<T, TOUT, 1, NT, EPI, WV, false, HALVES>(acc, y, M, N, I, rope, nullptr, norm.pend, norm.n_pend, &early,
+                                                              defer, factors);
     }
 }
 
@@ -761,11 +877,12 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));    // 16 bytes tha
 template <typename T, typename TOUT, int MB, int NT, int EPI>
 __global__ __launch_bounds__(GV_THREADS) void skinny_rows_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                                  TOUT* __restrict__ y, int M, int N, int K, int I,
-                                                                 RopeArgs rope, int splits) {
+                                                                 RopeArgs rope, int splits, DeferArgs defer) {
     constexpr int EL = Piece<T>::ELEMS;
     constexpr int CH = 4 * EL;
     constexpr int WV = GV_WAVES;
     constexpr int ROWS = MB * 16;
+    __shared__ float factors[ROWS];    // of the rows, where the product makes the division of the norm before it
     constexpr int XL = ROWS / 8;                       // 16-byte loads of a lane for one piece of all rows
     constexpr int SLAB = ROWS * SLAB_ROW;
     constexpr int RED = NT * MB * WAVE * 4 * static_cast<int>(sizeof(float));
@@ -787,6 +904,7 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_rows_kernel(const T* __rest
         y += static_cast<size_t>(row0) * rope.H * rope.hd;
         rope.positions += row0;
         if (rope.slot_mapping) rope.slot_mapping += row0;
+        if (defer.ss_in != nullptr) defer.ss_in += static_cast<size_t>(row0) * defer.parts;
         M = min(M - row0, ROWS);
     }
     unsigned char* slab = lds + wave * SLAB;
@@ -852,8 +970,11 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_rows_kernel(const T* __rest
 
     Piece<T> wa_a[NT], wa_b[NT];
     u32x4_t xr_a[XL], xr_b[XL];
+    DeferTake<WV, ROWS> take;
+    if constexpr (EPI != EPI_RESIDUAL) take.ask(defer, M, wave, lane);      // cache hits, ahead of W
     load_w(p_begin + wave, wa_a);
     load_x(p_begin + wave, xr_a);
+    if constexpr (EPI != EPI_RESIDUAL) take.settle(defer, M, wave, lane, factors);
     for (int c = p_begin + wave; c < p_end; c += 2 * WV) {
         stage(xr_a);
         wave_sync();
@@ -871,7 +992,8 @@ __global__ __launch_bounds__(GV_THREADS) void skinny_rows_kernel(const T* __rest
         }
     }
     __syncthreads();                       // every wavefront is done with its slab: the partial sums take the memory
-    skinny_finish<T, TOUT, MB, NT, EPI, WV, true>(acc, y, M, N, I, rope, reinterpret_cast<float*>(lds));
+    skinny_finish<T, TOUT, MB, NT, EPI, WV, true>(acc, y, M, N, I, rope, reinterpret_cast<float*>(lds), nullptr, 0, nullptr,
+                                                  defer, factors);
 }
 
 template <typename T, typename TOUT, int MB, int EPI>
@@ -903,8 +1025,10 @@ static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K,
 // The decode kernel: NT as launch_nt chooses it.  XP: pieces per wavefront of the normalising prologue, 0 without.
 template <typename T, typename TOUT, int EPI, int XP>
 static int launch_decode(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream,
-                         RopeArgs rope = RopeArgs{}, NormArgs norm = NormArgs{}, int splits = 1) {
+                         RopeArgs rope = RopeArgs{}, NormArgs norm = NormArgs{}, int splits = 1, DeferArgs defer = DeferArgs{}) {
     if (splits != 1 && (XP != 0 || EPI != EPI_STORE)) return -8;      // shares are stored, not finished
+    if ((defer.xn != nullptr && (EPI != EPI_RESIDUAL || splits != 1)) || (defer.ss_in != nullptr && (XP != 0 || EPI == EPI_RESIDUAL)))
+        return -11;     // h * w and the sums of squares come from a whole product onto the stream; they are taken by a product on a given x
     if (norm.n_pend > 0) {
         // addends that the residual stream has not received: for the staged normalising prologue (up to
         // eight rows, at most two tiles a workgroup), or for the residual epilogue
@@ -918,6 +1042,7 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
     }
     const int out_width = (EPI == EPI_SWIGLU) ? I : N;
     const int tiles = (out_width + 15) / 16;
+    bool defer_mismatch = false;       // the caller sized the sums of squares for another number of workgroups
     auto run = [&](auto nt_tag) {
         constexpr int NTc = decltype(nt_tag)::value;
         constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
@@ -928,18 +1053,19 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
         // 256, the same was measured and gained nothing: not compiled.)
         constexpr bool CAN_HALVE = EPI == EPI_ROPE;
         const bool halve = CAN_HALVE && grid <= HALVE_BELOW;
+        if (defer.xn != nullptr && defer.parts != grid) { defer_mismatch = true; return; }
         auto launch = [&](auto wv_tag, auto sr_tag, auto halves_tag) {
             constexpr int WVc = decltype(wv_tag)::value, SRc = decltype(sr_tag)::value, Hc = decltype(halves_tag)::value;
             if constexpr (XP > 0 && SRc > 0) {
                 if (norm.n_pend > 0) {
                     skinny_decode_kernel<T, TOUT, NTc, EPI, XP, WVc, SRc, Hc, PRO_NORM, true>
                         <<<dim3(grid * Hc, splits), WVc * WAVE, 0, stream>>>((const T*)x, (const T*)W, (TOUT*)y, M, N, K, I,
-                                                                              rope, norm, splits);
+                                                                              rope, norm, splits, defer);
                     return;
                 }
             }
             skinny_decode_kernel<T, TOUT, NTc, EPI, XP, WVc, SRc, Hc><<<dim3(grid * Hc, splits), WVc * WAVE, 0, stream>>>(
-                (const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm, splits);
+                (const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, norm, splits, defer);
         };
         using One = std::integral_constant<int, 1>;
         using Two = std::integral_constant<int, 2>;
@@ -967,7 +1093,7 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
         with_halves(Waves8{}, std::integral_constant<int, 0>{});
     };
     if constexpr (EPI != EPI_ROPE) {
-        if (NT >= 4) { run(std::integral_constant<int, 4>{}); return NI_LAUNCH_RESULT(); }
+        if (NT >= 4) { run(std::integral_constant<int, 4>{}); return defer_mismatch ? -11 : NI_LAUNCH_RESULT(); }
     }
     if constexpr (EPI == EPI_SWIGLU || EPI == EPI_ROPE) {
         run(std::integral_constant<int, 2>{});
@@ -975,22 +1101,25 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
         if (NT >= 2) run(std::integral_constant<int, 2>{});
         else run(std::integral_constant<int, 1>{});
     }
-    return NI_LAUNCH_RESULT();
+    return defer_mismatch ? -11 : NI_LAUNCH_RESULT();
 }
 
 // The kernel for 17 to 64 rows: MB blocks of 16 rows, NT as launch_nt chooses it, within the eight
 // fragments of partial sums a wavefront may hold.
 template <typename T, typename TOUT, int MB, int EPI>
 static int launch_rows(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, hipStream_t stream,
-                       RopeArgs rope = RopeArgs{}, int splits = 1) {
+                       RopeArgs rope = RopeArgs{}, int splits = 1, DeferArgs defer = DeferArgs{}) {
+    if ((defer.xn != nullptr && (EPI != EPI_RESIDUAL || splits != 1)) || (defer.ss_in != nullptr && EPI == EPI_RESIDUAL)) return -11;
     const int out_width = (EPI == EPI_SWIGLU) ? I : N;
     const int tiles = (out_width + 15) / 16;
+    bool defer_mismatch = false;
     auto run = [&](auto nt_tag) {
         constexpr int NTc = decltype(nt_tag)::value;
         constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
         const int grid = (tiles + NOUT - 1) / NOUT;
+        if (defer.xn != nullptr && defer.parts != grid) { defer_mismatch = true; return; }
         skinny_rows_kernel<T, TOUT, MB, NTc, EPI><<<dim3(grid, splits, (M + MB * 16 - 1) / (MB * 16)), GV_THREADS, 0, stream>>>(
-            (const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, splits);
+            (const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, splits, defer);
     };
     if constexpr (EPI == EPI_SWIGLU) {
         // two pairs of gate and up tiles a workgroup where asked for: half the workgroups, and with them
@@ -1009,21 +1138,31 @@ static int launch_rows(const void* x, const void* W, void* y, int M, int N, int 
         if (NT >= 2) run(std::integral_constant<int, 2>{});
         else run(std::integral_constant<int, 1>{});
     }
-    return NI_LAUNCH_RESULT();
+    return defer_mismatch ? -11 : NI_LAUNCH_RESULT();
+}
+
+// Workgroups of a product onto the residual stream of M rows and N columns, which is how many sums of squares
+// a row gets where the product leaves them behind for the next norm (DeferArgs): the launchers above, mirrored.
+static int residual_parts(int M, int N, int tiles_per_group) {
+    const int tiles = (N + 15) / 16;
+    int nt = tiles_per_group >= 4 ? 4 : tiles_per_group >= 2 ? 2 : 1;
+    if (M > 32 && nt == 4) nt = 2;       // three and four blocks of sixteen rows hold at most two tiles a workgroup
+    return (tiles + nt - 1) / nt;
 }
 
 template <typename T, typename TOUT, int EPI>
 static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K, int I, int NT, bool tiled,
-                     hipStream_t stream, RopeArgs rope = RopeArgs{}, NormArgs addends = NormArgs{}) {
-    if (M <= 16 && tiled) return launch_decode<T, TOUT, EPI, 0>(x, W, y, M, N, K, I, NT, stream, rope, addends);
+                     hipStream_t stream, RopeArgs rope = RopeArgs{}, NormArgs addends = NormArgs{}, DeferArgs defer = DeferArgs{}) {
+    if (M <= 16 && tiled) return launch_decode<T, TOUT, EPI, 0>(x, W, y, M, N, K, I, NT, stream, rope, addends, 1, defer);
     if (addends.n_pend > 0) return -10;      // only the kernel of the decode step proper adds them
     if (tiled) {
         // (with the rotation epilogue the rows are dealt out 32 to a workgroup: see skinny_rows_kernel)
         // two, three or four blocks of sixteen rows: what a workgroup brings of x into its LDS grows with them
-        if (M <= 32 || EPI == EPI_ROPE) return launch_rows<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
-        if (M <= 48) return launch_rows<T, TOUT, 3, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
-        return launch_rows<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, stream, rope);
+        if (M <= 32 || EPI == EPI_ROPE) return launch_rows<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream, rope, 1, defer);
+        if (M <= 48) return launch_rows<T, TOUT, 3, EPI>(x, W, y, M, N, K, I, NT, stream, rope, 1, defer);
+        return launch_rows<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, stream, rope, 1, defer);
     }
+    if (defer.xn != nullptr || defer.ss_in != nullptr) return -11;      // re-tiled matrices only
     if constexpr (EPI == EPI_RESIDUAL) {
         return -7;      // the residual epilogue exists for re-tiled matrices only
     } else {
@@ -1062,8 +1201,18 @@ static int launch_normed(const NormArgs& norm, const void* W, void* y, int M, in
 // tiled: W is in the re-tiled order described at the top (swiglu then needs N/2 to be a multiple of 16).
 // pend, n_pend (epilogue 3, at most 16 rows): float32 [n_pend, M, N] that y has not received yet and that are
 // added before the product, y = ((y + pend[0]) + pend[1] ...) + x . W^T; null, 0: none.
+//
+// A norm in two halves (DeferArgs above; re-tiled W only).  Leaving: epilogue 3 with xn [M, N] of the input type,
+// next_w float32 [N] and ss float32 [M, parts], parts = ni_skinny_residual_parts(M, N, tiles_per_group): beside adding
+// into y the product stores xn = y * next_w and every workgroup's sums of squares of its columns of y.  Taking:
+// epilogues 0, 1, 2 with ss float32 [M, parts] of the product before, parts <= 256 and that norm's eps: x is the xn
+// that product left, and row m of the sums is multiplied by 1 / sqrt(sum_p ss[m, p] / K + eps) before the epilogue.
+// xn and ss null: neither.
+NI_EXPORT int ni_skinny_residual_parts(int M, int N, int tiles_per_group) { return residual_parts(M, N, tiles_per_group); }
+
 NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N, int K, int epilogue, int tiles_per_group,
-                             int tiled, int dtype, const void* pend, int n_pend, hipStream_t stream) {
+                             int tiled, int dtype, const void* pend, int n_pend, void* xn, const void* next_w, void* ss,
+                             int parts, float eps, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64) return -1;
     const int el = dtype == 0 ? 8 : 16;
@@ -1075,15 +1224,27 @@ NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N
     NormArgs addends{nullptr, nullptr, 0.f};
     addends.pend = (const float*)pend;
     addends.n_pend = n_pend;
-    if (dtype == 0) {
-        if (epilogue == 3) return launch_mb<float, float, EPI_RESIDUAL>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream, RopeArgs{}, addends);
-        if (epilogue == 2) return launch_mb<float, float, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
-        return launch_mb<float, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
+    DeferArgs defer;
+    if (xn != nullptr || ss != nullptr) {
+        if (!tiled || !ss || parts < 1) return -11;
+        if (epilogue == 3) {
+            if (!xn || !next_w || parts != residual_parts(M, N, tiles_per_group)) return -11;
+            defer.xn = xn; defer.w = (const float*)next_w; defer.ss_out = (float*)ss;
+        } else {
+            if (xn != nullptr || parts > DEFER_PARTS_MAX || !(eps > 0.f)) return -11;
+            defer.ss_in = (const float*)ss; defer.eps = eps; defer.width = K;
+        }
+        defer.parts = parts;
     }
-    if (epilogue == 3) return launch_mb<bf16_t, float, EPI_RESIDUAL>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream, RopeArgs{}, addends);
-    if (epilogue == 2) return launch_mb<bf16_t, bf16_t, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
-    if (epilogue == 1) return launch_mb<bf16_t, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
-    return launch_mb<bf16_t, bf16_t, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream);
+    if (dtype == 0) {
+        if (epilogue == 3) return launch_mb<float, float, EPI_RESIDUAL>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream, RopeArgs{}, addends, defer);
+        if (epilogue == 2) return launch_mb<float, float, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream, RopeArgs{}, NormArgs{}, defer);
+        return launch_mb<float, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream, RopeArgs{}, NormArgs{}, defer);
+    }
+    if (epilogue == 3) return launch_mb<bf16_t, float, EPI_RESIDUAL>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream, RopeArgs{}, addends, defer);
+    if (epilogue == 2) return launch_mb<bf16_t, bf16_t, EPI_SWIGLU>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream, RopeArgs{}, NormArgs{}, defer);
+    if (epilogue == 1) return launch_mb<bf16_t, float, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream, RopeArgs{}, NormArgs{}, defer);
+    return launch_mb<bf16_t, bf16_t, EPI_STORE>(x, W, y, M, N, K, I, tiles_per_group, tiled != 0, stream, RopeArgs{}, NormArgs{}, defer);
 }
 
 // Up to 64 rows, re-tiled W: the K range cut into `splits` shares of whole 128-byte pieces, the sums of share s
@@ -1153,12 +1314,14 @@ NI_EXPORT int ni_skinny_merge_ok(int M, int heads, int hd, int runs, int dtype) 
 }
 
 template <typename TOUT, int EPI>
-static int launch_merged(const NormArgs& merge, const void* W, void* y, int M, int N, int K, hipStream_t stream) {
+static int launch_merged(const NormArgs& merge, const void* W, void* y, int M, int N, int K, hipStream_t stream,
+                         DeferArgs defer = DeferArgs{}) {
     const int tiles = (N + 15) / 16;
+    if (defer.ss_in != nullptr || (defer.xn != nullptr && EPI != EPI_RESIDUAL)) return -11;
     auto go = [&](auto sr_tag) {
         constexpr int SRc = decltype(sr_tag)::value;
         skinny_decode_kernel<bf16_t, TOUT, 1, EPI, 4, GV_WAVES, SRc, 1, PRO_MERGE><<<tiles, GV_THREADS, 0, stream>>>(
-            nullptr, (const bf16_t*)W, (TOUT*)y, M, N, K, 0, RopeArgs{}, merge, 1);
+            nullptr, (const bf16_t*)W, (TOUT*)y, M, N, K, 0, RopeArgs{}, merge, 1, defer);
     };
     if (M == 1) go(std::integral_constant<int, 1>{});
     else if (M <= 4) go(std::integral_constant<int, 4>{});
@@ -1167,9 +1330,10 @@ static int launch_merged(const NormArgs& merge, const void* W, void* y, int M, i
 }
 
 // pend, n_pend (epilogue 3): as for ni_skinny_gemm.
+// xn, next_w, ss (epilogue 3): as for ni_skinny_gemm, with parts = the tiles of N.
 NI_EXPORT int ni_skinny_gemm_merged(const void* part_o, const void* part_ml, int runs, int heads, int hd, const void* W,
                                     void* y, int M, int N, int epilogue, int dtype, const void* pend, int n_pend,
-                                    hipStream_t stream) {
+                                    void* xn, const void* next_w, void* ss, int parts, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (!part_o || !part_ml || !ni_skinny_merge_ok(M, heads, hd, runs, dtype)) return -5;
     if (epilogue != 0 && epilogue != 3) return -6;
@@ -1180,7 +1344,12 @@ NI_EXPORT int ni_skinny_gemm_merged(const void* part_o, const void* part_ml, int
     merge.part_o = (const float*)part_o;
     merge.part_ml = (const float*)part_ml;
     merge.runs = runs; merge.heads = heads; merge.hd = hd;
-    if (epilogue == 3) return launch_merged<float, EPI_RESIDUAL>(merge, W, y, M, N, heads * hd, stream);
+    DeferArgs defer;
+    if (xn != nullptr || ss != nullptr) {
+        if (epilogue != 3 || !xn || !next_w || !ss || parts != (N + 15) / 16) return -11;
+        defer.xn = xn; defer.w = (const float*)next_w; defer.ss_out = (float*)ss; defer.parts = parts;
+    }
+    if (epilogue == 3) return launch_merged<float, EPI_RESIDUAL>(merge, W, y, M, N, heads * hd, stream, defer);
     return launch_merged<bf16_t, EPI_STORE>(merge, W, y, M, N, heads * hd, stream);
 }
 
@@ -1188,11 +1357,13 @@ NI_EXPORT int ni_skinny_gemm_merged(const void* part_o, const void* part_ml, int
 // heads by the rows' positions, queries to q_out [M, H * hd], keys and values into the pools at
 // slot_mapping (null: not stored).  hd must be a multiple of 32 and fully rotated.
 // With x null the product is taken on RMSNorm(h): h float32 [M <= 8, K], norm_weight [K], W re-tiled; pend, n_pend as
-// for ni_skinny_gemm_normed.
+// for ni_skinny_gemm_normed.  With x and ss: x is what the product before left for a norm with this eps, ss [M, parts]
+// its sums of squares, and the division is made here (as for ni_skinny_gemm).
 NI_EXPORT int ni_skinny_qkv_rope(const void* x, const void* h, const void* norm_weight, float eps, const void* W,
                                  void* q_out, const void* positions, const void* cos_t, const void* sin_t,
                                  const void* slot_mapping, void* kpool, void* vpool, int M, int K, int H, int KVH, int hd,
-                                 int page_size, int tiled, int dtype, const void* pend, int n_pend, hipStream_t stream) {
+                                 int page_size, int tiled, int dtype, const void* pend, int n_pend, const void* ss, int parts,
+                                 hipStream_t stream) {
     if (M <= 0) return 0;
     if (M > 64) return -1;
     if (K % (dtype == 0 ? 8 : 16) != 0) return -2;
@@ -1202,6 +1373,7 @@ NI_EXPORT int ni_skinny_qkv_rope(const void* x, const void* h, const void* norm_
     const int N = (H + 2 * KVH) * hd;
     // the grid is sized from the output width: one workgroup per two tiles
     if (!x) {
+        if (ss != nullptr) return -11;
         if (!h || !norm_weight || !tiled || !ni_skinny_prologue_ok(M, K, dtype)) return -5;
         if (n_pend < 0 || (n_pend > 0 && !pend)) return -10;
         NormArgs norm{(const float*)h, (const float*)norm_weight, eps};
@@ -1211,6 +1383,11 @@ NI_EXPORT int ni_skinny_qkv_rope(const void* x, const void* h, const void* norm_
         return launch_normed<bf16_t, EPI_ROPE>(norm, W, q_out, M, N, K, 0, 2, stream, rope);
     }
     if (n_pend != 0) return -10;      // addends go with the normalising prologue only
-    if (dtype == 0) return launch_mb<float, float, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, tiled != 0, stream, rope);
-    return launch_mb<bf16_t, bf16_t, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, tiled != 0, stream, rope);
+    DeferArgs defer;
+    if (ss != nullptr) {              // x is what the product before left for the norm: the division is made here
+        if (!tiled || parts < 1 || parts > DEFER_PARTS_MAX || !(eps > 0.f)) return -11;
+        defer.ss_in = (const float*)ss; defer.parts = parts; defer.eps = eps; defer.width = K;
+    }
+    if (dtype == 0) return launch_mb<float, float, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, tiled != 0, stream, rope, NormArgs{}, defer);
+    return launch_mb<bf16_t, bf16_t, EPI_ROPE>(x, W, q_out, M, N, K, 0, 2, tiled != 0, stream, rope, NormArgs{}, defer);
 }

@@ -66,9 +66,19 @@ class Model:
         ``writes_into`` a given tensor (any other head returns a tensor of its own)."""
         h = self.embedding.forward(ctx.token_ids, ctx)
         pending = None
-        for run in self.spec.order:
+        order = self.spec.order
+        T = h.shape[0]
+        for i, run in enumerate(order):
             cache: LayerCache = layer_cache(run.cache, run.writes_cache)
-            h, pending = self.blocks[run.block].forward(h, pending, ctx, cache)
+            block = self.blocks[run.block]
+            # what the block behind this one would like to find beside the stream (its first norm's input half
+            # done by this block's last product), if both blocks know of that
+            wants = getattr(self.blocks[order[i + 1].block], "wants_scaled", None) if i + 1 < len(order) else None
+            leave = wants(T) if wants is not None and getattr(block, "leaves_for_next", False) else None
+            if leave is not None:
+                h, pending = block.forward(h, pending, ctx, cache, leave=leave)
+            else:
+                h, pending = block.forward(h, pending, ctx, cache)
         if ctx.logit_rows is None or ctx.logit_rows.shape[0] == 0:
             return None
         x = self.final_norm.forward(h, pending_for(self.final_norm, pending, self.rt.dtype), rows=ctx.logit_rows)

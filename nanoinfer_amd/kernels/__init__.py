@@ -565,6 +565,7 @@ FUSE_NORMS = True           # residual sums and norms ride on the skinny product
 ADDENDS_IN_PROLOGUE = True  # the shares of a cut product are added by the next normalising prologue and residual epilogue
 MERGE_IN_PRODUCT = True     # the key runs of a decode step's attention are merged by the output product where it can
 SPLIT_K = True              # products of 17 to 64 rows on matrices of few tiles are cut along K, the next norm adds the shares
+DEFER_NORMS = True          # a product onto the residual stream leaves h * w and sums of squares for the next norm, whose division the product behind it makes
 
 
 def tile_weight(w: torch.Tensor) -> torch.Tensor:
@@ -657,6 +658,89 @@ class NormedInput:
     @property
     def device(self):
         return self.h.device
+
+
+class NormSpec:
+    """Weight and eps of an RMSNorm, for a product onto the residual stream that is to leave the norm's
+    input half done behind (:class:`ScaledInput`)."""
+
+    __slots__ = ("weight", "eps")
+
+    def __init__(self, weight: torch.Tensor, eps: float):
+        self.weight, self.eps = weight, float(eps)
+
+
+class ScaledInput:
+    """The input of a product that stands behind an RMSNorm, as the product before the norm left it:
+    ``x`` [M, K] = ``h * weight`` in the compute type (not yet divided by the rows' root mean squares) and
+    ``ss`` float32 [M, parts], the sums of ``h^2`` over the columns of each of that product's workgroups.
+    ``RMSNorm(h) . W^T = ((h * w) . W^T) / rms(h)`` row by row: the skinny product multiplies ``x`` and
+    divides in its epilogue, so no kernel normalises and none reads ``h`` for it.  The residual stream
+    itself is complete (nothing is pending), so whoever cannot take this computes the norm of ``h``."""
+
+    __slots__ = ("x", "ss", "norm")
+
+    def __init__(self, x: torch.Tensor, ss: torch.Tensor, norm: NormSpec):
+        self.x, self.ss, self.norm = x, ss, norm
+
+    @property
+    def shape(self):
+        return self.x.shape
+
+    @property
+    def dtype(self):
+        return self.x.dtype
+
+    @property
+    def device(self):
+        return self.x.device
+
+    def made_for(self, weight: torch.Tensor, eps: float) -> bool:
+        """Whether this is the input of the norm with that weight tensor and eps."""
+        return self.norm.weight is weight and self.norm.eps == float(eps)
+
+
+DEFER_PARTS_MAX = 256        # sums of squares a row may come in (the kernels' bound)
+
+
+def _residual_parts(M: int, N: int) -> int:
+    return int(skinny_lib().ni_skinny_residual_parts(int(M), int(N), _tiles_per_group(N)))
+
+
+def leaves_scaled_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
+    """Whether a product of M rows of K elements onto the residual stream should leave a :class:`ScaledInput`
+    for the next norm; it then runs whole (its K range uncut) with the residual epilogue.  Measured in decode
+    steps of the 1B / 3B / 8B shapes against the ways it replaces (ms a step without : with).  Up to 16 rows
+    where the product runs whole anyway: the product behind the norm then needs neither a normalising
+    prologue (every workgroup reading all of h) nor a norm kernel (1B bfloat16 at batch 8 / 12 / 16
+    0.926 : 0.901, 1.057 : 1.008, 1.162 : 1.097, batch 1 the same; 1B float32 at batch 12 / 16 1.916 : 1.865,
+    1.997 : 1.941; 3B bfloat16 at batch 1 / 8 / 16 2.101 : 1.981, 2.412 : 2.275, 2.980 : 2.845).  Not where the
+    product would be cut along K to fill the chip (the down product of the 1B shape): whole it loses more than
+    the norm saves (1B at batch 1 0.742 : 0.776, float32 at batch 8 1.622 : 1.722).  From 17 to 32 rows the
+    products with rows of up to 4,096 elements (the o products), which whole beat their K shares plus the norm
+    kernel that adds them (1B at batch 24 / 32 1.263 : 1.251, 1.400 : 1.389); past 32 rows they do not."""
+    if not (DEFER_NORMS and isinstance(weight, Weight) and weight.tiles is not None and skinny_ok(M, K, dtype)):
+        return False
+    if _residual_parts(M, weight.rows.shape[0]) > DEFER_PARTS_MAX:
+        return False
+    if M <= SKINNY_BEST_ROWS:
+        return skinny_ksplit(M, K, dtype, weight)[0] == 1
+    return M <= 32 and K <= 4096 and skinny_wins(M, K, dtype, weight)
+
+
+def takes_scaled_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
+    """Whether the skinny product of M rows with this matrix can take a :class:`ScaledInput` for x."""
+    return (DEFER_NORMS and isinstance(weight, Weight) and weight.tiles is not None
+            and skinny_wins(M, K, dtype, weight))
+
+
+def _scaled_args(x: "ScaledInput", M: int, Kd: int):
+    """(x, ss, parts, eps) of a scaled input, checked, for a kernel's arguments."""
+    _gpu(x.x, "x", None, (M, Kd))
+    _gpu(x.ss, "sums of squares", torch.float32)
+    if not (x.ss.dim() == 2 and x.ss.shape[0] == M and 1 <= x.ss.shape[1] <= DEFER_PARTS_MAX):
+        raise KernelError(f"sums of squares {tuple(x.ss.shape)} against [{M}, at most {DEFER_PARTS_MAX}]")
+    return x.x, x.ss, int(x.ss.shape[1]), x.norm.eps
 
 
 @functools.lru_cache(maxsize=None)
@@ -777,14 +861,16 @@ def _check_normed(x: NormedInput, Kd: int) -> None:
 
 
 def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bool = False,
-                pending: Optional[torch.Tensor] = None) -> torch.Tensor:
+                pending: Optional[torch.Tensor] = None, leave: Optional[NormSpec] = None):
     """``x . weight^T`` for at most 64 rows of ``x``, streaming ``weight`` once (MFMA).  ``out``
     may be float32 for bfloat16 inputs.  With ``swiglu`` the weight is a stacked [2I, K] matrix
     (gate rows, then up rows) and ``out`` [M, I] receives ``silu(gate) * up``.  With ``residual``
     ``out`` is the float32 residual stream [M, N] and the product is added into it, after the
     ``pending`` addends [S, M, N] that the stream has not received yet (at most 16 rows).  ``x`` may
-    be a :class:`NormedInput`."""
+    be a :class:`NormedInput` or a :class:`ScaledInput`.  With ``residual`` and ``leave`` (the norm that
+    stands behind the stream) a :class:`ScaledInput` for that norm is returned."""
     normed = isinstance(x, NormedInput)
+    scaled = isinstance(x, ScaledInput)
     M, Kd = x.shape
     dtype = x.dtype
     rows, tiles = _rows_and_tiles(weight)
@@ -815,6 +901,10 @@ def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bo
         epi = 1 if (out.dtype == torch.float32 and dtype != torch.float32) else 0
     if pending is not None and not (residual and M <= SKINNY_BEST_ROWS):
         raise KernelError("pending addends go with the residual epilogue of at most 16 rows")
+    if leave is not None and not residual:
+        raise KernelError("only a product onto the residual stream leaves the next norm's input behind")
+    if scaled and (residual or tiles is None):
+        raise KernelError("a scaled input goes into a product with a re-tiled matrix that does not add into the stream")
     pend, n_pend = _check_addends(pending, M, N)
     per_group = _tiles_per_group(N // 2 if swiglu else N)
     if tiles is None and per_group == 4 and M <= 12:
@@ -835,11 +925,21 @@ def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bo
                                                   M, N, Kd, epi, per_group, dtype_code(dtype), _ptr(h_pend), h_n, _stream()),
                "skinny_gemm_normed")
         return out
+    xn = next_w = ss = None
+    parts, eps, left = 0, 0.0, None
+    if scaled:
+        x, ss, parts, eps = _scaled_args(x, M, Kd)
+    elif leave is not None:
+        _gpu(leave.weight, "next norm weight", torch.float32, (N,))
+        parts = _residual_parts(M, N)
+        xn = torch.empty(M, N, dtype=dtype, device=out.device)
+        ss = torch.empty(M, parts, dtype=torch.float32, device=out.device)
+        next_w, left = leave.weight, ScaledInput(xn, ss, leave)
     _gpu(x, "x")
     _check(skinny_lib().ni_skinny_gemm(_ptr(x), _ptr(rows if tiles is None else tiles), _ptr(out), M, N, Kd, epi,
                                        per_group, 0 if tiles is None else 1, dtype_code(dtype), _ptr(pend), n_pend,
-                                       _stream()), "skinny_gemm")
-    return out
+                                       _ptr(xn), _ptr(next_w), _ptr(ss), parts, ctypes.c_float(eps), _stream()), "skinny_gemm")
+    return left if left is not None else out
 
 
 def skinny_merge_ok(M: int, H: int, hd: int, nsplit: int, dtype: torch.dtype, weight) -> bool:
@@ -861,7 +961,7 @@ def skinny_merge_wins(M: int, H: int, hd: int, nsplit: int, dtype: torch.dtype, 
 
 
 def skinny_gemm_merged(workspace: torch.Tensor, nsplit: int, M: int, H: int, hd: int, weight, out: torch.Tensor,
-                       residual: bool = False, pending: Optional[torch.Tensor] = None) -> torch.Tensor:
+                       residual: bool = False, pending: Optional[torch.Tensor] = None, leave: Optional[NormSpec] = None):
     """``attn . weight^T`` where ``attn`` [M, H*hd] is still in the pieces that an attention kernel
     left in ``workspace`` for ``nsplit`` key runs (float32: outputs [M, H, nsplit, hd], then
     (maximum, sum) pairs [M, H, nsplit, 2]): the runs are merged in the product's prologue, with the
@@ -886,10 +986,21 @@ def skinny_gemm_merged(workspace: torch.Tensor, nsplit: int, M: int, H: int, hd:
     if pending is not None and not residual:
         raise KernelError("pending addends go with the residual epilogue")
     pend, n_pend = _check_addends(pending, M, N)
+    xn = next_w = ss = left = None
+    parts = 0
+    if leave is not None:
+        if not residual:
+            raise KernelError("only a product onto the residual stream leaves the next norm's input behind")
+        _gpu(leave.weight, "next norm weight", torch.float32, (N,))
+        parts = (N + 15) // 16
+        xn = torch.empty(M, N, dtype=dtype, device=out.device)
+        ss = torch.empty(M, parts, dtype=torch.float32, device=out.device)
+        next_w, left = leave.weight, ScaledInput(xn, ss, leave)
     _check(skinny_lib().ni_skinny_gemm_merged(_ptr(part_o), _ptr(part_ml), nsplit, H, hd, _ptr(tiles), _ptr(out), M, N,
-                                              3 if residual else 0, dtype_code(dtype), _ptr(pend), n_pend, _stream()),
+                                              3 if residual else 0, dtype_code(dtype), _ptr(pend), n_pend,
+                                              _ptr(xn), _ptr(next_w), _ptr(ss), parts, _stream()),
            "skinny_gemm_merged")
-    return out
+    return left if left is not None else out
 
 
 def qkv_rope_ok(M: int, K: int, hd: int, rotary_dim: int, dtype: torch.dtype) -> bool:
@@ -918,6 +1029,11 @@ def skinny_qkv_rope(x, w_qkv, positions: torch.Tensor, cos: torch.Tensor,
     M, Kd = x.shape
     dtype = x.dtype
     rows, tiles = _rows_and_tiles(w_qkv)
+    ss, parts, eps = None, 0, 0.0
+    if isinstance(x, ScaledInput):
+        if tiles is None:
+            raise KernelError("a scaled input goes into a product with a re-tiled matrix")
+        x, ss, parts, eps = _scaled_args(x, M, Kd)
     _gpu(rows, "w_qkv", dtype, ((H + 2 * KVH) * hd, Kd))
     if not (qkv_rope_ok(M, Kd, hd, 2 * cos.shape[1], dtype)):
         raise KernelError(f"skinny_qkv_rope does not take M={M}, K={Kd}, hd={hd}")
@@ -942,18 +1058,18 @@ def skinny_qkv_rope(x, w_qkv, positions: torch.Tensor, cos: torch.Tensor,
         device = x.h.device
     else:
         _gpu(x, "x")
-        x_ptr, h_ptr, nw_ptr, eps = _ptr(x), None, None, 0.0
+        x_ptr, h_ptr, nw_ptr = _ptr(x), None, None
         device = x.device
     q = torch.empty(M, H * hd, dtype=dtype, device=device)
     _check(skinny_lib().ni_skinny_qkv_rope(x_ptr, h_ptr, nw_ptr, ctypes.c_float(eps), _ptr(rows if tiles is None else tiles),
                                            _ptr(q), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping), _ptr(kpool),
                                            _ptr(vpool), M, Kd, H, KVH, hd, page_size, 0 if tiles is None else 1,
-                                           dtype_code(dtype), _ptr(pend), n_pend, _stream()), "skinny_qkv_rope")
+                                           dtype_code(dtype), _ptr(pend), n_pend, _ptr(ss), parts, _stream()), "skinny_qkv_rope")
     return q
 
 
 def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optional[torch.Tensor] = None,
-           pending: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
+           pending: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None, leave: Optional[NormSpec] = None):
     """``x . weight^T`` with ``weight`` stored [out, in].  Few rows go to the hand-written skinny
     product; many rows to the library (rocBLAS/hipBLASLt), where float32 inputs are multiplied in
     true float32 (the reduced-precision matrix modes of the library are switched off at import).
@@ -964,10 +1080,18 @@ def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optiona
     returned as float32 addends [S, M, N] that the next norm adds to the stream.  ``pending``: addends
     that ``residual`` has not received yet and that the product brings in with it (where
     :func:`residual_takes_addends` holds).  ``out``: where a plain product is to be written ([M, N] of the
-    output type) instead of a new tensor."""
+    output type) instead of a new tensor.  ``leave`` (with ``residual``, where :func:`leaves_scaled_ok`
+    holds; ignored elsewhere): the norm that stands behind the stream; the product then runs whole and
+    returns a :class:`ScaledInput` for that norm.  ``x`` may itself be a :class:`ScaledInput` where
+    :func:`takes_scaled_ok` holds."""
     rows, _ = _rows_and_tiles(weight)
-    if out is not None and (isinstance(x, NormedInput) or residual is not None):
+    if out is not None and (isinstance(x, (NormedInput, ScaledInput)) or residual is not None):
         raise KernelError("out= goes with a plain product")
+    if isinstance(x, ScaledInput):
+        if residual is not None or not takes_scaled_ok(x.shape[0], x.shape[1], x.dtype, weight):
+            raise KernelError("this product cannot take a scaled input")
+        y = torch.empty(x.shape[0], rows.shape[0], dtype=out_dtype or x.dtype, device=x.device)
+        return skinny_gemm(x, weight, y)
     if isinstance(x, NormedInput):
         if not (residual is None):
             raise KernelError("a normed input and a residual output in one product are not compiled")
@@ -982,6 +1106,10 @@ def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optiona
     if residual is not None:
         if not (residual_epilogue_ok(x.shape[0], x.shape[1], x.dtype, weight)):
             raise KernelError("the residual epilogue does not take this product")
+        if leave is not None and leaves_scaled_ok(x.shape[0], x.shape[1], x.dtype, weight):
+            if pending is not None and x.shape[0] > SKINNY_BEST_ROWS:
+                raise KernelError("this product cannot bring the residual stream's pending addends in")
+            return skinny_gemm(x, weight, residual, residual=True, pending=pending, leave=leave)
         if pending is not None and not residual_takes_addends(x.shape[0], x.shape[1], x.dtype, weight):
             raise KernelError("this product cannot bring the residual stream's pending addends in")
         shares, per = skinny_ksplit(x.shape[0], x.shape[1], x.dtype, weight)
@@ -1006,11 +1134,20 @@ def linear(x, weight, out_dtype: Optional[torch.dtype] = None, residual: Optiona
     return torch.mm(x, rows_t) if out is None else torch.mm(x, rows_t, out=out)
 
 
+def swiglu_takes_scaled(M: int, K: int, dtype: torch.dtype, weight_gate_up) -> bool:
+    """Whether :func:`linear_swiglu` can take a :class:`ScaledInput` of M rows: the fused skinny product on a
+    re-tiled stacked matrix whose halves start on tile boundaries."""
+    return takes_scaled_ok(M, K, dtype, weight_gate_up) and (weight_gate_up.shape[0] // 2) % 16 == 0
+
+
 def linear_swiglu(x, weight_gate_up) -> torch.Tensor:
     """``silu(x . Wg^T) * (x . Wu^T)`` for the stacked matrix [Wg; Wu]: fused into the product for
-    few rows, product then the SwiGLU kernel for many.  ``x`` may be a :class:`NormedInput`."""
+    few rows, product then the SwiGLU kernel for many.  ``x`` may be a :class:`NormedInput`, or a
+    :class:`ScaledInput` where :func:`swiglu_takes_scaled` holds."""
     inter = weight_gate_up.shape[0] // 2
     out = torch.empty(x.shape[0], inter, dtype=x.dtype, device=x.device)
+    if isinstance(x, ScaledInput) and not swiglu_takes_scaled(x.shape[0], x.shape[1], x.dtype, weight_gate_up):
+        raise KernelError("this product cannot take a scaled input")
     # (past 16 rows only a matrix whose halves start on tile boundaries is streamed re-tiled)
     if isinstance(x, NormedInput) or (skinny_wins(x.shape[0], x.shape[1], x.dtype, weight_gate_up)
                                       and (x.shape[0] <= SKINNY_BEST_ROWS or inter % 16 == 0)):

@@ -198,6 +198,8 @@ def pending_for(norm, pending: Optional[torch.Tensor], dtype: torch.dtype) -> Op
     """``pending`` as ``norm`` takes it.  A product of a few rows may hand its result on as float32
     addends [S, T, d] (its K range was cut into S shares); a norm that says ``takes_addends`` sums
     them itself, for any other they are summed here into one [T, d] of the compute type."""
+    if pending is not None and not isinstance(pending, torch.Tensor):
+        return None       # a norm's input left half done by the product before it: the stream itself is complete
     if pending is not None and pending.dim() == 3 and not getattr(norm, "takes_addends", False):
         return pending.sum(dim=0).to(dtype)
     return pending

@@ -81,11 +81,22 @@ class RMSNorm(Part):
         self.size = int(spec.params["size"])
         self.eps = float(spec.params["eps"])
         self.weight = rt.vector32(spec.weights["weight"], weights["weight"])
+        self._spec = None
 
     def forward(self, h: torch.Tensor, pending: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None):
+        if isinstance(pending, K.ScaledInput):
+            pending = None        # the stream is complete; what came with it was meant for a product, not for this kernel
         n = h.shape[0] if rows is None else rows.shape[0]
         out = torch.empty(n, self.size, dtype=self.rt.dtype, device=self.rt.device)
         return K.add_rmsnorm(h, pending, self.weight, self.eps, out, rows)
+
+    def as_deferred(self) -> "K.NormSpec":
+        """Weight and eps of this norm, for a product onto the residual stream that can leave ``h * weight``
+        and the rows' sums of squares behind (:class:`nanoinfer_amd.kernels.ScaledInput`): the product that
+        stands behind the norm then divides by the root mean squares in its epilogue."""
+        if self._spec is None:
+            self._spec = K.NormSpec(self.weight, self.eps)
+        return self._spec
 
     def as_prologue(self, h: torch.Tensor, pending: Optional[torch.Tensor] = None):
         """This norm of ``h`` as an input that a product can normalise itself; ``pending`` (float32
@@ -267,6 +278,19 @@ class Attention(Part):
                 and K.norm_prologue_ok(T, d, self.rt.dtype, self.w_qkv, addends)
                 and K.residual_takes_addends(T, self.H * self.hd, self.rt.dtype, self.w_o))
 
+    def takes_scaled(self, T: int) -> bool:
+        """Whether ``forward`` takes, for T tokens, the input that the product before the norm left half done
+        (a :class:`nanoinfer_amd.kernels.ScaledInput`): its first product divides by the rows' root mean squares."""
+        d = self.w_qkv.shape[1]
+        return (type(self).project is Attention.project and K.takes_scaled_ok(T, d, self.rt.dtype, self.w_qkv)
+                and (self._fused_projection(T, d, self.rt.dtype) or type(self).rotate_and_write is Attention.rotate_and_write))
+
+    def leaves_scaled(self, T: int) -> bool:
+        """Whether ``forward``, given ``residual=h`` and ``leave`` (the next norm's weight and eps), returns
+        that norm's input half done for T tokens."""
+        return (type(self).output is Attention.output and self.adds_residual(T)
+                and K.leaves_scaled_ok(T, self.H * self.hd, self.rt.dtype, self.w_o))
+
     def project(self, x, ctx) -> torch.Tensor:
         """Stage 1: ``x`` [T, d] -> [T, (H + 2 KVH) * hd], the query heads, then the key heads, then the
         value heads, as projected."""
@@ -328,27 +352,35 @@ class Attention(Part):
                self.H, self.KVH, self.hd, self.scale, self.window, nsplit, ws)
         return out
 
-    def output(self, attended, T: int, residual: Optional[torch.Tensor] = None, carried: Optional[torch.Tensor] = None):
+    def output(self, attended, T: int, residual: Optional[torch.Tensor] = None, carried: Optional[torch.Tensor] = None,
+               leave=None):
         """Stage 4: the o product of what :meth:`attend` returned.  With ``residual`` (the float32 stream) the
         product goes into it (None is returned) or comes back as float32 addends for the next norm; ``carried``
-        are addends that the stream has not received and that go in with it."""
+        are addends that the stream has not received and that go in with it; with ``leave`` (the next norm's
+        weight and eps, where :meth:`leaves_scaled` holds) that norm's input comes back half done."""
         if isinstance(attended, tuple):
             ws, nsplit = attended
             if residual is not None:
-                K.skinny_gemm_merged(ws, nsplit, T, self.H, self.hd, self.w_o, residual, residual=True, pending=carried)
-                return None
+                if leave is not None and not K.leaves_scaled_ok(T, self.H * self.hd, self.rt.dtype, self.w_o):
+                    leave = None
+                left = K.skinny_gemm_merged(ws, nsplit, T, self.H, self.hd, self.w_o, residual, residual=True,
+                                            pending=carried, leave=leave)
+                return left if isinstance(left, K.ScaledInput) else None
             y = torch.empty(T, self.w_o.rows.shape[0], dtype=self.rt.dtype, device=ws.device)
             return K.skinny_gemm_merged(ws, nsplit, T, self.H, self.hd, self.w_o, y)
-        return K.linear(attended, self.w_o, residual=residual, pending=carried)
+        return K.linear(attended, self.w_o, residual=residual, pending=carried, leave=leave)
 
-    def forward(self, x, ctx, cache: LayerCache, residual: Optional[torch.Tensor] = None):
+    def forward(self, x, ctx, cache: LayerCache, residual: Optional[torch.Tensor] = None, leave=None):
         T = x.shape[0]
         carried = getattr(x, "pending", None)       # addends of the residual stream that came with a normed input
         if carried is not None and residual is None:
             raise K.KernelError("pending addends of the residual stream need residual=h to go into")
         qkv = self.project_rotate_write(x, ctx, cache)
         leave_runs = type(self).output is Attention.output      # a replaced output stage gets the merged rows
-        return self.output(self.attend(qkv, ctx, cache, leave_runs=leave_runs), T, residual, carried)
+        attended = self.attend(qkv, ctx, cache, leave_runs=leave_runs)
+        if leave is not None:
+            return self.output(attended, T, residual, carried, leave)
+        return self.output(attended, T, residual, carried)
 
 
 # ------------------------------------------------------------------ feed-forward
@@ -388,11 +420,17 @@ class SwiGLU(Part):
                 and K.norm_prologue_ok(T, d, self.rt.dtype, self.w_gate_up, addends, swiglu=True)
                 and K.residual_takes_addends(T, self.intermediate_size, self.rt.dtype, self.w_down))
 
-    def forward(self, x, ctx, residual: Optional[torch.Tensor] = None):
+    def takes_scaled(self, T: int) -> bool:
+        return K.swiglu_takes_scaled(T, self.w_gate_up.shape[1], self.rt.dtype, self.w_gate_up)
+
+    def leaves_scaled(self, T: int) -> bool:
+        return self.adds_residual(T) and K.leaves_scaled_ok(T, self.intermediate_size, self.rt.dtype, self.w_down)
+
+    def forward(self, x, ctx, residual: Optional[torch.Tensor] = None, leave=None):
         carried = getattr(x, "pending", None)       # addends of the residual stream that came with a normed input
         if carried is not None and residual is None:
             raise K.KernelError("pending addends of the residual stream need residual=h to go into")
-        return K.linear(K.linear_swiglu(x, self.w_gate_up), self.w_down, residual=residual, pending=carried)
+        return K.linear(K.linear_swiglu(x, self.w_gate_up), self.w_down, residual=residual, pending=carried, leave=leave)
 
 
 # ------------------------------------------------------------------ block
@@ -420,6 +458,12 @@ class PreNormBlock(Block):
         output.  Float32 addends go along with the prologue where the part ``carries_addends``: its first product
         normalises ``h`` plus the addends, its last one adds them into ``h`` (it is then run with ``residual=h``)."""
         T = h.shape[0]
+        if isinstance(pending, K.ScaledInput):
+            # the stream is complete, and the product before left this norm's input half done
+            takes = getattr(part, "takes_scaled", None)
+            if takes is not None and takes(T) and pending.made_for(getattr(norm, "weight", None), getattr(norm, "eps", 0.0)):
+                return pending
+            pending = None
         takes = getattr(part, "takes_normed", None)
         prologue = getattr(norm, "as_prologue", None)
         if takes is not None and prologue is not None and takes(T):
@@ -431,18 +475,41 @@ class PreNormBlock(Block):
                 return prologue(h, pending)
         return norm.forward(h, pending_for(norm, pending, self.rt.dtype))
 
-    def forward(self, h, pending, ctx, cache: LayerCache):
+    @staticmethod
+    def _deferred(norm, producer, consumer, T: int):
+        """``norm``'s weight and eps if, for T tokens, ``producer`` (which adds into the stream) can leave the
+        norm's input half done and ``consumer`` can take it so; else None."""
+        spec = getattr(norm, "as_deferred", None)
+        leaves = getattr(producer, "leaves_scaled", None)
+        takes = getattr(consumer, "takes_scaled", None)
+        if spec is None or leaves is None or takes is None or not (leaves(T) and takes(T)):
+            return None
+        return spec()
+
+    leaves_for_next = True      # ``forward`` takes ``leave=``: what ``wants_scaled`` of the block behind this one returned
+
+    def wants_scaled(self, T: int):
+        """For the block that runs before this one: weight and eps of this block's first norm if its mixer can
+        take that norm's input half done for T tokens (see :meth:`_deferred`), else None."""
+        spec = getattr(self.mixer_norm, "as_deferred", None)
+        takes = getattr(self.mixer, "takes_scaled", None)
+        return spec() if spec is not None and takes is not None and takes(T) else None
+
+    def forward(self, h, pending, ctx, cache: LayerCache, leave=None):
         T = h.shape[0]
         x = self._normed_input(self.mixer_norm, self.mixer, h, pending)
         adds = getattr(self.mixer, "adds_residual", None)
         if adds is not None and adds(T):
-            a = self.mixer.forward(x, ctx, cache, residual=h)
+            spec = self._deferred(self.ffn_norm, self.mixer, self.ffn, T)
+            a = self.mixer.forward(x, ctx, cache, residual=h, **({} if spec is None else {"leave": spec}))
         else:
             a = self.mixer.forward(x, ctx, cache)
         x = self._normed_input(self.ffn_norm, self.ffn, h, a)
         adds = getattr(self.ffn, "adds_residual", None)
         if adds is not None and adds(T):
-            f = self.ffn.forward(x, ctx, residual=h)
+            leaves = getattr(self.ffn, "leaves_scaled", None)
+            spec = leave if (leave is not None and leaves is not None and leaves(T)) else None
+            f = self.ffn.forward(x, ctx, residual=h, **({} if spec is None else {"leave": spec}))
         else:
             f = self.ffn.forward(x, ctx)
         return h, f

@@ -834,6 +834,84 @@ def test_skinny_product_with_norm_prologue_and_residual_epilogue(K, dtype, M, N,
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("M,d,Ko,N2,S", [(1, 64, 32, 96, 0), (5, 192, 528, 1000, 2), (8, 2048, 2048, 256, 0), (16, 100 * 16, 48, 64, 1),
+                                         (3, 4096, 512, 128, 0), (24, 528, 64, 160, 0), (33, 2064, 192, 96, 0), (64, 2048, 2048, 512, 0),
+                                         (48, 272, 4096, 64, 0), (12, 3072, 256, 64, 2), (32, 2048, 2048, 512, 0),
+                                         (20, 3072, 3072, 256, 0), (8, 2048, 8192, 64, 0), (17, 272, 4112, 64, 0)])
+def test_a_norm_done_in_two_halves_by_the_products_around_it(K, dtype, M, d, Ko, N2, S):
+    """A product onto the residual stream leaves ``h * w`` and every workgroup's sums of squares of its columns
+    behind; the product after the norm takes them and divides by the rows' root mean squares in its epilogue
+    (store, float32 store, SwiGLU, rotation + cache write).  Against the plain steps in float64: stream, then
+    RMSNorm, rounded to the compute type, then the product.  With addends that the stream has not received (S),
+    widths that are no multiple of a tile or a piece, and one to four blocks of rows."""
+    g = torch.Generator().manual_seed(M * 131 + d + Ko)
+    dt = DT[dtype]
+    h = torch.randn(M + 1, d, generator=g) * 2
+    x = torch.randn(M, Ko, generator=g).to(dt)
+    wo = (torch.randn(d, Ko, generator=g) / math.sqrt(Ko)).to(dt)
+    nw = 1 + 0.1 * torch.randn(d, generator=g)
+    eps = 3e-6
+    pend = torch.randn(S, M, d, generator=g) if S else None
+    Wo = K.Weight(dev(wo))
+    # up to 16 rows a product that would not be cut along K anyway, up to 32 one with rows of up to 4,096 elements
+    assert K.leaves_scaled_ok(M, Ko, dt, Wo) == (K.skinny_ksplit(M, Ko, dt, Wo)[0] == 1 if M <= 16 else
+                                                 (M <= 32 and Ko <= 4096 and K.skinny_wins(M, Ko, dt, Wo)))
+    if dtype == "bfloat16":     # (in float32 the skinny kernels stream rows of up to 2,048 elements only, past 16 rows)
+        assert K.leaves_scaled_ok(M, Ko, dt, Wo) == ((M, Ko) not in ((33, 192), (64, 2048), (48, 4096), (8, 8192), (17, 4112)))
+    assert not K.leaves_scaled_ok(M, Ko, dt, dev(wo)), "only a re-tiled matrix"
+    if not K.leaves_scaled_ok(M, Ko, dt, Wo):
+        if K.residual_epilogue_ok(M, Ko, dt, Wo):       # the product goes its other way, whatever is asked for the norm
+            assert not isinstance(K.linear(dev(x), Wo, residual=dev(h.clone())[:M], leave=K.NormSpec(dev(nw), eps)),
+                                  K.ScaledInput)
+        return
+    stream = dev(h.clone())
+    spec = K.NormSpec(dev(nw), eps)
+    left = K.linear(dev(x), Wo, residual=stream[:M], pending=None if pend is None else dev(pend), leave=spec)
+    assert isinstance(left, K.ScaledInput) and left.made_for(spec.weight, eps) and not left.made_for(dev(nw), eps)
+    want_h = h[:M].double() + x.double() @ wo.double().t()
+    if pend is not None:
+        want_h = (h[:M].double() + pend.double().sum(0)) + x.double() @ wo.double().t()
+    assert rel(stream[:M], want_h) < 3e-6 and torch.equal(stream[M:].cpu(), h[M:]), "the stream itself, and no other row"
+    got_h = stream[:M].double().cpu()
+    assert rel(left.x, got_h * nw.double()) < KTOL[dtype], "h * w"
+    assert left.ss.shape[0] == M and rel(left.ss.double().sum(1), (got_h ** 2).sum(1)) < 3e-6, "sums of squares"
+    xn = P.rmsnorm(got_h, nw, eps).to(dt).double()
+    # the products behind the norm
+    w2 = (torch.randn(N2, d, generator=g) / math.sqrt(d)).to(dt)
+    W2 = K.Weight(dev(w2))
+    want = xn @ w2.double().t()
+    takes = K.takes_scaled_ok(M, d, dt, W2)
+    assert takes == K.skinny_wins(M, d, dt, W2)
+    if not takes:
+        with pytest.raises(K.KernelError):
+            K.linear(left, W2)
+        return
+    assert rel(K.linear(left, W2), want) < KTOL[dtype], "store"
+    assert rel(K.linear(left, W2, out_dtype=torch.float32), want) < KTOL[dtype], "float32 store"
+    if N2 % 32 == 0:
+        assert K.swiglu_takes_scaled(M, d, dt, W2)
+        assert rel(K.linear_swiglu(left, W2), P.swiglu(want[:, :N2 // 2], want[:, N2 // 2:])) < KTOL[dtype], "swiglu"
+    with pytest.raises(K.KernelError):
+        K.linear(left, dev(w2))                 # as stored: not taken
+    # rotation and cache write behind the norm: the same queries and pages as from the normalised rows
+    H, KVH, hd, ps = 2, 1, 32, 4
+    wq = (torch.randn((H + 2 * KVH) * hd, d, generator=g) / math.sqrt(d)).to(dt)
+    Wq = K.Weight(dev(wq))
+    if K.qkv_rope_ok(M, d, hd, hd, dt) and K.takes_scaled_ok(M, d, dt, Wq):
+        cos, sin = K.rope_table(dev(torch.rand(hd // 2, generator=g)), 128)
+        pos = dev(torch.arange(M, dtype=torch.int32) + 7)
+        slots = dev(torch.randperm(M + 3, generator=g)[:M].to(torch.int32))
+        pools = [[torch.zeros(-(-(M + 3) // ps), KVH, ps, hd, device="cuda", dtype=dt) for _ in range(2)] for _ in range(2)]
+        q_scaled = K.skinny_qkv_rope(left, Wq, pos, cos, sin, slots, pools[0][0], pools[0][1], H, KVH, hd)
+        q_plain = K.skinny_qkv_rope(dev(xn.to(dt)), Wq, pos, cos, sin, slots, pools[1][0], pools[1][1], H, KVH, hd)
+        scale = float(q_plain.double().abs().max())
+        assert float((q_scaled.double() - q_plain.double()).abs().max()) < KTOL[dtype] * scale
+        for a, b in zip(pools[0], pools[1]):
+            assert float((a.double() - b.double()).abs().max()) < KTOL[dtype] * max(scale, float(b.double().abs().max()))
+            assert float(b.double().abs().max()) > 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("M,N,Kd", [(17, 96, 2048), (33, 778, 528), (64, 2064, 192), (40, 50, 4096), (24, 64, 8192), (64, 2048, 8192),
                                     (20, 3000, 2048), (48, 272, 4112)])
 def test_skinny_product_of_17_to_64_rows_adds_into_the_residual_stream(K, dtype, M, N, Kd):
