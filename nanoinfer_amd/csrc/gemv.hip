@@ -319,7 +319,7 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
     constexpr int NOUT = (EPI == EPI_SWIGLU) ? NT / 2 : NT;      // output tiles of the workgroup
     const int out_n0 = wg * NOUT * 16;
     const int out_width = (EPI == EPI_SWIGLU) ? I : N;
-    if constexpr (EPI == EPI_RESIDUAL && HALVES == 1) {
+    if constexpr (EPI == EPI_RESIDUAL) {
         if (defer.xn != nullptr) {
             // The stream's new values, and with them what the next norm needs of them: h * w in the compute type, and
             // the sum of squares of each row over this workgroup's columns.  The items of a row are ROWW neighbouring
@@ -327,7 +327,8 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
             // goes through the same code (lanes without a row or a column add zero and store nothing).
             constexpr int ROWW = NT * 16;
             static_assert(ROWW <= WAVE && WAVE % ROWW == 0, "the items of a row lie within a wavefront");
-            const int parts = gridDim.x;
+            static_assert(HALVES == 1 || NT == 1, "halved tiles come one to a workgroup");
+            const int parts = gridDim.x;          // with HALVES == 2 every half of a tile is a part of its own
             for (int base = 0; base < MB * 16 * ROWW; base += WV * WAVE) {
                 const int item = base + tid;
                 if (item - lane >= MB * 16 * ROWW) break;           // the whole wavefront is past the items
@@ -335,7 +336,7 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
                 const int ot = n_in / 16, n_local = n_in % 16;
                 const int mb = m / 16, m_local = m % 16;
                 const int n = out_n0 + n_in;
-                const bool live = m < M && n < N;
+                const bool live = m < M && n < N && (HALVES == 1 || (n_local >> 3) == wg_half);
                 float sq = 0.f;
                 if (live) {
                     const int src = ((n_local / 4) * 16 + m_local) * 4 + (n_local % 4);
@@ -365,7 +366,8 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
                 }
 #pragma unroll
                 for (int off = ROWW / 2; off > 0; off >>= 1) sq += __shfl_xor(sq, off, WAVE);
-                if (n_in == 0 && m < M) defer.ss_out[static_cast<size_t>(m) * parts + wg] = sq;
+                if (n_in == (HALVES == 2 ? wg_half * 8 : 0) && m < M && n < N)
+                    defer.ss_out[static_cast<size_t>(m) * parts + blockIdx.x] = sq;
             }
             return;
         }
@@ -1021,6 +1023,7 @@ static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K,
 }
 
 #define HALVE_BELOW 160       // workgroups: a launch of no more than this many is doubled by halving the tiles
+#define HALVE_RESIDUAL_FROM 4096      // (the whole product onto the residual stream: from rows of this many elements)
 
 // The decode kernel: NT as launch_nt chooses it.  XP: pieces per wavefront of the normalising prologue, 0 without.
 template <typename T, typename TOUT, int EPI, int XP>
@@ -1051,9 +1054,13 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
         // rotation), which leaves a small model few workgroups (96 at the 1B shape): then two
         // workgroups share every pair of tiles.  (For one tile a workgroup, 128 workgroups against
         // 256, the same was measured and gained nothing: not compiled.)
-        constexpr bool CAN_HALVE = EPI == EPI_ROPE;
-        const bool halve = CAN_HALVE && grid <= HALVE_BELOW;
-        if (defer.xn != nullptr && defer.parts != grid) { defer_mismatch = true; return; }
+        // A whole product of long rows onto the residual stream (one that leaves the next norm's input behind, and
+        // so cannot be cut along K to fill the chip) is doubled the same way.
+        constexpr bool CAN_HALVE = EPI == EPI_ROPE || (EPI == EPI_RESIDUAL && NTc == 1 && XP == 0);
+        const bool halve = CAN_HALVE && grid <= HALVE_BELOW &&
+                           (EPI == EPI_ROPE || (K >= HALVE_RESIDUAL_FROM && splits == 1 && defer.xn != nullptr &&
+                                                2 * grid <= DEFER_PARTS_MAX));
+        if (defer.xn != nullptr && defer.parts != grid * (halve ? 2 : 1)) { defer_mismatch = true; return; }
         auto launch = [&](auto wv_tag, auto sr_tag, auto halves_tag) {
             constexpr int WVc = decltype(wv_tag)::value, SRc = decltype(sr_tag)::value, Hc = decltype(halves_tag)::value;
             if constexpr (XP > 0 && SRc > 0) {
@@ -1143,11 +1150,12 @@ static int launch_rows(const void* x, const void* W, void* y, int M, int N, int 
 
 // Workgroups of a product onto the residual stream of M rows and N columns, which is how many sums of squares
 // a row gets where the product leaves them behind for the next norm (DeferArgs): the launchers above, mirrored.
-static int residual_parts(int M, int N, int tiles_per_group) {
+static int residual_parts(int M, int N, int K, int tiles_per_group) {
     const int tiles = (N + 15) / 16;
     int nt = tiles_per_group >= 4 ? 4 : tiles_per_group >= 2 ? 2 : 1;
     if (M > 32 && nt == 4) nt = 2;       // three and four blocks of sixteen rows hold at most two tiles a workgroup
-    return (tiles + nt - 1) / nt;
+    const int grid = (tiles + nt - 1) / nt;
+    return (M <= 16 && nt == 1 && grid <= HALVE_BELOW && 2 * grid <= DEFER_PARTS_MAX && K >= HALVE_RESIDUAL_FROM) ? 2 * grid : grid;
 }
 
 template <typename T, typename TOUT, int EPI>
@@ -1203,12 +1211,12 @@ static int launch_normed(const NormArgs& norm, const void* W, void* y, int M, in
 // added before the product, y = ((y + pend[0]) + pend[1] ...) + x . W^T; null, 0: none.
 //
 // A norm in two halves (DeferArgs above; re-tiled W only).  Leaving: epilogue 3 with xn [M, N] of the input type,
-// next_w float32 [N] and ss float32 [M, parts], parts = ni_skinny_residual_parts(M, N, tiles_per_group): beside adding
+// next_w float32 [N] and ss float32 [M, parts], parts = ni_skinny_residual_parts(M, N, K, tiles_per_group): beside adding
 // into y the product stores xn = y * next_w and every workgroup's sums of squares of its columns of y.  Taking:
 // epilogues 0, 1, 2 with ss float32 [M, parts] of the product before, parts <= 256 and that norm's eps: x is the xn
 // that product left, and row m of the sums is multiplied by 1 / sqrt(sum_p ss[m, p] / K + eps) before the epilogue.
 // xn and ss null: neither.
-NI_EXPORT int ni_skinny_residual_parts(int M, int N, int tiles_per_group) { return residual_parts(M, N, tiles_per_group); }
+NI_EXPORT int ni_skinny_residual_parts(int M, int N, int K, int tiles_per_group) { return residual_parts(M, N, K, tiles_per_group); }
 
 NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N, int K, int epilogue, int tiles_per_group,
                              int tiled, int dtype, const void* pend, int n_pend, void* xn, const void* next_w, void* ss,
@@ -1228,7 +1236,7 @@ NI_EXPORT int ni_skinny_gemm(const void* x, const void* W, void* y, int M, int N
     if (xn != nullptr || ss != nullptr) {
         if (!tiled || !ss || parts < 1) return -11;
         if (epilogue == 3) {
-            if (!xn || !next_w || parts != residual_parts(M, N, tiles_per_group)) return -11;
+            if (!xn || !next_w || parts != residual_parts(M, N, K, tiles_per_group)) return -11;
             defer.xn = xn; defer.w = (const float*)next_w; defer.ss_out = (float*)ss;
         } else {
             if (xn != nullptr || parts > DEFER_PARTS_MAX || !(eps > 0.f)) return -11;

@@ -703,8 +703,8 @@ class ScaledInput:
 DEFER_PARTS_MAX = 256        # sums of squares a row may come in (the kernels' bound)
 
 
-def _residual_parts(M: int, N: int) -> int:
-    return int(skinny_lib().ni_skinny_residual_parts(int(M), int(N), _tiles_per_group(N)))
+def _residual_parts(M: int, N: int, K: int) -> int:
+    return int(skinny_lib().ni_skinny_residual_parts(int(M), int(N), int(K), _tiles_per_group(N)))
 
 
 def leaves_scaled_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
@@ -721,10 +721,19 @@ def leaves_scaled_ok(M: int, K: int, dtype: torch.dtype, weight) -> bool:
     kernel that adds them (1B at batch 24 / 32 1.263 : 1.251, 1.400 : 1.389); past 32 rows they do not."""
     if not (DEFER_NORMS and isinstance(weight, Weight) and weight.tiles is not None and skinny_ok(M, K, dtype)):
         return False
-    if _residual_parts(M, weight.rows.shape[0]) > DEFER_PARTS_MAX:
+    if _residual_parts(M, weight.rows.shape[0], K) > DEFER_PARTS_MAX:
         return False
     if M <= SKINNY_BEST_ROWS:
-        return skinny_ksplit(M, K, dtype, weight)[0] == 1
+        if skinny_ksplit(M, K, dtype, weight)[0] == 1:
+            return True
+        # A matrix of few tiles and long rows, which would be cut along K to fill the chip (the down product of the 1B
+        # shape): whole, it fills the chip by halved tiles instead (two workgroups a tile, each loading all of x),
+        # which costs more than the cut and, from five rows on in bfloat16, less than what the next product saves
+        # without a prologue that adds the shares or a norm kernel (a step of the 1B shape at batch 1 / 4 / 6 / 8 / 16,
+        # cut : whole, 0.747 : 0.772, 0.818 : 0.823, 0.871 : 0.857, 0.903 : 0.890, 1.118 : 1.095; in float32, whose
+        # matrices are twice the bytes, 1.364 : 1.504, 1.455 : 1.573, 1.613 : 1.717, 1.948 : 2.024)
+        N = weight.rows.shape[0]
+        return (dtype == torch.bfloat16 and M >= 5 and _tiles_per_group(N) == 1 and (N + 15) // 16 <= DEFER_PARTS_MAX // 2 and K >= 4096)
     return M <= 32 and K <= 4096 and skinny_wins(M, K, dtype, weight)
 
 
@@ -931,7 +940,7 @@ def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bo
         x, ss, parts, eps = _scaled_args(x, M, Kd)
     elif leave is not None:
         _gpu(leave.weight, "next norm weight", torch.float32, (N,))
-        parts = _residual_parts(M, N)
+        parts = _residual_parts(M, N, Kd)
         xn = torch.empty(M, N, dtype=dtype, device=out.device)
         ss = torch.empty(M, parts, dtype=torch.float32, device=out.device)
         next_w, left = leave.weight, ScaledInput(xn, ss, leave)

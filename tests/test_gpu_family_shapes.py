@@ -148,9 +148,11 @@ def test_decode_steps_whose_norms_are_done_in_two_halves(name, dtype, monkeypatc
                 got[(i, len(prompts[i]) - k)] = out[i].clone()
         if not graphs:
             # two layers: o and down of the first, o of the second leave; gate/up twice and the second q/k/v take
-            # (at the 1B sizes the down product is cut along K to fill the chip and leaves nothing)
-            n = 2 if name == "1B" else 3
+            # (at the 1B sizes in float32 the down product is cut along K to fill the chip and leaves nothing; in
+            # bfloat16 it runs whole on halved tiles from five rows on)
+            n = 2 if (name, dtype) == ("1B", "float32") else 3
             assert sorted(set(left)) == [1, 3, 8, 16] and left.count(8) == n and taken.count(8) == n, (left, taken)
+            assert left.count(3) == (2 if name == "1B" else 3)
             assert norms.count(8) <= 2, "the first layer's first norm at most, and the last norm on the wanted rows"
         rows = [(i, 5) for i in range(16, 24)] + [(i, 3) for i in range(8, 16)] + [(i, 2) for i in range(3, 8)]      # 21 rows
         out = runner.step([StepEntry(i, [prompts[i][-k]], [0]) for i, k in rows])
