@@ -366,7 +366,8 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
                 }
 #pragma unroll
                 for (int off = ROWW / 2; off > 0; off >>= 1) sq += __shfl_xor(sq, off, WAVE);
-                if (n_in == (HALVES == 2 ? wg_half * 8 : 0) && m < M && n < N)
+                // (a half tile that lies past the matrix's last column still writes its part: zero)
+                if (n_in == (HALVES == 2 ? wg_half * 8 : 0) && m < M)
                     defer.ss_out[static_cast<size_t>(m) * parts + blockIdx.x] = sq;
             }
             return;

@@ -838,7 +838,8 @@ def test_skinny_product_with_norm_prologue_and_residual_epilogue(K, dtype, M, N,
                                          (3, 4096, 512, 128, 0), (24, 528, 64, 160, 0), (33, 2064, 192, 96, 0), (64, 2048, 2048, 512, 0),
                                          (48, 272, 4096, 64, 0), (12, 3072, 256, 64, 2), (32, 2048, 2048, 512, 0),
                                          (20, 3072, 3072, 256, 0), (8, 2048, 8192, 64, 2), (17, 272, 4112, 64, 0),
-                                         (16, 528, 4096, 64, 0), (4, 2048, 8192, 64, 0), (13, 2560, 4112, 96, 1)])
+                                         (16, 528, 4096, 64, 0), (4, 2048, 8192, 64, 0), (13, 2560, 4112, 96, 1),
+                                         (9, 2040, 4096, 64, 0), (7, 24, 4096, 64, 1)])
 def test_a_norm_done_in_two_halves_by_the_products_around_it(K, dtype, M, d, Ko, N2, S):
     """A product onto the residual stream leaves ``h * w`` and every workgroup's sums of squares of its columns
     behind; the product after the norm takes them and divides by the rows' root mean squares in its epilogue
@@ -871,7 +872,11 @@ def test_a_norm_done_in_two_halves_by_the_products_around_it(K, dtype, M, d, Ko,
         return
     stream = dev(h.clone())
     spec = K.NormSpec(dev(nw), eps)
-    left = K.linear(dev(x), Wo, residual=stream[:M], pending=None if pend is None else dev(pend), leave=spec)
+    args = (dev(x), None if pend is None else dev(pend))
+    for size in (M * 64, M * 256, M * d):       # what the product allocates for itself starts out as NaN, not as zeros
+        del_me = torch.full((size,), float("nan"), device="cuda")
+        del del_me
+    left = K.linear(args[0], Wo, residual=stream[:M], pending=args[1], leave=spec)
     assert isinstance(left, K.ScaledInput) and left.made_for(spec.weight, eps) and not left.made_for(dev(nw), eps)
     want_h = h[:M].double() + x.double() @ wo.double().t()
     if pend is not None:
