@@ -703,6 +703,7 @@ class ScaledInput:
 DEFER_PARTS_MAX = 256        # sums of squares a row may come in (the kernels' bound)
 
 
+@functools.lru_cache(maxsize=None)
 def _residual_parts(M: int, N: int, K: int) -> int:
     return int(skinny_lib().ni_skinny_residual_parts(int(M), int(N), int(K), _tiles_per_group(N)))
 
