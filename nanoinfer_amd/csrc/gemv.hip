@@ -1023,7 +1023,13 @@ static int launch_nt(const void* x, const void* W, void* y, int M, int N, int K,
     return NI_LAUNCH_RESULT();
 }
 
-#define HALVE_BELOW 160       // workgroups: a launch of no more than this many is doubled by halving the tiles
+// Workgroups: a launch of no more than this many is doubled by halving the tiles.  A halved workgroup issues the loads of a
+// whole tile (the lanes of the other eight rows ask for the same bytes again, and a vector load costs the texture path the
+// same time whatever it fetches), so the doubled launch must still be one workgroup a compute unit: 160 pairs of tiles
+// as 320 halves put two on a quarter of the units and took 15.2 us where the 160 whole ones take 9 (the 3B shape's
+// [5120, 3072] with rotation at eight rows).
+#define HALVE_BELOW 128
+#define WIDE_BELOW 256        // workgroups: a product of one tile a workgroup and no more workgroups than this takes sixteen wavefronts
 #define HALVE_RESIDUAL_FROM 4096      // (the whole product onto the residual stream: from rows of this many elements)
 
 // The decode kernel: NT as launch_nt chooses it.  XP: pieces per wavefront of the normalising prologue, 0 without.
@@ -1086,7 +1092,7 @@ static int launch_decode(const void* x, const void* W, void* y, int M, int N, in
         };
         if constexpr (XP == 0 && NTc == 1) {
             // rows of 2,048 elements or more in few workgroups: sixteen wavefronts each
-            if (grid <= HALVE_BELOW && K >= 2048) {
+            if (grid <= WIDE_BELOW && K >= 2048) {
                 with_halves(std::integral_constant<int, 16>{}, std::integral_constant<int, 0>{});
                 return;
             }
