@@ -1195,7 +1195,10 @@ def test_skinny_product_reference_vector(K):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("M,H,KVH,hd,Kd,ps", [(1, 4, 2, 32, 64, 8), (8, 32, 8, 64, 2048, 16), (5, 6, 1, 32, 192, 8),
                                              (40, 3, 3, 128, 96, 4), (64, 8, 2, 96, 256, 16), (14, 32, 8, 64, 2048, 16),
-                                             (2, 24, 8, 128, 1024, 16), (16, 8, 8, 64, 2048, 16)])
+                                             (2, 24, 8, 128, 1024, 16), (16, 8, 8, 64, 2048, 16),
+                                             # pairs of tiles x blocks of 32 rows past 256 workgroups: three and four
+                                             # blocks of sixteen rows a workgroup instead; and just below: dealt out
+                                             (64, 24, 8, 128, 512, 16), (40, 32, 8, 128, 256, 16), (33, 40, 8, 64, 128, 8)])
 def test_product_with_rotation_and_cache_write(K, dtype, M, H, KVH, hd, Kd, ps):
     """The fused epilogue against the plain steps: product, rotation of pairs (j, j + hd/2), write by slot."""
     g = torch.Generator().manual_seed(M + hd)
