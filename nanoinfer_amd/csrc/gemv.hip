@@ -1176,6 +1176,11 @@ static int launch_mb(const void* x, const void* W, void* y, int M, int N, int K,
         // (dealt out only while that is still at most one workgroup a compute unit: the 160 pairs of tiles of the 3B
         // shape as 320 workgroups of 32 rows took 15.0 us at 64 rows, the 192 pairs of the 8B shape as 384 22.3 us)
         const bool dealt = EPI == EPI_ROPE && ((N + 31) / 32) * ((M + 31) / 32) <= 256;
+        if constexpr (EPI == EPI_ROPE) {
+            // up to 32 rows of a matrix of few pairs of tiles (96 at the 1B shape): 16 rows a workgroup
+            if (M <= 32 && ((N + 31) / 32) * ((M + 15) / 16) <= 256)
+                return launch_rows<T, TOUT, 1, EPI>(x, W, y, M, N, K, I, NT, stream, rope, 1, defer);
+        }
         if (M <= 32 || dealt) return launch_rows<T, TOUT, 2, EPI>(x, W, y, M, N, K, I, NT, stream, rope, 1, defer);
         if (M <= 48) return launch_rows<T, TOUT, 3, EPI>(x, W, y, M, N, K, I, NT, stream, rope, 1, defer);
         return launch_rows<T, TOUT, 4, EPI>(x, W, y, M, N, K, I, NT, stream, rope, 1, defer);

@@ -1198,7 +1198,9 @@ def test_skinny_product_reference_vector(K):
                                              (2, 24, 8, 128, 1024, 16), (16, 8, 8, 64, 2048, 16),
                                              # pairs of tiles x blocks of 32 rows past 256 workgroups: three and four
                                              # blocks of sixteen rows a workgroup instead; and just below: dealt out
-                                             (64, 24, 8, 128, 512, 16), (40, 32, 8, 128, 256, 16), (33, 40, 8, 64, 128, 8)])
+                                             (64, 24, 8, 128, 512, 16), (40, 32, 8, 128, 256, 16), (33, 40, 8, 64, 128, 8),
+                                             # 17 to 32 rows: sixteen a workgroup where that keeps within 256 workgroups
+                                             (24, 32, 8, 64, 2048, 16), (32, 6, 1, 32, 192, 8), (20, 24, 8, 128, 1024, 16)])
 def test_product_with_rotation_and_cache_write(K, dtype, M, H, KVH, hd, Kd, ps):
     """The fused epilogue against the plain steps: product, rotation of pairs (j, j + hd/2), write by slot."""
     g = torch.Generator().manual_seed(M + hd)
