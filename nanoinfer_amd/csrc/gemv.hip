@@ -293,9 +293,15 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
                     c = rope.cos_t[static_cast<size_t>(pos) * half + j];
                     sn = rope.sin_t[static_cast<size_t>(pos) * half + j];
                 }
-                const float y0 = x0 * c - x1 * sn;
-                const float y1 = x0 * sn + x1 * c;
-                x0 = y0; x1 = y1;
+                {
+                    // two products and their difference or sum, each rounded on its own: left to itself the compiler
+                    // fuses one product of each line into the addition in some instances of this function and the other
+                    // in others, and the same rows then turn out a last bit apart from kernel to kernel
+#pragma clang fp contract(off)
+                    const float y0 = x0 * c - x1 * sn;
+                    const float y1 = x0 * sn + x1 * c;
+                    x0 = y0; x1 = y1;
+                }
             }
             if (head < rope.H) {
                 TOUT* dst = y + static_cast<size_t>(m) * rope.H * rope.hd + static_cast<size_t>(head) * rope.hd;
