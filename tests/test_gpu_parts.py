@@ -86,7 +86,7 @@ def test_position_part_shares_one_table():
 # ------------------------------------------------------------------ a model from a spec written here
 
 def tiny_spec(mixer_kinds, order, d=64, H=4, KVH=2, hd=16, I=96, V=128, window=None, position="rope", state_size=None,
-              ffn_kinds=None, experts=3):
+              ffn_kinds=None, experts=3, norm_kinds=None):
     from nanoinfer_amd.config.spec import BlockSpec, LayerRun, ModelSpec, PartSpec
     if position == "rope":
         pos = PartSpec("rope", {"rotary_dim": hd, "theta": 10000.0, "scaling": None, "max_positions": 256})
@@ -109,10 +109,11 @@ def tiny_spec(mixer_kinds, order, d=64, H=4, KVH=2, hd=16, I=96, V=128, window=N
         else:
             ffn = PartSpec(ffn_kinds[i], {"hidden_size": d, "intermediate_size": I, "experts": experts},
                            {"router": pre + "router", "w1": pre + "w1", "w2": pre + "w2"})
-        blocks.append(BlockSpec("prenorm", {"mixer_norm": PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": pre + "n1"}),
-                                            "mixer": mixer,
-                                            "ffn_norm": PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": pre + "n2"}),
-                                            "ffn": ffn}))
+        def norm(name):
+            if norm_kinds is None or norm_kinds[i] == "rmsnorm":
+                return PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": pre + name})
+            return PartSpec(norm_kinds[i], {"size": d, "eps": 1e-5}, {"weight": pre + name, "bias": pre + name + "b"})
+        blocks.append(BlockSpec("prenorm", {"mixer_norm": norm("n1"), "mixer": mixer, "ffn_norm": norm("n2"), "ffn": ffn}))
     return ModelSpec(V, d, 256, PartSpec("table", {"vocab_size": V, "hidden_size": d}, {"weight": "emb"}), blocks,
                      [LayerRun(*o) for o in order], PartSpec("rmsnorm", {"size": d, "eps": 1e-5}, {"weight": "nf"}),
                      PartSpec("linear", {"vocab_size": V, "hidden_size": d}, {"weight": "emb"}))
@@ -133,15 +134,20 @@ def SpecRunner(spec, tensors, dtype, page_size=8, max_tokens=512, max_step_token
                                  max_step_tokens=max_step_tokens)
 
 
-def plain_spec_forward(spec, tensors, tokens, extra_mixers=None, extra_ffns=None, extra_positions=None):
+def plain_spec_forward(spec, tensors, tokens, extra_mixers=None, extra_ffns=None, extra_positions=None, extra_norms=None):
     """The plain implementation applied to a spec: same functions, parts chosen by the spec."""
     T = len(tokens)
     t64 = {k: v.double() for k, v in tensors.items()}
     h = P.embedding(t64[spec.embedding.weights["weight"]], tokens)
     kv = {}
+
+    def normed(part, h):
+        if part.kind == "rmsnorm":
+            return P.rmsnorm(h, t64[part.weights["weight"]], part.params["eps"])
+        return extra_norms[part.kind](h, t64, part)
     for run in spec.order:
         b = spec.blocks[run.block]
-        x = P.rmsnorm(h, t64[b.mixer_norm.weights["weight"]], b.mixer_norm.params["eps"])
+        x = normed(b.mixer_norm, h)
         m = b.mixer
         if m.kind == "attention":
             p = m.params
@@ -168,7 +174,7 @@ def plain_spec_forward(spec, tensors, tokens, extra_mixers=None, extra_ffns=None
         else:
             a = extra_mixers[m.kind](x, t64, m)
         h = h + a
-        x = P.rmsnorm(h, t64[b.ffn_norm.weights["weight"]], b.ffn_norm.params["eps"])
+        x = normed(b.ffn_norm, h)
         f = b.ffn
         if f.kind == "swiglu":
             h = h + P.linear(P.swiglu(P.linear(x, t64[f.weights["gate"]]), P.linear(x, t64[f.weights["up"]])), t64[f.weights["down"]])
@@ -430,6 +436,79 @@ def test_toy_feed_forward_with_routing_beside_a_dense_one():
         got = step_in_portions(runner, tokens, sizes)
         assert rel(got, want) < TOL["float32"], sizes
     assert len(set(choices.tolist())) >= 2                  # the tokens do go to different experts
+    runner.cache.check()
+
+
+# ------------------------------------------------------------------ a toy norm
+
+def register_toy_norm():
+    from nanoinfer_amd.parts.base import Part, WeightRequest
+    from nanoinfer_amd.registry import register_part
+
+    @register_part("norm", "toy_centered")
+    class ToyCenteredNorm(Part):
+        """``(x - mean(x)) / sqrt(var(x) + eps) * w + b`` in float32, by library tensor operations: a norm with the
+        family's interface and none of the optional abilities (no prologue, no addends, no half-done input): the
+        block sums what is pending for it and runs it as a step of its own."""
+
+        @classmethod
+        def weight_requests(cls, spec):
+            return [WeightRequest(spec.weights["weight"], (spec.params["size"],)),
+                    WeightRequest(spec.weights["bias"], (spec.params["size"],))]
+
+        def __init__(self, spec, weights, rt):
+            super().__init__(spec, weights, rt)
+            self.eps = float(spec.params["eps"])
+            self.weight = rt.vector32(spec.weights["weight"], weights["weight"])
+            self.bias = rt.vector32(spec.weights["bias"], weights["bias"])
+
+        def forward(self, h, pending, rows=None):
+            if rows is None and pending is not None:
+                h += pending.float()                     # the residual sum, in float32, in place
+            x = h if rows is None else h[rows.long()]
+            mean = x.mean(dim=-1, keepdim=True)
+            var = ((x - mean) ** 2).mean(dim=-1, keepdim=True)
+            return (((x - mean) / torch.sqrt(var + self.eps)) * self.weight + self.bias).to(self.rt.dtype)
+
+    return ToyCenteredNorm
+
+
+def plain_centered(h, t64, part):
+    mean = h.mean(dim=-1, keepdim=True)
+    var = ((h - mean) ** 2).mean(dim=-1, keepdim=True)
+    return (h - mean) / torch.sqrt(var + part.params["eps"]) * t64[part.weights["weight"]] + t64[part.weights["bias"]]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("kinds", [("toy_centered", "rmsnorm"), ("rmsnorm", "toy_centered"), ("rmsnorm", "toy_centered", "rmsnorm")])
+def test_toy_norm_beside_the_frameworks_own(kinds, dtype, monkeypatch):
+    """Layers whose norms are a toy norm defined here beside layers with the framework's RMSNorm, in both orders.
+    Around the framework's norm the products do the norm in two halves (the one before it leaves ``h * w`` and the
+    sums of squares, the one behind it divides), and where such a layer follows one with the toy norm the toy
+    layer's last product leaves them for it; around the toy norm, which offers nothing of the kind, the block adds
+    what is pending and runs the norm as a step of its own.  Portions, single tokens and steps of a few rows."""
+    from nanoinfer_amd import kernels
+    register_toy_norm()
+    n = len(kinds)
+    spec = tiny_spec(["attention"] * n, [(i, i) for i in range(n)], norm_kinds=list(kinds))
+    tensors = random_tensors(spec, 21)
+    tokens = list(random_tokens(128, 70, 6))
+    if dtype == "bfloat16":
+        tensors = {k: (v.to(torch.bfloat16).float() if v.dim() == 2 else v) for k, v in tensors.items()}
+    want = plain_spec_forward(spec, tensors, tokens, extra_norms={"toy_centered": plain_centered})
+    left = []
+    gemm = kernels.skinny_gemm
+    monkeypatch.setattr(kernels, "skinny_gemm", lambda x, w, out, *a, **kw: (
+        lambda r: (left.append(tuple(out.shape)) if isinstance(r, kernels.ScaledInput) else None, r)[1])(gemm(x, w, out, *a, **kw)))
+    runner = SpecRunner(spec, tensors, dtype)
+    for sizes in ([70], [9, 2, 1, 1, 17, 1, 5]):
+        got = step_in_portions(runner, tokens, sizes)
+        assert rel(got, want) < TOL[dtype], (kinds, sizes)
+    # per step of few rows: the product before every RMSNorm that stands inside the model left its input half done
+    # (the o product where the layer's norms are the framework's, the down product where the next layer's are)
+    inner = sum(k == "rmsnorm" for k in kinds) + sum(k == "rmsnorm" for k in kinds[1:])
+    assert len([shape for shape in left if shape[0] == 1]) % inner == 0 and any(shape[0] == 1 for shape in left)
+    assert not any(shape[0] == 70 for shape in left)
     runner.cache.check()
 
 
