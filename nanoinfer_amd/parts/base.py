@@ -148,7 +148,12 @@ class Block:
     answers for the whole block what each part answers for itself.  ``forward(h, pending, ctx,
     cache) -> (h, pending)`` is the subclass's: ``h`` is the float32 residual stream [T, d],
     ``pending`` an addend that the stream has not received yet (or None), which the next norm sums
-    in; the cache goes to the block's ``mixer``."""
+    in; the cache goes to the block's ``mixer``.  ``pending`` may also be something that is no tensor:
+    the next norm's input as the last product left it half done, beside a stream that is complete
+    (:class:`nanoinfer_amd.kernels.ScaledInput`); :func:`pending_for` turns that into None for a norm
+    that runs as a step of its own.  A block that sets ``leaves_for_next = True`` takes ``leave=`` in
+    its ``forward``: what ``wants_scaled(T)`` of the block that runs next returned, if that block has
+    such a method and returned anything."""
 
     family = "block"
     kind = ""
