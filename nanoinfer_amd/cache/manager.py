@@ -132,11 +132,12 @@ class KVCacheManager:
     (the most tokens one request brings to one step) is given, such a group's pool is only as
     large as ``max_requests`` requests can fill, and no larger than ``num_pages``; without it every
     group gets ``num_pages``.  ``device=None`` keeps the books without allocating pools.
+    ``scatter_pages`` hands page ids out in a fixed pseudo-random order (see :class:`BlockManager`).
     """
 
     def __init__(self, needs: Dict[int, CacheNeed], page_size: int, num_pages: int, max_requests: int,
                  dtype: torch.dtype = torch.float32, device: Optional[torch.device] = None,
-                 max_step_tokens: Optional[int] = None):
+                 max_step_tokens: Optional[int] = None, scatter_pages: bool = False):
         if page_size < 1:
             raise ValueError(f"page_size must be at least 1, got {page_size}")
         self.page_size = int(page_size)
@@ -156,7 +157,7 @@ class KVCacheManager:
                 if gi is None:
                     gi = len(self.groups)
                     by_need[need.kv] = gi
-                    self.groups.append(KVGroup(need.kv, [], self.page_size, BlockManager(self.pages_of_group(need.kv, max_requests))))
+                    self.groups.append(KVGroup(need.kv, [], self.page_size, BlockManager(self.pages_of_group(need.kv, max_requests), scatter=scatter_pages)))
                 self.groups[gi].cache_ids.append(cid)
                 self.group_of_cache[cid] = gi
             if need.state is not None:

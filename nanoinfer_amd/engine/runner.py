@@ -311,7 +311,8 @@ class ModelRunner:
         # large as their windows need; a longer portion is then refused
         self.max_step_tokens = None if max_step_tokens is None else int(max_step_tokens)
         self.cache = KVCacheManager(self.model.cache_needs(), self.page_size, num_pages, max_requests,
-                                    dtype=torch_dtype, device=self.device, max_step_tokens=self.max_step_tokens)
+                                    dtype=torch_dtype, device=self.device, max_step_tokens=self.max_step_tokens,
+                                    scatter_pages=True)   # requests of equal length would else hold runs at regular distances
         self.vocab_size = self.spec.vocab_size
         self.max_positions = self.model.max_positions
         self.eos_token_ids = tuple(self.spec.eos_token_ids)

@@ -45,6 +45,24 @@ def test_block_manager_all_or_nothing_and_double_free():
     assert bm.num_free == 3 and bm.allocate(1) == [0]
 
 
+def test_block_manager_scattered_ids():
+    """With ``scatter`` the ids come in a fixed pseudo-random order: every id once, the same order for the
+    same pool (also after a reset), not the ascending one, and a freed id is still the next one out."""
+    bm = BlockManager(64, scatter=True)
+    first = bm.allocate(64)
+    assert sorted(first) == list(range(64)) and first != list(range(64))
+    assert max(b - a for a, b in zip(first, first[1:])) > 1 and bm.num_free == 0
+    with pytest.raises(OutOfPages):
+        bm.allocate(1)
+    bm.free([first[5], first[9]])
+    assert bm.allocate(1) == [first[9]] and bm.is_taken(first[9]) and not bm.is_taken(first[5])
+    with pytest.raises(PageError):
+        bm.free([first[5]])
+    bm.reset()
+    assert bm.allocate(64) == first == BlockManager(64, scatter=True).allocate(64)
+    assert BlockManager(65, scatter=True).allocate(64) != first           # the order belongs to the pool's size
+
+
 # ------------------------------------------------------------------ reserve / release
 
 def test_pages_follow_tokens():
@@ -143,7 +161,7 @@ def test_random_orders_keep_the_books(seed):
     window = rng.choice([None, 6, 20])
     needs = {0: CacheNeed(kv=KVNeed(2, 16)), 1: CacheNeed(kv=KVNeed(2, 16, window=window))}
     ps = rng.choice([1, 4, 16])
-    m = KVCacheManager(needs, page_size=ps, num_pages=rng.randint(6, 20), max_requests=4)
+    m = KVCacheManager(needs, page_size=ps, num_pages=rng.randint(6, 20), max_requests=4, scatter_pages=seed % 2 == 1)
     live = {}
     next_id = 0
     for _ in range(600):
