@@ -179,6 +179,17 @@ struct DeferTake {
 // What an epilogue reads from memory, asked for while W is still streaming instead of at the end, where every
 // load is a round trip that nothing hides (the rotation's are two in a row: the position, then its angle).
 // For the first item of a thread (item == threadIdx.x), which with at most 16 rows and few tiles is its only one.
+// Four consecutive elements from floats in one access (p aligned to it), each rounded as st() rounds it.
+__device__ __forceinline__ void store_exact4(float* p, const float (&v)[4]) {
+    *reinterpret_cast<floatx4_t*>(p) = floatx4_t{v[0], v[1], v[2], v[3]};
+}
+__device__ __forceinline__ void store_exact4(bf16_t* p, const float (&v)[4]) {
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    *reinterpret_cast<u32x2_t*>(p) =
+        u32x2_t{static_cast<uint32_t>(f32_to_bf16_bits(v[0])) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16),
+                static_cast<uint32_t>(f32_to_bf16_bits(v[2])) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16)};
+}
+
 struct EpiEarly {
     bool have = false;       // the values below are those of item threadIdx.x
     int pos = 0, slot = -1;  // rotation: the row's position and cache slot
@@ -264,6 +275,120 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
     auto factor_of = [&](int m) { return scaled ? factors[m] : 1.0f; };
 
     // D[n_local][m_local] of a tile sits at lane = (n_local / 4) * 16 + m_local, register n_local % 4
+    constexpr bool DEFERS = EPI == EPI_RESIDUAL;       // (decided at run time: defer.xn)
+    if constexpr (MB >= 2) {
+        // Several blocks of rows: the sums are taken in the layout of the accumulators, a thread adding up the four
+        // registers of one lane of one tile over the wavefronts with 16-byte reads of neighbouring lanes (read item by
+        // item, sixteen lanes of a wavefront would meet in the same few banks, and with four blocks of rows the
+        // workgroup spent longer here than on a quarter of its matrix).  The four values are columns n0 .. n0 + 3 of row m;
+        // where two tiles belong together (gate and up, the two halves of a rotated head) the thread takes both.
+        static_assert(HALVES == 1, "halved tiles come with one block of rows");
+        if (!(DEFERS && defer.xn != nullptr)) {
+            constexpr bool PAIRS = EPI == EPI_ROPE || EPI == EPI_SWIGLU;
+            constexpr int OUT_T = PAIRS ? NT / 2 : NT;
+            for (int q = tid; q < OUT_T * MB * WAVE; q += WV * WAVE) {
+                const int ot = (q / WAVE) / MB, mb = (q / WAVE) % MB;
+                const int m = mb * 16 + lane % 16;
+                const int c0 = (lane / 16) * 4;                     // first of the lane's four columns within the tile
+                const int ta = (PAIRS ? 2 * ot : ot) * MB + mb;
+                floatx4_t a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int w = 0; w < WV; ++w) {
+                    a += *reinterpret_cast<const floatx4_t*>(&red[w][ta][lane * 4]);
+                    if constexpr (PAIRS) b += *reinterpret_cast<const floatx4_t*>(&red[w][ta + MB][lane * 4]);
+                }
+                if (m >= M) continue;
+                if (scaled) {
+                    const float f = factor_of(m);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { a[i] *= f; b[i] *= f; }
+                }
+                float v[4];
+                if constexpr (EPI == EPI_ROPE) {
+                    const int per_head = rope.hd / 32;
+                    const int head = wg / per_head;                 // among H query, KVH key, KVH value heads
+                    const int j = (wg % per_head) * 16 + c0;        // first of the lane's four pairs
+                    const int half = rope.hd / 2;
+                    float v1[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { v[i] = a[i]; v1[i] = b[i]; }
+                    if (head < rope.H + rope.KVH) {                 // queries and keys turn, values do not
+                        const int pos = rope.positions[m];
+                        const floatx4_t c = *reinterpret_cast<const floatx4_t*>(rope.cos_t + static_cast<size_t>(pos) * half + j);
+                        const floatx4_t sn = *reinterpret_cast<const floatx4_t*>(rope.sin_t + static_cast<size_t>(pos) * half + j);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            // (each product rounded on its own: see the single block of rows below)
+#pragma clang fp contract(off)
+                            v[i] = a[i] * c[i] - b[i] * sn[i];
+                            v1[i] = a[i] * sn[i] + b[i] * c[i];
+                        }
+                    }
+                    TOUT* dst = nullptr;
+                    if (head < rope.H) {
+                        dst = y + static_cast<size_t>(m) * rope.H * rope.hd + static_cast<size_t>(head) * rope.hd;
+                    } else if (rope.slot_mapping) {
+                        const int slot = rope.slot_mapping[m];
+                        if (slot >= 0) {
+                            const bool is_k = head < rope.H + rope.KVH;
+                            const int g = is_k ? head - rope.H : head - rope.H - rope.KVH;
+                            TOUT* pool = static_cast<TOUT*>(is_k ? rope.kpool : rope.vpool);
+                            dst = pool + ((static_cast<size_t>(slot / rope.page_size) * rope.KVH + g) * rope.page_size +
+                                          slot % rope.page_size) * rope.hd;
+                        }
+                    }
+                    if (dst != nullptr) {       // head sizes are multiples of 16 and j of 4: both runs are aligned
+                        store_exact4(dst + j, v);
+                        store_exact4(dst + j + half, v1);
+                    }
+                    continue;
+                }
+                const int out_n0 = wg * OUT_T * 16;
+                const int out_width = (EPI == EPI_SWIGLU) ? I : N;
+                const int n0 = out_n0 + ot * 16 + c0;
+                if (n0 >= out_width) continue;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if constexpr (EPI == EPI_SWIGLU) v[i] = a[i] / (1.0f + expf(-a[i])) * b[i];
+                    else v[i] = a[i];
+                }
+                TOUT* dst = y + static_cast<size_t>(m) * out_width + n0;
+                const bool whole = n0 + 3 < out_width && out_width % 4 == 0;      // four columns in one aligned access
+                if constexpr (EPI == EPI_RESIDUAL) {      // float32 residual stream, this workgroup's own columns
+                    float* hd = reinterpret_cast<float*>(dst);
+                    float sum[4];
+                    if (whole) {
+                        const floatx4_t h4 = *reinterpret_cast<const floatx4_t*>(hd);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) sum[i] = h4[i];
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) sum[i] = n0 + i < out_width ? hd[i] : 0.f;
+                    }
+                    // what the stream has not received yet, in its order, then the product
+                    for (int p = 0; p < n_pend; ++p) {
+                        const float* ad = pend + static_cast<size_t>(p) * M * N + static_cast<size_t>(m) * N + n0;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) if (n0 + i < out_width) sum[i] += ad[i];
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) sum[i] += v[i];
+                    if (whole) {
+                        *reinterpret_cast<floatx4_t*>(hd) = floatx4_t{sum[0], sum[1], sum[2], sum[3]};
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) if (n0 + i < out_width) hd[i] = sum[i];
+                    }
+                } else if (whole) {
+                    store_exact4(dst, v);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) if (n0 + i < out_width) st(dst + i, v[i]);
+                }
+            }
+            return;
+        }
+    }
     if constexpr (EPI == EPI_ROPE) {
         const int per_head = rope.hd / 32;
         const int head = wg / per_head;                 // among H query, KVH key, KVH value heads
