@@ -276,20 +276,23 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
 
     // D[n_local][m_local] of a tile sits at lane = (n_local / 4) * 16 + m_local, register n_local % 4
     constexpr bool DEFERS = EPI == EPI_RESIDUAL;       // (decided at run time: defer.xn)
-    if constexpr (MB >= 2) {
+    if constexpr (MB >= 2 && EPI != EPI_ROPE) {
         // Several blocks of rows: the sums are taken in the layout of the accumulators, a thread adding up the four
         // registers of one lane of one tile over the wavefronts with 16-byte reads of neighbouring lanes (read item by
         // item, sixteen lanes of a wavefront would meet in the same few banks, and with four blocks of rows the
         // workgroup spent longer here than on a quarter of its matrix).  The four values are columns n0 .. n0 + 3 of row m;
-        // where two tiles belong together (gate and up, the two halves of a rotated head) the thread takes both.
+        // a gate tile and its up tile are taken by the same thread.  (The rotation epilogue, 32 rows a workgroup, was
+        // no faster this way and keeps the items below.)
         static_assert(HALVES == 1, "halved tiles come with one block of rows");
         if (!(DEFERS && defer.xn != nullptr)) {
-            constexpr bool PAIRS = EPI == EPI_ROPE || EPI == EPI_SWIGLU;
+            constexpr bool PAIRS = EPI == EPI_SWIGLU;
             constexpr int OUT_T = PAIRS ? NT / 2 : NT;
+            const int out_n0 = wg * OUT_T * 16;
+            const int out_width = PAIRS ? I : N;
             for (int q = tid; q < OUT_T * MB * WAVE; q += WV * WAVE) {
                 const int ot = (q / WAVE) / MB, mb = (q / WAVE) % MB;
                 const int m = mb * 16 + lane % 16;
-                const int c0 = (lane / 16) * 4;                     // first of the lane's four columns within the tile
+                const int n0 = out_n0 + ot * 16 + (lane / 16) * 4;      // first of the lane's four columns
                 const int ta = (PAIRS ? 2 * ot : ot) * MB + mb;
                 floatx4_t a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -297,59 +300,16 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
                     a += *reinterpret_cast<const floatx4_t*>(&red[w][ta][lane * 4]);
                     if constexpr (PAIRS) b += *reinterpret_cast<const floatx4_t*>(&red[w][ta + MB][lane * 4]);
                 }
-                if (m >= M) continue;
+                if (m >= M || n0 >= out_width) continue;
                 if (scaled) {
                     const float f = factor_of(m);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) { a[i] *= f; b[i] *= f; }
                 }
                 float v[4];
-                if constexpr (EPI == EPI_ROPE) {
-                    const int per_head = rope.hd / 32;
-                    const int head = wg / per_head;                 // among H query, KVH key, KVH value heads
-                    const int j = (wg % per_head) * 16 + c0;        // first of the lane's four pairs
-                    const int half = rope.hd / 2;
-                    float v1[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) { v[i] = a[i]; v1[i] = b[i]; }
-                    if (head < rope.H + rope.KVH) {                 // queries and keys turn, values do not
-                        const int pos = rope.positions[m];
-                        const floatx4_t c = *reinterpret_cast<const floatx4_t*>(rope.cos_t + static_cast<size_t>(pos) * half + j);
-                        const floatx4_t sn = *reinterpret_cast<const floatx4_t*>(rope.sin_t + static_cast<size_t>(pos) * half + j);
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            // (each product rounded on its own: see the single block of rows below)
-#pragma clang fp contract(off)
-                            v[i] = a[i] * c[i] - b[i] * sn[i];
-                            v1[i] = a[i] * sn[i] + b[i] * c[i];
-                        }
-                    }
-                    TOUT* dst = nullptr;
-                    if (head < rope.H) {
-                        dst = y + static_cast<size_t>(m) * rope.H * rope.hd + static_cast<size_t>(head) * rope.hd;
-                    } else if (rope.slot_mapping) {
-                        const int slot = rope.slot_mapping[m];
-                        if (slot >= 0) {
-                            const bool is_k = head < rope.H + rope.KVH;
-                            const int g = is_k ? head - rope.H : head - rope.H - rope.KVH;
-                            TOUT* pool = static_cast<TOUT*>(is_k ? rope.kpool : rope.vpool);
-                            dst = pool + ((static_cast<size_t>(slot / rope.page_size) * rope.KVH + g) * rope.page_size +
-                                          slot % rope.page_size) * rope.hd;
-                        }
-                    }
-                    if (dst != nullptr) {       // head sizes are multiples of 16 and j of 4: both runs are aligned
-                        store_exact4(dst + j, v);
-                        store_exact4(dst + j + half, v1);
-                    }
-                    continue;
-                }
-                const int out_n0 = wg * OUT_T * 16;
-                const int out_width = (EPI == EPI_SWIGLU) ? I : N;
-                const int n0 = out_n0 + ot * 16 + c0;
-                if (n0 >= out_width) continue;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    if constexpr (EPI == EPI_SWIGLU) v[i] = a[i] / (1.0f + expf(-a[i])) * b[i];
+                    if constexpr (PAIRS) v[i] = a[i] / (1.0f + expf(-a[i])) * b[i];
                     else v[i] = a[i];
                 }
                 TOUT* dst = y + static_cast<size_t>(m) * out_width + n0;
