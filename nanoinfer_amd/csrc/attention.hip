@@ -270,43 +270,6 @@ __global__ void merge_splits_kernel(const float* __restrict__ part_o, const floa
     constexpr bool FAST = sizeof(T) == 2;
     const int t = blockIdx.x, h = blockIdx.y;
     const size_t p0 = (static_cast<size_t>(t) * H + h) * nsplit;
-    constexpr int FEW = 8;
-    if (nsplit <= FEW && HEAD_DIM <= 4 * 64) {
-        // few runs: everything the thread will read is asked for at once, the outputs of the runs beside their
-        // (maximum, sum) pairs, instead of one round trip for the maxima and another for the rest; the arithmetic
-        // and its order are those of the loops below
-        constexpr int DIMS = (HEAD_DIM + 63) / 64;
-        float2 ml[FEW];
-        float o[DIMS][FEW];
-#pragma unroll
-        for (int s = 0; s < FEW; ++s) {
-            const int sc = min(s, nsplit - 1);
-            ml[s] = *reinterpret_cast<const float2*>(part_ml + (p0 + sc) * 2);
-#pragma unroll
-            for (int d = 0; d < DIMS; ++d) {
-                const int dim = min(static_cast<int>(threadIdx.x) + d * 64, HEAD_DIM - 1);
-                o[d][s] = part_o[(p0 + sc) * HEAD_DIM + dim];
-            }
-        }
-        float M = NEG_BIG;
-#pragma unroll
-        for (int s = 0; s < FEW; ++s) if (s < nsplit) M = fmaxf(M, ml[s].x);
-#pragma unroll
-        for (int d = 0; d < DIMS; ++d) {
-            const int dim = static_cast<int>(threadIdx.x) + d * 64;
-            float Lsum = 0.f, O = 0.f;
-#pragma unroll
-            for (int s = 0; s < FEW; ++s) {
-                if (s < nsplit) {
-                    const float f = ex<FAST>(ml[s].x - M);
-                    Lsum += ml[s].y * f;
-                    O += o[d][s] * f;
-                }
-            }
-            if (dim < HEAD_DIM) st(out + static_cast<size_t>(t) * H * HEAD_DIM + static_cast<size_t>(h) * HEAD_DIM + dim, O / Lsum);
-        }
-        return;
-    }
     float M = NEG_BIG;
     for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[(p0 + s) * 2]);
     for (int dim = threadIdx.x; dim < HEAD_DIM; dim += blockDim.x) {
