@@ -9,7 +9,7 @@ argmax kernels pick the next ones, and they come back to the host, as in greedy 
 is decoded tokens per second.  The same line carries the prefill of one 2,048-token prompt in
 portions of 512 (``prefill``; ``--prefill-chunk`` changes the cut), in one portion, the engine's
 default (``prefill_one_portion``, and ``prefill_one_portion_eager`` with every kernel launched from
-the host instead of a recorded step), the decode step's fraction of the HBM roofline, and in
+the host instead of a recorded step; a longer ``--prompt-len`` goes in portions of 2,048 there), the decode step's fraction of the HBM roofline, and in
 ``points`` decode at batch 1 and 64 (``rooflines`` holds the roofline fraction of every point by
 its name).  The default line (1B shape, bfloat16) adds further points, each timed over 96 steps:
 decode at batch 8 and 64 from contexts of 8,192 and 32,768 tokens; prompts of 8,192 and 32,768
@@ -472,10 +472,11 @@ def main() -> int:
     log("prefill ...")
     prefill_s = rig.prefill(PROMPT_LEN, args.prefill_chunk)
     log(f"prefill of {PROMPT_LEN} in portions of {args.prefill_chunk}: {prefill_s * 1e3:.2f} ms")
+    how = "in one portion" if PROMPT_LEN <= ENGINE_CHUNK else f"in portions of {ENGINE_CHUNK}"      # the engine's default cut
     whole_s = rig.prefill(PROMPT_LEN, ENGINE_CHUNK)
-    log(f"prefill of {PROMPT_LEN} in one portion: {whole_s * 1e3:.2f} ms")
+    log(f"prefill of {PROMPT_LEN} {how}: {whole_s * 1e3:.2f} ms")
     eager_s = rig.prefill(PROMPT_LEN, ENGINE_CHUNK, recorded=False)
-    log(f"prefill of {PROMPT_LEN} in one portion, launched kernel by kernel: {eager_s * 1e3:.2f} ms")
+    log(f"prefill of {PROMPT_LEN} {how}, launched kernel by kernel: {eager_s * 1e3:.2f} ms")
     step_s, mean_ctx = rig.decode(args.batch, PROMPT_LEN, args.steps, args.warmup)
     log(f"decode batch {args.batch}: {step_s * 1e3:.3f} ms a step")
     points = {}
