@@ -211,7 +211,7 @@ class Scheduler:
         # 1. running requests, decode tokens before prompt portions, each group in admission order
         order = [r for r in self.running if r.remaining == 1] + [r for r in self.running if r.remaining > 1]
         for req in order:
-            if req not in self.running:      # preempted while making room for an earlier one
+            if req.state is not RequestState.RUNNING:      # preempted while making room for an earlier one
                 continue
             if len(batch.items) >= cfg.max_batch_size or budget <= 0:
                 break
