@@ -922,9 +922,11 @@ def skinny_gemm(x, weight, out: torch.Tensor, swiglu: bool = False, residual: bo
         # workgroup (measured at [128256, 2048], us for 1 / 2 / 4 tiles: one row 83.9 / 87.4 / 90.3, four rows
         # 86.0 / 87.3 / 94.3, eight rows 97.9 / 90.5 / 94.1, twelve 109.9 / 98.8 / 100.0, sixteen 118.6 / 103.2 / 100.5)
         per_group = 1 if M <= 4 else 2
-    if swiglu and M > 32 and tiles is not None:
-        # past 32 rows a workgroup that multiplies two pairs of gate and up tiles halves the loads of x,
-        # which every workgroup brings in whole (measured at [16384, 2048]: 64 rows 22.0 -> 20.9 us, 17 and 32 rows lose)
+    if swiglu and M > SKINNY_BEST_ROWS and tiles is not None:
+        # past 16 rows a workgroup that multiplies two pairs of gate and up tiles halves the loads of x, which
+        # every workgroup brings in whole (measured, one pair : two pairs in us, at [16384, 2048]: 17 rows 15.9 : 15.9,
+        # 32 rows 16.6 : 16.2, 64 rows 21.3 : 18.9; at [16384, 3072]: 17 rows 22.1 : 21.4, 32 rows 23.4 : 21.1, 64 rows
+        # 29.6 : 24.5; at [28672, 4096]: 17 rows 49.1 : 48.2, 32 rows 54.6 : 48.4, 64 rows 67.4 : 54.4)
         per_group = max(per_group, 4)
     if normed:
         h_pend, h_n = _check_addends(x.pending, M, Kd)
