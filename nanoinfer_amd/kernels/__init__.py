@@ -823,7 +823,11 @@ def skinny_ksplit(M: int, K: int, dtype: torch.dtype, weight):
         # float32 past 16 rows: only matrices of at most 128 tiles gain by the cut; the library's product is faster on the
         # others ([3072, 8192] at 64 rows in two shares 54.6 us against 45.2, [4096, 4096] 33.5 : 26.8, [4096, 14336] 93.8 : 86.2)
         return 1, 1
-    per = 2 if (M > 32 and K >= 4096) else 1
+    # two tiles a workgroup (half the workgroups' loads of x, twice the shares) past 32 rows of 4,096 elements or more,
+    # and in bfloat16 from 17 rows of 3,072 or more (product and the norm kernel behind it in us at 17 / 32 rows, whole or
+    # one tile a workgroup : two, [3072, 8192] 22.2 : 19.1 / 21.3 : 19.1, [4096, 14336] 32.0 : 28.1 / 33.4 : 28.6, [2048, 8192]
+    # 12.9 : 12.5 / 13.4 : 12.9; [3072, 3072] at 48 / 64 rows 11.4 : 10.7 / 12.7 : 11.4)
+    per = 2 if (M > 32 and K >= 4096) or (dtype == torch.bfloat16 and M > SKINNY_BEST_ROWS and K >= 3072) else 1
     groups = -(-((N + 15) // 16) // per)
     pieces = (K + 63) // 64
     # as many shares as keep the workgroups within one to a compute unit (192 groups in two shares are one and a

@@ -943,10 +943,10 @@ def test_skinny_product_of_17_to_64_rows_adds_into_the_residual_stream(K, dtype,
     assert ok == (K.skinny_wins(M, Kd, DT[dtype], W) or K.skinny_ksplit(M, Kd, DT[dtype], W)[0] > 1)
     assert ok
     got = K.linear(dev(x), W, residual=buf[:M])
-    shares = K.skinny_ksplit(M, Kd, DT[dtype], W)[0]
-    groups = -(-((N + 15) // 16) // (2 if M > 32 and Kd >= 4096 else 1))
-    assert shares == (max(1, min(256 // groups, Kd // 64 // 16, 16)) if Kd >= 2048 else 1), \
-        "rows of 2,048 elements or more are cut, towards 256 workgroups"
+    shares, per = K.skinny_ksplit(M, Kd, DT[dtype], W)
+    groups = -(-((N + 15) // 16) // per)
+    assert 1 <= shares <= 16 and (shares == 1 or (shares * groups <= 256 and Kd // 64 // shares >= 16)), \
+        "a cut leaves no more than a workgroup for every compute unit and at least sixteen pieces a share"
     if shares > 1:
         # the K range was cut: float32 addends for the next norm, the stream itself untouched
         assert got.dtype == torch.float32 and tuple(got.shape) == (shares, M, N)
