@@ -128,10 +128,11 @@ struct RopeArgs {
 // A norm done in two halves by the products on either side of it.  RMSNorm(h) . W^T = ((h * w) . W^T) / rms(h) row by
 // row, so the product that completes the residual stream (residual epilogue, `xn` set) also stores
 // xn[m, n] = h[m, n] * w[n] in the compute type and the sum of h[m, n]^2 over its own columns, ss_out[m * parts + wg]
-// (parts = its workgroups); and the product behind the norm (`ss_in` set) takes xn for its x and multiplies its sums
+// (parts = its workgroups; past sixteen rows ss_out[m * parts + tile], parts = the tiles of all workgroups: there a
+// tile's sums are one wavefront's, and need not meet another's); and the product behind the norm (`ss_in` set) takes xn for its x and multiplies its sums
 // by 1 / sqrt(sum over the parts / width + eps) in its epilogue.  No kernel normalises and none reads h for it.
 // The sums of squares are float32 of the float32 stream, added in a fixed order.
-#define DEFER_PARTS_MAX 256       // workgroups whose sums of squares the product behind the norm adds up for a row
+#define DEFER_PARTS_MAX 256       // sums of squares that the product behind the norm adds up for a row
 struct DeferArgs {
     void* xn = nullptr;            // [M, N] compute type: the stream times the next norm's weight
     const float* w = nullptr;      // [N] that weight
@@ -284,6 +285,67 @@ __device__ __forceinline__ void skinny_finish(const floatx4_t (&acc)[NT][MB], TO
         // a gate tile and its up tile are taken by the same thread.  (The rotation epilogue, 32 rows a workgroup, was
         // no faster this way and keeps the items below.)
         static_assert(HALVES == 1, "halved tiles come with one block of rows");
+        if constexpr (DEFERS) {
+            if (defer.xn != nullptr) {
+                // The stream's new values and what the next norm needs of them (see DeferArgs): h * w in the compute
+                // type, and of every tile its own sum of squares of each row, so that no wavefront has to meet another:
+                // ss_out[m * parts + tile], parts = the tiles of all workgroups.  A row's sixteen columns of a tile are
+                // the four values of the four lanes m % 16, + 16, + 32, + 48; every lane of a wavefront goes through the
+                // same code (a lane without a row or a column adds zero and stores nothing).
+                const int parts = static_cast<int>(gridDim.x) * NT;
+                for (int q = tid; q < NT * MB * WAVE; q += WV * WAVE) {
+                    const int ot = (q / WAVE) / MB, mb = (q / WAVE) % MB;
+                    const int m = mb * 16 + lane % 16;
+                    const int n0 = (wg * NT + ot) * 16 + (lane / 16) * 4;
+                    floatx4_t a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int w = 0; w < WV; ++w) a += *reinterpret_cast<const floatx4_t*>(&red[w][ot * MB + mb][lane * 4]);
+                    float sq = 0.f;
+                    if (m < M && n0 < N) {
+                        float* hd = reinterpret_cast<float*>(y) + static_cast<size_t>(m) * N + n0;
+                        T* xd = static_cast<T*>(defer.xn) + static_cast<size_t>(m) * N + n0;
+                        const bool whole = n0 + 3 < N && N % 4 == 0;      // four columns in one aligned access
+                        float sum[4], wn[4];
+                        if (whole) {
+                            const floatx4_t h4 = *reinterpret_cast<const floatx4_t*>(hd);
+                            const floatx4_t w4 = *reinterpret_cast<const floatx4_t*>(defer.w + n0);
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) { sum[i] = h4[i]; wn[i] = w4[i]; }
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) {
+                                sum[i] = n0 + i < N ? hd[i] : 0.f;
+                                wn[i] = n0 + i < N ? defer.w[n0 + i] : 0.f;
+                            }
+                        }
+                        for (int p = 0; p < n_pend; ++p) {       // what the stream has not received yet, in its order
+                            const float* ad = pend + static_cast<size_t>(p) * M * N + static_cast<size_t>(m) * N + n0;
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) if (n0 + i < N) sum[i] += ad[i];
+                        }
+                        float xv[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            sum[i] += a[i];
+                            xv[i] = sum[i] * wn[i];
+                            if (n0 + i < N) sq += sum[i] * sum[i];
+                        }
+                        if (whole) {
+                            *reinterpret_cast<floatx4_t*>(hd) = floatx4_t{sum[0], sum[1], sum[2], sum[3]};
+                            store_exact4(xd, xv);
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) if (n0 + i < N) { hd[i] = sum[i]; st(xd + i, xv[i]); }
+                        }
+                    }
+                    sq += __shfl_xor(sq, 16, WAVE);
+                    sq += __shfl_xor(sq, 32, WAVE);
+                    // (a tile that lies past the matrix's last column still writes its part: zero)
+                    if (lane < 16 && m < M) defer.ss_out[static_cast<size_t>(m) * parts + wg * NT + ot] = sq;
+                }
+                return;
+            }
+        }
         if (!(DEFERS && defer.xn != nullptr)) {
             constexpr bool PAIRS = EPI == EPI_SWIGLU;
             constexpr int OUT_T = PAIRS ? NT / 2 : NT;
@@ -1222,7 +1284,8 @@ static int launch_rows(const void* x, const void* W, void* y, int M, int N, int 
         constexpr int NTc = decltype(nt_tag)::value;
         constexpr int NOUT = (EPI == EPI_SWIGLU) ? NTc / 2 : NTc;
         const int grid = (tiles + NOUT - 1) / NOUT;
-        if (defer.xn != nullptr && defer.parts != grid) { defer_mismatch = true; return; }
+        // (several blocks of rows leave a sum of squares for every tile, not for every workgroup)
+        if (defer.xn != nullptr && defer.parts != (MB >= 2 ? grid * NTc : grid)) { defer_mismatch = true; return; }
         skinny_rows_kernel<T, TOUT, MB, NTc, EPI><<<dim3(grid, splits, (M + MB * 16 - 1) / (MB * 16)), GV_THREADS, 0, stream>>>(
             (const T*)x, (const T*)W, (TOUT*)y, M, N, K, I, rope, splits, defer);
     };
@@ -1253,7 +1316,8 @@ static int residual_parts(int M, int N, int K, int tiles_per_group) {
     int nt = tiles_per_group >= 4 ? 4 : tiles_per_group >= 2 ? 2 : 1;
     if (M > 32 && nt == 4) nt = 2;       // three and four blocks of sixteen rows hold at most two tiles a workgroup
     const int grid = (tiles + nt - 1) / nt;
-    return (M <= 16 && nt == 1 && grid <= HALVE_BELOW && 2 * grid <= DEFER_PARTS_MAX && K >= HALVE_RESIDUAL_FROM) ? 2 * grid : grid;
+    if (M > 16) return grid * nt;        // past sixteen rows every tile leaves its own sums
+    return (nt == 1 && grid <= HALVE_BELOW && 2 * grid <= DEFER_PARTS_MAX && K >= HALVE_RESIDUAL_FROM) ? 2 * grid : grid;
 }
 
 template <typename T, typename TOUT, int EPI>
