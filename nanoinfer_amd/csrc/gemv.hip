@@ -129,8 +129,8 @@ struct RopeArgs {
 // row, so the product that completes the residual stream (residual epilogue, `xn` set) also stores
 // xn[m, n] = h[m, n] * w[n] in the compute type and the sum of h[m, n]^2 over its own columns, ss_out[m * parts + wg]
 // (parts = its workgroups; past sixteen rows ss_out[m * parts + tile], parts = the tiles of all workgroups: there a
-// tile's sums are one wavefront's, and need not meet another's); and the product behind the norm (`ss_in` set) takes xn for its x and multiplies its sums
-// by 1 / sqrt(sum over the parts / width + eps) in its epilogue.  No kernel normalises and none reads h for it.
+// tile's sums are one wavefront's, and need not meet another's); and the product behind the norm (`ss_in` set) takes
+// xn for its x and multiplies its sums by 1 / sqrt(sum over the parts / width + eps) in its epilogue.  No kernel normalises and none reads h for it.
 // The sums of squares are float32 of the float32 stream, added in a fixed order.
 #define DEFER_PARTS_MAX 256       // sums of squares that the product behind the norm adds up for a row
 struct DeferArgs {
